@@ -1,0 +1,109 @@
+/*
+ * Internal declarations shared by the HIP sources of libkmx_hip.so (not part of the C ABI).
+ */
+#ifndef KMX_INTERNAL_H
+#define KMX_INTERNAL_H
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+#include <cstdio>
+
+#include "kmx.h"
+
+namespace kmx {
+
+constexpr int WAVE = 64; /* gfx950 wavefront width */
+
+/* Records the message returned by kmx_last_error() and passes `code` through. */
+int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+void clear_error();
+
+/* The stream every kernel of the library is launched on. */
+hipStream_t stream();
+
+/* Properties of the current device, queried once. */
+struct DeviceInfo {
+	int device = -1;
+	uint32_t compute_units = 0;
+	uint32_t lds_bytes = 0;      /* LDS available to one work-group */
+	uint32_t max_threads = 0;
+};
+int device_info(const DeviceInfo** out);
+
+/*
+ * Work space owned by the library (grown on demand, released by kmx_shutdown):
+ *   recheck queue : indices of the points the fast assignment kernels hand to the exact pass
+ *   counters      : [0] = queue length of the current call
+ *   packed means  : centroids re-laid-out (scaled by -2, padded) for the fast assignment kernels
+ *   norms         : |c|^2 per (padded) centroid followed by max_j |c_j|^2
+ *   partials      : per-work-group partial sums/counts of the update kernels that need them
+ */
+struct Workspace {
+	uint32_t* queue = nullptr;      size_t queue_cap = 0;      /* entries */
+	uint32_t* counters = nullptr;                               /* 16 words */
+	float* packed_means = nullptr;  size_t packed_cap = 0;     /* floats  */
+	float* norms = nullptr;         size_t norms_cap = 0;      /* floats  */
+	float* partials = nullptr;      size_t partials_cap = 0;   /* floats  */
+};
+int workspace(Workspace** ws);
+int reserve_queue(Workspace* ws, size_t entries);
+int reserve_packed(Workspace* ws, size_t packed_floats, size_t norm_floats);
+int reserve_partials(Workspace* ws, size_t floats);
+
+#define KMX_HIP(call)                                                                                         \
+	do {                                                                                                      \
+		hipError_t kmx_e_ = (call);                                                                           \
+		if (kmx_e_ != hipSuccess)                                                                             \
+			return ::kmx::fail(KMX_ERR_DEVICE, "%s failed: %s", #call, hipGetErrorString(kmx_e_));           \
+	} while (0)
+
+#define KMX_LAUNCH_CHECK(name)                                                                                \
+	do {                                                                                                      \
+		hipError_t kmx_e_ = hipGetLastError();                                                                \
+		if (kmx_e_ != hipSuccess)                                                                             \
+			return ::kmx::fail(KMX_ERR_DEVICE, "launch of %s failed: %s", name, hipGetErrorString(kmx_e_));  \
+	} while (0)
+
+/* Element address in either layout (layout_policies.hpp:22-25 SoA, :46-49 AoS of the reference). */
+template <int LAYOUT>
+__host__ __device__ __forceinline__ size_t elem(size_t stride, size_t idx, size_t dim)
+{
+	return LAYOUT == KMX_AOS ? idx * stride + dim : dim * stride + idx;
+}
+
+/* Argument bundle of one assignment call after validation. */
+struct AssignArgs {
+	const float* data; int layout; size_t stride;
+	const float* means; int layout_means; size_t stride_means;
+	uint32_t* assignment;
+	uint32_t dim, k, n;
+};
+
+struct UpdateArgs {
+	const float* data; int layout; size_t stride;
+	const uint32_t* assignment;
+	float* means; int layout_means; size_t stride_means;
+	uint32_t* cluster_sizes;
+	uint32_t dim, k, n;
+};
+
+/* assign_exact.hip */
+int launch_assign_base(const AssignArgs& a, kmx_exec_params* exec);
+/* Re-evaluates the points listed in ws->queue[0 .. counters[0]) with the serial arithmetic. */
+int launch_recheck(const AssignArgs& a, Workspace* ws);
+
+/* assign_mfma.hip / assign_lds_fma.hip: return KMX_ERR_UNSUPPORTED (without message side effects
+ * beyond kmx_last_error) when the shape does not fit the variant. */
+bool mfma_supports(const AssignArgs& a, const DeviceInfo& dev);
+int launch_assign_mfma(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev);
+bool lds_fma_supports(const AssignArgs& a, const DeviceInfo& dev);
+int launch_assign_lds_fma(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev);
+
+/* update.hip */
+int launch_update(int variant, const UpdateArgs& u, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev);
+
+} // namespace kmx
+
+#endif

@@ -1,0 +1,369 @@
+/*
+ * C ABI entry points of libkmx_hip.so: device / memory / stream / event plumbing, argument
+ * validation and dispatch to the kernel launchers. Declared in include/kmx.h.
+ */
+#include "kmx_internal.h"
+
+#include <cstdarg>
+#include <cstring>
+
+namespace kmx {
+
+static thread_local char g_error[512] = "";
+static hipStream_t g_stream = nullptr;
+static DeviceInfo g_dev;
+static Workspace g_ws;
+
+int fail(int code, const char* fmt, ...)
+{
+	va_list ap;
+	va_start(ap, fmt);
+	vsnprintf(g_error, sizeof(g_error), fmt, ap);
+	va_end(ap);
+	return code;
+}
+
+void clear_error() { g_error[0] = '\0'; }
+
+hipStream_t stream() { return g_stream; }
+
+int device_info(const DeviceInfo** out)
+{
+	int dev = 0;
+	KMX_HIP(hipGetDevice(&dev));
+	if (g_dev.device != dev) {
+		hipDeviceProp_t p;
+		KMX_HIP(hipGetDeviceProperties(&p, dev));
+		g_dev.device = dev;
+		g_dev.compute_units = (uint32_t)p.multiProcessorCount;
+		g_dev.lds_bytes = (uint32_t)p.sharedMemPerBlock;
+		g_dev.max_threads = (uint32_t)p.maxThreadsPerBlock;
+	}
+	*out = &g_dev;
+	return KMX_OK;
+}
+
+int workspace(Workspace** ws)
+{
+	if (!g_ws.counters) {
+		KMX_HIP(hipMalloc((void**)&g_ws.counters, 16 * sizeof(uint32_t)));
+		KMX_HIP(hipMemset(g_ws.counters, 0, 16 * sizeof(uint32_t)));
+	}
+	*ws = &g_ws;
+	return KMX_OK;
+}
+
+template <typename T>
+static int grow(T** ptr, size_t* cap, size_t want)
+{
+	if (want <= *cap) return KMX_OK;
+	if (*ptr) {
+		/* earlier launches may still be reading the old buffer */
+		KMX_HIP(hipStreamSynchronize(g_stream));
+		KMX_HIP(hipFree(*ptr));
+		*ptr = nullptr;
+		*cap = 0;
+	}
+	KMX_HIP(hipMalloc((void**)ptr, want * sizeof(T)));
+	*cap = want;
+	return KMX_OK;
+}
+
+int reserve_queue(Workspace* ws, size_t entries) { return grow(&ws->queue, &ws->queue_cap, entries); }
+
+int reserve_packed(Workspace* ws, size_t packed_floats, size_t norm_floats)
+{
+	int rc = grow(&ws->packed_means, &ws->packed_cap, packed_floats);
+	if (rc) return rc;
+	return grow(&ws->norms, &ws->norms_cap, norm_floats);
+}
+
+int reserve_partials(Workspace* ws, size_t floats) { return grow(&ws->partials, &ws->partials_cap, floats); }
+
+static int release_workspace()
+{
+	if (g_ws.queue) KMX_HIP(hipFree(g_ws.queue));
+	if (g_ws.counters) KMX_HIP(hipFree(g_ws.counters));
+	if (g_ws.packed_means) KMX_HIP(hipFree(g_ws.packed_means));
+	if (g_ws.norms) KMX_HIP(hipFree(g_ws.norms));
+	if (g_ws.partials) KMX_HIP(hipFree(g_ws.partials));
+	g_ws = Workspace();
+	return KMX_OK;
+}
+
+/* counterpart of fillZeros (reference kernels.cu:12-17), grid-stride, 128-bit stores where aligned */
+__global__ void fill_zero_kernel(uint32_t* __restrict__ p, size_t count)
+{
+	size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+	size_t step = (size_t)gridDim.x * blockDim.x;
+	for (; i < count; i += step) p[i] = 0u;
+}
+
+} // namespace kmx
+
+using namespace kmx;
+
+extern "C" {
+
+const char* kmx_last_error(void) { return g_error; }
+
+int kmx_device_count(int* count)
+{
+	clear_error();
+	if (!count) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_device_count: null pointer");
+	int c = 0;
+	hipError_t e = hipGetDeviceCount(&c);
+	if (e != hipSuccess) { (void)hipGetLastError(); c = 0; }
+	*count = c;
+	return KMX_OK;
+}
+
+int kmx_set_device(int device)
+{
+	clear_error();
+	int c = 0;
+	if (hipGetDeviceCount(&c) != hipSuccess || c == 0) {
+		(void)hipGetLastError();
+		return fail(KMX_ERR_NO_DEVICE, "No HIP devices found!");
+	}
+	KMX_HIP(hipSetDevice(device));
+	return KMX_OK;
+}
+
+int kmx_device_props(kmx_props* props)
+{
+	clear_error();
+	if (!props) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_device_props: null pointer");
+	int dev = 0;
+	KMX_HIP(hipGetDevice(&dev));
+	hipDeviceProp_t p;
+	KMX_HIP(hipGetDeviceProperties(&p, dev));
+	std::memset(props, 0, sizeof(*props));
+	std::strncpy(props->name, p.name, sizeof(props->name) - 1);
+	std::strncpy(props->arch, p.gcnArchName, sizeof(props->arch) - 1);
+	props->compute_units = (uint32_t)p.multiProcessorCount;
+	props->wavefront_size = (uint32_t)p.warpSize;
+	props->max_threads_per_block = (uint32_t)p.maxThreadsPerBlock;
+	props->lds_bytes_per_block = (uint32_t)p.sharedMemPerBlock;
+	props->clock_khz = (uint32_t)p.clockRate;
+	props->global_mem_bytes = (uint64_t)p.totalGlobalMem;
+	return KMX_OK;
+}
+
+int kmx_malloc(void** dptr, size_t bytes)
+{
+	clear_error();
+	if (!dptr) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_malloc: null pointer");
+	*dptr = nullptr;
+	if (bytes == 0) return KMX_OK;
+	KMX_HIP(hipMalloc(dptr, bytes));
+	return KMX_OK;
+}
+
+int kmx_free(void* dptr)
+{
+	clear_error();
+	if (!dptr) return KMX_OK;
+	KMX_HIP(hipFree(dptr));
+	return KMX_OK;
+}
+
+int kmx_h2d(void* dst_device, const void* src_host, size_t bytes)
+{
+	clear_error();
+	if (bytes == 0) return KMX_OK;
+	if (!dst_device || !src_host) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_h2d: null pointer");
+	KMX_HIP(hipMemcpyAsync(dst_device, src_host, bytes, hipMemcpyHostToDevice, stream()));
+	return KMX_OK;
+}
+
+int kmx_d2h(void* dst_host, const void* src_device, size_t bytes)
+{
+	clear_error();
+	if (bytes == 0) return KMX_OK;
+	if (!dst_host || !src_device) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_d2h: null pointer");
+	KMX_HIP(hipMemcpyAsync(dst_host, src_device, bytes, hipMemcpyDeviceToHost, stream()));
+	KMX_HIP(hipStreamSynchronize(stream()));
+	return KMX_OK;
+}
+
+int kmx_d2d(void* dst_device, const void* src_device, size_t bytes)
+{
+	clear_error();
+	if (bytes == 0) return KMX_OK;
+	if (!dst_device || !src_device) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_d2d: null pointer");
+	KMX_HIP(hipMemcpyAsync(dst_device, src_device, bytes, hipMemcpyDeviceToDevice, stream()));
+	return KMX_OK;
+}
+
+int kmx_sync(void)
+{
+	clear_error();
+	KMX_HIP(hipDeviceSynchronize());
+	return KMX_OK;
+}
+
+int kmx_set_stream(void* hip_stream)
+{
+	clear_error();
+	g_stream = (hipStream_t)hip_stream;
+	return KMX_OK;
+}
+
+int kmx_shutdown(void)
+{
+	clear_error();
+	KMX_HIP(hipDeviceSynchronize());
+	return release_workspace();
+}
+
+int kmx_fill_zero_u32(void* dptr, size_t count)
+{
+	clear_error();
+	if (count == 0) return KMX_OK;
+	if (!dptr) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_fill_zero_u32: null pointer");
+	const unsigned block = 256;
+	size_t blocks = (count + block - 1) / block;
+	if (blocks > 4096) blocks = 4096;
+	hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)blocks), dim3(block), 0, stream(), (uint32_t*)dptr, count);
+	KMX_LAUNCH_CHECK("fill_zero_kernel");
+	return KMX_OK;
+}
+
+static int check_layout(const char* who, const char* what, int layout, size_t stride, uint32_t count, uint32_t dim)
+{
+	if (layout != KMX_AOS && layout != KMX_SOA) return fail(KMX_ERR_INVALID_ARGUMENT, "%s: unknown %s layout %d", who, what, layout);
+	if (layout == KMX_AOS && stride < dim) return fail(KMX_ERR_INVALID_ARGUMENT, "%s: %s stride %zu < dim %u", who, what, stride, dim);
+	if (layout == KMX_SOA && stride < count) return fail(KMX_ERR_INVALID_ARGUMENT, "%s: %s stride %zu < count %u", who, what, stride, count);
+	return KMX_OK;
+}
+
+int kmx_assign_f32(int variant,
+                   const float* data, int layout, size_t stride,
+                   const float* means, int layout_means, size_t stride_means,
+                   const uint32_t* last_assignment, uint32_t* assignment,
+                   uint32_t dim, uint32_t k, uint32_t n, kmx_exec_params* exec)
+{
+	clear_error();
+	(void)last_assignment;
+	if (!exec) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_assign_f32: exec is null");
+	if (dim == 0 || k == 0) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_assign_f32: dim and k must be positive");
+	if (n == 0) { exec->block_count = 0; return KMX_OK; }
+	if (!data || !means || !assignment) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_assign_f32: null device pointer");
+	int rc = check_layout("kmx_assign_f32", "data", layout, stride, n, dim);
+	if (rc) return rc;
+	rc = check_layout("kmx_assign_f32", "means", layout_means, stride_means, k, dim);
+	if (rc) return rc;
+
+	const DeviceInfo* dev = nullptr;
+	rc = device_info(&dev);
+	if (rc) return rc;
+	Workspace* ws = nullptr;
+	rc = workspace(&ws);
+	if (rc) return rc;
+
+	AssignArgs a{ data, layout, stride, means, layout_means, stride_means, assignment, dim, k, n };
+	switch (variant) {
+	case KMX_ASSIGN_BASE:
+		return launch_assign_base(a, exec);
+	case KMX_ASSIGN_LDS_FMA:
+		if (!lds_fma_supports(a, *dev))
+			return fail(KMX_ERR_UNSUPPORTED, "kmx_assign_f32: shape dim=%u k=%u is not supported by the LDS/FMA variant", dim, k);
+		return launch_assign_lds_fma(a, exec, ws, *dev);
+	case KMX_ASSIGN_MFMA:
+		if (!mfma_supports(a, *dev))
+			return fail(KMX_ERR_UNSUPPORTED, "kmx_assign_f32: shape dim=%u k=%u is not supported by the MFMA variant", dim, k);
+		return launch_assign_mfma(a, exec, ws, *dev);
+	case KMX_ASSIGN_BEST:
+		/* counterpart of BestCachedAssignmentKernel::run (reference kernels.cu:706-717): pick by shape */
+		if (mfma_supports(a, *dev) && dim >= 16) return launch_assign_mfma(a, exec, ws, *dev);
+		if (lds_fma_supports(a, *dev)) return launch_assign_lds_fma(a, exec, ws, *dev);
+		if (mfma_supports(a, *dev)) return launch_assign_mfma(a, exec, ws, *dev);
+		return launch_assign_base(a, exec);
+	default:
+		return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_assign_f32: unknown variant %d", variant);
+	}
+}
+
+int kmx_assign_last_rechecked(uint64_t* count)
+{
+	clear_error();
+	if (!count) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_assign_last_rechecked: null pointer");
+	*count = 0;
+	Workspace* ws = nullptr;
+	int rc = workspace(&ws);
+	if (rc) return rc;
+	uint32_t c = 0;
+	KMX_HIP(hipMemcpyAsync(&c, ws->counters, sizeof(c), hipMemcpyDeviceToHost, stream()));
+	KMX_HIP(hipStreamSynchronize(stream()));
+	*count = c;
+	return KMX_OK;
+}
+
+int kmx_update_f32(int variant,
+                   const float* data, int layout, size_t stride,
+                   const uint32_t* assignment,
+                   float* means, int layout_means, size_t stride_means,
+                   uint32_t* cluster_sizes,
+                   uint32_t dim, uint32_t k, uint32_t n, kmx_exec_params* exec)
+{
+	clear_error();
+	if (!exec) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_update_f32: exec is null");
+	if (dim == 0 || k == 0) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_update_f32: dim and k must be positive");
+	if (!means || !cluster_sizes) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_update_f32: null device pointer");
+	if (n > 0 && (!data || !assignment)) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_update_f32: null device pointer");
+	int rc = check_layout("kmx_update_f32", "data", layout, stride, n, dim);
+	if (rc) return rc;
+	rc = check_layout("kmx_update_f32", "means", layout_means, stride_means, k, dim);
+	if (rc) return rc;
+	if (variant < KMX_UPDATE_ATOMIC_POINT || variant > KMX_UPDATE_ATOMIC_SHM)
+		return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_update_f32: unknown variant %d", variant);
+	if (exec->privatized_copies == 0) exec->privatized_copies = 1;
+
+	const DeviceInfo* dev = nullptr;
+	rc = device_info(&dev);
+	if (rc) return rc;
+	Workspace* ws = nullptr;
+	rc = workspace(&ws);
+	if (rc) return rc;
+
+	UpdateArgs u{ data, layout, stride, assignment, means, layout_means, stride_means, cluster_sizes, dim, k, n };
+	return launch_update(variant, u, exec, ws, *dev);
+}
+
+int kmx_event_create(void** event)
+{
+	clear_error();
+	if (!event) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_event_create: null pointer");
+	hipEvent_t e;
+	KMX_HIP(hipEventCreate(&e));
+	*event = (void*)e;
+	return KMX_OK;
+}
+
+int kmx_event_destroy(void* event)
+{
+	clear_error();
+	if (!event) return KMX_OK;
+	KMX_HIP(hipEventDestroy((hipEvent_t)event));
+	return KMX_OK;
+}
+
+int kmx_event_record(void* event)
+{
+	clear_error();
+	if (!event) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_event_record: null event");
+	KMX_HIP(hipEventRecord((hipEvent_t)event, stream()));
+	return KMX_OK;
+}
+
+int kmx_event_elapsed_ms(void* start, void* stop, float* ms)
+{
+	clear_error();
+	if (!start || !stop || !ms) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_event_elapsed_ms: null argument");
+	KMX_HIP(hipEventSynchronize((hipEvent_t)stop));
+	KMX_HIP(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+	return KMX_OK;
+}
+
+} // extern "C"

@@ -1,0 +1,146 @@
+/*
+ * kmx -- C ABI of the MI355X (gfx950) Lloyd-iteration kernels.
+ *
+ * This is the device boundary of the k-means harness: the only thing the C++ host side (or any
+ * other caller: ctypes, cgo, JNI ...) links against. It replaces the reference's kernel-runner
+ * boundary, experimental/k-means/k-means/headers/kernels.cuh, whose entry points are the static
+ * `KERNEL::run(const *ProblemInstance&, CudaExecParameters&)` policy functions and runFillZeros(),
+ * plus the small part of bpplib's CudaBuffer/CUCH the reference's algorithm objects use
+ * (experimental/k-means/k-means/headers/cuda.hpp:25-28,44-68,105-110).
+ *
+ * Conventions
+ *   - Every function returns 0 on success or a non-zero kmx_status; kmx_last_error() then holds a
+ *     message for the calling thread. Nothing throws across this boundary; the C++ host wrappers
+ *     rethrow as std::runtime_error like the reference's runners (kernels.cu:281-282,666,675,701).
+ *   - Device pointers are plain `void*`/`float*`/`uint32_t*` obtained from kmx_malloc (or from any
+ *     other HIP allocation of the current device). Runners borrow them and never free them.
+ *   - All work is enqueued on one stream (the legacy default stream unless kmx_set_stream() was
+ *     called) and the calls return without waiting, except kmx_sync, kmx_d2h and
+ *     kmx_event_elapsed_ms. Stream order is the only dependency mechanism, as in the reference
+ *     (cuda.hpp:70-88: one cudaDeviceSynchronize after the iteration loop).
+ *   - Not thread-safe: one host thread drives one device, as in the reference.
+ *   - layout: KMX_AOS element (idx, dim) = base[idx*stride + dim]; KMX_SOA = base[dim*stride + idx]
+ *     (layout_policies.hpp:22-25,46-49); stride = LAYOUT::precomputeConstants(count, dim).
+ */
+#ifndef KMX_H
+#define KMX_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum kmx_status {
+	KMX_OK = 0,
+	KMX_ERR_INVALID_ARGUMENT = 1, /* bad pointer / size / enum value                              */
+	KMX_ERR_UNSUPPORTED = 2,      /* shape not supported by the requested variant                  */
+	KMX_ERR_DEVICE = 3,           /* a HIP call failed; message carries hipGetErrorString          */
+	KMX_ERR_NO_DEVICE = 4         /* no GPU visible (cuda.hpp:50-51 "No CUDA devices found!")      */
+} kmx_status;
+
+typedef enum kmx_layout { KMX_AOS = 0, KMX_SOA = 1 } kmx_layout;
+
+/* = CudaExecParameters (kernels.cuh:55-70). In/out: runners overwrite block_count like the reference
+ * (kernels.cu:203,311,750). Unlike the reference (kernels.cu:384,676,713) they never write the
+ * other fields back, so one struct can serve the assignment and the update of every iteration. */
+typedef struct kmx_exec_params {
+	uint32_t block_size;        /* work-group size for the variants that honour it (default 256)   */
+	uint32_t block_count;       /* out: number of work-groups of the main kernel last launched      */
+	uint32_t shared_mem_bytes;  /* LDS budget per work-group; 0 = device maximum                    */
+	uint32_t privatized_copies; /* global replicas of the k x d accumulator (update variants 0, 1)  */
+	uint32_t items_per_thread;
+	uint32_t regs_cache;
+} kmx_exec_params;
+
+/* Assignment variants (reference counterparts: kernels.cuh:81-93). */
+typedef enum kmx_assign_variant {
+	KMX_ASSIGN_BASE = 0,    /* BaseAssignmentKernel: one lane per point, the serial arithmetic op for op */
+	KMX_ASSIGN_LDS_FMA = 1, /* CachedFixed/CachedRegs counterpart: centroids in LDS, register tile, fp32 FMA */
+	KMX_ASSIGN_MFMA = 2,    /* dense-contraction path: fp32 MFMA tiles of -2 x.c + |c|^2                */
+	KMX_ASSIGN_BEST = 3     /* BestCachedAssignmentKernel: shape-based selector between 1 and 2         */
+} kmx_assign_variant;
+
+/* Update variants (reference counterparts: kernels.cuh:96-105). */
+typedef enum kmx_update_variant {
+	KMX_UPDATE_ATOMIC_POINT = 0, /* UpdateAtomicPointKernel: one lane per point, global atomics      */
+	KMX_UPDATE_ATOMIC_FINE = 1,  /* UpdateAtomicFineKernel: one lane per (point, dim) element        */
+	KMX_UPDATE_ATOMIC_SHM = 2    /* UpdateAtomicShmKernel: LDS-privatised partial sums, wave-aggregated flush */
+} kmx_update_variant;
+
+typedef struct kmx_props {
+	char name[128];
+	char arch[64];             /* gcnArchName, e.g. "gfx950:sramecc+:xnack-" */
+	uint32_t compute_units;
+	uint32_t wavefront_size;
+	uint32_t max_threads_per_block;
+	uint32_t lds_bytes_per_block;
+	uint32_t clock_khz;
+	uint64_t global_mem_bytes;
+} kmx_props;
+
+/* ---- device + memory (bpp::CudaDevice::count / cudaSetDevice / bpp::CudaBuffer; cuda.hpp:50-64,105-110;
+ *      cudaGetDeviceProperties k-means.cpp:24-25) ---- */
+int kmx_device_count(int* count);
+int kmx_set_device(int device);
+int kmx_device_props(kmx_props* props);
+int kmx_malloc(void** dptr, size_t bytes);
+int kmx_free(void* dptr);
+int kmx_h2d(void* dst_device, const void* src_host, size_t bytes);          /* CudaBuffer::write; enqueued, host buffer must stay valid until kmx_sync */
+int kmx_d2h(void* dst_host, const void* src_device, size_t bytes);          /* CudaBuffer::read; waits for the stream            */
+int kmx_d2d(void* dst_device, const void* src_device, size_t bytes);        /* device copy on the stream                          */
+int kmx_sync(void);                                                         /* cudaDeviceSynchronize (cuda.hpp:67,87)             */
+int kmx_set_stream(void* hip_stream);                                       /* NULL = legacy default stream                       */
+int kmx_shutdown(void);                                                     /* frees the library's internal work space            */
+
+/* ---- runFillZeros<float|uint32_t> (kernels.cuh:74-75, kernels.cu:12-28): count 32-bit words := 0 ---- */
+int kmx_fill_zero_u32(void* dptr, size_t count);
+
+/*
+ * ---- ASGN_KERNEL::run(AssignmentProblemInstance, CudaExecParameters&) (kernels.cuh:7-20,81-93) ----
+ * assignment[i] = index of the centroid nearest to point i under the reference metric
+ * sqrt(sum_d (x_d - c_d)^2) with the serial tie-break (lowest index on equal distances;
+ * serial.hpp:21-35). Every variant returns exactly that index: the fast variants rank centroids
+ * with |c|^2 - 2 x.c and re-evaluate with the serial arithmetic every point whose two best
+ * candidates are closer than the rounding-error bound of that ranking.
+ * last_assignment is accepted for signature parity and ignored (no reference kernel reads it).
+ */
+int kmx_assign_f32(int variant,
+                   const float* data, int layout, size_t stride,
+                   const float* means, int layout_means, size_t stride_means,
+                   const uint32_t* last_assignment, uint32_t* assignment,
+                   uint32_t dim, uint32_t k, uint32_t n, kmx_exec_params* exec);
+
+/* Number of points the last kmx_assign_f32 call re-evaluated with the serial arithmetic (waits for the stream). */
+int kmx_assign_last_rechecked(uint64_t* count);
+
+/*
+ * ---- UPDATE_KERNEL::run(UpdateProblemInstance, CudaExecParameters&) (kernels.cuh:23-36,96-105) ----
+ * Precondition as in the reference (cuda.hpp:78-79): means (k x dim, times privatized_copies for
+ * variants 0 and 1) and cluster_sizes (k) are zero. Accumulates member sums and counts, merges
+ * the privatised replicas and divides every non-empty cluster by its count; empty clusters stay
+ * at zero (kernels.cu:149-163, serial.hpp:66-67).
+ */
+int kmx_update_f32(int variant,
+                   const float* data, int layout, size_t stride,
+                   const uint32_t* assignment,
+                   float* means, int layout_means, size_t stride_means,
+                   uint32_t* cluster_sizes,
+                   uint32_t dim, uint32_t k, uint32_t n, kmx_exec_params* exec);
+
+/* ---- events on the library's stream (for the assignment / update split; the reference only has
+ *      a wall-clock Stopwatch around run(), k-means.cpp:155-158) ---- */
+int kmx_event_create(void** event);
+int kmx_event_destroy(void* event);
+int kmx_event_record(void* event);
+int kmx_event_elapsed_ms(void* start, void* stop, float* ms); /* waits for `stop` */
+
+/* Message of the last failed call on this thread ("" if none). */
+const char* kmx_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif
