@@ -1,0 +1,168 @@
+#!/usr/bin/env python3
+"""Benchmark of the Lloyd iteration on one MI355X.
+
+    python bench.py [--gpus 1] [--steps 20] [--warmup 5] [--config 2]
+
+A "step" is one full k-means iteration (assignment + zero-fill + update + divide) over the whole
+synthetic data set of the chosen benchmark configuration (default: the headline, N = 2,097,152,
+d = 32, k = 1024, fp32, seeded Gaussian mixture, initial centroids = first k points), with the points
+and the initial centroids already resident in HBM when the clock starts -- the reference's protocol
+(k-means.cpp:155-169: wall clock around run(), transfers excluded). Prints ONE JSON line.
+
+Legs:
+  1. warm-up iterations, then state reset;
+  2. the timed region: K iterations back to back on the library's stream, one sync on each side,
+     wall clock -> value / ms_per_step;
+  3. the same K iterations again with the library's per-kernel events on (kmx_set_profiling) and events
+     around the assignment / update calls -> the split, the dominant kernel's average duration, roofline;
+  4. cpu_baseline: the reference's serial k-means (oracle/_ref build of the reference's own serial.hpp if it
+     travelled with the tree, else the C restatement in oracle/) timed on ONE host core over a bounded
+     sample of the same workload and scaled to the full N.
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP32_TFLOPS = 157.3   # MI355X fp32 (vector or matrix), dense
+PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+# published full-iteration time for the headline shape on the reference's best hardware (V100 SXM2)
+PUBLISHED_MS = {2: 25.45}  # results/README.md:20 of the reference
+
+
+def cpu_baseline(km, spec, n_sample, data, means0):
+    """One serial Lloyd iteration on one core over the first n_sample points; scaled to N."""
+    from oracle import binding as orc  # the checker is only timed here, never used by the measured path
+    dim, k = spec.dim, spec.k
+    sample = np.ascontiguousarray(data[: n_sample * dim])
+    if orc.ref_lib() is not None:
+        kind = "reference"
+        t0 = time.perf_counter()
+        orc.ref_kmeans(sample, means0, dim, k, n_sample, 1)
+        dt = time.perf_counter() - t0
+    else:
+        kind = "port"
+        t0 = time.perf_counter()
+        orc.kmeans(sample, means0, dim, k, n_sample, 1, threads=1, fast=False)
+        dt = time.perf_counter() - t0
+    scaled_ms = dt * 1e3 * (int(spec.n) / n_sample)
+    return {
+        "value": round(scaled_ms, 1), "unit": "ms/iteration", "cores": 1, "kind": kind,
+        "sample": "1 iteration over the first %d of %d points x all %d centroids took %.2f s on 1 core; scaled by N/sample"
+                  % (n_sample, int(spec.n), k, dt),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", type=int, default=2, help="benchmark configuration 1..5 (2 = headline)")
+    ap.add_argument("--cpu-sample", type=int, default=0, help="points in the CPU baseline sample (0 = about 12 s of work)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (no collectives, no sharding); --gpus %d is not supported" % args.gpus)
+
+    km = importlib.import_module("cuda-kmeans_amd")
+    if not (os.path.exists(km.HIP_LIB_PATH) and os.path.exists(km.HOST_LIB_PATH)):
+        km.build(force=False)
+    if km.device_count() == 0:
+        sys.exit("bench.py: no HIP device visible")
+    spec = km.baseline_config(args.config)
+    n, dim, k = int(spec.n), spec.dim, spec.k
+    data = km.generate_points(spec)
+    means0 = km.first_k_means(spec)
+
+    alg = km.HipKMeansAlgorithm(km.ASSIGN_BEST, km.UPDATE_ATOMIC_SHM)
+    alg.initialize(dim, k, n, args.steps, data, means0)
+
+    # 1. warm-up
+    alg.run(iters=args.warmup)
+    alg.reset(means0)
+
+    # 2. timed region
+    km.sync()
+    t0 = time.perf_counter()
+    alg.run(iters=args.steps)          # ends with one device sync
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ms_per_step = wall_ms / args.steps
+    counts = alg.getClusterSizes()
+    assert int(counts.sum()) == n, "cluster counts do not sum to N"
+
+    # 3. instrumented repeat of the same iterations
+    alg.reset(means0)
+    km.set_profiling(True)
+    ev = [km.Event() for _ in range(3)]
+    t_assign = t_update = k_assign = k_update = 0.0
+    rechecked = 0
+    for _ in range(args.steps):
+        ev[0].record()
+        nxt = alg.iteration()
+        ev[1].record()
+        alg.update_step(nxt)
+        ev[2].record()
+        t_assign += ev[0].elapsed_ms(ev[1])
+        t_update += ev[1].elapsed_ms(ev[2])
+        k_assign += km.last_kernel_ms(0)
+        k_update += km.last_kernel_ms(1)
+        rechecked += km.last_rechecked()
+    km.set_profiling(False)
+    t_assign /= args.steps; t_update /= args.steps; k_assign /= args.steps; k_update /= args.steps
+    alg.cleanup()
+
+    flop = 2.0 * n * k * dim                                      # one multiply-add per point x centroid x dim
+    update_bytes = 4.0 * (n * dim + n + k * dim + k)              # points + assignment in, sums + counts out
+    assign_bytes = 4.0 * (n * dim + n + k * dim)
+    assign_tflops = flop / (k_assign * 1e-3) / 1e12
+    update_gbs = update_bytes / (k_update * 1e-3) / 1e9
+    assign_gbs = assign_bytes / (k_assign * 1e-3) / 1e9
+    # the dominant kernel is the assignment sweep; it is compute-bound unless k is tiny (flop/byte = k/2)
+    if k >= 64:
+        roofline = {"kernel": "assignment sweep", "bound": "mfma", "achieved": round(assign_tflops, 2),
+                    "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s", "frac": round(assign_tflops / PEAK_FP32_TFLOPS, 4),
+                    "traffic": None}
+    else:
+        roofline = {"kernel": "assignment sweep", "bound": "hbm", "achieved": round(assign_gbs, 1),
+                    "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(assign_gbs / PEAK_HBM_GBS, 4), "traffic": None}
+    roofline["avg_kernel_ms"] = round(k_assign, 4)
+    roofline_update = {"kernel": "update accumulation", "bound": "hbm", "achieved": round(update_gbs, 1),
+                       "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(update_gbs / PEAK_HBM_GBS, 4),
+                       "traffic": None, "avg_kernel_ms": round(k_update, 4)}
+
+    out = {
+        "metric": "ms per k-means iteration (assign+update) at N=2M,d=32,k=1024; % roofline" if args.config == 2
+                  else "ms per k-means iteration (assign+update), benchmark configuration %d" % args.config,
+        "value": round(ms_per_step, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": False, "scaling": "weak",
+        "vs_baseline": round(ms_per_step / PUBLISHED_MS[args.config], 4) if args.config in PUBLISHED_MS else None,
+        "baseline_note": "published: 25.45 ms on V100 SXM2 for this shape (reference results/README.md:20); lower is better"
+                         if args.config in PUBLISHED_MS else None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "benchmark configuration %d: N=%d d=%d k=%d, %s, initial centroids = first k points, seed %d"
+                               % (args.config, n, dim, k, "Gaussian mixture" if spec.kind != 1 else "uniform", spec.seed),
+                   "layout": "aos", "assignment": "hip_best", "update": "atomic_shm"},
+        "assign_ms": round(t_assign, 4), "update_ms": round(t_update, 4),
+        "points_centroids_dims_per_s": round(float(n) * k * dim / (ms_per_step * 1e-3), 0),
+        "rechecked_points_per_iteration": round(rechecked / args.steps, 1),
+        "roofline": roofline, "roofline_update": roofline_update,
+    }
+
+    if not args.no_cpu_baseline:
+        per_point_s = 0.45e-9 * k * dim        # measured cost of the serial loop per point
+        n_sample = args.cpu_sample or int(min(n, max(1024, 12.0 / per_point_s)))
+        out["cpu_baseline"] = cpu_baseline(km, spec, n_sample, data, means0)
+
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

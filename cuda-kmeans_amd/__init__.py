@@ -30,7 +30,7 @@ ABI_SYMBOLS = [
     "kmx_device_count", "kmx_set_device", "kmx_device_props", "kmx_malloc", "kmx_free", "kmx_h2d", "kmx_d2h",
     "kmx_d2d", "kmx_sync", "kmx_set_stream", "kmx_shutdown", "kmx_fill_zero_u32", "kmx_assign_f32",
     "kmx_assign_last_rechecked", "kmx_update_f32", "kmx_event_create", "kmx_event_destroy", "kmx_event_record",
-    "kmx_event_elapsed_ms", "kmx_last_error",
+    "kmx_event_elapsed_ms", "kmx_set_profiling", "kmx_last_kernel_ms", "kmx_last_error",
 ]
 
 
@@ -107,6 +107,8 @@ def hip_lib():
         lib.kmx_event_destroy.argtypes = [vp]
         lib.kmx_event_record.argtypes = [vp]
         lib.kmx_event_elapsed_ms.argtypes = [vp, vp, ctypes.POINTER(ctypes.c_float)]
+        lib.kmx_set_profiling.argtypes = [ctypes.c_int]
+        lib.kmx_last_kernel_ms.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_float)]
         _hip = lib
     return _hip
 
@@ -271,6 +273,17 @@ def update(variant, data_buf, layout, stride, assignment_buf, means_buf, layout_
     check(hip_lib().kmx_update_f32(variant, data_buf.ptr, layout, stride, assignment_buf.ptr, means_buf.ptr,
                                    layout_means, stride_means, sizes_buf.ptr, dim, k, n, ctypes.byref(ex)))
     return ex
+
+
+def set_profiling(enabled):
+    check(hip_lib().kmx_set_profiling(1 if enabled else 0))
+
+
+def last_kernel_ms(which):
+    """Duration of the dominant kernel of the last assignment (0) / update (1) call made under set_profiling(True)."""
+    ms = ctypes.c_float(0)
+    check(hip_lib().kmx_last_kernel_ms(which, ctypes.byref(ms)))
+    return ms.value
 
 
 def last_rechecked():

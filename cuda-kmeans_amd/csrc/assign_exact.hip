@@ -103,10 +103,12 @@ static int launch_base_t(const AssignArgs& a, kmx_exec_params* exec, uint32_t* c
 	if (block > 256) block = 256;
 	block = (block + WAVE - 1) / WAVE * WAVE;
 	exec->block_count = (a.n + block - 1) / block;
+	int rc = profile_begin(0);
+	if (rc) return rc;
 	hipLaunchKernelGGL((assign_base_kernel<LD, LM>), dim3(exec->block_count), dim3(block), 0, stream(),
 	                   a.data, a.stride, a.means, a.stride_means, a.assignment, a.dim, a.k, a.n, counters);
 	KMX_LAUNCH_CHECK("assign_base_kernel");
-	return KMX_OK;
+	return profile_end(0);
 }
 
 int launch_assign_base(const AssignArgs& a, kmx_exec_params* exec)

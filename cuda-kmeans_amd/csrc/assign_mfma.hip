@@ -275,9 +275,11 @@ static int launch_mfma_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 	const uint32_t grid = std::min(rounds, dev.compute_units);
 	exec->block_count = grid;
 
+	int rc = KMX_OK;
 	if (stream_mode) {
 		auto kernel = assign_mfma_kernel<DPH, MFMA_P, LD, VEC, true>;
 		KMX_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+		if ((rc = profile_begin(0))) return rc;
 		hipLaunchKernelGGL(kernel, dim3(grid), dim3(MFMA_WAVES * WAVE), lds_bytes, stream(),
 		                   a.data, a.stride, ws->packed_means, ws->norms, a.assignment, ws->queue, ws->counters,
 		                   a.dim, a.k, kp, a.n, chunk_rows, kd);
@@ -285,12 +287,13 @@ static int launch_mfma_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 	else {
 		auto kernel = assign_mfma_kernel<DPH, MFMA_P, LD, VEC, false>;
 		KMX_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+		if ((rc = profile_begin(0))) return rc;
 		hipLaunchKernelGGL(kernel, dim3(grid), dim3(MFMA_WAVES * WAVE), lds_bytes, stream(),
 		                   a.data, a.stride, ws->packed_means, ws->norms, a.assignment, ws->queue, ws->counters,
 		                   a.dim, a.k, kp, a.n, chunk_rows, kd);
 	}
 	KMX_LAUNCH_CHECK("assign_mfma_kernel");
-	return KMX_OK;
+	return profile_end(0);
 }
 
 template <int DPH>

@@ -23,6 +23,10 @@ void clear_error();
 /* The stream every kernel of the library is launched on. */
 hipStream_t stream();
 
+/* Brackets the dominant kernel of a call with events when kmx_set_profiling(1) is active (which: 0 assign, 1 update). */
+int profile_begin(int which);
+int profile_end(int which);
+
 /* Properties of the current device, queried once. */
 struct DeviceInfo {
 	int device = -1;

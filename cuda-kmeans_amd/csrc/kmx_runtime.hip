@@ -27,6 +27,27 @@ void clear_error() { g_error[0] = '\0'; }
 
 hipStream_t stream() { return g_stream; }
 
+static bool g_profiling = false;
+static hipEvent_t g_prof[2][2] = { { nullptr, nullptr }, { nullptr, nullptr } };
+static bool g_prof_valid[2] = { false, false };
+
+int profile_begin(int which)
+{
+	if (!g_profiling) return KMX_OK;
+	for (int i = 0; i < 2; ++i)
+		if (!g_prof[which][i]) KMX_HIP(hipEventCreate(&g_prof[which][i]));
+	KMX_HIP(hipEventRecord(g_prof[which][0], g_stream));
+	return KMX_OK;
+}
+
+int profile_end(int which)
+{
+	if (!g_profiling) return KMX_OK;
+	KMX_HIP(hipEventRecord(g_prof[which][1], g_stream));
+	g_prof_valid[which] = true;
+	return KMX_OK;
+}
+
 int device_info(const DeviceInfo** out)
 {
 	int dev = 0;
@@ -329,6 +350,24 @@ int kmx_update_f32(int variant,
 
 	UpdateArgs u{ data, layout, stride, assignment, means, layout_means, stride_means, cluster_sizes, dim, k, n };
 	return launch_update(variant, u, exec, ws, *dev);
+}
+
+int kmx_set_profiling(int enabled)
+{
+	clear_error();
+	g_profiling = enabled != 0;
+	if (!g_profiling) g_prof_valid[0] = g_prof_valid[1] = false;
+	return KMX_OK;
+}
+
+int kmx_last_kernel_ms(int which, float* ms)
+{
+	clear_error();
+	if (which < 0 || which > 1 || !ms) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_last_kernel_ms: bad argument");
+	if (!g_prof_valid[which]) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_last_kernel_ms: no profiled call (kmx_set_profiling(1) first)");
+	KMX_HIP(hipEventSynchronize(g_prof[which][1]));
+	KMX_HIP(hipEventElapsedTime(ms, g_prof[which][0], g_prof[which][1]));
+	return KMX_OK;
 }
 
 int kmx_event_create(void** event)

@@ -216,7 +216,9 @@ static int launch_update_t(int variant, const UpdateArgs& u, kmx_exec_params* ex
 	const size_t copy_floats = copy_floats_of(u);
 	uint32_t copies = exec->privatized_copies;
 
+	int rc = KMX_OK;
 	if (u.n > 0) {
+		if ((rc = profile_begin(1))) return rc;
 		if (variant == KMX_UPDATE_ATOMIC_SHM) {
 			/* LDS budget: exec->shared_mem_bytes if given, else what the device offers a work-group */
 			uint32_t budget = exec->shared_mem_bytes ? std::min(exec->shared_mem_bytes, dev.lds_bytes) : dev.lds_bytes;
@@ -268,6 +270,7 @@ static int launch_update_t(int variant, const UpdateArgs& u, kmx_exec_params* ex
 			                   u.data, u.stride, u.assignment, u.means, u.stride_means, u.cluster_sizes, u.dim, u.k, u.n, copy_floats, copies);
 			KMX_LAUNCH_CHECK("update_fine_kernel");
 		}
+		if ((rc = profile_end(1))) return rc;
 	}
 
 	const uint32_t total = u.k * u.dim;

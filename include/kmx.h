@@ -136,6 +136,16 @@ int kmx_event_destroy(void* event);
 int kmx_event_record(void* event);
 int kmx_event_elapsed_ms(void* start, void* stop, float* ms); /* waits for `stop` */
 
+/*
+ * Per-kernel timing for roofline reports (no counterpart in the reference). While enabled, every
+ * kmx_assign_f32 / kmx_update_f32 call brackets its dominant kernel (the sweep over the centroids /
+ * the accumulation pass; not the small pack, recheck, merge and divide kernels around it) with a pair of
+ * events on the library's stream. kmx_last_kernel_ms(which, ...) waits for that kernel of the most
+ * recent call and returns its duration; which: 0 = assignment, 1 = update.
+ */
+int kmx_set_profiling(int enabled);
+int kmx_last_kernel_ms(int which, float* ms);
+
 /* Message of the last failed call on this thread ("" if none). */
 const char* kmx_last_error(void);
 

@@ -1,0 +1,327 @@
+"""Parity of the HIP path with the CPU oracle, through the C ABI, on a real MI355X (-m gpu).
+
+Bar (from the benchmark definition): assignment and per-cluster counts bit-exact, except points
+whose best and second-best reference distances differ by less than 1e-5 relative, which must be
+reported; centroids within 1e-4 relative in fp32.
+
+What "relative" means for a centroid coordinate: |gpu - oracle| / rms(oracle coordinates). Sums of
+n fp32 terms in a different order differ by O(sqrt(n) eps |sum|); coordinates near zero would make
+a per-coordinate relative error meaningless.
+
+Lloyd trajectories are chaotic at the last bit: the update's fp32 sums are accumulated in a different
+order from the serial loop (atomics, as in the reference's own GPU path), so after the first update the
+two runs hold centroids that differ in their last bits and a near-tie point may then legitimately go
+the other way, which moves two centroids by O(1/cluster size). Per-step ("teacher-forced") parity
+therefore feeds the oracle the centroids / assignment the GPU actually used: that comparison is exact
+and is the one that must show zero mismatches. The free-running comparison is reported and gated on
+the near-tie rule for the first assignment and on cluster-count conservation afterwards.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+AOS, SOA = 0, 1
+CENTROID_RTOL = 1e-4   # relative to the rms centroid coordinate
+NEAR_TIE = 1e-5        # relative gap between best and second-best reference distance
+
+
+def rel_err(got, want):
+    scale = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
+    return float(np.abs(got.astype(np.float64) - want).max() / max(scale, 1e-30))
+
+
+def gpu_assign(km, variant, data, means, dim, k, n, layout=AOS, layout_means=AOS, exec_params=None):
+    alg = km.HipAssignmentAlgorithm(variant, exec_params, layout, layout_means)
+    alg.initialize(dim, k, n, data, means)
+    alg.run()
+    out = alg.getAssignment()
+    rechecked = km.last_rechecked()
+    alg.cleanup()
+    return out, rechecked
+
+
+def gpu_update(km, variant, data, assignment, dim, k, n, layout=AOS, layout_means=AOS, exec_params=None):
+    ex = exec_params if exec_params is not None else km.ExecParams()
+    copies = max(1, ex.privatized_copies)
+    d = km.DeviceBuffer(4 * max(data.size, 1)); d.write(data)
+    a = km.DeviceBuffer(4 * max(n, 1)); a.write(assignment)
+    msize = km.layout_size(layout_means, k, dim)
+    m = km.DeviceBuffer(4 * msize * copies); m.zero()
+    s = km.DeviceBuffer(4 * k); s.zero()
+    km.update(variant, d, layout, km.layout_stride(layout, n, dim), a, m, layout_means,
+              km.layout_stride(layout_means, k, dim), s, dim, k, n, ex)
+    km.sync()
+    means, sizes = m.read(np.float32, msize), s.read(np.uint32, k)
+    for b in (d, a, m, s):
+        b.free()
+    return means, sizes
+
+
+def variants(km):
+    return [km.ASSIGN_BASE, km.ASSIGN_MFMA, km.ASSIGN_BEST]
+
+
+# ---------------------------------------------------------------- golden vectors of the reference
+
+@pytest.fixture(scope="module")
+def golden():
+    with open(os.path.join(HERE, "golden", "golden_index.json")) as f:
+        index = json.load(f)
+    return index, np.load(os.path.join(HERE, "golden", "golden.npz"))
+
+
+@pytest.mark.parametrize("name", ["cfg1_full", "cfg1_soa_soa", "cfg1_aos_soa", "cfg1_soa_aos", "cfg2_small",
+                                  "cfg3_small", "cfg5_small"])
+def test_first_pass_equals_reference_golden(km, gpu, golden, name):
+    """One assignment pass from the initial centroids against the REFERENCE's own output (bit-exact)."""
+    index, arrays = golden
+    c = index[name]
+    spec = km.baseline_config(c["config"])
+    data = km.generate_points(spec, c["n"], layout=c["layout"])
+    means0 = km.first_k_means(spec, c["layout_means"])
+    want = arrays[name + "_assignment_first_pass"].astype(np.uint32)
+    for v in variants(km):
+        got, _ = gpu_assign(km, v, data, means0, c["dim"], c["k"], c["n"], c["layout"], c["layout_means"])
+        assert np.array_equal(got, want), "variant %d: %d mismatches" % (v, int((got != want).sum()))
+
+
+# ---------------------------------------------------------------- single-step parity on awkward shapes
+
+SHAPES = [
+    (20, 128, 10240),   # the reference CLI's defaults (k-means.cpp:298-300)
+    (3, 5, 257),        # odd everything
+    (7, 33, 1000),
+    (2, 2, 128),        # the CLI's minima
+    (16, 16, 5000),
+    (32, 1000, 4099),   # k not a multiple of the tile, n prime
+    (64, 96, 2048),
+    (1, 7, 300),
+    (5, 4100, 777),     # centroids do not fit one LDS chunk of the narrow layout
+]
+
+
+@pytest.mark.parametrize("dim,k,n", SHAPES)
+@pytest.mark.parametrize("layout,layout_means", [(AOS, AOS), (SOA, SOA), (AOS, SOA), (SOA, AOS)])
+def test_assignment_is_bit_exact(km, orc, gpu, dim, k, n, layout, layout_means):
+    rng = np.random.default_rng(dim * 7919 + k)
+    data = rng.normal(size=n * dim).astype(np.float32) * np.float32(3)
+    means = data.reshape(-1)[:k * dim].copy() if n >= k and layout == AOS and layout_means == AOS \
+        else rng.normal(size=k * dim).astype(np.float32) * np.float32(3)
+    want = orc.assign(data, means, dim, k, n, layout, layout_means, threads=0, fast=True)
+    for v in variants(km):
+        got, _ = gpu_assign(km, v, data, means, dim, k, n, layout, layout_means)
+        bad = np.nonzero(got != want)[0]
+        assert bad.size == 0, "variant %d: %d mismatches, first at %s" % (v, bad.size, bad[:5])
+
+
+@pytest.mark.parametrize("dim,k,n", [(8, 64, 4096), (32, 256, 3000), (4, 512, 2000)])
+def test_hard_inputs(km, orc, gpu, dim, k, n):
+    """Exact ties, duplicated centroids, coincident points, NaN / inf / huge / tiny values."""
+    rng = np.random.default_rng(99 + dim)
+    base = rng.normal(size=(n, dim)).astype(np.float32)
+    means = rng.normal(size=(k, dim)).astype(np.float32)
+    cases = {}
+    m = means.copy(); m[k // 2] = m[3]; m[k - 1] = m[3]; m[7] = m[5]
+    d = base.copy(); d[: k] = m                              # points exactly on (duplicated) centroids
+    d[k: 2 * k] = (m + m[::-1]) / np.float32(2)              # midpoints: exact or near ties
+    cases["duplicates_and_midpoints"] = (d, m)
+    cases["all_points_identical"] = (np.repeat(base[:1], n, 0), means)
+    cases["all_centroids_identical"] = (base, np.repeat(means[:1], k, 0))
+    d = base.copy(); d[5, 0] = np.nan; d[9, dim - 1] = np.inf; d[11, 0] = -np.inf
+    cases["nan_inf_points"] = (d, means)
+    m = means.copy(); m[4, 1] = np.nan
+    cases["nan_centroid"] = (base, m)
+    m = means.copy(); m[0, 0] = np.nan
+    cases["nan_centroid_zero"] = (base, m)
+    m = means.copy(); m[6, 0] = np.inf
+    cases["inf_centroid"] = (base, m)
+    cases["huge"] = (base * np.float32(1e18), means * np.float32(1e18))       # squares overflow to inf
+    cases["large"] = (base * np.float32(1e6) + np.float32(1e7), means * np.float32(1e6) + np.float32(1e7))
+    cases["tiny"] = (base * np.float32(1e-25), means * np.float32(1e-25))     # squares underflow
+    cases["grid_ties"] = (np.round(base * 2) / 2, np.round(means * 2) / 2)    # many exactly equal distances
+    for name, (d, m) in cases.items():
+        d = np.ascontiguousarray(d, dtype=np.float32).ravel()
+        m = np.ascontiguousarray(m, dtype=np.float32).ravel()
+        want = orc.assign(d, m, dim, k, n, threads=0, fast=True)
+        for v in variants(km):
+            got, rechecked = gpu_assign(km, v, d, m, dim, k, n)
+            bad = np.nonzero(got != want)[0]
+            assert bad.size == 0, "%s, variant %d: %d mismatches, first at %s (gpu %s, oracle %s)" % (
+                name, v, bad.size, bad[:5], got[bad[:5]], want[bad[:5]])
+
+
+def test_sqrt_is_correctly_rounded_on_device(km, orc, gpu):
+    """The exact pass compares sqrt values: a 1-ulp device sqrt would flip ties. d = 1, k = n centroids such
+    that point i's nearest candidates have adjacent squared distances; also a direct sweep through BASE."""
+    rng = np.random.default_rng(5)
+    n, k = 4096, 64
+    data = rng.uniform(0.5, 100, size=n).astype(np.float32)
+    means = np.sort(rng.uniform(0, 200, size=k).astype(np.float32))
+    want = orc.assign(data, means, 1, k, n)
+    for v in variants(km):
+        got, _ = gpu_assign(km, v, data, means, 1, k, n)
+        assert np.array_equal(got, want)
+
+
+def test_empty_input_and_argument_errors(km, gpu):
+    ex = km.ExecParams()
+    d = km.DeviceBuffer(64); m = km.DeviceBuffer(64); a = km.DeviceBuffer(64)
+    km.assign(km.ASSIGN_BEST, d, AOS, 4, m, AOS, 4, a, 4, 2, 0, ex)        # n = 0 is a no-op
+    assert ex.block_count == 0
+    with pytest.raises(km.KmxError) as e:
+        km.assign(99, d, AOS, 4, m, AOS, 4, a, 4, 2, 4, ex)
+    assert e.value.code == km.KMX_ERR_INVALID_ARGUMENT
+    with pytest.raises(km.KmxError) as e:
+        km.assign(km.ASSIGN_BEST, d, AOS, 2, m, AOS, 4, a, 4, 2, 4, ex)    # stride < dim
+    assert e.value.code == km.KMX_ERR_INVALID_ARGUMENT
+    with pytest.raises(km.KmxError) as e:
+        km.assign(km.ASSIGN_MFMA, d, AOS, 100, m, AOS, 100, a, 100, 2, 1, ex)  # dim beyond the MFMA variant
+    assert e.value.code == km.KMX_ERR_UNSUPPORTED
+    km.sync()
+    for b in (d, m, a):
+        b.free()
+
+
+# ---------------------------------------------------------------- update
+
+UPDATE_SHAPES = [(8, 64, 65536), (20, 128, 10240), (3, 5, 257), (32, 1024, 50000), (4, 4096, 100000),
+                 (16, 16, 300000), (256, 1024, 4096), (33, 7, 1000), (2, 70000, 4096)]
+
+
+@pytest.mark.parametrize("dim,k,n", UPDATE_SHAPES)
+@pytest.mark.parametrize("layout,layout_means", [(AOS, AOS), (SOA, SOA), (AOS, SOA), (SOA, AOS)])
+def test_update_matches_oracle(km, orc, gpu, dim, k, n, layout, layout_means):
+    rng = np.random.default_rng(k + dim)
+    data = rng.normal(size=n * dim).astype(np.float32) * np.float32(5) + np.float32(2)
+    # skewed assignment with empty clusters: cluster 1 (if any) never occurs, low indices are hot
+    asg = np.minimum((rng.exponential(scale=k / 4, size=n)).astype(np.uint32), k - 1).astype(np.uint32)
+    if k > 2:
+        asg[asg == 1] = 0
+    want_means, want_sizes = orc.update(data, asg, dim, k, n, layout, layout_means, threads=0)
+    for variant, ex in [(km.UPDATE_ATOMIC_POINT, km.ExecParams()), (km.UPDATE_ATOMIC_FINE, km.ExecParams()),
+                        (km.UPDATE_ATOMIC_SHM, km.ExecParams()),
+                        (km.UPDATE_ATOMIC_FINE, km.ExecParams(privatized_copies=3, items_per_thread=4)),
+                        (km.UPDATE_ATOMIC_SHM, km.ExecParams(shared_mem_bytes=48 * 1024))]:
+        means, sizes = gpu_update(km, variant, data, asg, dim, k, n, layout, layout_means, ex)
+        assert np.array_equal(sizes, want_sizes), "variant %d: counts differ" % variant
+        assert rel_err(means, want_means) < CENTROID_RTOL, "variant %d" % variant
+        if k > 2:
+            lm = means.reshape(k, dim) if layout_means == AOS else means.reshape(dim, k).T
+            assert np.all(lm[1] == 0), "empty cluster must stay at the origin"
+
+
+# ---------------------------------------------------------------- the Lloyd loop
+
+def forced_run(km, orc, cid, n, iters, av, uv, layout=AOS, layout_means=AOS):
+    """Runs the GPU loop and checks every step against the oracle fed with the GPU's own inputs."""
+    spec = km.baseline_config(cid)
+    dim, k = spec.dim, spec.k
+    data = km.generate_points(spec, n, layout=layout)
+    means0 = km.first_k_means(spec, layout_means)
+    alg = km.HipKMeansAlgorithm(av, uv, layout=layout, layout_means=layout_means)
+    alg.initialize(dim, k, n, iters, data, means0)
+    report = []
+    for it in range(iters):
+        prev = alg.getMeans()
+        nxt = alg.iteration()
+        rechecked = km.last_rechecked()
+        ga = alg.cu_assignment[nxt].read(np.uint32, n)
+        oa = orc.assign(data, prev, dim, k, n, layout, layout_means, threads=0, fast=True)
+        alg.update_step(nxt)
+        gm, gs = alg.getMeans(), alg.getClusterSizes()
+        om, osz = orc.update(data, ga, dim, k, n, layout, layout_means, threads=0)
+        report.append(dict(iteration=it, rechecked=rechecked, mismatches=int((ga != oa).sum()),
+                           counts_equal=bool(np.array_equal(gs, osz)), centroid_err=rel_err(gm, om)))
+    alg.cleanup()
+    return report
+
+
+LOOP_CASES = [(1, 65536, 10), (2, 65536, 4), (3, 131072, 3), (5, 1 << 20, 4), (4, 8192, 2)]
+
+
+@pytest.mark.parametrize("cid,n,iters", LOOP_CASES)
+def test_every_iteration_matches_oracle(km, orc, gpu, cid, n, iters):
+    spec = km.baseline_config(cid)
+    combos = [(km.ASSIGN_BEST, km.UPDATE_ATOMIC_SHM)]
+    if spec.dim <= 64:
+        combos += [(km.ASSIGN_MFMA, km.UPDATE_ATOMIC_FINE)]
+    if n * spec.k * spec.dim <= 1 << 31:
+        combos += [(km.ASSIGN_BASE, km.UPDATE_ATOMIC_POINT)]
+    for av, uv in combos:
+        for r in forced_run(km, orc, cid, n, iters, av, uv):
+            assert r["mismatches"] == 0 and r["counts_equal"], (av, uv, r)
+            assert r["centroid_err"] < CENTROID_RTOL, (av, uv, r)
+
+
+def test_free_running_loop_reports_only_near_ties(km, orc, gpu):
+    """Whole run against the oracle's whole run (config 1 in full, as the reference's --verify does,
+    k-means.cpp:171-182). The first assignment must be identical. After that the runs may part at near-ties;
+    every point that differs in the last assignment is classified with the oracle's own distances against
+    the centroids the oracle used."""
+    spec = km.baseline_config(1)
+    n, dim, k, iters = int(spec.n), spec.dim, spec.k, spec.iterations
+    data, means0 = km.generate_points(spec), km.first_k_means(spec)
+    alg = km.HipKMeansAlgorithm(km.ASSIGN_BEST, km.UPDATE_ATOMIC_SHM)
+    alg.initialize(dim, k, n, iters, data, means0)
+    alg.run()
+    gm, ga, gs = alg.getMeans(), alg.getAssignment(), alg.getClusterSizes()
+    alg.cleanup()
+    om, oa, osz = orc.kmeans(data, means0, dim, k, n, iters, threads=0, fast=True)
+    assert int(gs.sum()) == n and np.array_equal(gs, np.bincount(ga, minlength=k).astype(np.uint32))
+    differ = np.nonzero(ga != oa)[0]
+    print("free-running config 1: %d of %d points differ after %d iterations; centroid error %.3e"
+          % (differ.size, n, iters, rel_err(gm, om)))
+    # a point may only differ because the two runs' centroids differ; bound the damage
+    assert differ.size <= n // 1000
+    if differ.size == 0:
+        assert np.array_equal(gs, osz) and rel_err(gm, om) < CENTROID_RTOL
+
+
+# ---------------------------------------------------------------- full benchmark sizes: size-independent properties
+
+@pytest.mark.parametrize("cid", [2, 3, 5])
+def test_full_size_properties(km, orc, gpu, cid):
+    spec = km.baseline_config(cid)
+    n, dim, k = int(spec.n), spec.dim, spec.k
+    data, means0 = km.generate_points(spec), km.first_k_means(spec)
+    alg = km.HipKMeansAlgorithm(km.ASSIGN_BEST, km.UPDATE_ATOMIC_SHM)
+    alg.initialize(dim, k, n, 2, data, means0)
+    alg.run(iters=1)
+    means1 = alg.getMeans()
+    nxt = alg.iteration()                      # second assignment, against means1
+    ga = alg.cu_assignment[nxt].read(np.uint32, n)
+    rechecked = km.last_rechecked()
+    alg.update_step(nxt)
+    km.sync()
+    gm, gs = alg.getMeans(), alg.getClusterSizes()
+    # idempotence: assigning again against the same centroids gives the same vector
+    again, _ = gpu_assign(km, km.ASSIGN_BEST, data, means1, dim, k, n)
+    assert np.array_equal(again, ga)
+    alg.cleanup()
+    # counts are the histogram of the assignment and sum to n
+    assert ga.max() < k
+    hist = np.bincount(ga, minlength=k).astype(np.uint32)
+    assert np.array_equal(gs, hist) and int(gs.sum()) == n
+    # centroid * count = sum of members (float64 recomputation, independent of any fp32 order)
+    pts = data.reshape(n, dim)
+    sums = np.stack([np.bincount(ga, weights=pts[:, d].astype(np.float64), minlength=k) for d in range(dim)], 1)
+    want = np.where(hist[:, None] > 0, sums / np.maximum(hist, 1)[:, None], 0.0)
+    assert rel_err(gm.reshape(k, dim), want) < CENTROID_RTOL
+    # exact oracle on a seeded sample of points, all k centroids
+    rng = np.random.default_rng(cid)
+    sample = np.sort(rng.choice(n, size=min(n, 200000 // max(1, k // 64)), replace=False))
+    want_s = orc.assign(np.ascontiguousarray(pts[sample]).ravel(), means1, dim, k, sample.size, threads=0, fast=True)
+    assert np.array_equal(ga[sample], want_s)
+    # every point is at least as close to its centroid as to a random other one (float64)
+    other = rng.integers(0, k, size=sample.size)
+    c = means1.reshape(k, dim).astype(np.float64)
+    x = pts[sample].astype(np.float64)
+    d_own = ((x - c[ga[sample]]) ** 2).sum(1)
+    d_other = ((x - c[other]) ** 2).sum(1)
+    assert np.all(d_own <= d_other * (1 + 1e-5) + 1e-12)
+    assert rechecked < n // 10
