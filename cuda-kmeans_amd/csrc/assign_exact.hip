@@ -54,45 +54,91 @@ assign_base_kernel(const float* __restrict__ data, size_t stride, const float* _
 }
 
 /*
- * One wavefront per queued point. Lane l evaluates centroids l, l+64, ... in ascending order and
- * keeps its own (distance, index) minimum; the 64 candidates are merged by (smaller distance, then
- * smaller index), which is the serial scan's result: the first centroid attaining the minimum.
- * A NaN distance to centroid 0 pins the point to centroid 0, as `minDist > dist` is then never true.
+ * Exact pass over the queued points. A group of L lanes (L = 16, 32 or 64, chosen from k) owns a batch of PB
+ * queued points: the points' coordinates are staged in LDS (every lane of the group reads the same
+ * word: a broadcast), lane l evaluates centroids l, l+L, ... in ascending order against all PB points
+ * (one coalesced load of the transposed centroid block per (centroid, dim), reused PB times) and keeps its
+ * own (distance, index) minimum per point; the L candidates are merged by (smaller distance, then smaller
+ * index), which is the serial scan's result: the first centroid attaining the minimum. A NaN distance to
+ * centroid 0 pins the point to centroid 0, as `minDist > dist` is then never true.
+ * means_t is the exact transposed copy [dim][kp] written by pack_means_kernel.
  */
-template <int LD, int LM>
+template <int LD, int L, int PB>
 __global__ void __launch_bounds__(256)
-recheck_kernel(const float* __restrict__ data, size_t stride, const float* __restrict__ means, size_t stride_means,
+recheck_kernel(const float* __restrict__ data, size_t stride, const float* __restrict__ means_t, uint32_t kp,
                uint32_t* __restrict__ assignment, uint32_t dim, uint32_t k,
                const uint32_t* __restrict__ queue, const uint32_t* __restrict__ counters)
 {
-	const uint32_t lane = threadIdx.x & (WAVE - 1);
-	const uint32_t wave = (blockIdx.x * blockDim.x + threadIdx.x) / WAVE;
-	const uint32_t waves = gridDim.x * blockDim.x / WAVE;
+	extern __shared__ float xs[];
+	constexpr uint32_t GROUPS = 256 / L;
+	const uint32_t group = threadIdx.x / L;
+	const uint32_t gl = threadIdx.x % L;
+	float* gx = xs + (size_t)group * PB * dim;
 	const uint32_t count = counters[0];
+	const uint32_t batches = (count + PB - 1) / PB;
 
-	for (uint32_t q = wave; q < count; q += waves) {
-		const uint32_t idx = queue[q];
-		float best = __builtin_inff();
-		uint32_t bestIdx = 0xFFFFFFFFu;
-		for (uint32_t m = lane; m < k; m += WAVE) {
-			float dist = exact_distance<LD, LM>(data, stride, idx, means, stride_means, m, dim);
-			if (dist < best || (dist == best && m < bestIdx)) {
-				best = dist;
-				bestIdx = m;
+	for (uint32_t first = blockIdx.x * GROUPS; first < batches; first += gridDim.x * GROUPS) {
+		const uint32_t batch = first + group;
+		const bool active = batch < batches;
+		__syncthreads(); /* the previous batch's coordinates are no longer needed */
+		if (active) {
+			for (uint32_t i = gl; i < PB * dim; i += L) {
+				const uint32_t p = i / dim, d = i - p * dim;
+				const uint32_t idx = queue[min(batch * PB + p, count - 1)];
+				gx[i] = data[elem<LD>(stride, idx, d)];
 			}
 		}
-		/* is the distance to centroid 0 NaN? (every lane repeats that one sum; the point index is wave-uniform) */
-		float d0 = exact_distance<LD, LM>(data, stride, idx, means, stride_means, 0, dim);
-		bool pinned = d0 != d0;
-		for (int off = WAVE / 2; off > 0; off >>= 1) {
-			float ob = __shfl_xor(best, off);
-			uint32_t oi = __shfl_xor(bestIdx, off);
-			if (ob < best || (ob == best && oi < bestIdx)) {
-				best = ob;
-				bestIdx = oi;
+		__syncthreads();
+		if (!active) continue;
+
+		float best[PB];
+		uint32_t bestIdx[PB];
+		uint32_t pinned = 0;
+#pragma unroll
+		for (int p = 0; p < PB; ++p) {
+			best[p] = __builtin_inff();
+			bestIdx[p] = 0xFFFFFFFFu;
+		}
+		for (uint32_t m = gl; m < k; m += L) {
+			float sum[PB];
+#pragma unroll
+			for (int p = 0; p < PB; ++p) sum[p] = 0.0f;
+			for (uint32_t d = 0; d < dim; ++d) {
+				const float c = means_t[(size_t)d * kp + m];
+#pragma unroll
+				for (int p = 0; p < PB; ++p) {
+					float diff = gx[p * dim + d] - c;
+					float sq = diff * diff;
+					sum[p] = sum[p] + sq;
+				}
+			}
+#pragma unroll
+			for (int p = 0; p < PB; ++p) {
+				float dist = __builtin_sqrtf(sum[p]);
+				if (m == 0 && dist != dist) pinned |= 1u << p;
+				if (dist < best[p] || (dist == best[p] && m < bestIdx[p])) {
+					best[p] = dist;
+					bestIdx[p] = m;
+				}
 			}
 		}
-		if (lane == 0) assignment[idx] = pinned ? 0u : (bestIdx == 0xFFFFFFFFu ? 0u : bestIdx);
+		pinned = (uint32_t)__shfl((int)pinned, 0, L); /* lane 0 of the group evaluated centroid 0 */
+#pragma unroll
+		for (int p = 0; p < PB; ++p) {
+			for (int off = L / 2; off > 0; off >>= 1) {
+				float ob = __shfl_xor(best[p], off, L);
+				uint32_t oi = (uint32_t)__shfl_xor((int)bestIdx[p], off, L);
+				if (ob < best[p] || (ob == best[p] && oi < bestIdx[p])) {
+					best[p] = ob;
+					bestIdx[p] = oi;
+				}
+			}
+			const uint32_t q = batch * PB + p;
+			if (gl == 0 && q < count) {
+				const bool pin = (pinned >> p) & 1u;
+				assignment[queue[q]] = (pin || bestIdx[p] == 0xFFFFFFFFu) ? 0u : bestIdx[p];
+			}
+		}
 	}
 }
 
@@ -122,22 +168,36 @@ int launch_assign_base(const AssignArgs& a, kmx_exec_params* exec)
 	return launch_base_t<KMX_SOA, KMX_SOA>(a, exec, ws->counters);
 }
 
-template <int LD, int LM>
-static int launch_recheck_t(const AssignArgs& a, Workspace* ws)
+template <int LD, int L, int PB>
+static int launch_recheck_t(const AssignArgs& a, Workspace* ws, uint32_t kp)
 {
 	const unsigned block = 256, blocks = 1024;
-	hipLaunchKernelGGL((recheck_kernel<LD, LM>), dim3(blocks), dim3(block), 0, stream(),
-	                   a.data, a.stride, a.means, a.stride_means, a.assignment, a.dim, a.k, ws->queue, ws->counters);
+	const size_t lds = (size_t)(256 / L) * PB * a.dim * sizeof(float);
+	auto kernel = recheck_kernel<LD, L, PB>;
+	if (lds > 65536) KMX_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+	hipLaunchKernelGGL(kernel, dim3(blocks), dim3(block), lds, stream(),
+	                   a.data, a.stride, ws->means_t, kp, a.assignment, a.dim, a.k, ws->queue, ws->counters);
 	KMX_LAUNCH_CHECK("recheck_kernel");
 	return KMX_OK;
 }
 
-int launch_recheck(const AssignArgs& a, Workspace* ws)
+template <int LD>
+static int launch_recheck_l(const AssignArgs& a, Workspace* ws, uint32_t kp)
 {
-	if (a.layout == KMX_AOS && a.layout_means == KMX_AOS) return launch_recheck_t<KMX_AOS, KMX_AOS>(a, ws);
-	if (a.layout == KMX_AOS && a.layout_means == KMX_SOA) return launch_recheck_t<KMX_AOS, KMX_SOA>(a, ws);
-	if (a.layout == KMX_SOA && a.layout_means == KMX_AOS) return launch_recheck_t<KMX_SOA, KMX_AOS>(a, ws);
-	return launch_recheck_t<KMX_SOA, KMX_SOA>(a, ws);
+	if (a.k >= 48) {
+		if (a.dim <= 512) return launch_recheck_t<LD, 64, 8>(a, ws, kp);
+		return launch_recheck_t<LD, 64, 1>(a, ws, kp);
+	}
+	if (a.k >= 24) return launch_recheck_t<LD, 32, 1>(a, ws, kp);
+	return launch_recheck_t<LD, 16, 1>(a, ws, kp);
+}
+
+int launch_recheck(const AssignArgs& a, Workspace* ws, uint32_t kp)
+{
+	if ((size_t)a.dim * sizeof(float) * 16 > 160 * 1024)
+		return fail(KMX_ERR_UNSUPPORTED, "assign: dim %u is too large for the exact pass", a.dim);
+	if (a.layout == KMX_AOS) return launch_recheck_l<KMX_AOS>(a, ws, kp);
+	return launch_recheck_l<KMX_SOA>(a, ws, kp);
 }
 
 } // namespace kmx

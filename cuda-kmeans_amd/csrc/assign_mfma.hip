@@ -57,7 +57,7 @@ static uint32_t pick_dph(uint32_t dim)
 template <int LM>
 __global__ void __launch_bounds__(256)
 pack_means_kernel(const float* __restrict__ means, size_t stride_means, float* __restrict__ packed, float* __restrict__ norms,
-                  uint32_t dim, uint32_t k, uint32_t kp, uint32_t dp, uint32_t* __restrict__ counters)
+                  float* __restrict__ means_t, uint32_t dim, uint32_t k, uint32_t kp, uint32_t dp, uint32_t* __restrict__ counters)
 {
 	const uint32_t j = blockIdx.x * blockDim.x + threadIdx.x;
 	if (j == 0) counters[0] = 0u; /* the recheck queue of this call starts empty */
@@ -68,6 +68,7 @@ pack_means_kernel(const float* __restrict__ means, size_t stride_means, float* _
 		float v = (j < k && q < dim) ? means[elem<LM>(stride_means, j, q)] : 0.0f;
 		c2 += v * v;
 		packed[(size_t)j * rs + q] = -2.0f * v;
+		if (q < dim) means_t[(size_t)q * kp + j] = v; /* exact copy for the recheck pass */
 	}
 	norms[j] = j < k ? c2 : __builtin_inff();
 }
@@ -311,7 +312,7 @@ int launch_assign_mfma(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws
 	const uint32_t dph = pick_dph(a.dim);
 	const uint32_t dp = 2 * dph;
 	const uint32_t kp = round_up(a.k, TILE);
-	int rc = reserve_packed(ws, (size_t)kp * (dp + ROW_PAD), kp);
+	int rc = reserve_packed(ws, (size_t)kp * (dp + ROW_PAD), kp, (size_t)kp * a.dim);
 	if (rc) return rc;
 	rc = reserve_queue(ws, a.n);
 	if (rc) return rc;
@@ -319,10 +320,10 @@ int launch_assign_mfma(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws
 	const uint32_t pack_blocks = (kp + 255) / 256;
 	if (a.layout_means == KMX_AOS)
 		hipLaunchKernelGGL((pack_means_kernel<KMX_AOS>), dim3(pack_blocks), dim3(256), 0, stream(),
-		                   a.means, a.stride_means, ws->packed_means, ws->norms, a.dim, a.k, kp, dp, ws->counters);
+		                   a.means, a.stride_means, ws->packed_means, ws->norms, ws->means_t, a.dim, a.k, kp, dp, ws->counters);
 	else
 		hipLaunchKernelGGL((pack_means_kernel<KMX_SOA>), dim3(pack_blocks), dim3(256), 0, stream(),
-		                   a.means, a.stride_means, ws->packed_means, ws->norms, a.dim, a.k, kp, dp, ws->counters);
+		                   a.means, a.stride_means, ws->packed_means, ws->norms, ws->means_t, a.dim, a.k, kp, dp, ws->counters);
 	KMX_LAUNCH_CHECK("pack_means_kernel");
 
 	/* tau = kd (|x|^2 + max|c|^2), kd = (8 d + 64) 2^-23 (see the bound at the top of the file) */
@@ -338,7 +339,7 @@ int launch_assign_mfma(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws
 	default: return fail(KMX_ERR_UNSUPPORTED, "assign (MFMA): dim %u is not supported", a.dim);
 	}
 	if (rc) return rc;
-	return launch_recheck(a, ws);
+	return launch_recheck(a, ws, kp);
 }
 
 } // namespace kmx

@@ -49,11 +49,12 @@ struct Workspace {
 	uint32_t* counters = nullptr;                               /* 16 words */
 	float* packed_means = nullptr;  size_t packed_cap = 0;     /* floats  */
 	float* norms = nullptr;         size_t norms_cap = 0;      /* floats  */
+	float* means_t = nullptr;       size_t means_t_cap = 0;    /* floats: exact transposed centroids [dim][kp] */
 	float* partials = nullptr;      size_t partials_cap = 0;   /* floats  */
 };
 int workspace(Workspace** ws);
 int reserve_queue(Workspace* ws, size_t entries);
-int reserve_packed(Workspace* ws, size_t packed_floats, size_t norm_floats);
+int reserve_packed(Workspace* ws, size_t packed_floats, size_t norm_floats, size_t transposed_floats);
 int reserve_partials(Workspace* ws, size_t floats);
 
 #define KMX_HIP(call)                                                                                         \
@@ -95,8 +96,9 @@ struct UpdateArgs {
 
 /* assign_exact.hip */
 int launch_assign_base(const AssignArgs& a, kmx_exec_params* exec);
-/* Re-evaluates the points listed in ws->queue[0 .. counters[0]) with the serial arithmetic. */
-int launch_recheck(const AssignArgs& a, Workspace* ws);
+/* Re-evaluates the points listed in ws->queue[0 .. counters[0]) with the serial arithmetic, reading the
+ * exact transposed centroids ws->means_t ([dim][kp]) that pack_means wrote for this call. */
+int launch_recheck(const AssignArgs& a, Workspace* ws, uint32_t kp);
 
 /* assign_mfma.hip / assign_lds_fma.hip: return KMX_ERR_UNSUPPORTED (without message side effects
  * beyond kmx_last_error) when the shape does not fit the variant. */

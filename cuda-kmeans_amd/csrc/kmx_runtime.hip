@@ -92,11 +92,13 @@ static int grow(T** ptr, size_t* cap, size_t want)
 
 int reserve_queue(Workspace* ws, size_t entries) { return grow(&ws->queue, &ws->queue_cap, entries); }
 
-int reserve_packed(Workspace* ws, size_t packed_floats, size_t norm_floats)
+int reserve_packed(Workspace* ws, size_t packed_floats, size_t norm_floats, size_t transposed_floats)
 {
 	int rc = grow(&ws->packed_means, &ws->packed_cap, packed_floats);
 	if (rc) return rc;
-	return grow(&ws->norms, &ws->norms_cap, norm_floats);
+	rc = grow(&ws->norms, &ws->norms_cap, norm_floats);
+	if (rc) return rc;
+	return grow(&ws->means_t, &ws->means_t_cap, transposed_floats);
 }
 
 int reserve_partials(Workspace* ws, size_t floats) { return grow(&ws->partials, &ws->partials_cap, floats); }
@@ -107,6 +109,7 @@ static int release_workspace()
 	if (g_ws.counters) KMX_HIP(hipFree(g_ws.counters));
 	if (g_ws.packed_means) KMX_HIP(hipFree(g_ws.packed_means));
 	if (g_ws.norms) KMX_HIP(hipFree(g_ws.norms));
+	if (g_ws.means_t) KMX_HIP(hipFree(g_ws.means_t));
 	if (g_ws.partials) KMX_HIP(hipFree(g_ws.partials));
 	g_ws = Workspace();
 	return KMX_OK;

@@ -1,21 +1,31 @@
 /*
  * Update step: per-cluster sums and counts of the assigned points, then the divide.
  *
- *   update_point_kernel - one lane per point, global atomics
- *                         (counterpart of updateAtomicPointKernel, reference kernels.cu:726-743)
- *   update_fine_kernel  - one lane per (point, dim) element, global atomics
- *                         (counterpart of updateAtomicFineKernel, reference kernels.cu:770-791)
- *   update_lds_kernel   - the tuned variant (counterpart of updateAtomicShmKernel, reference
- *                         kernels.cu:817-858): every work-group owns a contiguous chunk of points and
- *                         a slice of the dimensions, accumulates the WHOLE k x slice block (and the
- *                         counts) in LDS with ds_add, and flushes one aggregated atomic per non-zero
- *                         element to HBM. Points are read exactly once, fully coalesced.
+ *   update_point_kernel   - one lane per point, global atomics
+ *                           (counterpart of updateAtomicPointKernel, reference kernels.cu:726-743)
+ *   update_fine_kernel    - one lane per (point, dim) element, global atomics
+ *                           (counterpart of updateAtomicFineKernel, reference kernels.cu:770-791)
+ *   KMX_UPDATE_ATOMIC_SHM - the tuned variant (counterpart of updateAtomicShmKernel, reference
+ *                           kernels.cu:817-858), three kernels chosen by shape. Measured on gfx950: an LDS
+ *                           ds_add_f32 costs ~194 cycles per wavefront instruction whatever the address
+ *                           pattern (lanes are serialised), ds_add_u32 4.4 cycles, a plain LDS
+ *                           read-add-write 8.2 cycles. Floating-point LDS atomics are therefore avoided:
+ *       update_private_kernel  small k*dim: every lane group (one lane per dimension) owns a PRIVATE copy
+ *                              of the k x dim block in LDS and accumulates with plain read-add-write; the
+ *                              copies are merged at the end, one global atomic per element and work-group.
+ *       update_sorted_kernel   larger k: the work-group counting-sorts its chunk of points by cluster
+ *                              with integer LDS atomics, then lane groups walk the sorted list and sum each
+ *                              cluster's rows in registers (no atomics at all); per-chunk sums go to a partial
+ *                              buffer with plain coalesced stores and reduce_partials_kernel folds them.
+ *       update_lds_kernel      fallback for the shapes/layouts the two above do not take (SoA points):
+ *                              LDS-privatised ds_add_f32.
+ *     Points are read exactly once in all three.
  *   reduce_copies_kernel / divide_means_kernel
- *                       - counterparts of reducePrivCopiesKernel / divideMeansKernel
- *                         (reference kernels.cu:115-135,149-163); empty clusters keep their zero.
+ *                         - counterparts of reducePrivCopiesKernel / divideMeansKernel
+ *                           (reference kernels.cu:115-135,149-163); empty clusters keep their zero.
  *
- * Sums are fp32 and their order differs from the serial order (atomics), exactly as in the
- * reference's GPU path; counts are integers and exact.
+ * Sums are fp32 and their order differs from the serial order, exactly as in the reference's GPU path
+ * (atomics); counts are integers and exact.
  */
 #include "kmx_internal.h"
 
@@ -172,6 +182,230 @@ update_lds_kernel(const float* __restrict__ data, size_t stride, const uint32_t*
 	}
 }
 
+/*
+ * Small k*dim. Lane group = GW lanes (GW = power of two >= dim), lane gl < dim owns dimension gl. Every group
+ * has a private block [k*dim sums | k counts] in LDS; consecutive groups take consecutive points, so a
+ * wavefront reads 64/GW consecutive rows per step. LDS operations of one wavefront execute in order, so a
+ * plain read-add-write is correct even when consecutive points fall into the same cluster. copy_stride is
+ * chosen so that the groups of one wavefront start GW banks apart: equal targets (the hot-cluster case) are
+ * conflict-free.
+ */
+template <int LM>
+__global__ void __launch_bounds__(256)
+update_private_kernel(const float* __restrict__ data, size_t stride, const uint32_t* __restrict__ assignment,
+                      float* __restrict__ means, size_t stride_means, uint32_t* __restrict__ sizes,
+                      uint32_t dim, uint32_t k, uint32_t n, uint32_t gw, uint32_t copy_stride, uint32_t chunk_points)
+{
+	extern __shared__ float lds[];
+	const uint32_t groups = blockDim.x / gw;
+	const uint32_t group = threadIdx.x / gw;
+	const uint32_t gl = threadIdx.x - group * gw;
+	for (uint32_t i = threadIdx.x; i < groups * copy_stride; i += blockDim.x) lds[i] = 0.0f;
+	__syncthreads();
+
+	float* acc = lds + (size_t)group * copy_stride;
+	uint32_t* cnt = (uint32_t*)(acc + (size_t)k * dim);
+	const uint32_t p_begin = (uint32_t)min((uint64_t)blockIdx.x * chunk_points, (uint64_t)n);
+	const uint32_t p_end = (uint32_t)min((uint64_t)p_begin + chunk_points, (uint64_t)n);
+	const bool lane_on = gl < dim;
+	const float* src = data + (lane_on ? gl : 0);
+	uint32_t p = p_begin + group;
+	for (; p + (UPDATE_UNROLL - 1) * groups < p_end; p += UPDATE_UNROLL * groups) {
+		float v[UPDATE_UNROLL];
+		uint32_t t[UPDATE_UNROLL];
+#pragma unroll
+		for (int u = 0; u < UPDATE_UNROLL; ++u) {
+			v[u] = src[(size_t)(p + u * groups) * stride];
+			t[u] = assignment[p + u * groups];
+		}
+#pragma unroll
+		for (int u = 0; u < UPDATE_UNROLL; ++u) {
+			if (lane_on) acc[t[u] * dim + gl] += v[u];
+			if (gl == 0) cnt[t[u]] += 1u;
+		}
+	}
+	for (; p < p_end; p += groups) {
+		float v = src[(size_t)p * stride];
+		uint32_t t = assignment[p];
+		if (lane_on) acc[t * dim + gl] += v;
+		if (gl == 0) cnt[t] += 1u;
+	}
+	__syncthreads();
+
+	for (uint32_t e = threadIdx.x; e < k * dim; e += blockDim.x) {
+		float s = 0.0f;
+		for (uint32_t g = 0; g < groups; ++g) s += lds[(size_t)g * copy_stride + e];
+		const uint32_t c = e / dim, d = e - c * dim;
+		if (s != 0.0f) atomic_add_f32(&means[elem<LM>(stride_means, c, d)], s);
+	}
+	for (uint32_t c = threadIdx.x; c < k; c += blockDim.x) {
+		uint32_t s = 0;
+		for (uint32_t g = 0; g < groups; ++g) s += ((const uint32_t*)lds)[(size_t)g * copy_stride + (size_t)k * dim + c];
+		if (s) atomicAdd(&sizes[c], s);
+	}
+}
+
+/*
+ * Larger k. Grid = (point chunks, 32-wide dimension slices); work-group = 1024 lanes.
+ *   1. histogram of the chunk's assignments with ds_add_rtn_u32 (the returned value is the point's rank
+ *      inside its cluster); 2. exclusive scan -> cluster offsets; 3. scatter (cluster << 15 | local index)
+ *      into the sorted list; 4. the sorted list is cut into one range of whole clusters per lane group
+ *      (groups of GW lanes, lane = dimension), balanced by entry count; a group walks its range in batches
+ *      of 8 entries (8 row loads in flight), adds in a register and stores a cluster's row of sums when the
+ *      cluster changes -- zero rows for clusters without members, so the partial buffer needs no clearing.
+ * Per-chunk counts go to cluster_sizes with integer global atomics (dimension slice 0 only).
+ * partial layout: [chunk][cluster][dim].
+ */
+constexpr uint32_t SORT_SHIFT = 15; /* local point index bits: chunk_points <= 32768 */
+
+template <int ITEMS, int GW>
+__global__ void __launch_bounds__(1024)
+update_sorted_kernel(const float* __restrict__ data, size_t stride, const uint32_t* __restrict__ assignment,
+                     float* __restrict__ partial, uint32_t* __restrict__ sizes,
+                     uint32_t dim, uint32_t k, uint32_t n, uint32_t chunk_points)
+{
+	extern __shared__ uint32_t sm[];
+	uint32_t* offsets = sm;                   /* k + 1 words: histogram, then exclusive offsets */
+	uint32_t* scratch = sm + k + 1;           /* 32 words */
+	uint32_t* sorted = scratch + 32;          /* chunk_points words */
+	const uint32_t tid = threadIdx.x;
+	const uint32_t lane = tid & (WAVE - 1), wave = tid / WAVE;
+	const uint32_t p_begin = (uint32_t)min((uint64_t)blockIdx.x * chunk_points, (uint64_t)n);
+	const uint32_t count = min(chunk_points, n - p_begin);
+	const uint32_t d0 = blockIdx.y * 32;
+	const uint32_t width = min(32u, dim - d0);
+
+	for (uint32_t i = tid; i <= k; i += 1024) offsets[i] = 0;
+	__syncthreads();
+
+	/* 1. histogram + rank */
+	uint32_t target[ITEMS], rank[ITEMS];
+#pragma unroll
+	for (int it = 0; it < ITEMS; ++it) {
+		const uint32_t i = it * 1024 + tid;
+		target[it] = i < count ? assignment[p_begin + i] : 0xFFFFFFFFu;
+	}
+#pragma unroll
+	for (int it = 0; it < ITEMS; ++it) {
+		rank[it] = 0;
+		if (target[it] < k) rank[it] = atomicAdd(&offsets[target[it]], 1u);
+	}
+	__syncthreads();
+
+	/* counts of this chunk */
+	if (blockIdx.y == 0)
+		for (uint32_t c = tid; c < k; c += 1024) {
+			const uint32_t s = offsets[c];
+			if (s) atomicAdd(&sizes[c], s);
+		}
+
+	/* 2. exclusive scan of offsets[0..k) in place; offsets[k] = number of entries */
+	const uint32_t per = (k + 1023) / 1024;
+	const uint32_t b = tid * per;
+	uint32_t local = 0;
+	for (uint32_t i = 0; i < per; ++i)
+		if (b + i < k) local += offsets[b + i];
+	uint32_t incl = local;
+	for (int off = 1; off < WAVE; off <<= 1) {
+		const uint32_t up = (uint32_t)__shfl_up((int)incl, off);
+		if (lane >= (uint32_t)off) incl += up;
+	}
+	if (lane == WAVE - 1) scratch[wave] = incl;
+	__syncthreads();
+	uint32_t wave_prefix = 0;
+	for (uint32_t w = 0; w < wave; ++w) wave_prefix += scratch[w];
+	uint32_t run = wave_prefix + incl - local;
+	for (uint32_t i = 0; i < per; ++i)
+		if (b + i < k) {
+			const uint32_t c = offsets[b + i];
+			offsets[b + i] = run;
+			run += c;
+		}
+	if (b <= k && k < b + per) offsets[k] = run;        /* the thread that owns the last entries */
+	if (tid == 1023 && b + per <= k) offsets[k] = run;   /* k a multiple of 1024: last thread closes the list */
+	__syncthreads();
+
+	/* 3. scatter */
+#pragma unroll
+	for (int it = 0; it < ITEMS; ++it)
+		if (target[it] < k) sorted[offsets[target[it]] + rank[it]] = (target[it] << SORT_SHIFT) | (uint32_t)(it * 1024 + tid);
+	__syncthreads();
+
+	/* 4. segment sums */
+	constexpr uint32_t GROUPS = 1024 / GW;
+	const uint32_t group = tid / GW, gl = tid % GW;
+	const uint32_t entries = offsets[k];
+	auto first_cluster = [&](uint32_t g) -> uint32_t {
+		/* smallest c in [0, k] with offsets[c] >= g * entries / GROUPS */
+		if (g >= GROUPS) return k;
+		const uint32_t want = (uint32_t)((uint64_t)g * entries / GROUPS);
+		uint32_t lo = 0, hi = k;
+		while (lo < hi) {
+			const uint32_t mid = (lo + hi) / 2;
+			if (offsets[mid] >= want) hi = mid; else lo = mid + 1;
+		}
+		return lo;
+	};
+	const uint32_t c_lo = first_cluster(group), c_hi = first_cluster(group + 1);
+	const bool lane_on = gl < width;
+	const float* src = data + (size_t)p_begin * stride + d0 + (lane_on ? gl : 0);
+	float* out = partial + ((size_t)blockIdx.x * k) * dim + d0 + gl;
+	uint32_t cur = c_lo;
+	float acc = 0.0f;
+	uint32_t e = offsets[c_lo];
+	const uint32_t e_end = offsets[c_hi];
+	for (; e + UPDATE_UNROLL <= e_end; e += UPDATE_UNROLL) {
+		uint32_t ent[UPDATE_UNROLL];
+		float v[UPDATE_UNROLL];
+#pragma unroll
+		for (int u = 0; u < UPDATE_UNROLL; ++u) ent[u] = sorted[e + u];
+#pragma unroll
+		for (int u = 0; u < UPDATE_UNROLL; ++u) v[u] = src[(size_t)(ent[u] & ((1u << SORT_SHIFT) - 1u)) * stride];
+#pragma unroll
+		for (int u = 0; u < UPDATE_UNROLL; ++u) {
+			const uint32_t t = ent[u] >> SORT_SHIFT;
+			while (cur < t) {
+				if (lane_on) out[(size_t)cur * dim] = acc;
+				acc = 0.0f;
+				++cur;
+			}
+			acc += v[u];
+		}
+	}
+	for (; e < e_end; ++e) {
+		const uint32_t ent = sorted[e];
+		const float v = src[(size_t)(ent & ((1u << SORT_SHIFT) - 1u)) * stride];
+		const uint32_t t = ent >> SORT_SHIFT;
+		while (cur < t) {
+			if (lane_on) out[(size_t)cur * dim] = acc;
+			acc = 0.0f;
+			++cur;
+		}
+		acc += v;
+	}
+	while (cur < c_hi) {
+		if (lane_on) out[(size_t)cur * dim] = acc;
+		acc = 0.0f;
+		++cur;
+	}
+}
+
+/* means[c][d] += sum over a share of the chunks of partial[chunk][c][d]; grid = (elements / 256, shares) */
+template <int LM>
+__global__ void __launch_bounds__(256)
+reduce_partials_kernel(const float* __restrict__ partial, float* __restrict__ means, size_t stride_means,
+                       uint32_t dim, uint32_t k, uint32_t chunks)
+{
+	const uint32_t e = blockIdx.x * blockDim.x + threadIdx.x;
+	if (e >= k * dim) return;
+	const uint32_t per = (chunks + gridDim.y - 1) / gridDim.y;
+	const uint32_t c0 = blockIdx.y * per, c1 = min(c0 + per, chunks);
+	float s = 0.0f;
+	for (uint32_t c = c0; c < c1; ++c) s += partial[(size_t)c * k * dim + e];
+	const uint32_t cl = e / dim, d = e - cl * dim;
+	if (s != 0.0f) atomic_add_f32(&means[elem<LM>(stride_means, cl, d)], s);
+}
+
 template <int LM>
 __global__ void __launch_bounds__(256)
 reduce_copies_kernel(float* __restrict__ means, size_t stride_means, size_t copy_floats, uint32_t dim, uint32_t k, uint32_t copies)
@@ -207,8 +441,123 @@ static size_t copy_floats_of(const UpdateArgs& u)
 	return u.layout_means == KMX_AOS ? (size_t)u.k * u.stride_means : (size_t)u.dim * u.stride_means;
 }
 
+static uint32_t pow2_at_least(uint32_t v)
+{
+	uint32_t p = 1;
+	while (p < v) p <<= 1;
+	return p;
+}
+
+template <int ITEMS, int LM>
+static int launch_sorted(const UpdateArgs& u, Workspace* ws, uint32_t chunks, uint32_t slices, uint32_t chunk_points, uint32_t gw, uint32_t lds_bytes)
+{
+	void (*kernel)(const float*, size_t, const uint32_t*, float*, uint32_t*, uint32_t, uint32_t, uint32_t, uint32_t) = nullptr;
+	switch (gw) {
+	case 4: kernel = update_sorted_kernel<ITEMS, 4>; break;
+	case 8: kernel = update_sorted_kernel<ITEMS, 8>; break;
+	case 16: kernel = update_sorted_kernel<ITEMS, 16>; break;
+	default: kernel = update_sorted_kernel<ITEMS, 32>; break;
+	}
+	KMX_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+	hipLaunchKernelGGL(kernel, dim3(chunks, slices), dim3(1024), lds_bytes, stream(),
+	                   u.data, u.stride, u.assignment, ws->partials, u.cluster_sizes, u.dim, u.k, u.n, chunk_points);
+	KMX_LAUNCH_CHECK("update_sorted_kernel");
+	const uint32_t total = u.k * u.dim;
+	const uint32_t shares = std::max<uint32_t>(1, std::min<uint32_t>(chunks, 8));
+	hipLaunchKernelGGL((reduce_partials_kernel<LM>), dim3((total + 255) / 256, shares), dim3(256), 0, stream(),
+	                   ws->partials, u.means, u.stride_means, u.dim, u.k, chunks);
+	KMX_LAUNCH_CHECK("reduce_partials_kernel");
+	return KMX_OK;
+}
+
+/* Picks and launches the kernel of KMX_UPDATE_ATOMIC_SHM; *done = false if no LDS variant fits the shape. */
 template <int LD, int LM>
-static int launch_update_t(int variant, const UpdateArgs& u, kmx_exec_params* exec, const DeviceInfo& dev)
+static int launch_update_tuned(const UpdateArgs& u, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev, bool* done)
+{
+	*done = true;
+	const uint32_t budget = exec->shared_mem_bytes ? std::min(exec->shared_mem_bytes, dev.lds_bytes) : dev.lds_bytes;
+
+	if (LD == KMX_AOS && u.dim <= 64) {
+		/* private copies: 256 / gw groups, each k*dim sums + k counts, padded so that groups start gw banks apart */
+		const uint32_t gw = pow2_at_least(u.dim);
+		const uint32_t groups = 256 / gw;
+		const uint64_t copy_words = (uint64_t)u.k * (u.dim + 1);
+		const uint64_t copy_stride = (copy_words + 63) / 64 * 64 + gw;
+		const uint64_t lds_bytes = groups * copy_stride * 4;
+		if (lds_bytes <= std::min<uint32_t>(budget, 96 * 1024)) {
+			const uint32_t wg_per_cu = std::max<uint32_t>(1, std::min<uint32_t>(8, (uint32_t)(dev.lds_bytes / lds_bytes)));
+			uint32_t chunks = dev.compute_units * wg_per_cu;
+			const uint32_t quantum = groups * UPDATE_UNROLL;
+			uint32_t chunk_points = (u.n + chunks - 1) / chunks;
+			chunk_points = (chunk_points + quantum - 1) / quantum * quantum;
+			chunks = (u.n + chunk_points - 1) / chunk_points;
+			exec->block_count = chunks;
+			hipLaunchKernelGGL((update_private_kernel<LM>), dim3(chunks), dim3(256), (uint32_t)lds_bytes, stream(),
+			                   u.data, u.stride, u.assignment, u.means, u.stride_means, u.cluster_sizes,
+			                   u.dim, u.k, u.n, gw, (uint32_t)copy_stride, chunk_points);
+			KMX_LAUNCH_CHECK("update_private_kernel");
+			return KMX_OK;
+		}
+	}
+
+	if (LD == KMX_AOS && u.k < (1u << (32 - SORT_SHIFT)) && (uint64_t)(u.k + 33) * 4 + 1024 * 4 <= budget) {
+		const uint32_t slices = (u.dim + 31) / 32;
+		const uint32_t gw = u.dim > 16 ? 32 : pow2_at_least(std::max<uint32_t>(u.dim, 4));
+		const uint32_t max_points = std::min<uint32_t>(1u << SORT_SHIFT, (budget - (u.k + 33) * 4) / 4 / 1024 * 1024);
+		uint32_t chunks = std::max<uint32_t>(1, dev.compute_units / slices);
+		uint32_t chunk_points = (u.n + chunks - 1) / chunks;
+		chunk_points = std::min(max_points, (chunk_points + 1023) / 1024 * 1024);
+		chunks = (u.n + chunk_points - 1) / chunk_points;
+		const uint32_t lds_bytes = (u.k + 33 + chunk_points) * 4;
+		int rc = reserve_partials(ws, (size_t)chunks * u.k * u.dim);
+		if (rc) return rc;
+		exec->block_count = chunks * slices;
+		const uint32_t items = chunk_points / 1024;
+		if (items <= 4) return launch_sorted<4, LM>(u, ws, chunks, slices, chunk_points, gw, lds_bytes);
+		if (items <= 8) return launch_sorted<8, LM>(u, ws, chunks, slices, chunk_points, gw, lds_bytes);
+		if (items <= 16) return launch_sorted<16, LM>(u, ws, chunks, slices, chunk_points, gw, lds_bytes);
+		return launch_sorted<32, LM>(u, ws, chunks, slices, chunk_points, gw, lds_bytes);
+	}
+
+	/* fallback: LDS-privatised floating-point atomics */
+	const uint32_t pad = LD == KMX_AOS ? 0 : 1;
+	const uint32_t words = budget / 4;
+	uint32_t slice = 0;
+	if (words > u.k) slice = std::min<uint32_t>(u.dim, (words - u.k) / u.k > pad ? (words - u.k) / u.k - pad : 0);
+	if (LD == KMX_AOS) slice = std::min<uint32_t>(slice, 1024);
+	if (slice < u.dim) {
+		for (uint32_t nice : { 32u, 16u, 8u, 4u })
+			if (slice >= nice) { slice = slice / nice * nice; break; }
+	}
+	if (slice == 0) {
+		*done = false;
+		return KMX_OK;
+	}
+	const uint32_t slices = (u.dim + slice - 1) / slice;
+	const uint32_t row = slice + pad;
+	const uint32_t wg = 1024;
+	const uint32_t slots = LD == KMX_AOS ? wg / slice : wg;
+	/* replicas only pay for small k: keep them within 16 KB and one per point slot */
+	uint32_t replicas = std::max<uint32_t>(1, std::min<uint32_t>({ 16384u / ((row + 1) * u.k * 4), LD == KMX_AOS ? slots : 16u, 16u }));
+	const uint32_t lds_bytes = replicas * u.k * (row + 1) * 4;
+	const uint32_t wg_per_cu = std::max<uint32_t>(1, std::min<uint32_t>(2, dev.lds_bytes / std::max(lds_bytes, 1u)));
+	uint32_t chunks = std::max<uint32_t>(1, dev.compute_units * wg_per_cu / slices);
+	uint32_t chunk_points = (u.n + chunks - 1) / chunks;
+	const uint32_t quantum = slots * UPDATE_UNROLL;
+	chunk_points = (chunk_points + quantum - 1) / quantum * quantum;
+	chunks = (u.n + chunk_points - 1) / chunk_points;
+	auto kernel = update_lds_kernel<LD, LM>;
+	KMX_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+	exec->block_count = chunks * slices;
+	hipLaunchKernelGGL(kernel, dim3(chunks, slices), dim3(wg), lds_bytes, stream(),
+	                   u.data, u.stride, u.assignment, u.means, u.stride_means, u.cluster_sizes,
+	                   u.dim, u.k, u.n, slice, chunk_points, replicas);
+	KMX_LAUNCH_CHECK("update_lds_kernel");
+	return KMX_OK;
+}
+
+template <int LD, int LM>
+static int launch_update_t(int variant, const UpdateArgs& u, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev)
 {
 	uint32_t block = exec->block_size ? exec->block_size : 256;
 	block = std::min<uint32_t>((block + WAVE - 1) / WAVE * WAVE, 1024);
@@ -220,39 +569,13 @@ static int launch_update_t(int variant, const UpdateArgs& u, kmx_exec_params* ex
 	if (u.n > 0) {
 		if ((rc = profile_begin(1))) return rc;
 		if (variant == KMX_UPDATE_ATOMIC_SHM) {
-			/* LDS budget: exec->shared_mem_bytes if given, else what the device offers a work-group */
-			uint32_t budget = exec->shared_mem_bytes ? std::min(exec->shared_mem_bytes, dev.lds_bytes) : dev.lds_bytes;
-			const uint32_t pad = LD == KMX_AOS ? 0 : 1;
-			const uint32_t words = budget / 4;
-			uint32_t slice = 0;
-			if (words > u.k) slice = std::min<uint32_t>(u.dim, (words - u.k) / u.k > pad ? (words - u.k) / u.k - pad : 0);
-			if (slice >= 32 && slice < u.dim) slice = slice / 32 * 32; /* whole 128-byte lines per point and slice */
-			if (slice == 0 || (LD == KMX_AOS && slice > 1024)) {
-				variant = KMX_UPDATE_ATOMIC_FINE; /* k too large for LDS privatisation */
-				copies = 1;
-			}
+			bool done = false;
+			rc = launch_update_tuned<LD, LM>(u, exec, ws, dev, &done);
+			if (rc) return rc;
+			if (done) copies = 1; /* the tuned kernels write replica 0 only */
 			else {
-				const uint32_t slices = (u.dim + slice - 1) / slice;
-				const uint32_t row = slice + pad;
-				const uint32_t wg = 1024;
-				const uint32_t slots = LD == KMX_AOS ? wg / slice : wg;
-				/* replicas only pay for small k: keep them within 16 KB and one per point slot */
-				uint32_t replicas = std::max<uint32_t>(1, std::min<uint32_t>({ 16384u / ((row + 1) * u.k * 4), LD == KMX_AOS ? slots : 16u, 16u }));
-				const uint32_t lds_bytes = replicas * u.k * (row + 1) * 4;
-				const uint32_t wg_per_cu = std::max<uint32_t>(1, std::min<uint32_t>(2, dev.lds_bytes / std::max(lds_bytes, 1u)));
-				uint32_t chunks = std::max<uint32_t>(1, dev.compute_units * wg_per_cu / slices);
-				uint32_t chunk_points = (u.n + chunks - 1) / chunks;
-				const uint32_t quantum = slots * UPDATE_UNROLL;
-				chunk_points = (chunk_points + quantum - 1) / quantum * quantum;
-				chunks = (u.n + chunk_points - 1) / chunk_points;
-				auto kernel = update_lds_kernel<LD, LM>;
-				KMX_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-				exec->block_count = chunks * slices;
-				hipLaunchKernelGGL(kernel, dim3(chunks, slices), dim3(wg), lds_bytes, stream(),
-				                   u.data, u.stride, u.assignment, u.means, u.stride_means, u.cluster_sizes,
-				                   u.dim, u.k, u.n, slice, chunk_points, replicas);
-				KMX_LAUNCH_CHECK("update_lds_kernel");
-				copies = 1; /* this variant writes replica 0 only */
+				variant = KMX_UPDATE_ATOMIC_FINE; /* k too large for any LDS privatisation */
+				copies = 1;
 			}
 		}
 		if (variant == KMX_UPDATE_ATOMIC_POINT) {
@@ -286,11 +609,10 @@ static int launch_update_t(int variant, const UpdateArgs& u, kmx_exec_params* ex
 
 int launch_update(int variant, const UpdateArgs& u, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev)
 {
-	(void)ws;
-	if (u.layout == KMX_AOS && u.layout_means == KMX_AOS) return launch_update_t<KMX_AOS, KMX_AOS>(variant, u, exec, dev);
-	if (u.layout == KMX_AOS && u.layout_means == KMX_SOA) return launch_update_t<KMX_AOS, KMX_SOA>(variant, u, exec, dev);
-	if (u.layout == KMX_SOA && u.layout_means == KMX_AOS) return launch_update_t<KMX_SOA, KMX_AOS>(variant, u, exec, dev);
-	return launch_update_t<KMX_SOA, KMX_SOA>(variant, u, exec, dev);
+	if (u.layout == KMX_AOS && u.layout_means == KMX_AOS) return launch_update_t<KMX_AOS, KMX_AOS>(variant, u, exec, ws, dev);
+	if (u.layout == KMX_AOS && u.layout_means == KMX_SOA) return launch_update_t<KMX_AOS, KMX_SOA>(variant, u, exec, ws, dev);
+	if (u.layout == KMX_SOA && u.layout_means == KMX_AOS) return launch_update_t<KMX_SOA, KMX_AOS>(variant, u, exec, ws, dev);
+	return launch_update_t<KMX_SOA, KMX_SOA>(variant, u, exec, ws, dev);
 }
 
 } // namespace kmx
