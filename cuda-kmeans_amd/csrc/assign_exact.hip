@@ -142,6 +142,87 @@ recheck_kernel(const float* __restrict__ data, size_t stride, const float* __res
 	}
 }
 
+/*
+ * Exact pass for dim <= DPAD <= 64 without LDS: the PB points of a batch live in registers (every lane of the
+ * group loads the same words, a broadcast), all DPAD centroid coordinates of a lane's centroid are requested
+ * before the first add, so their latency overlaps. Dimensions beyond dim are fed as x = c = 0: adding
+ * (0-0)^2 = +0 leaves every partial sum unchanged, so the padding is exact.
+ */
+template <int LD, int L, int PB, int DPAD>
+__global__ void __launch_bounds__(256)
+recheck_reg_kernel(const float* __restrict__ data, size_t stride, const float* __restrict__ means_t, uint32_t kp,
+                   uint32_t* __restrict__ assignment, uint32_t dim, uint32_t k,
+                   const uint32_t* __restrict__ queue, const uint32_t* __restrict__ counters)
+{
+	constexpr uint32_t GROUPS = 256 / L;
+	const uint32_t group = threadIdx.x / L;
+	const uint32_t gl = threadIdx.x % L;
+	const uint32_t count = counters[0];
+	const uint32_t batches = (count + PB - 1) / PB;
+
+	for (uint32_t batch = blockIdx.x * GROUPS + group; batch < batches; batch += gridDim.x * GROUPS) {
+		float x[PB][DPAD];
+		uint32_t idx[PB];
+#pragma unroll
+		for (int p = 0; p < PB; ++p) {
+			idx[p] = queue[min(batch * PB + p, count - 1)];
+#pragma unroll
+			for (int d = 0; d < DPAD; ++d) x[p][d] = (uint32_t)d < dim ? data[elem<LD>(stride, idx[p], d)] : 0.0f;
+		}
+		float best[PB];
+		uint32_t bestIdx[PB];
+		uint32_t pinned = 0;
+#pragma unroll
+		for (int p = 0; p < PB; ++p) {
+			best[p] = __builtin_inff();
+			bestIdx[p] = 0xFFFFFFFFu;
+		}
+		for (uint32_t m = gl; m < k; m += L) {
+			float c[DPAD];
+#pragma unroll
+			for (int d = 0; d < DPAD; ++d) c[d] = (uint32_t)d < dim ? means_t[(size_t)d * kp + m] : 0.0f;
+			float sum[PB];
+#pragma unroll
+			for (int p = 0; p < PB; ++p) sum[p] = 0.0f;
+#pragma unroll
+			for (int d = 0; d < DPAD; ++d) {
+#pragma unroll
+				for (int p = 0; p < PB; ++p) {
+					float diff = x[p][d] - c[d];
+					float sq = diff * diff;
+					sum[p] = sum[p] + sq;
+				}
+			}
+#pragma unroll
+			for (int p = 0; p < PB; ++p) {
+				float dist = __builtin_sqrtf(sum[p]);
+				if (m == 0 && dist != dist) pinned |= 1u << p;
+				if (dist < best[p] || (dist == best[p] && m < bestIdx[p])) {
+					best[p] = dist;
+					bestIdx[p] = m;
+				}
+			}
+		}
+		pinned = (uint32_t)__shfl((int)pinned, 0, L); /* lane 0 of the group evaluated centroid 0 */
+#pragma unroll
+		for (int p = 0; p < PB; ++p) {
+			for (int off = L / 2; off > 0; off >>= 1) {
+				float ob = __shfl_xor(best[p], off, L);
+				uint32_t oi = (uint32_t)__shfl_xor((int)bestIdx[p], off, L);
+				if (ob < best[p] || (ob == best[p] && oi < bestIdx[p])) {
+					best[p] = ob;
+					bestIdx[p] = oi;
+				}
+			}
+			const uint32_t q = batch * PB + p;
+			if (gl == 0 && q < count) {
+				const bool pin = (pinned >> p) & 1u;
+				assignment[idx[p]] = (pin || bestIdx[p] == 0xFFFFFFFFu) ? 0u : bestIdx[p];
+			}
+		}
+	}
+}
+
 template <int LD, int LM>
 static int launch_base_t(const AssignArgs& a, kmx_exec_params* exec, uint32_t* counters)
 {
@@ -181,9 +262,32 @@ static int launch_recheck_t(const AssignArgs& a, Workspace* ws, uint32_t kp)
 	return KMX_OK;
 }
 
+template <int LD, int L, int PB, int DPAD>
+static int launch_recheck_reg(const AssignArgs& a, Workspace* ws, uint32_t kp)
+{
+	hipLaunchKernelGGL((recheck_reg_kernel<LD, L, PB, DPAD>), dim3(2048), dim3(256), 0, stream(),
+	                   a.data, a.stride, ws->means_t, kp, a.assignment, a.dim, a.k, ws->queue, ws->counters);
+	KMX_LAUNCH_CHECK("recheck_reg_kernel");
+	return KMX_OK;
+}
+
+template <int LD, int L>
+static int launch_recheck_dpad(const AssignArgs& a, Workspace* ws, uint32_t kp)
+{
+	if (a.dim <= 8) return launch_recheck_reg<LD, L, 4, 8>(a, ws, kp);
+	if (a.dim <= 16) return launch_recheck_reg<LD, L, 4, 16>(a, ws, kp);
+	if (a.dim <= 32) return launch_recheck_reg<LD, L, 4, 32>(a, ws, kp);
+	return launch_recheck_reg<LD, L, 2, 64>(a, ws, kp);
+}
+
 template <int LD>
 static int launch_recheck_l(const AssignArgs& a, Workspace* ws, uint32_t kp)
 {
+	if (a.dim <= 64) {
+		if (a.k >= 48) return launch_recheck_dpad<LD, 64>(a, ws, kp);
+		if (a.k >= 24) return launch_recheck_dpad<LD, 32>(a, ws, kp);
+		return launch_recheck_dpad<LD, 16>(a, ws, kp);
+	}
 	if (a.k >= 48) {
 		if (a.dim <= 512) return launch_recheck_t<LD, 64, 8>(a, ws, kp);
 		return launch_recheck_t<LD, 64, 1>(a, ws, kp);
