@@ -1,0 +1,138 @@
+/*
+ * Kernel-runner boundary of the harness, host side: the same policy classes the reference declares in
+ * experimental/k-means/k-means/headers/kernels.cuh (problem-instance structs :7-52, CudaExecParameters
+ * :55-70, runFillZeros :74-75, DECLARE_ASSIGNMENT_KERNEL :81-93, DECLARE_UPDATE_KERNEL :96-105), each
+ * with one static run(instance, exec). Here run() forwards to the C ABI of libkmx_hip.so
+ * (include/kmx.h); no HIP header is needed on this side. Failures come back as error codes and are
+ * rethrown as std::runtime_error, which is how the reference's runners report unsupported shapes
+ * (kernels.cu:281-282,666,675,701) and how CUCH() reports device errors.
+ *
+ * Only F = float is built (the reference's --double path is not).
+ */
+#ifndef KMX_HOST_HIP_KERNELS_HPP
+#define KMX_HOST_HIP_KERNELS_HPP
+
+#include "kmx.h"
+#include "layouts.hpp"
+
+#include <cstddef>
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+#include <type_traits>
+
+/* throws with the library's message when a kmx call fails */
+inline void KMX_CHECK(int rc)
+{
+	if (rc != KMX_OK) throw std::runtime_error(std::string(kmx_last_error()));
+}
+
+template<typename F, typename IDX_T>
+struct AssignmentProblemInstance {
+	const F* data;
+	const F* means;
+	const IDX_T* lastAssignment;
+	IDX_T* assignment; /* the result */
+	IDX_T dim, k, n;
+
+	AssignmentProblemInstance(const F* _data, const F* _means, const IDX_T* _lastAssignment, IDX_T* _assignment,
+		std::size_t _dim, std::size_t _k, std::size_t _n)
+		: data(_data), means(_means), lastAssignment(_lastAssignment), assignment(_assignment),
+		dim((IDX_T)_dim), k((IDX_T)_k), n((IDX_T)_n) {}
+};
+
+template<typename F, typename IDX_T>
+struct UpdateProblemInstance {
+	const F* data;
+	const IDX_T* assignment;
+	F* means; /* the result; zeroed by the caller */
+	IDX_T* clusterSizes; /* zeroed by the caller */
+	IDX_T dim, k, n;
+
+	UpdateProblemInstance(const F* _data, const IDX_T* _assignment, F* _means, IDX_T* _clusterSizes,
+		std::size_t _dim, std::size_t _k, std::size_t _n)
+		: data(_data), assignment(_assignment), means(_means), clusterSizes(_clusterSizes),
+		dim((IDX_T)_dim), k((IDX_T)_k), n((IDX_T)_n) {}
+};
+
+/* = CudaExecParameters; the field order is that of kmx_exec_params */
+struct HipExecParameters {
+	unsigned int blockSize;
+	unsigned int blockCount;
+	unsigned int sharedMemorySize;
+	std::uint32_t privatizedCopies;
+	std::uint32_t itemsPerThread;
+	std::uint32_t regsCache;
+
+	HipExecParameters(unsigned int _blockSize = 256, unsigned int _blockCount = 0, unsigned int _sharedMemorySize = 0,
+		std::uint32_t _privatizedCopies = 1, std::uint32_t _itemsPerThread = 1, std::uint32_t _regsCache = 1)
+		: blockSize(_blockSize), blockCount(_blockCount), sharedMemorySize(_sharedMemorySize),
+		privatizedCopies(_privatizedCopies), itemsPerThread(_itemsPerThread), regsCache(_regsCache) {}
+};
+using CudaExecParameters = HipExecParameters; /* the reference's name */
+
+static_assert(sizeof(HipExecParameters) == sizeof(kmx_exec_params), "HipExecParameters must mirror kmx_exec_params");
+
+/* runFillZeros<F>(data, n): n 32-bit elements := 0 on the stream */
+template<typename T>
+void runFillZeros(T* data, std::size_t n)
+{
+	static_assert(sizeof(T) == 4, "only 32-bit element types are built");
+	KMX_CHECK(kmx_fill_zero_u32(data, n));
+}
+
+namespace hip_detail {
+
+template<typename F, typename IDX_T, class LAYOUT, class LAYOUT_MEANS>
+void assign(int variant, const AssignmentProblemInstance<F, IDX_T>& in, HipExecParameters& exec)
+{
+	static_assert(std::is_same<F, float>::value && sizeof(IDX_T) == 4, "built for float data and 32-bit indices");
+	KMX_CHECK(kmx_assign_f32(variant,
+		in.data, LAYOUT::ID, LAYOUT::precomputeConstants(in.n, in.dim),
+		in.means, LAYOUT_MEANS::ID, LAYOUT_MEANS::precomputeConstants(in.k, in.dim),
+		(const std::uint32_t*)in.lastAssignment, (std::uint32_t*)in.assignment,
+		in.dim, in.k, in.n, reinterpret_cast<kmx_exec_params*>(&exec)));
+}
+
+template<typename F, typename IDX_T, class LAYOUT, class LAYOUT_MEANS>
+void update(int variant, const UpdateProblemInstance<F, IDX_T>& in, HipExecParameters& exec)
+{
+	static_assert(std::is_same<F, float>::value && sizeof(IDX_T) == 4, "built for float data and 32-bit indices");
+	KMX_CHECK(kmx_update_f32(variant,
+		in.data, LAYOUT::ID, LAYOUT::precomputeConstants(in.n, in.dim),
+		(const std::uint32_t*)in.assignment,
+		in.means, LAYOUT_MEANS::ID, LAYOUT_MEANS::precomputeConstants(in.k, in.dim),
+		(std::uint32_t*)in.clusterSizes, in.dim, in.k, in.n, reinterpret_cast<kmx_exec_params*>(&exec)));
+}
+
+} // namespace hip_detail
+
+#define KMX_DEFINE_ASSIGNMENT_KERNEL(NAME, VARIANT)\
+template<typename F, typename IDX_T, class LAYOUT, class LAYOUT_MEANS, class METRIC>\
+class NAME {\
+public:\
+	static void run(const AssignmentProblemInstance<F, IDX_T>& in, HipExecParameters& exec)\
+	{ hip_detail::assign<F, IDX_T, LAYOUT, LAYOUT_MEANS>(VARIANT, in, exec); }\
+};
+
+KMX_DEFINE_ASSIGNMENT_KERNEL(BaseAssignmentKernel, KMX_ASSIGN_BASE)       /* kernels.cu:180-207 */
+KMX_DEFINE_ASSIGNMENT_KERNEL(LdsFmaAssignmentKernel, KMX_ASSIGN_LDS_FMA)  /* role of CachedFixed / CachedRegs, kernels.cu:216-319,546-703 */
+KMX_DEFINE_ASSIGNMENT_KERNEL(MfmaAssignmentKernel, KMX_ASSIGN_MFMA)       /* no counterpart: matrix-core path */
+KMX_DEFINE_ASSIGNMENT_KERNEL(BestCachedAssignmentKernel, KMX_ASSIGN_BEST) /* kernels.cu:706-717 */
+
+#define KMX_DEFINE_UPDATE_KERNEL(NAME, VARIANT)\
+template<typename F, typename IDX_T, class LAYOUT, class LAYOUT_MEANS, int EMUL = false>\
+class NAME {\
+public:\
+	static void run(const UpdateProblemInstance<F, IDX_T>& in, HipExecParameters& exec)\
+	{\
+		static_assert(!EMUL, "CAS-emulated atomics are not built: gfx950 has native fp32 atomics");\
+		hip_detail::update<F, IDX_T, LAYOUT, LAYOUT_MEANS>(VARIANT, in, exec);\
+	}\
+};
+
+KMX_DEFINE_UPDATE_KERNEL(UpdateAtomicPointKernel, KMX_UPDATE_ATOMIC_POINT) /* kernels.cu:726-761 */
+KMX_DEFINE_UPDATE_KERNEL(UpdateAtomicFineKernel, KMX_UPDATE_ATOMIC_FINE)   /* kernels.cu:770-809 */
+KMX_DEFINE_UPDATE_KERNEL(UpdateAtomicShmKernel, KMX_UPDATE_ATOMIC_SHM)     /* kernels.cu:817-878 */
+
+#endif
