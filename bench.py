@@ -35,6 +35,9 @@ PEAK_FP32_TFLOPS = 157.3   # MI355X fp32 (vector or matrix), dense
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # published full-iteration time for the headline shape on the reference's best hardware (V100 SXM2)
 PUBLISHED_MS = {2: 25.45}  # results/README.md:20 of the reference
+# HBM bytes per launch of the dominant kernels at configuration 2, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# scaled by the readings for a 256 MiB device copy (profiles/headline_cfg2_kernels.md); None where not measured
+MEASURED_TRAFFIC = {2: {"assign": 278.5e6, "update": 311.5e6}}
 
 
 def cpu_baseline(km, spec, n_sample, data, means0):
@@ -68,6 +71,9 @@ def main():
     ap.add_argument("--config", type=int, default=2, help="benchmark configuration 1..5 (2 = headline)")
     ap.add_argument("--cpu-sample", type=int, default=0, help="points in the CPU baseline sample (0 = about 12 s of work)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="one device-to-device copy of the point array before the timed region (a copy kernel of known "
+                         "size, to scale FETCH_SIZE / WRITE_SIZE counter readings)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (no collectives, no sharding); --gpus %d is not supported" % args.gpus)
@@ -84,6 +90,12 @@ def main():
 
     alg = km.HipKMeansAlgorithm(km.ASSIGN_BEST, km.UPDATE_ATOMIC_SHM)
     alg.initialize(dim, k, n, args.steps, data, means0)
+
+    if args.calibrate_copy:
+        scratch = km.DeviceBuffer(alg.cu_data.nbytes)
+        km.check(km.hip_lib().kmx_d2d(scratch.ptr, alg.cu_data.ptr, alg.cu_data.nbytes))
+        km.sync()
+        scratch.free()
 
     # 1. warm-up
     alg.run(iters=args.warmup)
@@ -133,10 +145,14 @@ def main():
     else:
         roofline = {"kernel": "assignment sweep", "bound": "hbm", "achieved": round(assign_gbs, 1),
                     "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(assign_gbs / PEAK_HBM_GBS, 4), "traffic": None}
+    traffic = MEASURED_TRAFFIC.get(args.config, {})
+    roofline["traffic"] = traffic.get("assign")
+    roofline["algorithmic_bytes"] = assign_bytes
     roofline["avg_kernel_ms"] = round(k_assign, 4)
     roofline_update = {"kernel": "update accumulation", "bound": "hbm", "achieved": round(update_gbs, 1),
                        "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(update_gbs / PEAK_HBM_GBS, 4),
-                       "traffic": None, "avg_kernel_ms": round(k_update, 4)}
+                       "traffic": traffic.get("update"), "algorithmic_bytes": update_bytes,
+                       "avg_kernel_ms": round(k_update, 4)}
 
     out = {
         "metric": "ms per k-means iteration (assign+update) at N=2M,d=32,k=1024; % roofline" if args.config == 2
