@@ -103,13 +103,23 @@ recheck_kernel(const float* __restrict__ data, size_t stride, const float* __res
 			float sum[PB];
 #pragma unroll
 			for (int p = 0; p < PB; ++p) sum[p] = 0.0f;
-			for (uint32_t d = 0; d < dim; ++d) {
-				const float c = means_t[(size_t)d * kp + m];
+			/* 16 centroid coordinates are requested before the first of them is used; dimensions beyond dim are
+			 * fed as x = c = 0, which adds +0 and leaves the sums unchanged */
+			for (uint32_t d0 = 0; d0 < dim; d0 += 16) {
+				float c[16];
 #pragma unroll
-				for (int p = 0; p < PB; ++p) {
-					float diff = gx[p * dim + d] - c;
-					float sq = diff * diff;
-					sum[p] = sum[p] + sq;
+				for (int u = 0; u < 16; ++u) c[u] = d0 + u < dim ? means_t[(size_t)(d0 + u) * kp + m] : 0.0f;
+#pragma unroll
+				for (int u = 0; u < 16; ++u) {
+					const bool on = d0 + u < dim;
+					const uint32_t d = on ? d0 + u : dim - 1;
+#pragma unroll
+					for (int p = 0; p < PB; ++p) {
+						const float x = on ? gx[p * dim + d] : 0.0f;
+						float diff = x - c[u];
+						float sq = diff * diff;
+						sum[p] = sum[p] + sq;
+					}
 				}
 			}
 #pragma unroll

@@ -100,6 +100,9 @@ SHAPES = [
     (16, 16, 5000),
     (32, 1000, 4099),   # k not a multiple of the tile, n prime
     (64, 96, 2048),
+    (100, 40, 1500),    # wide rows: 128-dimension MFMA instantiation, padded
+    (256, 300, 700),    # widest supported row
+    (130, 2000, 400),   # wide rows, centroids streamed through LDS in chunks
     (1, 7, 300),
     (5, 4100, 777),     # centroids do not fit one LDS chunk of the narrow layout
 ]
@@ -170,7 +173,7 @@ def test_sqrt_is_correctly_rounded_on_device(km, orc, gpu):
 
 def test_empty_input_and_argument_errors(km, gpu):
     ex = km.ExecParams()
-    d = km.DeviceBuffer(64); m = km.DeviceBuffer(64); a = km.DeviceBuffer(64)
+    d = km.DeviceBuffer(8192); m = km.DeviceBuffer(8192); a = km.DeviceBuffer(64)
     km.assign(km.ASSIGN_BEST, d, AOS, 4, m, AOS, 4, a, 4, 2, 0, ex)        # n = 0 is a no-op
     assert ex.block_count == 0
     with pytest.raises(km.KmxError) as e:
@@ -180,7 +183,7 @@ def test_empty_input_and_argument_errors(km, gpu):
         km.assign(km.ASSIGN_BEST, d, AOS, 2, m, AOS, 4, a, 4, 2, 4, ex)    # stride < dim
     assert e.value.code == km.KMX_ERR_INVALID_ARGUMENT
     with pytest.raises(km.KmxError) as e:
-        km.assign(km.ASSIGN_MFMA, d, AOS, 100, m, AOS, 100, a, 100, 2, 1, ex)  # dim beyond the MFMA variant
+        km.assign(km.ASSIGN_MFMA, d, AOS, 300, m, AOS, 300, a, 300, 2, 1, ex)  # dim beyond the MFMA variant
     assert e.value.code == km.KMX_ERR_UNSUPPORTED
     km.sync()
     for b in (d, m, a):
