@@ -54,42 +54,40 @@ assign_base_kernel(const float* __restrict__ data, size_t stride, const float* _
 }
 
 /*
- * Exact pass over the queued points. A group of L lanes (L = 16, 32 or 64, chosen from k) owns a batch of PB
- * queued points: the points' coordinates are staged in LDS (every lane of the group reads the same
- * word: a broadcast), lane l evaluates centroids l, l+L, ... in ascending order against all PB points
- * (one coalesced load of the transposed centroid block per (centroid, dim), reused PB times) and keeps its
- * own (distance, index) minimum per point; the L candidates are merged by (smaller distance, then smaller
- * index), which is the serial scan's result: the first centroid attaining the minimum. A NaN distance to
- * centroid 0 pins the point to centroid 0, as `minDist > dist` is then never true.
+ * Exact pass over the queued points, any dimension. A work-group of 256 lanes owns a batch of PB queued points:
+ * their coordinates are staged in LDS (rows padded with zeros to a multiple of 4 floats, so that every lane
+ * fetches four coordinates with one broadcast 128-bit read), lane t evaluates centroids t, t+256, ... in
+ * ascending order against all PB points (16 coalesced loads of the transposed centroid block in flight,
+ * each value reused PB times) and keeps its own (distance, index) minimum per point; the 256 candidates are
+ * merged by (smaller distance, then smaller index), which is the serial scan's result: the first centroid
+ * attaining the minimum. A NaN distance to centroid 0 pins the point to centroid 0, as `minDist > dist` is
+ * then never true. Zero padding is exact: (0-0)^2 = +0 leaves a partial sum unchanged.
  * means_t is the exact transposed copy [dim][kp] written by pack_means_kernel.
  */
-template <int LD, int L, int PB>
+template <int LD, int PB>
 __global__ void __launch_bounds__(256)
 recheck_kernel(const float* __restrict__ data, size_t stride, const float* __restrict__ means_t, uint32_t kp,
                uint32_t* __restrict__ assignment, uint32_t dim, uint32_t k,
                const uint32_t* __restrict__ queue, const uint32_t* __restrict__ counters)
 {
-	extern __shared__ float xs[];
-	constexpr uint32_t GROUPS = 256 / L;
-	const uint32_t group = threadIdx.x / L;
-	const uint32_t gl = threadIdx.x % L;
-	float* gx = xs + (size_t)group * PB * dim;
+	extern __shared__ float xs[]; /* PB rows of dim4 floats */
+	__shared__ float cand_dist[4][PB];
+	__shared__ uint32_t cand_idx[4][PB];
+	__shared__ uint32_t pinned_mask;
+	typedef float f4 __attribute__((ext_vector_type(4)));
+	const uint32_t dim4 = (dim + 3) / 4 * 4;
+	const uint32_t lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
 	const uint32_t count = counters[0];
 	const uint32_t batches = (count + PB - 1) / PB;
 
-	for (uint32_t first = blockIdx.x * GROUPS; first < batches; first += gridDim.x * GROUPS) {
-		const uint32_t batch = first + group;
-		const bool active = batch < batches;
-		__syncthreads(); /* the previous batch's coordinates are no longer needed */
-		if (active) {
-			for (uint32_t i = gl; i < PB * dim; i += L) {
-				const uint32_t p = i / dim, d = i - p * dim;
-				const uint32_t idx = queue[min(batch * PB + p, count - 1)];
-				gx[i] = data[elem<LD>(stride, idx, d)];
-			}
+	for (uint32_t batch = blockIdx.x; batch < batches; batch += gridDim.x) {
+		__syncthreads(); /* the previous batch's coordinates and candidates are no longer needed */
+		for (uint32_t i = threadIdx.x; i < PB * dim4; i += blockDim.x) {
+			const uint32_t p = i / dim4, d = i - p * dim4;
+			const uint32_t idx = queue[min(batch * PB + p, count - 1)];
+			xs[i] = d < dim ? data[elem<LD>(stride, idx, d)] : 0.0f;
 		}
 		__syncthreads();
-		if (!active) continue;
 
 		float best[PB];
 		uint32_t bestIdx[PB];
@@ -99,26 +97,27 @@ recheck_kernel(const float* __restrict__ data, size_t stride, const float* __res
 			best[p] = __builtin_inff();
 			bestIdx[p] = 0xFFFFFFFFu;
 		}
-		for (uint32_t m = gl; m < k; m += L) {
+		for (uint32_t m = threadIdx.x; m < k; m += blockDim.x) {
 			float sum[PB];
 #pragma unroll
 			for (int p = 0; p < PB; ++p) sum[p] = 0.0f;
-			/* 16 centroid coordinates are requested before the first of them is used; dimensions beyond dim are
-			 * fed as x = c = 0, which adds +0 and leaves the sums unchanged */
-			for (uint32_t d0 = 0; d0 < dim; d0 += 16) {
+			for (uint32_t d0 = 0; d0 < dim4; d0 += 16) {
 				float c[16];
 #pragma unroll
 				for (int u = 0; u < 16; ++u) c[u] = d0 + u < dim ? means_t[(size_t)(d0 + u) * kp + m] : 0.0f;
 #pragma unroll
-				for (int u = 0; u < 16; ++u) {
-					const bool on = d0 + u < dim;
-					const uint32_t d = on ? d0 + u : dim - 1;
+				for (int u4 = 0; u4 < 4; ++u4) {
+					if (d0 + 4 * u4 < dim4) { /* uniform: whole groups of four padded coordinates */
 #pragma unroll
-					for (int p = 0; p < PB; ++p) {
-						const float x = on ? gx[p * dim + d] : 0.0f;
-						float diff = x - c[u];
-						float sq = diff * diff;
-						sum[p] = sum[p] + sq;
+						for (int p = 0; p < PB; ++p) {
+							const f4 x = *(const f4*)(xs + p * dim4 + d0 + 4 * u4);
+#pragma unroll
+							for (int q = 0; q < 4; ++q) {
+								float diff = x[q] - c[4 * u4 + q];
+								float sq = diff * diff;
+								sum[p] = sum[p] + sq;
+							}
+						}
 					}
 				}
 			}
@@ -132,21 +131,39 @@ recheck_kernel(const float* __restrict__ data, size_t stride, const float* __res
 				}
 			}
 		}
-		pinned = (uint32_t)__shfl((int)pinned, 0, L); /* lane 0 of the group evaluated centroid 0 */
+		if (threadIdx.x == 0) pinned_mask = pinned; /* lane 0 evaluated centroid 0 */
 #pragma unroll
 		for (int p = 0; p < PB; ++p) {
-			for (int off = L / 2; off > 0; off >>= 1) {
-				float ob = __shfl_xor(best[p], off, L);
-				uint32_t oi = (uint32_t)__shfl_xor((int)bestIdx[p], off, L);
+			for (int off = WAVE / 2; off > 0; off >>= 1) {
+				float ob = __shfl_xor(best[p], off);
+				uint32_t oi = (uint32_t)__shfl_xor((int)bestIdx[p], off);
 				if (ob < best[p] || (ob == best[p] && oi < bestIdx[p])) {
 					best[p] = ob;
 					bestIdx[p] = oi;
 				}
 			}
+			if (lane == 0) {
+				cand_dist[wave][p] = best[p];
+				cand_idx[wave][p] = bestIdx[p];
+			}
+		}
+		__syncthreads();
+		if (threadIdx.x < PB) {
+			const uint32_t p = threadIdx.x;
+			float b = cand_dist[0][p];
+			uint32_t bi = cand_idx[0][p];
+			for (int w = 1; w < 4; ++w) {
+				const float ob = cand_dist[w][p];
+				const uint32_t oi = cand_idx[w][p];
+				if (ob < b || (ob == b && oi < bi)) {
+					b = ob;
+					bi = oi;
+				}
+			}
 			const uint32_t q = batch * PB + p;
-			if (gl == 0 && q < count) {
-				const bool pin = (pinned >> p) & 1u;
-				assignment[queue[q]] = (pin || bestIdx[p] == 0xFFFFFFFFu) ? 0u : bestIdx[p];
+			if (q < count) {
+				const bool pin = (pinned_mask >> p) & 1u;
+				assignment[queue[q]] = (pin || bi == 0xFFFFFFFFu) ? 0u : bi;
 			}
 		}
 	}
@@ -259,13 +276,13 @@ int launch_assign_base(const AssignArgs& a, kmx_exec_params* exec)
 	return launch_base_t<KMX_SOA, KMX_SOA>(a, exec, ws->counters);
 }
 
-template <int LD, int L, int PB>
+template <int LD, int PB>
 static int launch_recheck_t(const AssignArgs& a, Workspace* ws, uint32_t kp)
 {
-	const unsigned block = 256, blocks = 1024;
-	const size_t lds = (size_t)(256 / L) * PB * a.dim * sizeof(float);
-	auto kernel = recheck_kernel<LD, L, PB>;
-	if (lds > 65536) KMX_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+	const unsigned block = 256, blocks = 2048;
+	const size_t lds = (size_t)PB * ((a.dim + 3) / 4 * 4) * sizeof(float);
+	auto kernel = recheck_kernel<LD, PB>;
+	if (lds > 48 * 1024) KMX_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
 	hipLaunchKernelGGL(kernel, dim3(blocks), dim3(block), lds, stream(),
 	                   a.data, a.stride, ws->means_t, kp, a.assignment, a.dim, a.k, ws->queue, ws->counters);
 	KMX_LAUNCH_CHECK("recheck_kernel");
@@ -298,12 +315,8 @@ static int launch_recheck_l(const AssignArgs& a, Workspace* ws, uint32_t kp)
 		if (a.k >= 24) return launch_recheck_dpad<LD, 32>(a, ws, kp);
 		return launch_recheck_dpad<LD, 16>(a, ws, kp);
 	}
-	if (a.k >= 48) {
-		if (a.dim <= 512) return launch_recheck_t<LD, 64, 8>(a, ws, kp);
-		return launch_recheck_t<LD, 64, 1>(a, ws, kp);
-	}
-	if (a.k >= 24) return launch_recheck_t<LD, 32, 1>(a, ws, kp);
-	return launch_recheck_t<LD, 16, 1>(a, ws, kp);
+	if ((size_t)a.dim * 8 * sizeof(float) <= 64 * 1024) return launch_recheck_t<LD, 8>(a, ws, kp);
+	return launch_recheck_t<LD, 1>(a, ws, kp);
 }
 
 int launch_recheck(const AssignArgs& a, Workspace* ws, uint32_t kp)

@@ -93,16 +93,13 @@ KMX_DECLARE_MFMA_LAUNCHER(2) KMX_DECLARE_MFMA_LAUNCHER(4) KMX_DECLARE_MFMA_LAUNC
 KMX_DECLARE_MFMA_LAUNCHER(16) KMX_DECLARE_MFMA_LAUNCHER(24) KMX_DECLARE_MFMA_LAUNCHER(32) KMX_DECLARE_MFMA_LAUNCHER(64)
 KMX_DECLARE_MFMA_LAUNCHER(128)
 
-int launch_assign_mfma(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev)
+/* packs the centroids of this call into the work space (rows of dp floats, kp rows) and empties the recheck queue */
+int launch_pack_means(const AssignArgs& a, Workspace* ws, uint32_t dp, uint32_t kp)
 {
-	const uint32_t dph = pick_dph(a.dim);
-	const uint32_t dp = 2 * dph;
-	const uint32_t kp = round_up(a.k, TILE);
 	int rc = reserve_packed(ws, (size_t)(kp / TILE) * tile_floats(dp + ROW_PAD), (size_t)(kp / TILE) * NORM_TILE, (size_t)kp * a.dim);
 	if (rc) return rc;
 	rc = reserve_queue(ws, a.n);
 	if (rc) return rc;
-
 	const uint32_t pack_blocks = (kp * WAVE + 255) / 256;
 	if (a.layout_means == KMX_AOS)
 		hipLaunchKernelGGL((pack_means_kernel<KMX_AOS>), dim3(pack_blocks), dim3(256), 0, stream(),
@@ -111,6 +108,16 @@ int launch_assign_mfma(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws
 		hipLaunchKernelGGL((pack_means_kernel<KMX_SOA>), dim3(pack_blocks), dim3(256), 0, stream(),
 		                   a.means, a.stride_means, ws->packed_means, ws->norms, ws->means_t, a.dim, a.k, kp, dp, ws->counters);
 	KMX_LAUNCH_CHECK("pack_means_kernel");
+	return KMX_OK;
+}
+
+int launch_assign_mfma(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev)
+{
+	const uint32_t dph = pick_dph(a.dim);
+	const uint32_t dp = 2 * dph;
+	const uint32_t kp = round_up(a.k, TILE);
+	int rc = launch_pack_means(a, ws, dp, kp);
+	if (rc) return rc;
 
 	/* tau = kd (|x|^2 + max|c|^2), kd = (8 d + 64) 2^-23 (see the bound at the top of the file) */
 	const float kd = (8.0f * (float)a.dim + 64.0f) * 1.1920929e-07f;

@@ -62,8 +62,9 @@ def gpu_update(km, variant, data, assignment, dim, k, n, layout=AOS, layout_mean
     return means, sizes
 
 
-def variants(km):
-    return [km.ASSIGN_BASE, km.ASSIGN_MFMA, km.ASSIGN_BEST]
+def variants(km, dim=1):
+    v = [km.ASSIGN_BASE, km.ASSIGN_MFMA, km.ASSIGN_BEST]
+    return v + [km.ASSIGN_LDS_FMA] if dim <= 64 else v
 
 
 # ---------------------------------------------------------------- golden vectors of the reference
@@ -85,7 +86,7 @@ def test_first_pass_equals_reference_golden(km, gpu, golden, name):
     data = km.generate_points(spec, c["n"], layout=c["layout"])
     means0 = km.first_k_means(spec, c["layout_means"])
     want = arrays[name + "_assignment_first_pass"].astype(np.uint32)
-    for v in variants(km):
+    for v in variants(km, c["dim"]):
         got, _ = gpu_assign(km, v, data, means0, c["dim"], c["k"], c["n"], c["layout"], c["layout_means"])
         assert np.array_equal(got, want), "variant %d: %d mismatches" % (v, int((got != want).sum()))
 
@@ -116,7 +117,7 @@ def test_assignment_is_bit_exact(km, orc, gpu, dim, k, n, layout, layout_means):
     means = data.reshape(-1)[:k * dim].copy() if n >= k and layout == AOS and layout_means == AOS \
         else rng.normal(size=k * dim).astype(np.float32) * np.float32(3)
     want = orc.assign(data, means, dim, k, n, layout, layout_means, threads=0, fast=True)
-    for v in variants(km):
+    for v in variants(km, dim):
         got, _ = gpu_assign(km, v, data, means, dim, k, n, layout, layout_means)
         bad = np.nonzero(got != want)[0]
         assert bad.size == 0, "variant %d: %d mismatches, first at %s" % (v, bad.size, bad[:5])
@@ -151,7 +152,7 @@ def test_hard_inputs(km, orc, gpu, dim, k, n):
         d = np.ascontiguousarray(d, dtype=np.float32).ravel()
         m = np.ascontiguousarray(m, dtype=np.float32).ravel()
         want = orc.assign(d, m, dim, k, n, threads=0, fast=True)
-        for v in variants(km):
+        for v in variants(km, dim):
             got, rechecked = gpu_assign(km, v, d, m, dim, k, n)
             bad = np.nonzero(got != want)[0]
             assert bad.size == 0, "%s, variant %d: %d mismatches, first at %s (gpu %s, oracle %s)" % (
@@ -166,7 +167,7 @@ def test_sqrt_is_correctly_rounded_on_device(km, orc, gpu):
     data = rng.uniform(0.5, 100, size=n).astype(np.float32)
     means = np.sort(rng.uniform(0, 200, size=k).astype(np.float32))
     want = orc.assign(data, means, 1, k, n)
-    for v in variants(km):
+    for v in variants(km, 1):
         got, _ = gpu_assign(km, v, data, means, 1, k, n)
         assert np.array_equal(got, want)
 
@@ -251,8 +252,9 @@ LOOP_CASES = [(1, 65536, 10), (2, 65536, 4), (3, 131072, 3), (5, 1 << 20, 4), (4
 def test_every_iteration_matches_oracle(km, orc, gpu, cid, n, iters):
     spec = km.baseline_config(cid)
     combos = [(km.ASSIGN_BEST, km.UPDATE_ATOMIC_SHM)]
+    combos += [(km.ASSIGN_MFMA, km.UPDATE_ATOMIC_FINE)]
     if spec.dim <= 64:
-        combos += [(km.ASSIGN_MFMA, km.UPDATE_ATOMIC_FINE)]
+        combos += [(km.ASSIGN_LDS_FMA, km.UPDATE_ATOMIC_SHM)]
     if n * spec.k * spec.dim <= 1 << 31:
         combos += [(km.ASSIGN_BASE, km.UPDATE_ATOMIC_POINT)]
     for av, uv in combos:

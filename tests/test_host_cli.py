@@ -104,7 +104,7 @@ def test_device_algorithms_verify(harness, gpu, algo):
 
 @pytest.mark.gpu
 def test_device_assignment_only_and_reference_dataset(harness, gpu):
-    for algo in ("hip_best", "hip_mfma", "hip_base", "cuda_cached_regs"):
+    for algo in ("hip_best", "hip_mfma", "hip_base", "hip_lds_fma", "cuda_cached_regs", "cuda_cached_fixed"):
         rc, out, err = run(harness, "--assignmentOnly", "--algorithm", algo, "--N", "64k", "--k", "256", "--dim", "16", "--verify", "--serialThreads", "8")
         assert rc == 0 and "Verifying results ... OK" in err, err
         assert len(out.split()) == 2
@@ -112,5 +112,5 @@ def test_device_assignment_only_and_reference_dataset(harness, gpu):
     for layout in ("aos", "soa"):
         rc, out, err = run(harness, "--algorithm", "hip_best", "--iterations", "1", "--layout", layout, "--verify")
         assert rc == 0 and "Verifying results ... OK" in err, err
-    rc, out, err = run(harness, "--algorithm", "hip_lds_fma", "--assignmentOnly")
+    rc, out, err = run(harness, "--algorithm", "hip_lds_fma", "--assignmentOnly", "--dim", "100")
     assert rc == 2 and "not supported" in out
