@@ -70,6 +70,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--config", type=int, default=2, help="benchmark configuration 1..5 (2 = headline)")
     ap.add_argument("--cpu-sample", type=int, default=0, help="points in the CPU baseline sample (0 = about 12 s of work)")
+    ap.add_argument("--assign-variant", default="best", choices=["base", "lds_fma", "mfma", "best"])
+    ap.add_argument("--update-variant", default="atomic_shm", choices=["atomic_point", "atomic_fine", "atomic_shm"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="one device-to-device copy of the point array before the timed region (a copy kernel of known "
@@ -88,7 +90,10 @@ def main():
     data = km.generate_points(spec)
     means0 = km.first_k_means(spec)
 
-    alg = km.HipKMeansAlgorithm(km.ASSIGN_BEST, km.UPDATE_ATOMIC_SHM)
+    assign_variant = {"base": km.ASSIGN_BASE, "lds_fma": km.ASSIGN_LDS_FMA, "mfma": km.ASSIGN_MFMA, "best": km.ASSIGN_BEST}[args.assign_variant]
+    update_variant = {"atomic_point": km.UPDATE_ATOMIC_POINT, "atomic_fine": km.UPDATE_ATOMIC_FINE,
+                      "atomic_shm": km.UPDATE_ATOMIC_SHM}[args.update_variant]
+    alg = km.HipKMeansAlgorithm(assign_variant, update_variant)
     alg.initialize(dim, k, n, args.steps, data, means0)
 
     if args.calibrate_copy:
@@ -145,7 +150,7 @@ def main():
     else:
         roofline = {"kernel": "assignment sweep", "bound": "hbm", "achieved": round(assign_gbs, 1),
                     "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(assign_gbs / PEAK_HBM_GBS, 4), "traffic": None}
-    traffic = MEASURED_TRAFFIC.get(args.config, {})
+    traffic = MEASURED_TRAFFIC.get(args.config, {}) if (args.assign_variant, args.update_variant) == ("best", "atomic_shm") else {}
     roofline["traffic"] = traffic.get("assign")
     roofline["algorithmic_bytes"] = assign_bytes
     roofline["avg_kernel_ms"] = round(k_assign, 4)
@@ -165,7 +170,7 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "benchmark configuration %d: N=%d d=%d k=%d, %s, initial centroids = first k points, seed %d"
                                % (args.config, n, dim, k, "Gaussian mixture" if spec.kind != 1 else "uniform", spec.seed),
-                   "layout": "aos", "assignment": "hip_best", "update": "atomic_shm"},
+                   "layout": "aos", "assignment": "hip_" + args.assign_variant, "update": args.update_variant},
         "assign_ms": round(t_assign, 4), "update_ms": round(t_update, 4),
         "points_centroids_dims_per_s": round(float(n) * k * dim / (ms_per_step * 1e-3), 0),
         "rechecked_points_per_iteration": round(rechecked / args.steps, 1),

@@ -257,6 +257,7 @@ update_private_kernel(const float* __restrict__ data, size_t stride, const uint3
  * partial layout: [chunk][cluster][dim].
  */
 constexpr uint32_t SORT_SHIFT = 15; /* local point index bits: chunk_points <= 32768 */
+constexpr int SORT_UNROLL = 8;      /* row loads in flight per lane group in the segment-sum phase */
 
 template <int ITEMS, int GW>
 __global__ void __launch_bounds__(1024)
@@ -354,15 +355,15 @@ update_sorted_kernel(const float* __restrict__ data, size_t stride, const uint32
 	float acc = 0.0f;
 	uint32_t e = offsets[c_lo];
 	const uint32_t e_end = offsets[c_hi];
-	for (; e + UPDATE_UNROLL <= e_end; e += UPDATE_UNROLL) {
-		uint32_t ent[UPDATE_UNROLL];
-		float v[UPDATE_UNROLL];
+	for (; e + SORT_UNROLL <= e_end; e += SORT_UNROLL) {
+		uint32_t ent[SORT_UNROLL];
+		float v[SORT_UNROLL];
 #pragma unroll
-		for (int u = 0; u < UPDATE_UNROLL; ++u) ent[u] = sorted[e + u];
+		for (int u = 0; u < SORT_UNROLL; ++u) ent[u] = sorted[e + u];
 #pragma unroll
-		for (int u = 0; u < UPDATE_UNROLL; ++u) v[u] = src[(size_t)(ent[u] & ((1u << SORT_SHIFT) - 1u)) * stride];
+		for (int u = 0; u < SORT_UNROLL; ++u) v[u] = src[(size_t)(ent[u] & ((1u << SORT_SHIFT) - 1u)) * stride];
 #pragma unroll
-		for (int u = 0; u < UPDATE_UNROLL; ++u) {
+		for (int u = 0; u < SORT_UNROLL; ++u) {
 			const uint32_t t = ent[u] >> SORT_SHIFT;
 			while (cur < t) {
 				if (lane_on) out[(size_t)cur * dim] = acc;
@@ -390,20 +391,42 @@ update_sorted_kernel(const float* __restrict__ data, size_t stride, const uint32
 	}
 }
 
-/* means[c][d] += sum over a share of the chunks of partial[chunk][c][d]; grid = (elements / 256, shares) */
+/*
+ * means[c][d] = (sum over the chunks of partial[chunk][c][d]) / count[c]  (0 for an empty cluster).
+ * Block = 64 consecutive elements x 4 chunk shares; every lane keeps 8 loads in flight; the shares meet in LDS.
+ * Overwrites means: the sorted path needs neither zeroed centroids nor the separate divide kernel.
+ */
 template <int LM>
 __global__ void __launch_bounds__(256)
 reduce_partials_kernel(const float* __restrict__ partial, float* __restrict__ means, size_t stride_means,
-                       uint32_t dim, uint32_t k, uint32_t chunks)
+                       const uint32_t* __restrict__ sizes, uint32_t dim, uint32_t k, uint32_t chunks)
 {
-	const uint32_t e = blockIdx.x * blockDim.x + threadIdx.x;
-	if (e >= k * dim) return;
-	const uint32_t per = (chunks + gridDim.y - 1) / gridDim.y;
-	const uint32_t c0 = blockIdx.y * per, c1 = min(c0 + per, chunks);
+	__shared__ float part[4][64];
+	const uint32_t col = threadIdx.x & 63, share = threadIdx.x >> 6;
+	const uint32_t e = blockIdx.x * 64 + col;
+	const size_t kd = (size_t)k * dim;
 	float s = 0.0f;
-	for (uint32_t c = c0; c < c1; ++c) s += partial[(size_t)c * k * dim + e];
-	const uint32_t cl = e / dim, d = e - cl * dim;
-	if (s != 0.0f) atomic_add_f32(&means[elem<LM>(stride_means, cl, d)], s);
+	if (e < kd) {
+		const uint32_t per = (chunks + 3) / 4;
+		const uint32_t c0 = share * per, c1 = min(c0 + per, chunks);
+		uint32_t c = c0;
+		for (; c + 8 <= c1; c += 8) {
+			float v[8];
+#pragma unroll
+			for (int u = 0; u < 8; ++u) v[u] = partial[(size_t)(c + u) * kd + e];
+#pragma unroll
+			for (int u = 0; u < 8; ++u) s += v[u];
+		}
+		for (; c < c1; ++c) s += partial[(size_t)c * kd + e];
+	}
+	part[share][col] = s;
+	__syncthreads();
+	if (share == 0 && e < kd) {
+		s = (part[0][col] + part[1][col]) + (part[2][col] + part[3][col]);
+		const uint32_t cl = e / dim, d = e - cl * dim;
+		const uint32_t count = sizes[cl];
+		means[elem<LM>(stride_means, cl, d)] = count ? s / (float)count : 0.0f;
+	}
 }
 
 template <int LM>
@@ -463,18 +486,18 @@ static int launch_sorted(const UpdateArgs& u, Workspace* ws, uint32_t chunks, ui
 	                   u.data, u.stride, u.assignment, ws->partials, u.cluster_sizes, u.dim, u.k, u.n, chunk_points);
 	KMX_LAUNCH_CHECK("update_sorted_kernel");
 	const uint32_t total = u.k * u.dim;
-	const uint32_t shares = std::max<uint32_t>(1, std::min<uint32_t>(chunks, 8));
-	hipLaunchKernelGGL((reduce_partials_kernel<LM>), dim3((total + 255) / 256, shares), dim3(256), 0, stream(),
-	                   ws->partials, u.means, u.stride_means, u.dim, u.k, chunks);
+	hipLaunchKernelGGL((reduce_partials_kernel<LM>), dim3((total + 63) / 64), dim3(256), 0, stream(),
+	                   ws->partials, u.means, u.stride_means, u.cluster_sizes, u.dim, u.k, chunks);
 	KMX_LAUNCH_CHECK("reduce_partials_kernel");
 	return KMX_OK;
 }
 
-/* Picks and launches the kernel of KMX_UPDATE_ATOMIC_SHM; *done = false if no LDS variant fits the shape. */
+/* Picks and launches the kernel of KMX_UPDATE_ATOMIC_SHM. *state: 0 = no LDS variant fits the shape, 1 = sums and
+ * counts accumulated (divide still to do), 2 = centroids finished (the sorted path divides while it folds the partials). */
 template <int LD, int LM>
-static int launch_update_tuned(const UpdateArgs& u, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev, bool* done)
+static int launch_update_tuned(const UpdateArgs& u, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev, int* state)
 {
-	*done = true;
+	*state = 1;
 	const uint32_t budget = exec->shared_mem_bytes ? std::min(exec->shared_mem_bytes, dev.lds_bytes) : dev.lds_bytes;
 
 	if (LD == KMX_AOS && u.dim <= 64) {
@@ -512,6 +535,7 @@ static int launch_update_tuned(const UpdateArgs& u, kmx_exec_params* exec, Works
 		int rc = reserve_partials(ws, (size_t)chunks * u.k * u.dim);
 		if (rc) return rc;
 		exec->block_count = chunks * slices;
+		*state = 2;
 		const uint32_t items = chunk_points / 1024;
 		if (items <= 4) return launch_sorted<4, LM>(u, ws, chunks, slices, chunk_points, gw, lds_bytes);
 		if (items <= 8) return launch_sorted<8, LM>(u, ws, chunks, slices, chunk_points, gw, lds_bytes);
@@ -530,7 +554,7 @@ static int launch_update_tuned(const UpdateArgs& u, kmx_exec_params* exec, Works
 			if (slice >= nice) { slice = slice / nice * nice; break; }
 	}
 	if (slice == 0) {
-		*done = false;
+		*state = 0;
 		return KMX_OK;
 	}
 	const uint32_t slices = (u.dim + slice - 1) / slice;
@@ -569,10 +593,11 @@ static int launch_update_t(int variant, const UpdateArgs& u, kmx_exec_params* ex
 	if (u.n > 0) {
 		if ((rc = profile_begin(1))) return rc;
 		if (variant == KMX_UPDATE_ATOMIC_SHM) {
-			bool done = false;
-			rc = launch_update_tuned<LD, LM>(u, exec, ws, dev, &done);
+			int state = 0;
+			rc = launch_update_tuned<LD, LM>(u, exec, ws, dev, &state);
 			if (rc) return rc;
-			if (done) copies = 1; /* the tuned kernels write replica 0 only */
+			if (state == 2) return profile_end(1); /* nothing left to merge or divide */
+			if (state == 1) copies = 1; /* the tuned kernels write replica 0 only */
 			else {
 				variant = KMX_UPDATE_ATOMIC_FINE; /* k too large for any LDS privatisation */
 				copies = 1;
