@@ -172,7 +172,7 @@ int launch_assign_lds_fma(const AssignArgs& a, kmx_exec_params* exec, Workspace*
 	const uint32_t kp = round_up(a.k, TILE);
 	int rc = launch_pack_means(a, ws, dp, kp);
 	if (rc) return rc;
-	const float kd = (8.0f * (float)a.dim + 64.0f) * 1.1920929e-07f;
+	const float kd = (8.0f * (float)a.dim + 24.0f) * 1.1920929e-07f;
 	switch (dp) {
 	case 4: rc = launch_fma_dp<4>(a, exec, ws, dev, kp, kd); break;
 	case 8: rc = launch_fma_dp<8>(a, exec, ws, dev, kp, kd); break;

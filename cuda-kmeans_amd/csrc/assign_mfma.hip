@@ -12,7 +12,7 @@
  *   - a_j as computed:     |a_j - (T_j - |x|^2)| <= (d+2) u' (|c_j|^2 + 2|x||c_j|),  u' = 2u allowed
  *                          for the accumulation order / rounding inside the matrix core
  *   - sqrt can merge two sums that differ by a few ulp, which would hand the win to a lower index
- * Putting these together, if  a_(2) - a_(1) > tau  with  tau = (8 d + 64) 2^-23 (|x|^2 + max_j |c_j|^2)
+ * Putting these together, if  a_(2) - a_(1) > tau  with  tau = (8 d + 24) 2^-23 (|x|^2 + max_j |c_j|^2)
  * then centroid (1) has the strictly smallest serial distance and is the serial result. Every other
  * point (including all NaN / overflow cases, for which the comparison is false) is appended to the
  * recheck queue and re-evaluated by the recheck kernels with the serial arithmetic.
@@ -119,8 +119,8 @@ int launch_assign_mfma(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws
 	int rc = launch_pack_means(a, ws, dp, kp);
 	if (rc) return rc;
 
-	/* tau = kd (|x|^2 + max|c|^2), kd = (8 d + 64) 2^-23 (see the bound at the top of the file) */
-	const float kd = (8.0f * (float)a.dim + 64.0f) * 1.1920929e-07f;
+	/* tau = kd (|x|^2 + max|c|^2), kd = (8 d + 24) 2^-23 (see the bound at the top of the file) */
+	const float kd = (8.0f * (float)a.dim + 24.0f) * 1.1920929e-07f;
 	switch (dph) {
 	case 2: rc = launch_mfma_2(a, exec, ws, dev, kp, kd); break;
 	case 4: rc = launch_mfma_4(a, exec, ws, dev, kp, kd); break;

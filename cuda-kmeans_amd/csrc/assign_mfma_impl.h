@@ -406,7 +406,7 @@ assign_mfma_kernel(const float* __restrict__ data, size_t stride, const float* _
 }
 
 /* points per wavefront and sweep, and whether the next sweep's points are prefetched: bounded by the register file */
-template <int DPH> struct SweepShape { static constexpr int P = DPH <= 32 ? 2 : 1; static constexpr bool PREFETCH = DPH <= 64; };
+template <int DPH> struct SweepShape { static constexpr int P = DPH <= 8 ? 4 : (DPH <= 32 ? 2 : 1); static constexpr bool PREFETCH = DPH <= 64; };
 
 template <int DPH, int LD, bool VEC>
 static int launch_mfma_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev, uint32_t kp, float kd)
@@ -426,9 +426,6 @@ static int launch_mfma_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 	const uint32_t lds_bytes = chunk_rows / TILE * tile_bytes;
 	const uint32_t unit_points = MFMA_WAVES * P * TILE;
 	const uint32_t units = (a.n + unit_points - 1) / unit_points;
-	const uint32_t grid = std::min(units, dev.compute_units);
-	exec->block_count = grid;
-
 	void (*kernel)(const float*, size_t, const float*, const float*, uint32_t*, uint32_t*, uint32_t*,
 	               uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, float, float) = nullptr;
 	if constexpr (DPH <= 32) {
@@ -440,6 +437,13 @@ static int launch_mfma_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 		kernel = assign_mfma_kernel<DPH, P, LD, VEC, true, false, PF>;
 	}
 	KMX_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+	/* persistent work-groups: as many as fit a CU at once (small k leaves room for several, which the
+	 * HBM-bound shapes need to keep enough loads in flight) */
+	int per_cu = 1;
+	KMX_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)kernel, (int)(MFMA_WAVES * WAVE), lds_bytes));
+	per_cu = std::max(1, std::min(per_cu, 4));
+	const uint32_t grid = std::min(units, dev.compute_units * (uint32_t)per_cu);
+	exec->block_count = grid;
 	int rc = profile_begin(0);
 	if (rc) return rc;
 	hipLaunchKernelGGL(kernel, dim3(grid), dim3(MFMA_WAVES * WAVE), lds_bytes, stream(),
