@@ -16,6 +16,8 @@ namespace kmx {
 
 constexpr int WAVE = 64; /* gfx950 wavefront width */
 
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
 /* Records the message returned by kmx_last_error() and passes `code` through. */
 int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 void clear_error();

@@ -257,9 +257,39 @@ update_private_kernel(const float* __restrict__ data, size_t stride, const uint3
  * partial layout: [chunk][cluster][dim].
  */
 constexpr uint32_t SORT_SHIFT = 15; /* local point index bits: chunk_points <= 32768 */
-constexpr int SORT_UNROLL = 8;      /* row loads in flight per lane group in the segment-sum phase */
+constexpr int SORT_UNROLL = 8;      /* row loads per batch and lane group in the segment-sum phase (two batches in flight) */
 
-template <int ITEMS, int GW>
+/* VEC consecutive floats of a row per lane: one 16-byte load when VEC = 4 (needs dim, stride % 4 == 0 and an aligned base). */
+template <int VEC> struct RowPart { float v[VEC]; };
+
+template <int VEC>
+__device__ __forceinline__ RowPart<VEC> load_part(const float* p)
+{
+	RowPart<VEC> r;
+	if constexpr (VEC == 4) {
+		const f32x4 t = *(const f32x4*)p;
+		r.v[0] = t.x; r.v[1] = t.y; r.v[2] = t.z; r.v[3] = t.w;
+	} else {
+#pragma unroll
+		for (int i = 0; i < VEC; ++i) r.v[i] = p[i];
+	}
+	return r;
+}
+
+template <int VEC>
+__device__ __forceinline__ void store_part(float* p, const RowPart<VEC>& r)
+{
+	if constexpr (VEC == 4) {
+		f32x4 t;
+		t.x = r.v[0]; t.y = r.v[1]; t.z = r.v[2]; t.w = r.v[3];
+		*(f32x4*)p = t;
+	} else {
+#pragma unroll
+		for (int i = 0; i < VEC; ++i) p[i] = r.v[i];
+	}
+}
+
+template <int ITEMS, int GW, int VEC>
 __global__ void __launch_bounds__(1024)
 update_sorted_kernel(const float* __restrict__ data, size_t stride, const uint32_t* __restrict__ assignment,
                      float* __restrict__ partial, uint32_t* __restrict__ sizes,
@@ -348,81 +378,106 @@ update_sorted_kernel(const float* __restrict__ data, size_t stride, const uint32
 		return lo;
 	};
 	const uint32_t c_lo = first_cluster(group), c_hi = first_cluster(group + 1);
-	const bool lane_on = gl < width;
-	const float* src = data + (size_t)p_begin * stride + d0 + (lane_on ? gl : 0);
-	float* out = partial + ((size_t)blockIdx.x * k) * dim + d0 + gl;
+	const bool lane_on = gl * VEC < width;
+	const float* src = data + (size_t)p_begin * stride + d0 + (lane_on ? gl * VEC : 0);
+	float* out = partial + ((size_t)blockIdx.x * k) * dim + d0 + gl * VEC;
 	uint32_t cur = c_lo;
-	float acc = 0.0f;
+	RowPart<VEC> acc;
+#pragma unroll
+	for (int i = 0; i < VEC; ++i) acc.v[i] = 0.0f;
+	auto flush_to = [&](uint32_t t) {
+		while (cur < t) {
+			if (lane_on) store_part<VEC>(out + (size_t)cur * dim, acc);
+#pragma unroll
+			for (int i = 0; i < VEC; ++i) acc.v[i] = 0.0f;
+			++cur;
+		}
+	};
 	uint32_t e = offsets[c_lo];
 	const uint32_t e_end = offsets[c_hi];
-	for (; e + SORT_UNROLL <= e_end; e += SORT_UNROLL) {
-		uint32_t ent[SORT_UNROLL];
-		float v[SORT_UNROLL];
+	/* software pipeline: the row loads of the next batch are issued before the current batch is summed */
+	constexpr uint32_t LOCAL_MASK = (1u << SORT_SHIFT) - 1u;
+	uint32_t ent[SORT_UNROLL];
+	RowPart<VEC> v[SORT_UNROLL];
+	bool have = e + SORT_UNROLL <= e_end;
+	if (have) {
 #pragma unroll
 		for (int u = 0; u < SORT_UNROLL; ++u) ent[u] = sorted[e + u];
 #pragma unroll
-		for (int u = 0; u < SORT_UNROLL; ++u) v[u] = src[(size_t)(ent[u] & ((1u << SORT_SHIFT) - 1u)) * stride];
+		for (int u = 0; u < SORT_UNROLL; ++u) v[u] = load_part<VEC>(src + (size_t)(ent[u] & LOCAL_MASK) * stride);
+	}
+	while (have) {
+		e += SORT_UNROLL;
+		const bool more = e + SORT_UNROLL <= e_end;
+		uint32_t ent_next[SORT_UNROLL];
+		RowPart<VEC> v_next[SORT_UNROLL];
+		if (more) {
+#pragma unroll
+			for (int u = 0; u < SORT_UNROLL; ++u) ent_next[u] = sorted[e + u];
+#pragma unroll
+			for (int u = 0; u < SORT_UNROLL; ++u) v_next[u] = load_part<VEC>(src + (size_t)(ent_next[u] & LOCAL_MASK) * stride);
+		}
 #pragma unroll
 		for (int u = 0; u < SORT_UNROLL; ++u) {
-			const uint32_t t = ent[u] >> SORT_SHIFT;
-			while (cur < t) {
-				if (lane_on) out[(size_t)cur * dim] = acc;
-				acc = 0.0f;
-				++cur;
-			}
-			acc += v[u];
+			flush_to(ent[u] >> SORT_SHIFT);
+#pragma unroll
+			for (int i = 0; i < VEC; ++i) acc.v[i] += v[u].v[i];
 		}
+		if (more) {
+#pragma unroll
+			for (int u = 0; u < SORT_UNROLL; ++u) {
+				ent[u] = ent_next[u];
+				v[u] = v_next[u];
+			}
+		}
+		have = more;
 	}
 	for (; e < e_end; ++e) {
-		const uint32_t ent = sorted[e];
-		const float v = src[(size_t)(ent & ((1u << SORT_SHIFT) - 1u)) * stride];
-		const uint32_t t = ent >> SORT_SHIFT;
-		while (cur < t) {
-			if (lane_on) out[(size_t)cur * dim] = acc;
-			acc = 0.0f;
-			++cur;
-		}
-		acc += v;
+		const uint32_t one = sorted[e];
+		const RowPart<VEC> row = load_part<VEC>(src + (size_t)(one & LOCAL_MASK) * stride);
+		flush_to(one >> SORT_SHIFT);
+#pragma unroll
+		for (int i = 0; i < VEC; ++i) acc.v[i] += row.v[i];
 	}
-	while (cur < c_hi) {
-		if (lane_on) out[(size_t)cur * dim] = acc;
-		acc = 0.0f;
-		++cur;
-	}
+	flush_to(c_hi);
 }
 
 /*
  * means[c][d] = (sum over the chunks of partial[chunk][c][d]) / count[c]  (0 for an empty cluster).
- * Block = 64 consecutive elements x 4 chunk shares; every lane keeps 8 loads in flight; the shares meet in LDS.
+ * Block = 64 consecutive elements x 16 chunk shares; every lane keeps up to 16 loads in flight; the shares meet in LDS.
  * Overwrites means: the sorted path needs neither zeroed centroids nor the separate divide kernel.
  */
+constexpr uint32_t REDUCE_SHARES = 16;
+
 template <int LM>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(64 * REDUCE_SHARES)
 reduce_partials_kernel(const float* __restrict__ partial, float* __restrict__ means, size_t stride_means,
                        const uint32_t* __restrict__ sizes, uint32_t dim, uint32_t k, uint32_t chunks)
 {
-	__shared__ float part[4][64];
+	__shared__ float part[REDUCE_SHARES][64];
 	const uint32_t col = threadIdx.x & 63, share = threadIdx.x >> 6;
 	const uint32_t e = blockIdx.x * 64 + col;
 	const size_t kd = (size_t)k * dim;
 	float s = 0.0f;
 	if (e < kd) {
-		const uint32_t per = (chunks + 3) / 4;
-		const uint32_t c0 = share * per, c1 = min(c0 + per, chunks);
+		const uint32_t per = (chunks + REDUCE_SHARES - 1) / REDUCE_SHARES;
+		const uint32_t c0 = min(share * per, chunks), c1 = min(c0 + per, chunks);
 		uint32_t c = c0;
-		for (; c + 8 <= c1; c += 8) {
-			float v[8];
+		for (; c + 16 <= c1; c += 16) {
+			float v[16];
 #pragma unroll
-			for (int u = 0; u < 8; ++u) v[u] = partial[(size_t)(c + u) * kd + e];
+			for (int u = 0; u < 16; ++u) v[u] = partial[(size_t)(c + u) * kd + e];
 #pragma unroll
-			for (int u = 0; u < 8; ++u) s += v[u];
+			for (int u = 0; u < 16; ++u) s += v[u];
 		}
 		for (; c < c1; ++c) s += partial[(size_t)c * kd + e];
 	}
 	part[share][col] = s;
 	__syncthreads();
 	if (share == 0 && e < kd) {
-		s = (part[0][col] + part[1][col]) + (part[2][col] + part[3][col]);
+		s = 0.0f;
+#pragma unroll
+		for (uint32_t i = 0; i < REDUCE_SHARES; ++i) s += part[i][col];
 		const uint32_t cl = e / dim, d = e - cl * dim;
 		const uint32_t count = sizes[cl];
 		means[elem<LM>(stride_means, cl, d)] = count ? s / (float)count : 0.0f;
@@ -472,21 +527,30 @@ static uint32_t pow2_at_least(uint32_t v)
 }
 
 template <int ITEMS, int LM>
-static int launch_sorted(const UpdateArgs& u, Workspace* ws, uint32_t chunks, uint32_t slices, uint32_t chunk_points, uint32_t gw, uint32_t lds_bytes)
+static int launch_sorted(const UpdateArgs& u, Workspace* ws, uint32_t chunks, uint32_t slices, uint32_t chunk_points, uint32_t gw, uint32_t vec, uint32_t lds_bytes)
 {
 	void (*kernel)(const float*, size_t, const uint32_t*, float*, uint32_t*, uint32_t, uint32_t, uint32_t, uint32_t) = nullptr;
-	switch (gw) {
-	case 4: kernel = update_sorted_kernel<ITEMS, 4>; break;
-	case 8: kernel = update_sorted_kernel<ITEMS, 8>; break;
-	case 16: kernel = update_sorted_kernel<ITEMS, 16>; break;
-	default: kernel = update_sorted_kernel<ITEMS, 32>; break;
+	if (vec == 4) {
+		switch (gw) {
+		case 1: kernel = update_sorted_kernel<ITEMS, 1, 4>; break;
+		case 2: kernel = update_sorted_kernel<ITEMS, 2, 4>; break;
+		case 4: kernel = update_sorted_kernel<ITEMS, 4, 4>; break;
+		default: kernel = update_sorted_kernel<ITEMS, 8, 4>; break;
+		}
+	} else {
+		switch (gw) {
+		case 4: kernel = update_sorted_kernel<ITEMS, 4, 1>; break;
+		case 8: kernel = update_sorted_kernel<ITEMS, 8, 1>; break;
+		case 16: kernel = update_sorted_kernel<ITEMS, 16, 1>; break;
+		default: kernel = update_sorted_kernel<ITEMS, 32, 1>; break;
+		}
 	}
 	KMX_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
 	hipLaunchKernelGGL(kernel, dim3(chunks, slices), dim3(1024), lds_bytes, stream(),
 	                   u.data, u.stride, u.assignment, ws->partials, u.cluster_sizes, u.dim, u.k, u.n, chunk_points);
 	KMX_LAUNCH_CHECK("update_sorted_kernel");
 	const uint32_t total = u.k * u.dim;
-	hipLaunchKernelGGL((reduce_partials_kernel<LM>), dim3((total + 63) / 64), dim3(256), 0, stream(),
+	hipLaunchKernelGGL((reduce_partials_kernel<LM>), dim3((total + 63) / 64), dim3(64 * REDUCE_SHARES), 0, stream(),
 	                   ws->partials, u.means, u.stride_means, u.cluster_sizes, u.dim, u.k, chunks);
 	KMX_LAUNCH_CHECK("reduce_partials_kernel");
 	return KMX_OK;
@@ -525,7 +589,9 @@ static int launch_update_tuned(const UpdateArgs& u, kmx_exec_params* exec, Works
 
 	if (LD == KMX_AOS && u.k < (1u << (32 - SORT_SHIFT)) && (uint64_t)(u.k + 33) * 4 + 1024 * 4 <= budget) {
 		const uint32_t slices = (u.dim + 31) / 32;
-		const uint32_t gw = u.dim > 16 ? 32 : pow2_at_least(std::max<uint32_t>(u.dim, 4));
+		/* 16-byte row parts where one slice covers the row and its alignment allows it (measured: no gain for sliced rows) */
+		const uint32_t vec = (u.dim <= 32 && u.dim % 4 == 0 && u.stride % 4 == 0 && ((uintptr_t)u.data & 15) == 0) ? 4 : 1;
+		const uint32_t gw = (u.dim > 16 ? 32 : pow2_at_least(std::max<uint32_t>(u.dim, 4))) / vec;
 		const uint32_t max_points = std::min<uint32_t>(1u << SORT_SHIFT, (budget - (u.k + 33) * 4) / 4 / 1024 * 1024);
 		uint32_t chunks = std::max<uint32_t>(1, dev.compute_units / slices);
 		uint32_t chunk_points = (u.n + chunks - 1) / chunks;
@@ -537,10 +603,10 @@ static int launch_update_tuned(const UpdateArgs& u, kmx_exec_params* exec, Works
 		exec->block_count = chunks * slices;
 		*state = 2;
 		const uint32_t items = chunk_points / 1024;
-		if (items <= 4) return launch_sorted<4, LM>(u, ws, chunks, slices, chunk_points, gw, lds_bytes);
-		if (items <= 8) return launch_sorted<8, LM>(u, ws, chunks, slices, chunk_points, gw, lds_bytes);
-		if (items <= 16) return launch_sorted<16, LM>(u, ws, chunks, slices, chunk_points, gw, lds_bytes);
-		return launch_sorted<32, LM>(u, ws, chunks, slices, chunk_points, gw, lds_bytes);
+		if (items <= 4) return launch_sorted<4, LM>(u, ws, chunks, slices, chunk_points, gw, vec, lds_bytes);
+		if (items <= 8) return launch_sorted<8, LM>(u, ws, chunks, slices, chunk_points, gw, vec, lds_bytes);
+		if (items <= 16) return launch_sorted<16, LM>(u, ws, chunks, slices, chunk_points, gw, vec, lds_bytes);
+		return launch_sorted<32, LM>(u, ws, chunks, slices, chunk_points, gw, vec, lds_bytes);
 	}
 
 	/* fallback: LDS-privatised floating-point atomics */
