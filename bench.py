@@ -70,7 +70,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--config", type=int, default=2, help="benchmark configuration 1..5 (2 = headline)")
     ap.add_argument("--cpu-sample", type=int, default=0, help="points in the CPU baseline sample (0 = about 12 s of work)")
-    ap.add_argument("--assign-variant", default="best", choices=["base", "lds_fma", "mfma", "best"])
+    ap.add_argument("--assign-variant", default="best", choices=["base", "lds_fma", "mfma", "mfma_bf16x3", "best"])
     ap.add_argument("--update-variant", default="atomic_shm", choices=["atomic_point", "atomic_fine", "atomic_shm"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -90,7 +90,8 @@ def main():
     data = km.generate_points(spec)
     means0 = km.first_k_means(spec)
 
-    assign_variant = {"base": km.ASSIGN_BASE, "lds_fma": km.ASSIGN_LDS_FMA, "mfma": km.ASSIGN_MFMA, "best": km.ASSIGN_BEST}[args.assign_variant]
+    assign_variant = {"base": km.ASSIGN_BASE, "lds_fma": km.ASSIGN_LDS_FMA, "mfma": km.ASSIGN_MFMA, "mfma_bf16x3": km.ASSIGN_MFMA_BF16X3,
+                      "best": km.ASSIGN_BEST}[args.assign_variant]
     update_variant = {"atomic_point": km.UPDATE_ATOMIC_POINT, "atomic_fine": km.UPDATE_ATOMIC_FINE,
                       "atomic_shm": km.UPDATE_ATOMIC_SHM}[args.update_variant]
     alg = km.HipKMeansAlgorithm(assign_variant, update_variant)

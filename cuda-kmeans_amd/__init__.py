@@ -20,7 +20,7 @@ HIP_LIB_PATH = os.path.join(_HERE, "csrc", "libkmx_hip.so")
 HOST_LIB_PATH = os.path.join(_HERE, "host", "libkmx_host.so")
 
 AOS, SOA = 0, 1
-ASSIGN_BASE, ASSIGN_LDS_FMA, ASSIGN_MFMA, ASSIGN_BEST = 0, 1, 2, 3
+ASSIGN_BASE, ASSIGN_LDS_FMA, ASSIGN_MFMA, ASSIGN_BEST, ASSIGN_MFMA_BF16X3 = 0, 1, 2, 3, 4
 UPDATE_ATOMIC_POINT, UPDATE_ATOMIC_FINE, UPDATE_ATOMIC_SHM = 0, 1, 2
 
 KMX_OK, KMX_ERR_INVALID_ARGUMENT, KMX_ERR_UNSUPPORTED, KMX_ERR_DEVICE, KMX_ERR_NO_DEVICE = 0, 1, 2, 3, 4

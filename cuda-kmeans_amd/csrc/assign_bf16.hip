@@ -1,0 +1,123 @@
+/*
+ * Assignment on the matrix cores at bf16 rate with fp32-level accuracy: a[j][i] = |c_j|^2 - 2 c_j . x_i as
+ * v_mfma_f32_32x32x16_bf16 tiles over SPLIT operands.
+ *
+ * Every fp32 value v is written as hi + mid + rest with hi = bf16(v), mid = bf16(v - hi) (round to nearest
+ * even), |rest| <= 2^-18 |v|. The contraction keeps the three largest of the four hi/mid products,
+ *      c'.x  ~  sum_i  c'hi_i x_mid_i + c'mid_i x_hi_i + c'hi_i x_hi_i ,       c' = -2c,
+ * each product exact in fp32 (8 x 8 significant bits), accumulated in fp32 by the matrix core. One block of
+ * 16 dimensions costs 3 MFMAs of 8 passes where the fp32 kernel (v_mfma_f32_32x32x2_f32) spends 8 MFMAs of
+ * 16 passes: 24 against 128 matrix-core passes per tile and block.
+ *
+ * Exactness. As in the fp32 kernel the result promised to the caller is the index the serial scan returns
+ * (reference serial.hpp:21-35, metric_policies.hpp:23-28,40-44), established by the same certification:
+ * a point whose two smallest a[j] are further apart than tau is decided, every other point goes to the
+ * recheck queue and is re-evaluated with the serial arithmetic. Only tau differs. With u' = 2^-23 (one
+ * unit allows for any rounding or truncation of the accumulator) and S = |x|^2 + max_j |c_j|^2:
+ *   - dropped terms:   |c'_i x_i - (three products)| <= (2^-18 + 2^-18 + 2^-18)(1 + 2^-8) |c'_i||x_i|,
+ *                      and sum_i |c'_i||x_i| <= 2|c||x| <= S            -> 3.02 * 2^-18 S  (= 96.6 u' S)
+ *   - accumulation of 3d products and |c|^2 in fp32                      -> (3d + 2) u' * 2 S
+ *   - the serial sum's own error and the sqrt collision margin           -> (2d + 12) u' S   (as for fp32)
+ * tau must exceed twice the error of a[j] plus the serial margin: (12d + 8 + 193.3 + 2d + 12) u' S, so
+ *      tau = (14 d + 224) 2^-23 (|x|^2 + max_j |c_j|^2).
+ * The refinement (winning row inside the winning tile) re-evaluates rows with v_dot2c_f32_bf16 on the same
+ * three products, so the same bound covers it.
+ *
+ * Data flow, tiling, tracking, flag buffering and the recheck hand-over are those of the fp32 kernel
+ * (assign_mfma.hip); the packed centroid row holds hi and mid parts of -2c, 4 bytes per dimension as before.
+ */
+#include "assign_bf16_impl.h"
+
+namespace kmx {
+
+/* supported blocks of 16 dimensions per row */
+static uint32_t pick_kb(uint32_t dim)
+{
+	const uint32_t need = (dim + KBLOCK - 1) / KBLOCK;
+	const uint32_t options[] = { 1, 2, 3, 4, 8, 16 };
+	for (uint32_t o : options)
+		if (need <= o) return o;
+	return 0;
+}
+
+/*
+ * One wavefront per (padded) centroid row: hi/mid parts of -2c in the unit order tile_step_bf16 reads,
+ * |c|^2 by a wavefront reduction, and the exact transposed copy for the recheck pass.
+ */
+template <int LM>
+__global__ void __launch_bounds__(256)
+pack_means_bf16_kernel(const float* __restrict__ means, size_t stride_means, float* __restrict__ packed, float* __restrict__ norms,
+                       float* __restrict__ means_t, uint32_t dim, uint32_t k, uint32_t kp, uint32_t dp, uint32_t* __restrict__ counters)
+{
+	const uint32_t lane = threadIdx.x & (WAVE - 1);
+	const uint32_t j = (blockIdx.x * blockDim.x + threadIdx.x) / WAVE;
+	if (blockIdx.x == 0 && threadIdx.x == 0) counters[0] = 0u; /* the recheck queue of this call starts empty */
+	if (j >= kp) return;
+	const uint32_t rs = dp + ROW_PAD;
+	float* row = packed + packed_row(j, rs);
+	__bf16* parts = (__bf16*)row;
+	float c2 = 0.0f;
+	for (uint32_t q = lane; q < dp; q += WAVE) {
+		const float v = (j < k && q < dim) ? means[elem<LM>(stride_means, j, q)] : 0.0f;
+		c2 += v * v;
+		__bf16 hi, mid;
+		split_bf16(-2.0f * v, hi, mid);
+		/* block q / 16, half-wave (q % 16) / 8: 16-byte unit 4 kb + 2 h (hi), + 1 (mid) */
+		const uint32_t unit = 4 * (q / KBLOCK) + 2 * ((q % KBLOCK) / 8);
+		parts[8 * unit + q % 8] = hi;
+		parts[8 * (unit + 1) + q % 8] = mid;
+		if (q < dim) means_t[(size_t)q * kp + j] = v; /* exact copy for the recheck pass */
+	}
+	const uint32_t pad_floats = ROW_PAD + (j % TILE == TILE - 1 ? TILE_PAD : 0);
+	if (lane < pad_floats) row[dp + lane] = 0.0f;
+	for (int off = WAVE / 2; off > 0; off >>= 1) c2 += __shfl_xor(c2, off);
+	if (lane == 0) norms[norm_at(j)] = j < k ? c2 : __builtin_inff();
+	if (lane < NORM_TILE - TILE && j % TILE == 0) norms[(j / TILE) * NORM_TILE + TILE + lane] = __builtin_inff();
+}
+
+bool bf16_supports(const AssignArgs& a, const DeviceInfo& dev)
+{
+	const uint32_t kb = pick_kb(a.dim);
+	if (kb == 0) return false;
+	return (size_t)(tile_floats(KBLOCK * kb + ROW_PAD) + NORM_TILE) * 4 + 8192 <= dev.lds_bytes;
+}
+
+#define KMX_DECLARE_BF16_LAUNCHER(W) \
+	int launch_bf16_##W(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev, uint32_t kp, float kd);
+KMX_DECLARE_BF16_LAUNCHER(1) KMX_DECLARE_BF16_LAUNCHER(2) KMX_DECLARE_BF16_LAUNCHER(3) KMX_DECLARE_BF16_LAUNCHER(4)
+KMX_DECLARE_BF16_LAUNCHER(8) KMX_DECLARE_BF16_LAUNCHER(16)
+
+int launch_assign_bf16(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev)
+{
+	const uint32_t kb = pick_kb(a.dim);
+	const uint32_t dp = KBLOCK * kb;
+	const uint32_t kp = round_up(a.k, TILE);
+	int rc = reserve_packed(ws, (size_t)(kp / TILE) * tile_floats(dp + ROW_PAD), (size_t)(kp / TILE) * NORM_TILE, (size_t)kp * a.dim);
+	if (rc) return rc;
+	rc = reserve_queue(ws, a.n);
+	if (rc) return rc;
+	const uint32_t pack_blocks = (kp * WAVE + 255) / 256;
+	if (a.layout_means == KMX_AOS)
+		hipLaunchKernelGGL((pack_means_bf16_kernel<KMX_AOS>), dim3(pack_blocks), dim3(256), 0, stream(),
+		                   a.means, a.stride_means, ws->packed_means, ws->norms, ws->means_t, a.dim, a.k, kp, dp, ws->counters);
+	else
+		hipLaunchKernelGGL((pack_means_bf16_kernel<KMX_SOA>), dim3(pack_blocks), dim3(256), 0, stream(),
+		                   a.means, a.stride_means, ws->packed_means, ws->norms, ws->means_t, a.dim, a.k, kp, dp, ws->counters);
+	KMX_LAUNCH_CHECK("pack_means_bf16_kernel");
+
+	/* tau = kd (|x|^2 + max|c|^2), kd = (14 d + 224) 2^-23 (see the bound at the top of the file) */
+	const float kd = (14.0f * (float)a.dim + 224.0f) * 1.1920929e-07f;
+	switch (kb) {
+	case 1: rc = launch_bf16_1(a, exec, ws, dev, kp, kd); break;
+	case 2: rc = launch_bf16_2(a, exec, ws, dev, kp, kd); break;
+	case 3: rc = launch_bf16_3(a, exec, ws, dev, kp, kd); break;
+	case 4: rc = launch_bf16_4(a, exec, ws, dev, kp, kd); break;
+	case 8: rc = launch_bf16_8(a, exec, ws, dev, kp, kd); break;
+	case 16: rc = launch_bf16_16(a, exec, ws, dev, kp, kd); break;
+	default: return fail(KMX_ERR_UNSUPPORTED, "assign (split-bf16 MFMA): dim %u is not supported", a.dim);
+	}
+	if (rc) return rc;
+	return launch_recheck(a, ws, kp);
+}
+
+} // namespace kmx

@@ -1,0 +1,398 @@
+/*
+ * Device code of the split-bf16 MFMA assignment (see assign_bf16.hip for the design notes and the error bound).
+ * Instantiated per row width in separate translation units (assign_bf16_inst.hip, one object per KMX_KB value).
+ * Tile geometry, padding, tracking and the recheck hand-over are those of the fp32 MFMA kernel.
+ */
+#ifndef KMX_ASSIGN_BF16_IMPL_H
+#define KMX_ASSIGN_BF16_IMPL_H
+
+#include "assign_mfma_impl.h"
+
+namespace kmx {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr uint32_t KBLOCK = 16; /* dimensions per v_mfma_f32_32x32x16_bf16 */
+
+/* value = hi + mid + (at most 2^-18 |value|), both parts bf16 (round to nearest even) */
+__device__ __forceinline__ void split_bf16(float v, __bf16& hi, __bf16& mid)
+{
+	hi = (__bf16)v;
+	mid = (__bf16)(v - (float)hi);
+}
+
+/* One tile of 32 points as B operands: per block of 16 dimensions the lane holds the 8 dimensions of its
+ * half-wave (lanes 0-31: the first 8, lanes 32-63: the second 8) of ONE point, as hi and mid parts. */
+template <int KB> struct SplitPoints {
+	bf16x8 hi[KB], mid[KB];
+};
+
+/* points of one sweep unit -> split B operands; xx = this lane's share of |x|^2; rows beyond n read as zero */
+template <int KB, int P, int LD, bool VEC>
+__device__ __forceinline__ void load_split_points(SplitPoints<KB> (&b)[P], float (&xx)[P], const float* __restrict__ data, size_t stride,
+                                                  uint32_t base, uint32_t col, uint32_t h, uint32_t dim, uint32_t n)
+{
+#pragma unroll
+	for (int p = 0; p < P; ++p) {
+		const uint32_t pt = base + p * TILE + col;
+		const bool valid = pt < n;
+		float part = 0.0f;
+#pragma unroll
+		for (int kb = 0; kb < KB; ++kb) {
+			const uint32_t d0 = kb * KBLOCK + h * 8;
+			float v[8];
+			if (LD == KMX_AOS && VEC) {
+				const float* src = data + (size_t)pt * stride + d0;
+				f32x4 lo = { 0.0f, 0.0f, 0.0f, 0.0f }, up = { 0.0f, 0.0f, 0.0f, 0.0f };
+				if (valid && d0 < dim) lo = *(const f32x4*)src;
+				if (valid && d0 + 4 < dim) up = *(const f32x4*)(src + 4);
+				v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w;
+				v[4] = up.x; v[5] = up.y; v[6] = up.z; v[7] = up.w;
+			}
+			else {
+#pragma unroll
+				for (int j = 0; j < 8; ++j) v[j] = (valid && d0 + j < dim) ? data[elem<LD>(stride, pt, d0 + j)] : 0.0f;
+			}
+#pragma unroll
+			for (int j = 0; j < 8; ++j) {
+				part += v[j] * v[j];
+				__bf16 hi, mid;
+				split_bf16(v[j], hi, mid);
+				b[p].hi[kb][j] = hi;
+				b[p].mid[kb][j] = mid;
+			}
+		}
+		xx[p] = part;
+	}
+}
+
+/* the 16 bytes (8 bf16) at 16-byte unit `unit` of a packed row */
+__device__ __forceinline__ bf16x8 row_unit(const float* row, uint32_t unit) { return *(const bf16x8*)(row + 4 * unit); }
+
+/*
+ * One step of the software pipeline: the MFMAs of tile `tile_new` into acc_new (three products per block of 16
+ * dimensions: hi*mid, mid*hi, hi*hi -- small terms first) and the tracking of the previous tile's results.
+ * Packed row layout, in 16-byte units: block kb, half-wave h -> unit 4 kb + 2 h holds the hi parts of the
+ * 8 dimensions, unit 4 kb + 2 h + 1 the mid parts.
+ */
+template <int KB, int P, bool TRACK, bool COARSE>
+__device__ __forceinline__ void tile_step_bf16(const float* __restrict__ lds, const float* __restrict__ lds_norms, uint32_t tile_new,
+                                               uint32_t col, uint32_t h, const SplitPoints<KB> (&b)[P],
+                                               f32x16 (&acc_new)[P], const f32x16 (&acc_old)[P], uint32_t tile_old,
+                                               Track (&st)[P], float neg_inf)
+{
+	constexpr uint32_t RS = KBLOCK * KB + ROW_PAD;
+	const float* arow = lds + (size_t)tile_new * tile_floats(RS) + (size_t)col * RS;
+	bf16x8 chi[KB], cmid[KB];
+#pragma unroll
+	for (int kb = 0; kb < KB; ++kb) {
+		chi[kb] = row_unit(arow, 4 * kb + 2 * h);
+		cmid[kb] = row_unit(arow, 4 * kb + 2 * h + 1);
+	}
+	/* C operand: |c|^2 of the 16 rows this lane receives: rows 8g + 4h + (0..3), g = 0..3 */
+	f32x16 cinit;
+#pragma unroll
+	for (int g = 0; g < 4; ++g) {
+		f32x4 v = *(const f32x4*)(lds_norms + tile_new * NORM_TILE + 8 * g + 4 * h);
+		cinit[4 * g] = v.x; cinit[4 * g + 1] = v.y; cinit[4 * g + 2] = v.z; cinit[4 * g + 3] = v.w;
+	}
+#pragma unroll
+	for (int p = 0; p < P; ++p) acc_new[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(chi[0], b[p].mid[0], cinit, 0, 0, 0);
+#pragma unroll
+	for (int kb = 0; kb < KB; ++kb) {
+		if (kb > 0) {
+#pragma unroll
+			for (int p = 0; p < P; ++p) acc_new[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(chi[kb], b[p].mid[kb], acc_new[p], 0, 0, 0);
+		}
+#pragma unroll
+		for (int p = 0; p < P; ++p) acc_new[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cmid[kb], b[p].hi[kb], acc_new[p], 0, 0, 0);
+#pragma unroll
+		for (int p = 0; p < P; ++p) acc_new[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(chi[kb], b[p].hi[kb], acc_new[p], 0, 0, 0);
+	}
+	if (TRACK) {
+#pragma unroll
+		for (int p = 0; p < P; ++p) track_tile<COARSE>(acc_old[p], st[p], tile_old, neg_inf);
+		constexpr int MFMAS = 3 * KB * P;
+		constexpr int VALU = (COARSE ? 16 : 67) * P;
+		if (KB <= 4) {
+			__builtin_amdgcn_sched_group_barrier(0x008, MFMAS, 0);
+			__builtin_amdgcn_sched_group_barrier(0x002, VALU, 0);
+		}
+	}
+}
+
+/* acc + a[2i] b[2i] + a[2i+1] b[2i+1] as one v_dot2c_f32_bf16 (pairs taken with constant shuffles: extracting a
+ * dword of the bit-cast vector by a loop index made the compiler read element 0 every time) */
+#define KMX_DOT2_PAIR(acc, a, b, i) \
+	__builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(a, a, 2 * (i), 2 * (i) + 1), __builtin_shufflevector(b, b, 2 * (i), 2 * (i) + 1), acc, false)
+
+/* this half-wave's share of the three-product dot of one packed row with one point (the same terms the MFMAs add) */
+template <int KB>
+__device__ __forceinline__ float row_dot_bf16(const float* row, uint32_t h, const SplitPoints<KB>& x)
+{
+	float part = 0.0f;
+#pragma unroll
+	for (int kb = 0; kb < KB; ++kb) {
+		const bf16x8 ch = row_unit(row, 4 * kb + 2 * h);
+		const bf16x8 cm = row_unit(row, 4 * kb + 2 * h + 1);
+		const bf16x8 xh = x.hi[kb];
+		const bf16x8 xm = x.mid[kb];
+		part = KMX_DOT2_PAIR(part, ch, xm, 0); part = KMX_DOT2_PAIR(part, cm, xh, 0); part = KMX_DOT2_PAIR(part, ch, xh, 0);
+		part = KMX_DOT2_PAIR(part, ch, xm, 1); part = KMX_DOT2_PAIR(part, cm, xh, 1); part = KMX_DOT2_PAIR(part, ch, xh, 1);
+		part = KMX_DOT2_PAIR(part, ch, xm, 2); part = KMX_DOT2_PAIR(part, cm, xh, 2); part = KMX_DOT2_PAIR(part, ch, xh, 2);
+		part = KMX_DOT2_PAIR(part, ch, xm, 3); part = KMX_DOT2_PAIR(part, cm, xh, 3); part = KMX_DOT2_PAIR(part, ch, xh, 3);
+	}
+	return part;
+}
+
+template <int KB, int P, int LD, bool VEC, bool STREAM, bool COARSE, bool PREFETCH>
+__global__ void __launch_bounds__(MFMA_WAVES * WAVE)
+assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* __restrict__ packed, const float* __restrict__ norms,
+                   uint32_t* __restrict__ assignment, uint32_t* __restrict__ queue, uint32_t* __restrict__ counters,
+                   uint32_t dim, uint32_t k, uint32_t kp, uint32_t n, uint32_t chunk_rows, float kd, float neg_inf)
+{
+	constexpr uint32_t RS = KBLOCK * KB + ROW_PAD;
+	extern __shared__ float lds[];
+	__shared__ uint32_t wave_max[MFMA_WAVES];
+	__shared__ uint32_t flag_list[MFMA_WAVES][FLAG_CAP];
+
+	const uint32_t lane = threadIdx.x & (WAVE - 1);
+	const uint32_t wave = threadIdx.x / WAVE;
+	const uint32_t col = lane & 31; /* point within a tile (B column) / centroid row fed to A */
+	const uint32_t h = lane >> 5;   /* half-wave: K split and the +4 row group of the result    */
+
+	/* max_j |c_j|^2 (bit pattern maximum: propagates NaN and +inf, which then flag every point) */
+	uint32_t cmax = 0;
+	for (uint32_t j = threadIdx.x; j < k; j += blockDim.x) cmax = max(cmax, __float_as_uint(norms[norm_at(j)]));
+	for (int off = WAVE / 2; off > 0; off >>= 1) cmax = max(cmax, (uint32_t)__shfl_xor((int)cmax, off));
+	if (lane == 0) wave_max[wave] = cmax;
+	__syncthreads();
+	cmax = 0;
+	for (uint32_t w = 0; w < MFMA_WAVES; ++w) cmax = max(cmax, wave_max[w]);
+	const float c2max = __uint_as_float(cmax);
+
+	float* lds_norms = lds + (size_t)(chunk_rows / TILE) * tile_floats(RS);
+	const uint32_t chunks = (kp + chunk_rows - 1) / chunk_rows;
+
+	auto stage = [&](uint32_t row0, uint32_t rows) {
+		const f32x4* src = (const f32x4*)(packed + packed_row(row0, RS));
+		f32x4* dst = (f32x4*)lds;
+		const uint32_t vecs = (rows / TILE) * tile_floats(RS) / 4;
+		for (uint32_t i = threadIdx.x; i < vecs; i += blockDim.x) dst[i] = src[i];
+		const f32x4* nsrc = (const f32x4*)(norms + (size_t)(row0 / TILE) * NORM_TILE);
+		f32x4* ndst = (f32x4*)lds_norms;
+		const uint32_t nvecs = (rows / TILE) * NORM_TILE / 4;
+		for (uint32_t i = threadIdx.x; i < nvecs; i += blockDim.x) ndst[i] = nsrc[i];
+	};
+
+	if (!STREAM) {
+		stage(0, kp);
+		__syncthreads();
+	}
+
+	uint32_t flagged = 0; /* wave-uniform */
+	auto flush_flags = [&]() {
+		__builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+		__builtin_amdgcn_wave_barrier();
+		uint32_t slot = 0;
+		if (lane == 0) slot = atomicAdd(&counters[0], flagged);
+		slot = (uint32_t)__shfl((int)slot, 0);
+		for (uint32_t i = lane; i < flagged; i += WAVE) queue[slot + i] = flag_list[wave][i];
+		__builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+		__builtin_amdgcn_wave_barrier();
+		flagged = 0;
+	};
+
+	const uint32_t unit_points = MFMA_WAVES * P * TILE;
+	const uint32_t units = (n + unit_points - 1) / unit_points;
+
+	auto sweep = [&](const SplitPoints<KB> (&b)[P], const float (&xx)[P], uint32_t base) {
+		float x2[P];
+		Track st[P];
+#pragma unroll
+		for (int p = 0; p < P; ++p) {
+			x2[p] = xx[p] + __shfl_xor(xx[p], 32);
+			st[p].m1 = __builtin_inff();
+			st[p].m2 = __builtin_inff();
+			st[p].tile = 0;
+			st[p].loc = 0;
+		}
+		f32x16 acc0[P], acc1[P];
+		for (uint32_t chunk = 0; chunk < chunks; ++chunk) {
+			const uint32_t row0 = chunk * chunk_rows;
+			const uint32_t rows = min(chunk_rows, kp - row0);
+			if (STREAM) {
+				__syncthreads(); /* everyone is done with the previous chunk */
+				stage(row0, rows);
+				__syncthreads();
+			}
+			const uint32_t tiles = rows / TILE;
+			const uint32_t tile0 = row0 / TILE;
+			tile_step_bf16<KB, P, false, COARSE>(lds, lds_norms, 0, col, h, b, acc0, acc1, 0, st, neg_inf);
+			uint32_t t = 0; /* acc0 holds tile t, not yet tracked */
+			while (t + 2 < tiles) {
+				tile_step_bf16<KB, P, true, COARSE>(lds, lds_norms, t + 1, col, h, b, acc1, acc0, tile0 + t, st, neg_inf);
+				tile_step_bf16<KB, P, true, COARSE>(lds, lds_norms, t + 2, col, h, b, acc0, acc1, tile0 + t + 1, st, neg_inf);
+				t += 2;
+			}
+			if (t + 1 < tiles) {
+				tile_step_bf16<KB, P, true, COARSE>(lds, lds_norms, t + 1, col, h, b, acc1, acc0, tile0 + t, st, neg_inf);
+#pragma unroll
+				for (int p = 0; p < P; ++p) track_tile<COARSE>(acc1[p], st[p], tile0 + t + 1, neg_inf);
+			}
+			else {
+#pragma unroll
+				for (int p = 0; p < P; ++p) track_tile<COARSE>(acc0[p], st[p], tile0 + t, neg_inf);
+			}
+		}
+
+#pragma unroll
+		for (int p = 0; p < P; ++p) {
+			const float o1 = __shfl_xor(st[p].m1, 32);
+			const float o2 = __shfl_xor(st[p].m2, 32);
+			const uint32_t ot = (uint32_t)__shfl_xor((int)st[p].tile, 32);
+			const bool win = st[p].m1 < o1 || (st[p].m1 == o1 && h == 0);
+			uint32_t idx;
+			float first, second;
+			if (COARSE) {
+				/* refinement of the winning 16-row subset (see assign_mfma_impl.h); the rows are re-evaluated with
+				 * v_dot2c_f32_bf16 on the same three products, so the error bound of the MFMA results covers them */
+				const uint32_t ts = win ? st[p].tile : ot;
+				const uint32_t wh = win ? h : 1u - h;
+				const float W = win ? fminf(o1, st[p].m2) : fminf(st[p].m1, o2);
+				const float* tile_base = STREAM ? packed + (size_t)ts * tile_floats(RS) : lds + (size_t)ts * tile_floats(RS);
+				const float* norm_base = STREAM ? norms + ts * NORM_TILE : lds_norms + ts * NORM_TILE;
+				float tot[16];
+#pragma unroll
+				for (int r = 0; r < 16; ++r)
+					tot[r] = row_dot_bf16<KB>(tile_base + (size_t)(8 * (r / 4) + 4 * wh + (r % 4)) * RS, h, b[p]);
+				float v1 = __builtin_inff(), v2 = __builtin_inff();
+				uint32_t rbest = 0;
+#pragma unroll
+				for (int g = 0; g < 4; ++g) {
+					const f32x4 c2 = *(const f32x4*)(norm_base + 8 * g + 4 * wh);
+#pragma unroll
+					for (int q = 0; q < 4; ++q) {
+						const int r = 4 * g + q;
+						const float v = (tot[r] + __shfl_xor(tot[r], 32)) + c2[q];
+						v2 = __builtin_amdgcn_fmed3f(v1, v2, v);
+						const bool lt = v < v1;
+						rbest = lt ? (uint32_t)r : rbest;
+						v1 = lt ? v : v1;
+					}
+				}
+				idx = ts * TILE + 8 * (rbest / 4) + 4 * wh + (rbest % 4);
+				first = v1;
+				second = fminf(v2, W);
+			}
+			else {
+				const uint32_t mine_idx = st[p].tile * TILE + st[p].loc + 4 * h;
+				const uint32_t oi = (uint32_t)__shfl_xor((int)mine_idx, 32);
+				idx = win ? mine_idx : oi;
+				first = fminf(st[p].m1, o1);
+				second = fminf(fmaxf(st[p].m1, o1), fminf(st[p].m2, o2));
+			}
+			const float tau = kd * (x2[p] + c2max);
+			const uint32_t pt = base + p * TILE + col;
+			const bool mine = h == 0 && pt < n;
+			const bool decided = (second - first > tau) && (x2[p] + c2max > 1e-30f);
+			if (mine) assignment[pt] = idx < k ? idx : 0u;
+			const bool flag = mine && !decided;
+			const unsigned long long mask = __ballot(flag);
+			if (mask) {
+				const uint32_t add = (uint32_t)__builtin_popcountll(mask);
+				if (flagged + add > FLAG_CAP) flush_flags();
+				if (flag) flag_list[wave][flagged + __builtin_popcountll(mask & ((1ull << lane) - 1ull))] = pt;
+				flagged += add;
+			}
+		}
+	};
+
+	if (PREFETCH) {
+		SplitPoints<KB> b0[P], b1[P];
+		float xx0[P], xx1[P];
+		uint32_t unit = blockIdx.x;
+		if (unit < units) load_split_points<KB, P, LD, VEC>(b0, xx0, data, stride, (unit * MFMA_WAVES + wave) * P * TILE, col, h, dim, n);
+		while (unit < units) {
+			uint32_t next = unit + gridDim.x;
+			if (next < units) load_split_points<KB, P, LD, VEC>(b1, xx1, data, stride, (next * MFMA_WAVES + wave) * P * TILE, col, h, dim, n);
+			sweep(b0, xx0, (unit * MFMA_WAVES + wave) * P * TILE);
+			unit = next;
+			if (unit >= units) break;
+			next = unit + gridDim.x;
+			if (next < units) load_split_points<KB, P, LD, VEC>(b0, xx0, data, stride, (next * MFMA_WAVES + wave) * P * TILE, col, h, dim, n);
+			sweep(b1, xx1, (unit * MFMA_WAVES + wave) * P * TILE);
+			unit = next;
+		}
+	}
+	else {
+		SplitPoints<KB> b0[P];
+		float xx0[P];
+		for (uint32_t unit = blockIdx.x; unit < units; unit += gridDim.x) {
+			load_split_points<KB, P, LD, VEC>(b0, xx0, data, stride, (unit * MFMA_WAVES + wave) * P * TILE, col, h, dim, n);
+			sweep(b0, xx0, (unit * MFMA_WAVES + wave) * P * TILE);
+		}
+	}
+	if (flagged) flush_flags();
+}
+
+/* point tiles per wavefront and sweep, and whether the next sweep's points are prefetched: bounded by the register file */
+template <int KB> struct SplitSweepShape {
+	static constexpr int P = KB <= 4 ? 2 : 1;
+	static constexpr bool PREFETCH = KB <= 8;
+};
+
+template <int KB, int LD, bool VEC>
+static int launch_bf16_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev, uint32_t kp, float kd)
+{
+	constexpr uint32_t RS = KBLOCK * KB + ROW_PAD;
+	constexpr int P = SplitSweepShape<KB>::P;
+	constexpr bool PF = SplitSweepShape<KB>::PREFETCH;
+	uint32_t budget = exec->shared_mem_bytes ? std::min(exec->shared_mem_bytes, dev.lds_bytes) : dev.lds_bytes;
+	const uint32_t static_bytes = (FLAG_CAP * MFMA_WAVES + 64) * 4;
+	const uint32_t tile_bytes = (tile_floats(RS) + NORM_TILE) * 4;
+	if (budget < static_bytes + tile_bytes) return fail(KMX_ERR_UNSUPPORTED, "assign (split-bf16 MFMA): LDS budget of %u bytes is too small", budget);
+	const uint32_t chunk_rows = std::min<uint32_t>(kp, (budget - static_bytes) / tile_bytes * TILE);
+	const bool stream_mode = chunk_rows < kp;
+	const bool coarse = kp / TILE >= COARSE_MIN_TILES && KB <= 4;
+	const uint32_t lds_bytes = chunk_rows / TILE * tile_bytes;
+	const uint32_t unit_points = MFMA_WAVES * P * TILE;
+	const uint32_t units = (a.n + unit_points - 1) / unit_points;
+	void (*kernel)(const float*, size_t, const float*, const float*, uint32_t*, uint32_t*, uint32_t*,
+	               uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, float, float) = nullptr;
+	if constexpr (KB <= 4) {
+		if (stream_mode) kernel = coarse ? assign_bf16_kernel<KB, P, LD, VEC, true, true, PF> : assign_bf16_kernel<KB, P, LD, VEC, true, false, PF>;
+		else kernel = coarse ? assign_bf16_kernel<KB, P, LD, VEC, false, true, PF> : assign_bf16_kernel<KB, P, LD, VEC, false, false, PF>;
+	}
+	else {
+		kernel = assign_bf16_kernel<KB, P, LD, VEC, true, false, PF>;
+	}
+	KMX_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+	int per_cu = 1;
+	KMX_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)kernel, (int)(MFMA_WAVES * WAVE), lds_bytes));
+	per_cu = std::max(1, std::min(per_cu, 4));
+	const uint32_t grid = std::min(units, dev.compute_units * (uint32_t)per_cu);
+	exec->block_count = grid;
+	int rc = profile_begin(0);
+	if (rc) return rc;
+	hipLaunchKernelGGL(kernel, dim3(grid), dim3(MFMA_WAVES * WAVE), lds_bytes, stream(),
+	                   a.data, a.stride, ws->packed_means, ws->norms, a.assignment, ws->queue, ws->counters,
+	                   a.dim, a.k, kp, a.n, chunk_rows, kd, -__builtin_inff());
+	KMX_LAUNCH_CHECK("assign_bf16_kernel");
+	return profile_end(0);
+}
+
+template <int KB>
+static int launch_bf16_kb(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev, uint32_t kp, float kd)
+{
+	if (a.layout == KMX_SOA) return launch_bf16_t<KB, KMX_SOA, false>(a, exec, ws, dev, kp, kd);
+	const bool aligned = a.dim % 4 == 0 && a.stride % 4 == 0 && ((uintptr_t)a.data % 16) == 0;
+	if (aligned) return launch_bf16_t<KB, KMX_AOS, true>(a, exec, ws, dev, kp, kd);
+	return launch_bf16_t<KB, KMX_AOS, false>(a, exec, ws, dev, kp, kd);
+}
+
+} // namespace kmx
+
+#endif

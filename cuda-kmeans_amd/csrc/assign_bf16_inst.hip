@@ -1,0 +1,21 @@
+/*
+ * One instantiation of the split-bf16 MFMA assignment kernel family: KMX_KB blocks of 16 dimensions per row
+ * (given on the command line).
+ */
+#include "assign_bf16_impl.h"
+
+#ifndef KMX_KB
+#error "compile with -DKMX_KB=<blocks of 16 dimensions per row>"
+#endif
+
+#define KMX_CAT2(a, b) a##b
+#define KMX_CAT(a, b) KMX_CAT2(a, b)
+
+namespace kmx {
+
+int KMX_CAT(launch_bf16_, KMX_KB)(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev, uint32_t kp, float kd)
+{
+	return launch_bf16_kb<KMX_KB>(a, exec, ws, dev, kp, kd);
+}
+
+} // namespace kmx

@@ -108,6 +108,8 @@ int launch_recheck(const AssignArgs& a, Workspace* ws, uint32_t kp);
 int launch_pack_means(const AssignArgs& a, Workspace* ws, uint32_t dp, uint32_t kp);
 bool mfma_supports(const AssignArgs& a, const DeviceInfo& dev);
 int launch_assign_mfma(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev);
+bool bf16_supports(const AssignArgs& a, const DeviceInfo& dev);
+int launch_assign_bf16(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev);
 bool lds_fma_supports(const AssignArgs& a, const DeviceInfo& dev);
 int launch_assign_lds_fma(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev);
 

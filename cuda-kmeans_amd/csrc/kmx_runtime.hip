@@ -298,6 +298,10 @@ int kmx_assign_f32(int variant,
 		if (!mfma_supports(a, *dev))
 			return fail(KMX_ERR_UNSUPPORTED, "kmx_assign_f32: shape dim=%u k=%u is not supported by the MFMA variant", dim, k);
 		return launch_assign_mfma(a, exec, ws, *dev);
+	case KMX_ASSIGN_MFMA_BF16X3:
+		if (!bf16_supports(a, *dev))
+			return fail(KMX_ERR_UNSUPPORTED, "kmx_assign_f32: shape dim=%u k=%u is not supported by the split-bf16 MFMA variant", dim, k);
+		return launch_assign_bf16(a, exec, ws, *dev);
 	case KMX_ASSIGN_BEST:
 		/* counterpart of BestCachedAssignmentKernel::run (reference kernels.cu:706-717): pick by shape */
 		/* the MFMA variant was the fastest at every shape measured (also at dim 4 and k 16) */

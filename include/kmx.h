@@ -59,7 +59,9 @@ typedef enum kmx_assign_variant {
 	KMX_ASSIGN_BASE = 0,    /* BaseAssignmentKernel: one lane per point, the serial arithmetic op for op */
 	KMX_ASSIGN_LDS_FMA = 1, /* CachedFixed/CachedRegs counterpart: centroids in LDS, register tile, fp32 FMA */
 	KMX_ASSIGN_MFMA = 2,    /* dense-contraction path: fp32 MFMA tiles of -2 x.c + |c|^2                */
-	KMX_ASSIGN_BEST = 3     /* BestCachedAssignmentKernel: shape-based selector between 1 and 2         */
+	KMX_ASSIGN_BEST = 3,    /* BestCachedAssignmentKernel: shape-based selector between the tuned variants */
+	KMX_ASSIGN_MFMA_BF16X3 = 4 /* dense-contraction path at bf16 MFMA rate: operands split into hi + mid bf16 parts,
+	                              three products per term, fp32 accumulation; same exact result (certify + recheck) */
 } kmx_assign_variant;
 
 /* Update variants (reference counterparts: kernels.cuh:96-105). */

@@ -63,7 +63,7 @@ def gpu_update(km, variant, data, assignment, dim, k, n, layout=AOS, layout_mean
 
 
 def variants(km, dim=1):
-    v = [km.ASSIGN_BASE, km.ASSIGN_MFMA, km.ASSIGN_BEST]
+    v = [km.ASSIGN_BASE, km.ASSIGN_MFMA, km.ASSIGN_MFMA_BF16X3, km.ASSIGN_BEST]
     return v + [km.ASSIGN_LDS_FMA] if dim <= 64 else v
 
 
@@ -252,7 +252,7 @@ LOOP_CASES = [(1, 65536, 10), (2, 65536, 4), (3, 131072, 3), (5, 1 << 20, 4), (4
 def test_every_iteration_matches_oracle(km, orc, gpu, cid, n, iters):
     spec = km.baseline_config(cid)
     combos = [(km.ASSIGN_BEST, km.UPDATE_ATOMIC_SHM)]
-    combos += [(km.ASSIGN_MFMA, km.UPDATE_ATOMIC_FINE)]
+    combos += [(km.ASSIGN_MFMA, km.UPDATE_ATOMIC_FINE), (km.ASSIGN_MFMA_BF16X3, km.UPDATE_ATOMIC_SHM)]
     if spec.dim <= 64:
         combos += [(km.ASSIGN_LDS_FMA, km.UPDATE_ATOMIC_SHM)]
     if n * spec.k * spec.dim <= 1 << 31:
