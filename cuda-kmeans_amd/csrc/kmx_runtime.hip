@@ -304,7 +304,10 @@ int kmx_assign_f32(int variant,
 		return launch_assign_bf16(a, exec, ws, *dev);
 	case KMX_ASSIGN_BEST:
 		/* counterpart of BestCachedAssignmentKernel::run (reference kernels.cu:706-717): pick by shape */
-		/* the MFMA variant was the fastest at every shape measured (also at dim 4 and k 16) */
+		/* measured: the split-bf16 sweep is about twice as fast as the fp32 one wherever the sweep dominates; it hands
+		 * 2-3 times as many points to the exact pass, which costs more than it saves for very short rows and for
+		 * few centroids (HBM-bound shapes). The fp32 MFMA sweep beat the plain-VALU variant at every shape. */
+		if (bf16_supports(a, *dev) && dim >= 8 && k >= 64) return launch_assign_bf16(a, exec, ws, *dev);
 		if (mfma_supports(a, *dev)) return launch_assign_mfma(a, exec, ws, *dev);
 		if (lds_fma_supports(a, *dev)) return launch_assign_lds_fma(a, exec, ws, *dev);
 		return launch_assign_base(a, exec);

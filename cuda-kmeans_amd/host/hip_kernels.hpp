@@ -118,6 +118,7 @@ public:\
 KMX_DEFINE_ASSIGNMENT_KERNEL(BaseAssignmentKernel, KMX_ASSIGN_BASE)       /* kernels.cu:180-207 */
 KMX_DEFINE_ASSIGNMENT_KERNEL(LdsFmaAssignmentKernel, KMX_ASSIGN_LDS_FMA)  /* role of CachedFixed / CachedRegs, kernels.cu:216-319,546-703 */
 KMX_DEFINE_ASSIGNMENT_KERNEL(MfmaAssignmentKernel, KMX_ASSIGN_MFMA)       /* no counterpart: matrix-core path */
+KMX_DEFINE_ASSIGNMENT_KERNEL(MfmaBf16AssignmentKernel, KMX_ASSIGN_MFMA_BF16X3) /* no counterpart: matrix-core path on split bf16 operands */
 KMX_DEFINE_ASSIGNMENT_KERNEL(BestCachedAssignmentKernel, KMX_ASSIGN_BEST) /* kernels.cu:706-717 */
 
 #define KMX_DEFINE_UPDATE_KERNEL(NAME, VARIANT)\

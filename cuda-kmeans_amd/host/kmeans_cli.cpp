@@ -103,6 +103,7 @@ void run_assignment(const ProgramArguments& args, std::vector<F>& data, std::vec
 	algorithms["hip_base"].reset(new HipAssignmentAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC, BaseAssignmentKernel<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC>>(exec));
 	algorithms["hip_lds_fma"].reset(new HipAssignmentAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC, LdsFmaAssignmentKernel<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC>>(exec));
 	algorithms["hip_mfma"].reset(new HipAssignmentAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC, MfmaAssignmentKernel<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC>>(exec));
+	algorithms["hip_mfma_bf16"].reset(new HipAssignmentAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC, MfmaBf16AssignmentKernel<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC>>(exec));
 	algorithms["hip_best"].reset(new HipAssignmentAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC, BestCachedAssignmentKernel<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC>>(exec));
 
 	auto it = algorithms.find(algoName);
@@ -157,6 +158,7 @@ void run_kmeans(const ProgramArguments& args, std::vector<F>& data, std::vector<
 	using Base = BaseAssignmentKernel<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC>;
 	using Best = BestCachedAssignmentKernel<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC>;
 	using Mfma = MfmaAssignmentKernel<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC>;
+	using MfmaBf16 = MfmaBf16AssignmentKernel<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC>;
 	using Point = UpdateAtomicPointKernel<F, IDX_T, LAYOUT, LAYOUT_MEANS>;
 	using Shm = UpdateAtomicShmKernel<F, IDX_T, LAYOUT, LAYOUT_MEANS>;
 	using map_t = std::map<std::string, std::unique_ptr<IKMeansAlgorithm<F, IDX_T>>>;
@@ -165,6 +167,7 @@ void run_kmeans(const ProgramArguments& args, std::vector<F>& data, std::vector<
 	algorithms["hip_base"].reset(new HipKMeansAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC, Base, Point>(exec, json));
 	algorithms["hip_base_shm"].reset(new HipKMeansAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC, Base, Shm>(exec, json));
 	algorithms["hip_mfma"].reset(new HipKMeansAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC, Mfma, Shm>(exec, json));
+	algorithms["hip_mfma_bf16"].reset(new HipKMeansAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC, MfmaBf16, Shm>(exec, json));
 	algorithms["hip_best"].reset(new HipKMeansAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC, Best, Shm>(exec, json));
 
 	auto it = algorithms.find(algoName);
@@ -292,7 +295,7 @@ int main(int argc, char* argv[])
 		args.registerInt("seed", "Random generator seed.", 42, 0);
 		args.registerBool("assignmentOnly", "Run only assignment part of the algorithm (microbenchmark).");
 		args.conflicts("assignmentOnly", "iterations");
-		args.registerString("algorithm", "Which algorithm is to be tested (serial, hip_base, hip_base_shm, hip_mfma, hip_best; assignment only: hip_lds_fma).", "serial");
+		args.registerString("algorithm", "Which algorithm is to be tested (serial, hip_base, hip_base_shm, hip_mfma, hip_mfma_bf16, hip_best; assignment only: hip_lds_fma).", "serial");
 		args.registerEnum("layout", "Type of data layout.", "aos", { "aos", "soa" });
 		args.registerEnum("layoutMeans", "Type of data layout (override for means only).", "aos", { "aos", "soa" });
 		args.registerBool("double", "Use doubles instead of floats (not built).");

@@ -93,7 +93,7 @@ def test_no_device_is_an_error_not_a_fallback(harness, km):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("algo", ["hip_best", "hip_mfma", "hip_base", "hip_base_shm", "cuda_best"])
+@pytest.mark.parametrize("algo", ["hip_best", "hip_mfma", "hip_mfma_bf16", "hip_base", "hip_base_shm", "cuda_best"])
 def test_device_algorithms_verify(harness, gpu, algo):
     rc, out, err = run(harness, "--config", "1", "--algorithm", algo, "--iterations", "1", "--verify", "--serialThreads", "8", "--json")
     assert rc == 0, out + err
@@ -104,7 +104,7 @@ def test_device_algorithms_verify(harness, gpu, algo):
 
 @pytest.mark.gpu
 def test_device_assignment_only_and_reference_dataset(harness, gpu):
-    for algo in ("hip_best", "hip_mfma", "hip_base", "hip_lds_fma", "cuda_cached_regs", "cuda_cached_fixed"):
+    for algo in ("hip_best", "hip_mfma", "hip_mfma_bf16", "hip_base", "hip_lds_fma", "cuda_cached_regs", "cuda_cached_fixed"):
         rc, out, err = run(harness, "--assignmentOnly", "--algorithm", algo, "--N", "64k", "--k", "256", "--dim", "16", "--verify", "--serialThreads", "8")
         assert rc == 0 and "Verifying results ... OK" in err, err
         assert len(out.split()) == 2
