@@ -32,6 +32,8 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_FP32_TFLOPS = 157.3   # MI355X fp32 (vector or matrix), dense
+PEAK_BF16_TFLOPS = 2500.0  # MI355X bf16 matrix, dense
+VARIANT_NAMES = {0: "base", 1: "lds_fma", 2: "mfma", 4: "mfma_bf16x3"}
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # published full-iteration time for the headline shape on the reference's best hardware (V100 SXM2)
 PUBLISHED_MS = {2: 25.45}  # results/README.md:20 of the reference
@@ -133,6 +135,7 @@ def main():
         k_assign += km.last_kernel_ms(0)
         k_update += km.last_kernel_ms(1)
         rechecked += km.last_rechecked()
+    ran_variant = km.last_assign_variant()
     km.set_profiling(False)
     t_assign /= args.steps; t_update /= args.steps; k_assign /= args.steps; k_update /= args.steps
     alg.cleanup()
@@ -144,7 +147,15 @@ def main():
     update_gbs = update_bytes / (k_update * 1e-3) / 1e9
     assign_gbs = assign_bytes / (k_assign * 1e-3) / 1e9
     # the dominant kernel is the assignment sweep; it is compute-bound unless k is tiny (flop/byte = k/2)
-    if k >= 64:
+    if k >= 64 and ran_variant == km.ASSIGN_MFMA_BF16X3:
+        # split operands: three bf16 products per algorithmic multiply-add, executed on the bf16 matrix pipeline
+        executed = 3.0 * assign_tflops
+        roofline = {"kernel": "assignment sweep (split-bf16 MFMA)", "bound": "mfma", "achieved": round(executed, 1),
+                    "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(executed / PEAK_BF16_TFLOPS, 4),
+                    "traffic": None, "flops_counted": "executed: 3 bf16 products per point x centroid x dim, x2",
+                    "algorithmic_tflops": round(assign_tflops, 1),
+                    "algorithmic_frac_of_fp32_peak": round(assign_tflops / PEAK_FP32_TFLOPS, 4)}
+    elif k >= 64:
         roofline = {"kernel": "assignment sweep", "bound": "mfma", "achieved": round(assign_tflops, 2),
                     "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s", "frac": round(assign_tflops / PEAK_FP32_TFLOPS, 4),
                     "traffic": None}
@@ -168,10 +179,13 @@ def main():
         "vs_baseline": round(ms_per_step / PUBLISHED_MS[args.config], 4) if args.config in PUBLISHED_MS else None,
         "baseline_note": "published: 25.45 ms on V100 SXM2 for this shape (reference results/README.md:20); lower is better"
                          if args.config in PUBLISHED_MS else None,
-        "dtype": "f32", "data": "synthetic",
+        "dtype": "f32 (sweep on bf16x3 split operands, f32 accumulate; exact f32 re-evaluation of uncertified points)"
+                 if ran_variant == km.ASSIGN_MFMA_BF16X3 else "f32",
+        "data": "synthetic",
         "config": {"workload": "benchmark configuration %d: N=%d d=%d k=%d, %s, initial centroids = first k points, seed %d"
                                % (args.config, n, dim, k, "Gaussian mixture" if spec.kind != 1 else "uniform", spec.seed),
-                   "layout": "aos", "assignment": "hip_" + args.assign_variant, "update": args.update_variant},
+                   "layout": "aos", "assignment": "hip_" + args.assign_variant,
+                   "assignment_kernel": VARIANT_NAMES.get(ran_variant, str(ran_variant)), "update": args.update_variant},
         "assign_ms": round(t_assign, 4), "update_ms": round(t_update, 4),
         "points_centroids_dims_per_s": round(float(n) * k * dim / (ms_per_step * 1e-3), 0),
         "rechecked_points_per_iteration": round(rechecked / args.steps, 1),

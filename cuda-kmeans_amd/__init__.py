@@ -29,7 +29,7 @@ KMX_OK, KMX_ERR_INVALID_ARGUMENT, KMX_ERR_UNSUPPORTED, KMX_ERR_DEVICE, KMX_ERR_N
 ABI_SYMBOLS = [
     "kmx_device_count", "kmx_set_device", "kmx_device_props", "kmx_malloc", "kmx_free", "kmx_h2d", "kmx_d2h",
     "kmx_d2d", "kmx_sync", "kmx_set_stream", "kmx_shutdown", "kmx_fill_zero_u32", "kmx_assign_f32",
-    "kmx_assign_last_rechecked", "kmx_update_f32", "kmx_event_create", "kmx_event_destroy", "kmx_event_record",
+    "kmx_assign_last_rechecked", "kmx_assign_last_variant", "kmx_update_f32", "kmx_event_create", "kmx_event_destroy", "kmx_event_record",
     "kmx_event_elapsed_ms", "kmx_set_profiling", "kmx_last_kernel_ms", "kmx_last_error",
 ]
 
@@ -101,6 +101,7 @@ def hip_lib():
         lib.kmx_assign_f32.argtypes = [ctypes.c_int, vp, ctypes.c_int, sz, vp, ctypes.c_int, sz, vp, vp, u32, u32, u32,
                                        ctypes.POINTER(ExecParams)]
         lib.kmx_assign_last_rechecked.argtypes = [ctypes.POINTER(ctypes.c_uint64)]
+        lib.kmx_assign_last_variant.argtypes = [ctypes.POINTER(ctypes.c_int)]
         lib.kmx_update_f32.argtypes = [ctypes.c_int, vp, ctypes.c_int, sz, vp, vp, ctypes.c_int, sz, vp, u32, u32, u32,
                                        ctypes.POINTER(ExecParams)]
         lib.kmx_event_create.argtypes = [ctypes.POINTER(vp)]
@@ -284,6 +285,13 @@ def last_kernel_ms(which):
     ms = ctypes.c_float(0)
     check(hip_lib().kmx_last_kernel_ms(which, ctypes.byref(ms)))
     return ms.value
+
+
+def last_assign_variant():
+    """The concrete variant the last assignment call ran (what ASSIGN_BEST selected)."""
+    v = ctypes.c_int(-1)
+    check(hip_lib().kmx_assign_last_variant(ctypes.byref(v)))
+    return v.value
 
 
 def last_rechecked():

@@ -254,6 +254,8 @@ int kmx_fill_zero_u32(void* dptr, size_t count)
 	return KMX_OK;
 }
 
+static int g_last_assign_variant = -1; /* concrete variant of the last kmx_assign_f32 call */
+
 static int check_layout(const char* who, const char* what, int layout, size_t stride, uint32_t count, uint32_t dim)
 {
 	if (layout != KMX_AOS && layout != KMX_SOA) return fail(KMX_ERR_INVALID_ARGUMENT, "%s: unknown %s layout %d", who, what, layout);
@@ -287,6 +289,17 @@ int kmx_assign_f32(int variant,
 	if (rc) return rc;
 
 	AssignArgs a{ data, layout, stride, means, layout_means, stride_means, assignment, dim, k, n };
+	if (variant == KMX_ASSIGN_BEST) {
+		/* counterpart of BestCachedAssignmentKernel::run (reference kernels.cu:706-717): pick by shape.
+		 * Measured: the split-bf16 sweep is about twice as fast as the fp32 one wherever the sweep dominates; it hands
+		 * 2-3 times as many points to the exact pass, which costs more than it saves for very short rows and for
+		 * few centroids (HBM-bound shapes). The fp32 MFMA sweep beat the plain-VALU variant at every shape. */
+		if (bf16_supports(a, *dev) && dim >= 8 && k >= 64) variant = KMX_ASSIGN_MFMA_BF16X3;
+		else if (mfma_supports(a, *dev)) variant = KMX_ASSIGN_MFMA;
+		else if (lds_fma_supports(a, *dev)) variant = KMX_ASSIGN_LDS_FMA;
+		else variant = KMX_ASSIGN_BASE;
+	}
+	g_last_assign_variant = variant;
 	switch (variant) {
 	case KMX_ASSIGN_BASE:
 		return launch_assign_base(a, exec);
@@ -302,18 +315,17 @@ int kmx_assign_f32(int variant,
 		if (!bf16_supports(a, *dev))
 			return fail(KMX_ERR_UNSUPPORTED, "kmx_assign_f32: shape dim=%u k=%u is not supported by the split-bf16 MFMA variant", dim, k);
 		return launch_assign_bf16(a, exec, ws, *dev);
-	case KMX_ASSIGN_BEST:
-		/* counterpart of BestCachedAssignmentKernel::run (reference kernels.cu:706-717): pick by shape */
-		/* measured: the split-bf16 sweep is about twice as fast as the fp32 one wherever the sweep dominates; it hands
-		 * 2-3 times as many points to the exact pass, which costs more than it saves for very short rows and for
-		 * few centroids (HBM-bound shapes). The fp32 MFMA sweep beat the plain-VALU variant at every shape. */
-		if (bf16_supports(a, *dev) && dim >= 8 && k >= 64) return launch_assign_bf16(a, exec, ws, *dev);
-		if (mfma_supports(a, *dev)) return launch_assign_mfma(a, exec, ws, *dev);
-		if (lds_fma_supports(a, *dev)) return launch_assign_lds_fma(a, exec, ws, *dev);
-		return launch_assign_base(a, exec);
 	default:
 		return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_assign_f32: unknown variant %d", variant);
 	}
+}
+
+int kmx_assign_last_variant(int* variant)
+{
+	clear_error();
+	if (!variant) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_assign_last_variant: null pointer");
+	*variant = g_last_assign_variant;
+	return KMX_OK;
 }
 
 int kmx_assign_last_rechecked(uint64_t* count)

@@ -117,6 +117,10 @@ int kmx_assign_f32(int variant,
 /* Number of points the last kmx_assign_f32 call re-evaluated with the serial arithmetic (waits for the stream). */
 int kmx_assign_last_rechecked(uint64_t* count);
 
+/* The concrete variant (never KMX_ASSIGN_BEST) the last kmx_assign_f32 call ran, -1 before the first call:
+ * what the selector chose, for reports such as the reference's per-algorithm benchmark lines (k-means.cpp:155-169). */
+int kmx_assign_last_variant(int* variant);
+
 /*
  * ---- UPDATE_KERNEL::run(UpdateProblemInstance, CudaExecParameters&) (kernels.cuh:23-36,96-105) ----
  * Precondition as in the reference (cuda.hpp:78-79): means (k x dim, times privatized_copies for
