@@ -156,7 +156,7 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 	constexpr uint32_t RS = KBLOCK * KB + ROW_PAD;
 	extern __shared__ float lds[];
 	__shared__ uint32_t wave_max[MFMA_WAVES];
-	__shared__ uint32_t flag_list[MFMA_WAVES][FLAG_CAP];
+	__shared__ uint32_t flag_list[MFMA_WAVES][2 * FLAG_CAP]; /* (point, threshold) pairs */
 
 	const uint32_t lane = threadIdx.x & (WAVE - 1);
 	const uint32_t wave = threadIdx.x / WAVE;
@@ -199,7 +199,7 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 		uint32_t slot = 0;
 		if (lane == 0) slot = atomicAdd(&counters[0], flagged);
 		slot = (uint32_t)__shfl((int)slot, 0);
-		for (uint32_t i = lane; i < flagged; i += WAVE) queue[slot + i] = flag_list[wave][i];
+		for (uint32_t i = lane; i < 2 * flagged; i += WAVE) queue[2 * (size_t)slot + i] = flag_list[wave][i];
 		__builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
 		__builtin_amdgcn_wave_barrier();
 		flagged = 0;
@@ -304,7 +304,11 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 			if (mask) {
 				const uint32_t add = (uint32_t)__builtin_popcountll(mask);
 				if (flagged + add > FLAG_CAP) flush_flags();
-				if (flag) flag_list[wave][flagged + __builtin_popcountll(mask & ((1ull << lane) - 1ull))] = pt;
+				if (flag) {
+					const uint32_t at = 2 * (flagged + __builtin_popcountll(mask & ((1ull << lane) - 1ull)));
+					flag_list[wave][at] = pt;
+					flag_list[wave][at + 1] = screening_threshold(first, tau);
+				}
 				flagged += add;
 			}
 		}
@@ -351,7 +355,7 @@ static int launch_bf16_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 	constexpr int P = SplitSweepShape<KB>::P;
 	constexpr bool PF = SplitSweepShape<KB>::PREFETCH;
 	uint32_t budget = exec->shared_mem_bytes ? std::min(exec->shared_mem_bytes, dev.lds_bytes) : dev.lds_bytes;
-	const uint32_t static_bytes = (FLAG_CAP * MFMA_WAVES + 64) * 4;
+	const uint32_t static_bytes = (2 * FLAG_CAP * MFMA_WAVES + 64) * 4;
 	const uint32_t tile_bytes = (tile_floats(RS) + NORM_TILE) * 4;
 	if (budget < static_bytes + tile_bytes) return fail(KMX_ERR_UNSUPPORTED, "assign (split-bf16 MFMA): LDS budget of %u bytes is too small", budget);
 	const uint32_t chunk_rows = std::min<uint32_t>(kp, (budget - static_bytes) / tile_bytes * TILE);

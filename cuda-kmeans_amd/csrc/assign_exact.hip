@@ -7,9 +7,8 @@
  *
  *   assign_base_kernel  - one lane per point; counterpart of baseAssignmentKernel
  *                         (reference kernels.cu:180-199) and the `hip_base` algorithm.
- *   recheck_kernel      - one wavefront per queued point; the exact pass behind the fast
- *                         variants (they queue the points whose ranking by |c|^2 - 2x.c is
- *                         not decided beyond rounding error).
+ *   recheck_kernel,     - the exact pass behind the fast variants (they queue the points whose
+ *   recheck_reg_kernel    ranking by |c|^2 - 2x.c is not decided beyond rounding error).
  *
  * Floating-point contraction is switched off for the whole file: a fused multiply-add here
  * would change low-order bits and with them the tie-breaks.
@@ -54,15 +53,29 @@ assign_base_kernel(const float* __restrict__ data, size_t stride, const float* _
 }
 
 /*
- * Exact pass over the queued points, any dimension. A work-group of 256 lanes owns a batch of PB queued points:
- * their coordinates are staged in LDS (rows padded with zeros to a multiple of 4 floats, so that every lane
- * fetches four coordinates with one broadcast 128-bit read), lane t evaluates centroids t, t+256, ... in
- * ascending order against all PB points (16 coalesced loads of the transposed centroid block in flight,
- * each value reused PB times) and keeps its own (distance, index) minimum per point; the 256 candidates are
- * merged by (smaller distance, then smaller index), which is the serial scan's result: the first centroid
- * attaining the minimum. A NaN distance to centroid 0 pins the point to centroid 0, as `minDist > dist` is
- * then never true. Zero padding is exact: (0-0)^2 = +0 leaves a partial sum unchanged.
- * means_t is the exact transposed copy [dim][kp] written by pack_means_kernel.
+ * The exact pass behind the fast variants. A queue entry is (point, threshold): the sweep's smallest ranking value
+ * a[j] = |c_j|^2 - 2 c_j.x plus its tau. The register kernel (rows up to 64 floats) first SCREENS a centroid with
+ * plain fused multiply-adds on the exact centroid copy (the value obeys the sweep's error bound, so a centroid whose
+ * value exceeds the threshold has a strictly larger serial distance than the sweep's best one and cannot be the
+ * result) and evaluates the serial arithmetic only for the centroids that pass: typically two or three of k. A lane
+ * notes up to SCREEN_CAP passing centroids and evaluates them after its scan, so that the wavefront runs the
+ * expensive block a few times instead of whenever any of its lanes has a hit; beyond SCREEN_CAP (duplicated
+ * centroids, NaN data: `!(a > threshold)` passes everything that is not a number) the lane evaluates on the spot.
+ * The kernel for wider rows evaluates every centroid (measured: screening did not pay there, the centroid block is
+ * read twice). The merge by (smaller distance, then smaller index) over all evaluated centroids is the serial scan's
+ * result: the first centroid attaining the minimum. A NaN distance to centroid 0 pins the point to centroid 0, as
+ * `minDist > dist` is then never true (centroid 0 always passes the screen in that case: its ranking value is NaN
+ * as well).
+ */
+constexpr int SCREEN_CAP = 4;
+
+/*
+ * Any dimension. A work-group of 256 lanes owns a batch of PB queued points: their coordinates are staged in LDS
+ * (rows padded with zeros to a multiple of 4 floats, so that every lane fetches four coordinates with one broadcast
+ * 128-bit read), lane t handles centroids t, t+256, ... against all PB points (16 coalesced loads of the transposed
+ * centroid block in flight, each value reused PB times) and keeps its own (distance, index) minimum per point.
+ * Zero padding is exact: (0-0)^2 = +0 leaves a partial sum unchanged.
+ * means_t is the exact transposed copy [dim][kp] written by the pack kernels.
  */
 template <int LD, int PB>
 __global__ void __launch_bounds__(256)
@@ -84,7 +97,7 @@ recheck_kernel(const float* __restrict__ data, size_t stride, const float* __res
 		__syncthreads(); /* the previous batch's coordinates and candidates are no longer needed */
 		for (uint32_t i = threadIdx.x; i < PB * dim4; i += blockDim.x) {
 			const uint32_t p = i / dim4, d = i - p * dim4;
-			const uint32_t idx = queue[min(batch * PB + p, count - 1)];
+			const uint32_t idx = queue[2 * (size_t)min(batch * PB + p, count - 1)];
 			xs[i] = d < dim ? data[elem<LD>(stride, idx, d)] : 0.0f;
 		}
 		__syncthreads();
@@ -97,7 +110,7 @@ recheck_kernel(const float* __restrict__ data, size_t stride, const float* __res
 			best[p] = __builtin_inff();
 			bestIdx[p] = 0xFFFFFFFFu;
 		}
-		for (uint32_t m = threadIdx.x; m < k; m += blockDim.x) {
+		auto evaluate = [&](uint32_t m) {
 			float sum[PB];
 #pragma unroll
 			for (int p = 0; p < PB; ++p) sum[p] = 0.0f;
@@ -130,8 +143,9 @@ recheck_kernel(const float* __restrict__ data, size_t stride, const float* __res
 					bestIdx[p] = m;
 				}
 			}
-		}
-		if (threadIdx.x == 0) pinned_mask = pinned; /* lane 0 evaluated centroid 0 */
+		};
+		for (uint32_t m = threadIdx.x; m < k; m += blockDim.x) evaluate(m);
+		if (threadIdx.x == 0) pinned_mask = pinned; /* lane 0 handles centroid 0 */
 #pragma unroll
 		for (int p = 0; p < PB; ++p) {
 			for (int off = WAVE / 2; off > 0; off >>= 1) {
@@ -163,16 +177,16 @@ recheck_kernel(const float* __restrict__ data, size_t stride, const float* __res
 			const uint32_t q = batch * PB + p;
 			if (q < count) {
 				const bool pin = (pinned_mask >> p) & 1u;
-				assignment[queue[q]] = (pin || bi == 0xFFFFFFFFu) ? 0u : bi;
+				assignment[queue[2 * (size_t)q]] = (pin || bi == 0xFFFFFFFFu) ? 0u : bi;
 			}
 		}
 	}
 }
 
 /*
- * Exact pass for dim <= DPAD <= 64 without LDS: the PB points of a batch live in registers (every lane of the
- * group loads the same words, a broadcast), all DPAD centroid coordinates of a lane's centroid are requested
- * before the first add, so their latency overlaps. Dimensions beyond dim are fed as x = c = 0: adding
+ * dim <= DPAD <= 64 without LDS: the PB points of a batch live in registers (every lane of the group of L lanes loads
+ * the same words, a broadcast), lane t of the group handles centroids t, t+L, ...; all DPAD coordinates of a centroid
+ * are requested before the first use, so their latency overlaps. Dimensions beyond dim are fed as x = c = 0: adding
  * (0-0)^2 = +0 leaves every partial sum unchanged, so the padding is exact.
  */
 template <int LD, int L, int PB, int DPAD>
@@ -189,10 +203,13 @@ recheck_reg_kernel(const float* __restrict__ data, size_t stride, const float* _
 
 	for (uint32_t batch = blockIdx.x * GROUPS + group; batch < batches; batch += gridDim.x * GROUPS) {
 		float x[PB][DPAD];
+		float thr[PB];
 		uint32_t idx[PB];
 #pragma unroll
 		for (int p = 0; p < PB; ++p) {
-			idx[p] = queue[min(batch * PB + p, count - 1)];
+			const size_t entry = 2 * (size_t)min(batch * PB + p, count - 1);
+			idx[p] = queue[entry];
+			thr[p] = __uint_as_float(queue[entry + 1]);
 #pragma unroll
 			for (int d = 0; d < DPAD; ++d) x[p][d] = (uint32_t)d < dim ? data[elem<LD>(stride, idx[p], d)] : 0.0f;
 		}
@@ -204,10 +221,7 @@ recheck_reg_kernel(const float* __restrict__ data, size_t stride, const float* _
 			best[p] = __builtin_inff();
 			bestIdx[p] = 0xFFFFFFFFu;
 		}
-		for (uint32_t m = gl; m < k; m += L) {
-			float c[DPAD];
-#pragma unroll
-			for (int d = 0; d < DPAD; ++d) c[d] = (uint32_t)d < dim ? means_t[(size_t)d * kp + m] : 0.0f;
+		auto evaluate = [&](uint32_t m, const float (&c)[DPAD]) {
 			float sum[PB];
 #pragma unroll
 			for (int p = 0; p < PB; ++p) sum[p] = 0.0f;
@@ -229,8 +243,46 @@ recheck_reg_kernel(const float* __restrict__ data, size_t stride, const float* _
 					bestIdx[p] = m;
 				}
 			}
+		};
+		uint32_t noted[SCREEN_CAP];
+		uint32_t notes = 0;
+		for (uint32_t m = gl; m < k; m += L) {
+			float c[DPAD];
+#pragma unroll
+			for (int d = 0; d < DPAD; ++d) c[d] = (uint32_t)d < dim ? means_t[(size_t)d * kp + m] : 0.0f;
+			float c2 = 0.0f;
+			float dot[PB];
+#pragma unroll
+			for (int p = 0; p < PB; ++p) dot[p] = 0.0f;
+#pragma unroll
+			for (int d = 0; d < DPAD; ++d) {
+				c2 = __builtin_fmaf(c[d], c[d], c2);
+#pragma unroll
+				for (int p = 0; p < PB; ++p) dot[p] = __builtin_fmaf(c[d], x[p][d], dot[p]);
+			}
+			bool pass = false;
+#pragma unroll
+			for (int p = 0; p < PB; ++p) pass = pass || !(__builtin_fmaf(-2.0f, dot[p], c2) > thr[p]);
+			if (pass) {
+				if (notes < SCREEN_CAP) {
+#pragma unroll
+					for (int i = 0; i < SCREEN_CAP; ++i)
+						if (notes == (uint32_t)i) noted[i] = m;
+					++notes;
+				}
+				else evaluate(m, c);
+			}
 		}
-		pinned = (uint32_t)__shfl((int)pinned, 0, L); /* lane 0 of the group evaluated centroid 0 */
+#pragma unroll
+		for (int i = 0; i < SCREEN_CAP; ++i) {
+			if ((uint32_t)i < notes) {
+				float c[DPAD];
+#pragma unroll
+				for (int d = 0; d < DPAD; ++d) c[d] = (uint32_t)d < dim ? means_t[(size_t)d * kp + noted[i]] : 0.0f;
+				evaluate(noted[i], c);
+			}
+		}
+		pinned = (uint32_t)__shfl((int)pinned, 0, L); /* lane 0 of the group handles centroid 0 */
 #pragma unroll
 		for (int p = 0; p < PB; ++p) {
 			for (int off = L / 2; off > 0; off >>= 1) {

@@ -98,7 +98,7 @@ int launch_pack_means(const AssignArgs& a, Workspace* ws, uint32_t dp, uint32_t 
 {
 	int rc = reserve_packed(ws, (size_t)(kp / TILE) * tile_floats(dp + ROW_PAD), (size_t)(kp / TILE) * NORM_TILE, (size_t)kp * a.dim);
 	if (rc) return rc;
-	rc = reserve_queue(ws, a.n);
+	rc = reserve_queue(ws, 2 * (size_t)a.n); /* (point, threshold) pairs */
 	if (rc) return rc;
 	const uint32_t pack_blocks = (kp * WAVE + 255) / 256;
 	if (a.layout_means == KMX_AOS)

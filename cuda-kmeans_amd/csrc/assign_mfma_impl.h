@@ -22,6 +22,18 @@ constexpr uint32_t TILE_PAD = 4;    /* floats appended to every packed tile of 3
 constexpr uint32_t NORM_TILE = 36;  /* floats per tile in the norms array (32 + 4 padding) */
 constexpr uint32_t MFMA_WAVES = 8;  /* wavefronts per work-group                      */
 constexpr uint32_t FLAG_CAP = 128;  /* per-wavefront list of points waiting for the recheck queue */
+
+/*
+ * A recheck queue entry is two words: the point index and, as float bits, the screening threshold of the point:
+ * the smallest ranking value a[j] the sweep saw plus tau. A centroid whose a[j] exceeds it cannot be the serial
+ * result (same argument as for the certification), so the exact pass only evaluates the others. Anything that is
+ * not a finite number (NaN, overflow) becomes +inf: every centroid is then evaluated.
+ */
+__device__ __forceinline__ uint32_t screening_threshold(float first, float tau)
+{
+	const float t = first + tau;
+	return __float_as_uint(__builtin_fabsf(t) < __builtin_inff() ? t : __builtin_inff());
+}
 constexpr uint32_t COARSE_MIN_TILES = 10; /* from this many centroid tiles on, track per tile and refine */
 
 __host__ __device__ constexpr uint32_t round_up(uint32_t v, uint32_t m) { return (v + m - 1) / m * m; }
@@ -189,7 +201,7 @@ assign_mfma_kernel(const float* __restrict__ data, size_t stride, const float* _
 	constexpr uint32_t RS = DP + ROW_PAD;
 	extern __shared__ float lds[];
 	__shared__ uint32_t wave_max[MFMA_WAVES];
-	__shared__ uint32_t flag_list[MFMA_WAVES][FLAG_CAP];
+	__shared__ uint32_t flag_list[MFMA_WAVES][2 * FLAG_CAP]; /* (point, threshold) pairs */
 
 	const uint32_t lane = threadIdx.x & (WAVE - 1);
 	const uint32_t wave = threadIdx.x / WAVE;
@@ -234,7 +246,7 @@ assign_mfma_kernel(const float* __restrict__ data, size_t stride, const float* _
 		uint32_t slot = 0;
 		if (lane == 0) slot = atomicAdd(&counters[0], flagged);
 		slot = (uint32_t)__shfl((int)slot, 0);
-		for (uint32_t i = lane; i < flagged; i += WAVE) queue[slot + i] = flag_list[wave][i];
+		for (uint32_t i = lane; i < 2 * flagged; i += WAVE) queue[2 * (size_t)slot + i] = flag_list[wave][i];
 		__builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
 		__builtin_amdgcn_wave_barrier();
 		flagged = 0;
@@ -372,7 +384,11 @@ assign_mfma_kernel(const float* __restrict__ data, size_t stride, const float* _
 			if (mask) {
 				const uint32_t add = (uint32_t)__builtin_popcountll(mask);
 				if (flagged + add > FLAG_CAP) flush_flags();
-				if (flag) flag_list[wave][flagged + __builtin_popcountll(mask & ((1ull << lane) - 1ull))] = pt;
+				if (flag) {
+					const uint32_t at = 2 * (flagged + __builtin_popcountll(mask & ((1ull << lane) - 1ull)));
+					flag_list[wave][at] = pt;
+					flag_list[wave][at + 1] = screening_threshold(first, tau);
+				}
 				flagged += add;
 			}
 		}
@@ -415,7 +431,7 @@ static int launch_mfma_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 	constexpr int P = SweepShape<DPH>::P;
 	constexpr bool PF = SweepShape<DPH>::PREFETCH;
 	uint32_t budget = exec->shared_mem_bytes ? std::min(exec->shared_mem_bytes, dev.lds_bytes) : dev.lds_bytes;
-	const uint32_t static_bytes = (FLAG_CAP * MFMA_WAVES + 64) * 4; /* static LDS of the kernel */
+	const uint32_t static_bytes = (2 * FLAG_CAP * MFMA_WAVES + 64) * 4; /* static LDS of the kernel */
 	const uint32_t tile_bytes = (tile_floats(RS) + NORM_TILE) * 4;
 	if (budget < static_bytes + tile_bytes) return fail(KMX_ERR_UNSUPPORTED, "assign (MFMA): LDS budget of %u bytes is too small", budget);
 	const uint32_t chunk_rows = std::min<uint32_t>(kp, (budget - static_bytes) / tile_bytes * TILE);
