@@ -21,6 +21,7 @@ HOST_LIB_PATH = os.path.join(_HERE, "host", "libkmx_host.so")
 
 AOS, SOA = 0, 1
 ASSIGN_BASE, ASSIGN_LDS_FMA, ASSIGN_MFMA, ASSIGN_BEST, ASSIGN_MFMA_BF16X3 = 0, 1, 2, 3, 4
+FUSED_TWO_PASS = 0
 UPDATE_ATOMIC_POINT, UPDATE_ATOMIC_FINE, UPDATE_ATOMIC_SHM = 0, 1, 2
 
 KMX_OK, KMX_ERR_INVALID_ARGUMENT, KMX_ERR_UNSUPPORTED, KMX_ERR_DEVICE, KMX_ERR_NO_DEVICE = 0, 1, 2, 3, 4
@@ -29,7 +30,7 @@ KMX_OK, KMX_ERR_INVALID_ARGUMENT, KMX_ERR_UNSUPPORTED, KMX_ERR_DEVICE, KMX_ERR_N
 ABI_SYMBOLS = [
     "kmx_device_count", "kmx_set_device", "kmx_device_props", "kmx_malloc", "kmx_free", "kmx_h2d", "kmx_d2h",
     "kmx_d2d", "kmx_sync", "kmx_set_stream", "kmx_shutdown", "kmx_fill_zero_u32", "kmx_assign_f32",
-    "kmx_assign_last_rechecked", "kmx_assign_last_variant", "kmx_update_f32", "kmx_event_create", "kmx_event_destroy", "kmx_event_record",
+    "kmx_assign_last_rechecked", "kmx_assign_last_variant", "kmx_update_f32", "kmx_fused_f32", "kmx_event_create", "kmx_event_destroy", "kmx_event_record",
     "kmx_event_elapsed_ms", "kmx_set_profiling", "kmx_last_kernel_ms", "kmx_last_error",
 ]
 
@@ -104,6 +105,8 @@ def hip_lib():
         lib.kmx_assign_last_variant.argtypes = [ctypes.POINTER(ctypes.c_int)]
         lib.kmx_update_f32.argtypes = [ctypes.c_int, vp, ctypes.c_int, sz, vp, vp, ctypes.c_int, sz, vp, u32, u32, u32,
                                        ctypes.POINTER(ExecParams)]
+        lib.kmx_fused_f32.argtypes = [ctypes.c_int, vp, ctypes.c_int, sz, vp, vp, ctypes.c_int, sz, vp, u32, u32, u32,
+                                      ctypes.POINTER(ExecParams)]
         lib.kmx_event_create.argtypes = [ctypes.POINTER(vp)]
         lib.kmx_event_destroy.argtypes = [vp]
         lib.kmx_event_record.argtypes = [vp]
@@ -276,6 +279,15 @@ def update(variant, data_buf, layout, stride, assignment_buf, means_buf, layout_
     return ex
 
 
+def fused(variant, data_buf, layout, stride, means_in_buf, means_out_buf, layout_means, stride_means, sizes_buf, dim, k,
+          n, exec_params=None):
+    """FUSED_KERNEL::run (kernels.cuh:107-116) through kmx_fused_f32; enqueues and returns."""
+    ex = exec_params if exec_params is not None else ExecParams()
+    check(hip_lib().kmx_fused_f32(variant, data_buf.ptr, layout, stride, means_in_buf.ptr, means_out_buf.ptr,
+                                  layout_means, stride_means, sizes_buf.ptr, dim, k, n, ctypes.byref(ex)))
+    return ex
+
+
 def set_profiling(enabled):
     check(hip_lib().kmx_set_profiling(1 if enabled else 0))
 
@@ -369,6 +381,70 @@ class HipKMeansAlgorithm:
 
     def getClusterSizes(self):
         return self.cu_sizes.read(np.uint32, self.k)
+
+    def cleanup(self):
+        for b in self._bufs:
+            b.free()
+        self._bufs = []
+
+
+class HipFusedKMeansAlgorithm:
+    """Mirror of CudaFusedKMeansAlgorithm (cuda.hpp:116-233): no assignment buffers; per iteration
+    zero(means[next]) -> zero(sizes) -> fused(means[last] -> means[next]); getAssignment() is computed afterwards
+    against the FINAL centroids (the reference does that on the host, cuda.hpp:199-221; here one more device pass)."""
+
+    def __init__(self, variant=FUSED_TWO_PASS, exec_params=None, layout=AOS, layout_means=AOS):
+        self.variant = variant
+        self.exec = exec_params if exec_params is not None else ExecParams()
+        self.layout, self.layout_means = layout, layout_means
+        self._bufs = []
+
+    def initialize(self, dim, k, n, iters, data, means):
+        if device_count() == 0:
+            raise KmxError(KMX_ERR_NO_DEVICE, "No HIP devices found!")
+        check(hip_lib().kmx_set_device(0))
+        self.dim, self.k, self.n, self.iters = int(dim), int(k), int(n), int(iters)
+        self.stride = layout_stride(self.layout, self.n, self.dim)
+        self.stride_means = layout_stride(self.layout_means, self.k, self.dim)
+        self.means_size = layout_size(self.layout_means, self.k, self.dim)
+        self.cu_data = DeviceBuffer(4 * layout_size(self.layout, self.n, self.dim))
+        self.cu_sizes = DeviceBuffer(4 * self.k)
+        self.cu_means = [DeviceBuffer(4 * self.means_size) for _ in range(2)]
+        self._bufs = [self.cu_data, self.cu_sizes] + self.cu_means
+        self.cu_data.write(data)
+        self.last = 0
+        self.cu_means[0].write(means)
+        self.cu_sizes.zero()
+        sync()
+
+    def iteration(self):
+        nxt = (self.last + 1) % 2
+        self.cu_means[nxt].zero()
+        self.cu_sizes.zero()
+        fused(self.variant, self.cu_data, self.layout, self.stride, self.cu_means[self.last], self.cu_means[nxt],
+              self.layout_means, self.stride_means, self.cu_sizes, self.dim, self.k, self.n, self.exec)
+        self.last = nxt
+
+    def run(self, iters=None):
+        for _ in range(self.iters if iters is None else iters):
+            self.iteration()
+        sync()
+
+    def getMeans(self):
+        return self.cu_means[self.last].read(np.float32, self.means_size)
+
+    def getClusterSizes(self):
+        return self.cu_sizes.read(np.uint32, self.k)
+
+    def getAssignment(self):
+        out = DeviceBuffer(4 * max(self.n, 1))
+        try:
+            assign(ASSIGN_BEST, self.cu_data, self.layout, self.stride, self.cu_means[self.last], self.layout_means,
+                   self.stride_means, out, self.dim, self.k, self.n, self.exec)
+            sync()
+            return out.read(np.uint32, self.n)
+        finally:
+            out.free()
 
     def cleanup(self):
         for b in self._bufs:

@@ -53,11 +53,13 @@ struct Workspace {
 	float* norms = nullptr;         size_t norms_cap = 0;      /* floats  */
 	float* means_t = nullptr;       size_t means_t_cap = 0;    /* floats: exact transposed centroids [dim][kp] */
 	float* partials = nullptr;      size_t partials_cap = 0;   /* floats  */
+	uint32_t* fused_assignment = nullptr; size_t fused_cap = 0; /* entries: assignment vector of kmx_fused_f32 */
 };
 int workspace(Workspace** ws);
 int reserve_queue(Workspace* ws, size_t entries);
 int reserve_packed(Workspace* ws, size_t packed_floats, size_t norm_floats, size_t transposed_floats);
 int reserve_partials(Workspace* ws, size_t floats);
+int reserve_fused_assignment(Workspace* ws, size_t entries);
 
 #define KMX_HIP(call)                                                                                         \
 	do {                                                                                                      \

@@ -102,6 +102,7 @@ int reserve_packed(Workspace* ws, size_t packed_floats, size_t norm_floats, size
 }
 
 int reserve_partials(Workspace* ws, size_t floats) { return grow(&ws->partials, &ws->partials_cap, floats); }
+int reserve_fused_assignment(Workspace* ws, size_t entries) { return grow(&ws->fused_assignment, &ws->fused_cap, entries); }
 
 static int release_workspace()
 {
@@ -111,6 +112,7 @@ static int release_workspace()
 	if (g_ws.norms) KMX_HIP(hipFree(g_ws.norms));
 	if (g_ws.means_t) KMX_HIP(hipFree(g_ws.means_t));
 	if (g_ws.partials) KMX_HIP(hipFree(g_ws.partials));
+	if (g_ws.fused_assignment) KMX_HIP(hipFree(g_ws.fused_assignment));
 	g_ws = Workspace();
 	return KMX_OK;
 }
@@ -372,6 +374,29 @@ int kmx_update_f32(int variant,
 
 	UpdateArgs u{ data, layout, stride, assignment, means, layout_means, stride_means, cluster_sizes, dim, k, n };
 	return launch_update(variant, u, exec, ws, *dev);
+}
+
+int kmx_fused_f32(int variant,
+                  const float* data, int layout, size_t stride,
+                  const float* means_in, float* means_out, int layout_means, size_t stride_means,
+                  uint32_t* cluster_sizes,
+                  uint32_t dim, uint32_t k, uint32_t n, kmx_exec_params* exec)
+{
+	clear_error();
+	if (!exec) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_fused_f32: exec is null");
+	if (variant != KMX_FUSED_TWO_PASS) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_fused_f32: unknown variant %d", variant);
+	if (!means_in || !means_out || !cluster_sizes) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_fused_f32: null device pointer");
+	if (means_in == means_out) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_fused_f32: means_in and means_out must differ");
+	Workspace* ws = nullptr;
+	int rc = workspace(&ws);
+	if (rc) return rc;
+	rc = reserve_fused_assignment(ws, n);
+	if (rc) return rc;
+	/* argument checks of the two halves apply unchanged (their messages name the half that objects) */
+	rc = kmx_assign_f32(KMX_ASSIGN_BEST, data, layout, stride, means_in, layout_means, stride_means, nullptr, ws->fused_assignment, dim, k, n, exec);
+	if (rc) return rc;
+	return kmx_update_f32(KMX_UPDATE_ATOMIC_SHM, data, layout, stride, ws->fused_assignment, means_out, layout_means, stride_means,
+	                      cluster_sizes, dim, k, n, exec);
 }
 
 int kmx_set_profiling(int enabled)

@@ -55,6 +55,21 @@ struct UpdateProblemInstance {
 		dim((IDX_T)_dim), k((IDX_T)_k), n((IDX_T)_n) {}
 };
 
+/* = FusedProblemInstance (kernels.cuh:38-53) */
+template<typename F, typename IDX_T>
+struct FusedProblemInstance {
+	const F* data;
+	const F* meansIn;
+	F* meansOut; /* the result; zeroed by the caller */
+	IDX_T* clusterSizes; /* zeroed by the caller */
+	IDX_T dim, k, n;
+
+	FusedProblemInstance(const F* _data, const F* _meansIn, F* _meansOut, IDX_T* _clusterSizes,
+		std::size_t _dim, std::size_t _k, std::size_t _n)
+		: data(_data), meansIn(_meansIn), meansOut(_meansOut), clusterSizes(_clusterSizes),
+		dim((IDX_T)_dim), k((IDX_T)_k), n((IDX_T)_n) {}
+};
+
 /* = CudaExecParameters; the field order is that of kmx_exec_params */
 struct HipExecParameters {
 	unsigned int blockSize;
@@ -105,6 +120,16 @@ void update(int variant, const UpdateProblemInstance<F, IDX_T>& in, HipExecParam
 		(std::uint32_t*)in.clusterSizes, in.dim, in.k, in.n, reinterpret_cast<kmx_exec_params*>(&exec)));
 }
 
+template<typename F, typename IDX_T, class LAYOUT, class LAYOUT_MEANS>
+void fused(int variant, const FusedProblemInstance<F, IDX_T>& in, HipExecParameters& exec)
+{
+	static_assert(std::is_same<F, float>::value && sizeof(IDX_T) == 4, "built for float data and 32-bit indices");
+	KMX_CHECK(kmx_fused_f32(variant,
+		in.data, LAYOUT::ID, LAYOUT::precomputeConstants(in.n, in.dim),
+		in.meansIn, in.meansOut, LAYOUT_MEANS::ID, LAYOUT_MEANS::precomputeConstants(in.k, in.dim),
+		(std::uint32_t*)in.clusterSizes, in.dim, in.k, in.n, reinterpret_cast<kmx_exec_params*>(&exec)));
+}
+
 } // namespace hip_detail
 
 #define KMX_DEFINE_ASSIGNMENT_KERNEL(NAME, VARIANT)\
@@ -120,6 +145,14 @@ KMX_DEFINE_ASSIGNMENT_KERNEL(LdsFmaAssignmentKernel, KMX_ASSIGN_LDS_FMA)  /* rol
 KMX_DEFINE_ASSIGNMENT_KERNEL(MfmaAssignmentKernel, KMX_ASSIGN_MFMA)       /* no counterpart: matrix-core path */
 KMX_DEFINE_ASSIGNMENT_KERNEL(MfmaBf16AssignmentKernel, KMX_ASSIGN_MFMA_BF16X3) /* no counterpart: matrix-core path on split bf16 operands */
 KMX_DEFINE_ASSIGNMENT_KERNEL(BestCachedAssignmentKernel, KMX_ASSIGN_BEST) /* kernels.cu:706-717 */
+
+/* role of FusedCachedFixedKernel / FusedCachedRegsKernel (kernels.cu:883-1190): one call per iteration, no assignment buffer */
+template<typename F, typename IDX_T, class LAYOUT, class LAYOUT_MEANS, class METRIC>
+class FusedTwoPassKernel {
+public:
+	static void run(const FusedProblemInstance<F, IDX_T>& in, HipExecParameters& exec)
+	{ hip_detail::fused<F, IDX_T, LAYOUT, LAYOUT_MEANS>(KMX_FUSED_TWO_PASS, in, exec); }
+};
 
 #define KMX_DEFINE_UPDATE_KERNEL(NAME, VARIANT)\
 template<typename F, typename IDX_T, class LAYOUT, class LAYOUT_MEANS, int EMUL = false>\

@@ -176,6 +176,91 @@ public:
 	}
 };
 
+/*
+ * Counterpart of CudaFusedKMeansAlgorithm (cuda.hpp:116-233): no assignment buffers; every iteration zero-fills the
+ * next centroid buffer and the counts and makes one FUSED kernel call. As in the reference, getAssignment() is not a
+ * by-product of the iterations: it is computed afterwards against the FINAL centroids (the reference scans on the
+ * host, cuda.hpp:199-221; here the device runs one more assignment pass, which returns the same indices).
+ */
+template<typename F = float, typename IDX_T = std::uint32_t, class LAYOUT = AoSLayoutPolicy<>,
+	class LAYOUT_MEANS = LAYOUT, class METRIC = EuclideanMetricPolicy<F, LAYOUT, LAYOUT_MEANS>,
+	class KERNEL = FusedTwoPassKernel<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC>>
+class HipFusedKMeansAlgorithm : public IKMeansAlgorithm<F, IDX_T>
+{
+	HipExecParameters mExecParams;
+	bool mMeansReady = false, mAssignmentReady = false;
+	HipBuffer<F> mDevData;
+	HipBuffer<F> mDevMeans[2];
+	HipBuffer<IDX_T> mDevClusterSizes;
+	unsigned mLast = 0;
+
+	std::size_t meansSize() const { return LAYOUT_MEANS::size(this->mK, this->mDim); }
+
+public:
+	explicit HipFusedKMeansAlgorithm(const HipExecParameters& exec) : mExecParams(exec) {}
+
+	void initialize(std::size_t dim, std::size_t k, std::size_t n, std::size_t iters,
+		const std::vector<F>& data, const std::vector<F>& means) override
+	{
+		IKMeansAlgorithm<F, IDX_T>::initialize(dim, k, n, iters, data, means);
+		mMeansReady = mAssignmentReady = false;
+		requireDevice();
+		mDevData.realloc(LAYOUT::size(n, dim));
+		mDevClusterSizes.realloc(k);
+		for (auto& b : mDevMeans) b.realloc(meansSize());
+		mDevData.write(data);
+		mLast = 0;
+		mDevMeans[mLast].write(means);
+		runFillZeros<IDX_T>(*mDevClusterSizes, k);
+		KMX_CHECK(kmx_sync());
+	}
+
+	void run() override
+	{
+		for (std::size_t iter = 0; iter < this->mIters; ++iter) {
+			const unsigned next = (mLast + 1) % 2;
+			runFillZeros<F>(*mDevMeans[next], meansSize());
+			runFillZeros<IDX_T>(*mDevClusterSizes, this->mK);
+			FusedProblemInstance<F, IDX_T> fused(*mDevData, *mDevMeans[mLast], *mDevMeans[next], *mDevClusterSizes,
+				this->mDim, this->mK, this->mN);
+			KERNEL::run(fused, mExecParams);
+			mLast = next;
+		}
+		KMX_CHECK(kmx_sync());
+	}
+
+	const std::vector<F>& getMeans() override
+	{
+		if (!mMeansReady) {
+			mDevMeans[mLast].read(this->mMeans, meansSize());
+			mMeansReady = true;
+		}
+		return this->mMeans;
+	}
+
+	const std::vector<IDX_T>& getAssignment() override
+	{
+		if (!mAssignmentReady) {
+			HipBuffer<IDX_T> out;
+			out.realloc(this->mN);
+			AssignmentProblemInstance<F, IDX_T> assignment(*mDevData, *mDevMeans[mLast], nullptr, *out, this->mDim, this->mK, this->mN);
+			BestCachedAssignmentKernel<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC>::run(assignment, mExecParams);
+			out.read(this->mAssignment, this->mN);
+			out.free();
+			mAssignmentReady = true;
+		}
+		return this->mAssignment;
+	}
+
+	void cleanup() override
+	{
+		IKMeansAlgorithm<F, IDX_T>::cleanup();
+		mDevData.free();
+		for (auto& b : mDevMeans) b.free();
+		mDevClusterSizes.free();
+	}
+};
+
 template<typename F = float, typename IDX_T = std::uint32_t, class LAYOUT = AoSLayoutPolicy<>,
 	class LAYOUT_MEANS = LAYOUT, class METRIC = EuclideanMetricPolicy<F, LAYOUT, LAYOUT_MEANS>,
 	class KERNEL = BaseAssignmentKernel<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC>>

@@ -56,6 +56,7 @@ std::string canonicalAlgorithm(const std::string& name)
 	static const std::map<std::string, std::string> aliases = {
 		{ "cuda_base", "hip_base" }, { "cuda_base_shm", "hip_base_shm" }, { "cuda_best", "hip_best" },
 		{ "cuda_cached_fixed", "hip_lds_fma" }, { "cuda_cached_regs", "hip_mfma" },
+		{ "cuda_fused_fixed", "hip_fused" }, { "cuda_fused_regs", "hip_fused" },
 	};
 	auto it = aliases.find(name);
 	return it == aliases.end() ? name : it->second;
@@ -169,6 +170,7 @@ void run_kmeans(const ProgramArguments& args, std::vector<F>& data, std::vector<
 	algorithms["hip_mfma"].reset(new HipKMeansAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC, Mfma, Shm>(exec, json));
 	algorithms["hip_mfma_bf16"].reset(new HipKMeansAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC, MfmaBf16, Shm>(exec, json));
 	algorithms["hip_best"].reset(new HipKMeansAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC, Best, Shm>(exec, json));
+	algorithms["hip_fused"].reset(new HipFusedKMeansAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC>(exec));
 
 	auto it = algorithms.find(algoName);
 	if (it == algorithms.end()) throw std::runtime_error("Unkown algorithm '" + algoName + "'.");
@@ -208,7 +210,15 @@ void run_kmeans(const ProgramArguments& args, std::vector<F>& data, std::vector<
 		SerialKMeansAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC> base(threads);
 		base.initialize(dim, k, n, iters, data, means);
 		base.run();
-		mismatches = verify_assignment<IDX_T>(algorithm->getAssignment(), base.getAssignment(), n);
+		if (algoName == "hip_fused") {
+			/* the fused algorithm reports the assignment against its FINAL centroids (cuda.hpp:199-221), the serial
+			 * algorithm the one its last iteration used: compare with a serial assignment pass over the same centroids */
+			SerialAssignmentAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC> last(threads);
+			last.initialize(dim, k, n, data, algorithm->getMeans());
+			last.run();
+			mismatches = verify_assignment<IDX_T>(algorithm->getAssignment(), last.getAssignment(), n);
+		}
+		else mismatches = verify_assignment<IDX_T>(algorithm->getAssignment(), base.getAssignment(), n);
 		errors = mismatches + verify_means<F, LAYOUT_MEANS>(algorithm->getMeans(), base.getMeans(), dim, k);
 		centroidErr = centroid_error<F, LAYOUT_MEANS>(algorithm->getMeans(), base.getMeans(), dim, k);
 		verified = true;
@@ -295,7 +305,7 @@ int main(int argc, char* argv[])
 		args.registerInt("seed", "Random generator seed.", 42, 0);
 		args.registerBool("assignmentOnly", "Run only assignment part of the algorithm (microbenchmark).");
 		args.conflicts("assignmentOnly", "iterations");
-		args.registerString("algorithm", "Which algorithm is to be tested (serial, hip_base, hip_base_shm, hip_mfma, hip_mfma_bf16, hip_best; assignment only: hip_lds_fma).", "serial");
+		args.registerString("algorithm", "Which algorithm is to be tested (serial, hip_base, hip_base_shm, hip_mfma, hip_mfma_bf16, hip_best, hip_fused; assignment only: hip_lds_fma).", "serial");
 		args.registerEnum("layout", "Type of data layout.", "aos", { "aos", "soa" });
 		args.registerEnum("layoutMeans", "Type of data layout (override for means only).", "aos", { "aos", "soa" });
 		args.registerBool("double", "Use doubles instead of floats (not built).");

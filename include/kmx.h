@@ -135,6 +135,25 @@ int kmx_update_f32(int variant,
                    uint32_t* cluster_sizes,
                    uint32_t dim, uint32_t k, uint32_t n, kmx_exec_params* exec);
 
+/*
+ * ---- FUSED_KERNEL::run(FusedProblemInstance, CudaExecParameters&) (kernels.cuh:38-53,107-116; called by
+ *      CudaFusedKMeansAlgorithm::run, cuda.hpp:174-191) ----
+ * One whole iteration without a caller-visible assignment vector: every point is assigned to its nearest centroid
+ * of means_in (same result as kmx_assign_f32) and accumulated into means_out / cluster_sizes, which are then merged
+ * and divided as by kmx_update_f32. Precondition as in the reference (cuda.hpp:178-179): means_out and cluster_sizes
+ * are zero. The assignment lives in the library's work space (n words, grown on demand).
+ */
+typedef enum kmx_fused_variant {
+	KMX_FUSED_TWO_PASS = 0 /* selector-chosen assignment sweep into the work space, then the tuned update (the points are
+	                          read twice; the reference's FusedCachedFixed / FusedCachedRegs read them once) */
+} kmx_fused_variant;
+
+int kmx_fused_f32(int variant,
+                  const float* data, int layout, size_t stride,
+                  const float* means_in, float* means_out, int layout_means, size_t stride_means,
+                  uint32_t* cluster_sizes,
+                  uint32_t dim, uint32_t k, uint32_t n, kmx_exec_params* exec);
+
 /* ---- events on the library's stream (for the assignment / update split; the reference only has
  *      a wall-clock Stopwatch around run(), k-means.cpp:155-158) ---- */
 int kmx_event_create(void** event);

@@ -263,6 +263,32 @@ def test_every_iteration_matches_oracle(km, orc, gpu, cid, n, iters):
             assert r["centroid_err"] < CENTROID_RTOL, (av, uv, r)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("cid,n,iters,layout,layout_means", [(1, 65536, 4, AOS, AOS), (2, 32768, 2, AOS, AOS),
+                                                             (5, 1 << 18, 3, AOS, AOS), (1, 20000, 2, SOA, AOS)])
+def test_fused_iterations_match_oracle(km, orc, gpu, cid, n, iters, layout, layout_means):
+    """FUSED kernel call (kernels.cuh:107-116): every iteration checked against the oracle fed with the same centroids;
+    the assignment it reports afterwards is the serial argmin against the FINAL centroids (cuda.hpp:199-221)."""
+    spec = km.baseline_config(cid)
+    dim, k = spec.dim, spec.k
+    data = km.generate_points(spec, n, layout=layout)
+    means0 = km.first_k_means(spec, layout_means)
+    alg = km.HipFusedKMeansAlgorithm(layout=layout, layout_means=layout_means)
+    alg.initialize(dim, k, n, iters, data, means0)
+    for _ in range(iters):
+        prev = alg.getMeans()
+        alg.iteration()
+        gm, gs = alg.getMeans(), alg.getClusterSizes()
+        oa = orc.assign(data, prev, dim, k, n, layout, layout_means, threads=0, fast=True)
+        om, osz = orc.update(data, oa, dim, k, n, layout, layout_means, threads=0)
+        assert np.array_equal(gs, osz)
+        assert rel_err(gm, om) < CENTROID_RTOL
+    final = alg.getMeans()
+    want = orc.assign(data, final, dim, k, n, layout, layout_means, threads=0, fast=True)
+    assert np.array_equal(alg.getAssignment(), want)
+    alg.cleanup()
+
+
 def test_free_running_loop_reports_only_near_ties(km, orc, gpu):
     """Whole run against the oracle's whole run (config 1 in full, as the reference's --verify does,
     k-means.cpp:171-182). The first assignment must be identical. After that the runs may part at near-ties;

@@ -93,7 +93,8 @@ def test_no_device_is_an_error_not_a_fallback(harness, km):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("algo", ["hip_best", "hip_mfma", "hip_mfma_bf16", "hip_base", "hip_base_shm", "cuda_best"])
+@pytest.mark.parametrize("algo", ["hip_best", "hip_mfma", "hip_mfma_bf16", "hip_base", "hip_base_shm", "cuda_best", "hip_fused",
+                                  "cuda_fused_regs"])
 def test_device_algorithms_verify(harness, gpu, algo):
     rc, out, err = run(harness, "--config", "1", "--algorithm", algo, "--iterations", "1", "--verify", "--serialThreads", "8", "--json")
     assert rc == 0, out + err
