@@ -54,12 +54,14 @@ struct Workspace {
 	float* means_t = nullptr;       size_t means_t_cap = 0;    /* floats: exact transposed centroids [dim][kp] */
 	float* partials = nullptr;      size_t partials_cap = 0;   /* floats  */
 	uint32_t* fused_assignment = nullptr; size_t fused_cap = 0; /* entries: assignment vector of kmx_fused_f32 */
+	uint32_t* bucket_sizes = nullptr;     size_t bucket_cap = 0; /* entries: member counts nobody asked for (kmx_bucket_sum_f32) */
 };
 int workspace(Workspace** ws);
 int reserve_queue(Workspace* ws, size_t entries);
 int reserve_packed(Workspace* ws, size_t packed_floats, size_t norm_floats, size_t transposed_floats);
 int reserve_partials(Workspace* ws, size_t floats);
 int reserve_fused_assignment(Workspace* ws, size_t entries);
+int reserve_bucket_sizes(Workspace* ws, size_t entries);
 
 #define KMX_HIP(call)                                                                                         \
 	do {                                                                                                      \
@@ -96,6 +98,7 @@ struct UpdateArgs {
 	float* means; int layout_means; size_t stride_means;
 	uint32_t* cluster_sizes;
 	uint32_t dim, k, n;
+	bool divide = true; /* false: leave the member sums in `means` (the update micro-benchmark) */
 };
 
 /* assign_exact.hip */

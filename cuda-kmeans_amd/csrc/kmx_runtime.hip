@@ -103,6 +103,7 @@ int reserve_packed(Workspace* ws, size_t packed_floats, size_t norm_floats, size
 
 int reserve_partials(Workspace* ws, size_t floats) { return grow(&ws->partials, &ws->partials_cap, floats); }
 int reserve_fused_assignment(Workspace* ws, size_t entries) { return grow(&ws->fused_assignment, &ws->fused_cap, entries); }
+int reserve_bucket_sizes(Workspace* ws, size_t entries) { return grow(&ws->bucket_sizes, &ws->bucket_cap, entries); }
 
 static int release_workspace()
 {
@@ -113,6 +114,7 @@ static int release_workspace()
 	if (g_ws.means_t) KMX_HIP(hipFree(g_ws.means_t));
 	if (g_ws.partials) KMX_HIP(hipFree(g_ws.partials));
 	if (g_ws.fused_assignment) KMX_HIP(hipFree(g_ws.fused_assignment));
+	if (g_ws.bucket_sizes) KMX_HIP(hipFree(g_ws.bucket_sizes));
 	g_ws = Workspace();
 	return KMX_OK;
 }
@@ -373,6 +375,42 @@ int kmx_update_f32(int variant,
 	if (rc) return rc;
 
 	UpdateArgs u{ data, layout, stride, assignment, means, layout_means, stride_means, cluster_sizes, dim, k, n };
+	return launch_update(variant, u, exec, ws, *dev);
+}
+
+int kmx_bucket_sum_f32(int variant,
+                       const float* data, int layout, size_t stride,
+                       const uint32_t* indices,
+                       float* result, int layout_result, size_t stride_result,
+                       uint32_t dim, uint32_t k, uint32_t n, kmx_exec_params* exec)
+{
+	clear_error();
+	if (!exec) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_bucket_sum_f32: exec is null");
+	if (dim == 0 || k == 0) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_bucket_sum_f32: dim and k must be positive");
+	if (!result) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_bucket_sum_f32: null device pointer");
+	if (n > 0 && (!data || !indices)) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_bucket_sum_f32: null device pointer");
+	int rc = check_layout("kmx_bucket_sum_f32", "data", layout, stride, n, dim);
+	if (rc) return rc;
+	rc = check_layout("kmx_bucket_sum_f32", "result", layout_result, stride_result, k, dim);
+	if (rc) return rc;
+	if (variant < KMX_UPDATE_ATOMIC_POINT || variant > KMX_UPDATE_ATOMIC_SHM)
+		return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_bucket_sum_f32: unknown variant %d", variant);
+	if (exec->privatized_copies == 0) exec->privatized_copies = 1;
+
+	const DeviceInfo* dev = nullptr;
+	rc = device_info(&dev);
+	if (rc) return rc;
+	Workspace* ws = nullptr;
+	rc = workspace(&ws);
+	if (rc) return rc;
+	/* the kernels count members as they go; the counts land in a scratch array */
+	rc = reserve_bucket_sizes(ws, k);
+	if (rc) return rc;
+	rc = kmx_fill_zero_u32(ws->bucket_sizes, k);
+	if (rc) return rc;
+
+	UpdateArgs u{ data, layout, stride, indices, result, layout_result, stride_result, ws->bucket_sizes, dim, k, n };
+	u.divide = false;
 	return launch_update(variant, u, exec, ws, *dev);
 }
 

@@ -446,13 +446,14 @@ update_sorted_kernel(const float* __restrict__ data, size_t stride, const uint32
  * means[c][d] = (sum over the chunks of partial[chunk][c][d]) / count[c]  (0 for an empty cluster).
  * Block = 64 consecutive elements x 16 chunk shares; every lane keeps up to 16 loads in flight; the shares meet in LDS.
  * Overwrites means: the sorted path needs neither zeroed centroids nor the separate divide kernel.
+ * divide = 0 stores the sums themselves.
  */
 constexpr uint32_t REDUCE_SHARES = 16;
 
 template <int LM>
 __global__ void __launch_bounds__(64 * REDUCE_SHARES)
 reduce_partials_kernel(const float* __restrict__ partial, float* __restrict__ means, size_t stride_means,
-                       const uint32_t* __restrict__ sizes, uint32_t dim, uint32_t k, uint32_t chunks)
+                       const uint32_t* __restrict__ sizes, uint32_t dim, uint32_t k, uint32_t chunks, uint32_t divide)
 {
 	__shared__ float part[REDUCE_SHARES][64];
 	const uint32_t col = threadIdx.x & 63, share = threadIdx.x >> 6;
@@ -480,7 +481,7 @@ reduce_partials_kernel(const float* __restrict__ partial, float* __restrict__ me
 		for (uint32_t i = 0; i < REDUCE_SHARES; ++i) s += part[i][col];
 		const uint32_t cl = e / dim, d = e - cl * dim;
 		const uint32_t count = sizes[cl];
-		means[elem<LM>(stride_means, cl, d)] = count ? s / (float)count : 0.0f;
+		means[elem<LM>(stride_means, cl, d)] = !divide ? s : (count ? s / (float)count : 0.0f);
 	}
 }
 
@@ -551,7 +552,7 @@ static int launch_sorted(const UpdateArgs& u, Workspace* ws, uint32_t chunks, ui
 	KMX_LAUNCH_CHECK("update_sorted_kernel");
 	const uint32_t total = u.k * u.dim;
 	hipLaunchKernelGGL((reduce_partials_kernel<LM>), dim3((total + 63) / 64), dim3(64 * REDUCE_SHARES), 0, stream(),
-	                   ws->partials, u.means, u.stride_means, u.cluster_sizes, u.dim, u.k, chunks);
+	                   ws->partials, u.means, u.stride_means, u.cluster_sizes, u.dim, u.k, chunks, u.divide ? 1u : 0u);
 	KMX_LAUNCH_CHECK("reduce_partials_kernel");
 	return KMX_OK;
 }
@@ -693,8 +694,10 @@ static int launch_update_t(int variant, const UpdateArgs& u, kmx_exec_params* ex
 		hipLaunchKernelGGL((reduce_copies_kernel<LM>), dim3(blocks), dim3(256), 0, stream(), u.means, u.stride_means, copy_floats, u.dim, u.k, copies);
 		KMX_LAUNCH_CHECK("reduce_copies_kernel");
 	}
-	hipLaunchKernelGGL((divide_means_kernel<LM>), dim3(blocks), dim3(256), 0, stream(), u.means, u.stride_means, u.cluster_sizes, u.dim, u.k);
-	KMX_LAUNCH_CHECK("divide_means_kernel");
+	if (u.divide) {
+		hipLaunchKernelGGL((divide_means_kernel<LM>), dim3(blocks), dim3(256), 0, stream(), u.means, u.stride_means, u.cluster_sizes, u.dim, u.k);
+		KMX_LAUNCH_CHECK("divide_means_kernel");
+	}
 	return KMX_OK;
 }
 

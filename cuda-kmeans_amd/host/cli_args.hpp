@@ -101,9 +101,10 @@ public:
 			if (i + 1 >= argc) throw ArgumentException("Argument '--" + name + "' needs a value.");
 			std::string value = argv[++i];
 			if (a.kind == Kind::Int) {
-				a.intValue = parseInt(name, value);
-				if (a.intValue < a.minValue || a.intValue > a.maxValue)
+				const std::int64_t parsed = parseInt(name, value);
+				if (parsed < a.minValue || parsed > a.maxValue)
 					throw ArgumentException("Argument '--" + name + "' is out of range [" + std::to_string(a.minValue) + ", " + std::to_string(a.maxValue) + "].");
+				a.intValue = parsed;
 			}
 			else if (a.kind == Kind::Enum) {
 				if (!a.options.count(value)) throw ArgumentException("Argument '--" + name + "': '" + value + "' is not one of the allowed values.");

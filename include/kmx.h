@@ -136,6 +136,21 @@ int kmx_update_f32(int variant,
                    uint32_t dim, uint32_t k, uint32_t n, kmx_exec_params* exec);
 
 /*
+ * ---- KERNEL::run(ProblemInstance, CudaExecParameters&) of the update micro-benchmark
+ *      (experimental/bucketing-cuda/bucketing-cuda/headers/kernels.cuh:7-22,44-63; called once per batch by
+ *      CudaBucketingAlgorithm::run, bucketing-cuda/headers/cuda.hpp:56-63) ----
+ * result[b][d] = sum of data[i][d] over the vectors with indices[i] == b: the accumulation of kmx_update_f32 without
+ * counts and without the divide, same variants (enum kmx_update_variant). Precondition as in the reference
+ * (cuda.hpp:48): result (k x dim, times privatized_copies for variants 0 and 1) is zero. The sums of the replicas
+ * are merged into replica 0.
+ */
+int kmx_bucket_sum_f32(int variant,
+                       const float* data, int layout, size_t stride,
+                       const uint32_t* indices,
+                       float* result, int layout_result, size_t stride_result,
+                       uint32_t dim, uint32_t k, uint32_t n, kmx_exec_params* exec);
+
+/*
  * ---- FUSED_KERNEL::run(FusedProblemInstance, CudaExecParameters&) (kernels.cuh:38-53,107-116; called by
  *      CudaFusedKMeansAlgorithm::run, cuda.hpp:174-191) ----
  * One whole iteration without a caller-visible assignment vector: every point is assigned to its nearest centroid
