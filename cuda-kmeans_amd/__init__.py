@@ -30,7 +30,7 @@ KMX_OK, KMX_ERR_INVALID_ARGUMENT, KMX_ERR_UNSUPPORTED, KMX_ERR_DEVICE, KMX_ERR_N
 ABI_SYMBOLS = [
     "kmx_device_count", "kmx_set_device", "kmx_device_props", "kmx_malloc", "kmx_free", "kmx_h2d", "kmx_d2h",
     "kmx_d2d", "kmx_sync", "kmx_set_stream", "kmx_shutdown", "kmx_fill_zero_u32", "kmx_assign_f32",
-    "kmx_assign_last_rechecked", "kmx_assign_last_variant", "kmx_update_f32", "kmx_bucket_sum_f32", "kmx_fused_f32", "kmx_event_create", "kmx_event_destroy", "kmx_event_record",
+    "kmx_assign_last_rechecked", "kmx_assign_last_variant", "kmx_update_f32", "kmx_bucket_sum_f32", "kmx_fused_f32", "kmx_graph_begin", "kmx_graph_end", "kmx_graph_launch", "kmx_graph_destroy", "kmx_event_create", "kmx_event_destroy", "kmx_event_record",
     "kmx_event_elapsed_ms", "kmx_set_profiling", "kmx_last_kernel_ms", "kmx_last_error",
 ]
 
@@ -109,6 +109,10 @@ def hip_lib():
                                            ctypes.POINTER(ExecParams)]
         lib.kmx_fused_f32.argtypes = [ctypes.c_int, vp, ctypes.c_int, sz, vp, vp, ctypes.c_int, sz, vp, u32, u32, u32,
                                       ctypes.POINTER(ExecParams)]
+        lib.kmx_graph_begin.argtypes = []
+        lib.kmx_graph_end.argtypes = [ctypes.POINTER(vp)]
+        lib.kmx_graph_launch.argtypes = [vp]
+        lib.kmx_graph_destroy.argtypes = [vp]
         lib.kmx_event_create.argtypes = [ctypes.POINTER(vp)]
         lib.kmx_event_destroy.argtypes = [vp]
         lib.kmx_event_record.argtypes = [vp]
@@ -299,6 +303,33 @@ def fused(variant, data_buf, layout, stride, means_in_buf, means_out_buf, layout
     return ex
 
 
+class Graph:
+    """A recording of library calls (kmx_graph_begin .. kmx_graph_end) that can be launched as one unit."""
+
+    def __init__(self):
+        self._g = ctypes.c_void_p()
+
+    def __enter__(self):
+        check(hip_lib().kmx_graph_begin())
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        rc = hip_lib().kmx_graph_end(ctypes.byref(self._g))
+        if exc_type is None:
+            check(rc)
+        elif rc == 0:
+            self.destroy()   # a recording that ended in an exception is not kept
+        return False
+
+    def launch(self):
+        check(hip_lib().kmx_graph_launch(self._g))
+
+    def destroy(self):
+        if self._g:
+            check(hip_lib().kmx_graph_destroy(self._g))
+            self._g = ctypes.c_void_p()
+
+
 def set_profiling(enabled):
     check(hip_lib().kmx_set_profiling(1 if enabled else 0))
 
@@ -376,8 +407,25 @@ class HipKMeansAlgorithm:
                self.layout_means, self.stride_means, self.cu_sizes, self.dim, self.k, self.n, self.exec)
         self.last = nxt
 
-    def run(self, iters=None, collect_rechecked=False):
-        for _ in range(self.iters if iters is None else iters):
+    def run(self, iters=None, collect_rechecked=False, use_graph=False):
+        """All iterations, one sync at the end. use_graph: the first iteration runs call by call (it sizes the work
+        space), then two ping-pong iterations are recorded once and replayed; an odd one out runs call by call."""
+        todo = self.iters if iters is None else iters
+        if use_graph and not collect_rechecked and todo >= 3:
+            self.update_step(self.iteration())
+            pairs = (todo - 1) // 2
+            with Graph() as g:
+                for _ in range(2):
+                    self.update_step(self.iteration())
+            for _ in range(pairs):
+                g.launch()
+            todo -= 1 + 2 * pairs
+            for _ in range(todo):
+                self.update_step(self.iteration())
+            sync()
+            g.destroy()
+            return
+        for _ in range(todo):
             nxt = self.iteration()
             if collect_rechecked:
                 self.rechecked.append(last_rechecked())

@@ -25,7 +25,16 @@ int fail(int code, const char* fmt, ...)
 
 void clear_error() { g_error[0] = '\0'; }
 
-hipStream_t stream() { return g_stream; }
+/* while a graph is being recorded every launch goes to the library's own capture stream */
+static hipStream_t g_capture_stream = nullptr;
+static bool g_capturing = false;
+
+hipStream_t stream() { return g_capturing ? g_capture_stream : g_stream; }
+
+#define KMX_NOT_WHILE_CAPTURING(name)                                                                          \
+	do {                                                                                                       \
+		if (g_capturing) return fail(KMX_ERR_INVALID_ARGUMENT, name ": not allowed between kmx_graph_begin and kmx_graph_end"); \
+	} while (0)
 
 static bool g_profiling = false;
 static hipEvent_t g_prof[2][2] = { { nullptr, nullptr }, { nullptr, nullptr } };
@@ -33,7 +42,7 @@ static bool g_prof_valid[2] = { false, false };
 
 int profile_begin(int which)
 {
-	if (!g_profiling) return KMX_OK;
+	if (!g_profiling || g_capturing) return KMX_OK;
 	for (int i = 0; i < 2; ++i)
 		if (!g_prof[which][i]) KMX_HIP(hipEventCreate(&g_prof[which][i]));
 	KMX_HIP(hipEventRecord(g_prof[which][0], g_stream));
@@ -42,7 +51,7 @@ int profile_begin(int which)
 
 int profile_end(int which)
 {
-	if (!g_profiling) return KMX_OK;
+	if (!g_profiling || g_capturing) return KMX_OK;
 	KMX_HIP(hipEventRecord(g_prof[which][1], g_stream));
 	g_prof_valid[which] = true;
 	return KMX_OK;
@@ -78,6 +87,9 @@ template <typename T>
 static int grow(T** ptr, size_t* cap, size_t want)
 {
 	if (want <= *cap) return KMX_OK;
+	if (g_capturing)
+		return fail(KMX_ERR_INVALID_ARGUMENT, "the call needs a larger work space, which cannot be allocated while a graph is recorded: "
+		                                      "make the same call once before kmx_graph_begin");
 	if (*ptr) {
 		/* earlier launches may still be reading the old buffer */
 		KMX_HIP(hipStreamSynchronize(g_stream));
@@ -149,6 +161,7 @@ int kmx_device_count(int* count)
 int kmx_set_device(int device)
 {
 	clear_error();
+	KMX_NOT_WHILE_CAPTURING("kmx_set_device");
 	int c = 0;
 	if (hipGetDeviceCount(&c) != hipSuccess || c == 0) {
 		(void)hipGetLastError();
@@ -181,6 +194,7 @@ int kmx_device_props(kmx_props* props)
 int kmx_malloc(void** dptr, size_t bytes)
 {
 	clear_error();
+	KMX_NOT_WHILE_CAPTURING("kmx_malloc");
 	if (!dptr) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_malloc: null pointer");
 	*dptr = nullptr;
 	if (bytes == 0) return KMX_OK;
@@ -191,6 +205,7 @@ int kmx_malloc(void** dptr, size_t bytes)
 int kmx_free(void* dptr)
 {
 	clear_error();
+	KMX_NOT_WHILE_CAPTURING("kmx_free");
 	if (!dptr) return KMX_OK;
 	KMX_HIP(hipFree(dptr));
 	return KMX_OK;
@@ -199,6 +214,7 @@ int kmx_free(void* dptr)
 int kmx_h2d(void* dst_device, const void* src_host, size_t bytes)
 {
 	clear_error();
+	KMX_NOT_WHILE_CAPTURING("kmx_h2d");
 	if (bytes == 0) return KMX_OK;
 	if (!dst_device || !src_host) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_h2d: null pointer");
 	KMX_HIP(hipMemcpyAsync(dst_device, src_host, bytes, hipMemcpyHostToDevice, stream()));
@@ -208,6 +224,7 @@ int kmx_h2d(void* dst_device, const void* src_host, size_t bytes)
 int kmx_d2h(void* dst_host, const void* src_device, size_t bytes)
 {
 	clear_error();
+	KMX_NOT_WHILE_CAPTURING("kmx_d2h");
 	if (bytes == 0) return KMX_OK;
 	if (!dst_host || !src_device) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_d2h: null pointer");
 	KMX_HIP(hipMemcpyAsync(dst_host, src_device, bytes, hipMemcpyDeviceToHost, stream()));
@@ -218,6 +235,7 @@ int kmx_d2h(void* dst_host, const void* src_device, size_t bytes)
 int kmx_d2d(void* dst_device, const void* src_device, size_t bytes)
 {
 	clear_error();
+	KMX_NOT_WHILE_CAPTURING("kmx_d2d");
 	if (bytes == 0) return KMX_OK;
 	if (!dst_device || !src_device) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_d2d: null pointer");
 	KMX_HIP(hipMemcpyAsync(dst_device, src_device, bytes, hipMemcpyDeviceToDevice, stream()));
@@ -227,6 +245,7 @@ int kmx_d2d(void* dst_device, const void* src_device, size_t bytes)
 int kmx_sync(void)
 {
 	clear_error();
+	KMX_NOT_WHILE_CAPTURING("kmx_sync");
 	KMX_HIP(hipDeviceSynchronize());
 	return KMX_OK;
 }
@@ -234,6 +253,7 @@ int kmx_sync(void)
 int kmx_set_stream(void* hip_stream)
 {
 	clear_error();
+	KMX_NOT_WHILE_CAPTURING("kmx_set_stream");
 	g_stream = (hipStream_t)hip_stream;
 	return KMX_OK;
 }
@@ -241,6 +261,7 @@ int kmx_set_stream(void* hip_stream)
 int kmx_shutdown(void)
 {
 	clear_error();
+	KMX_NOT_WHILE_CAPTURING("kmx_shutdown");
 	KMX_HIP(hipDeviceSynchronize());
 	return release_workspace();
 }
@@ -335,6 +356,7 @@ int kmx_assign_last_variant(int* variant)
 int kmx_assign_last_rechecked(uint64_t* count)
 {
 	clear_error();
+	KMX_NOT_WHILE_CAPTURING("kmx_assign_last_rechecked");
 	if (!count) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_assign_last_rechecked: null pointer");
 	*count = 0;
 	Workspace* ws = nullptr;
@@ -437,6 +459,61 @@ int kmx_fused_f32(int variant,
 	                      cluster_sizes, dim, k, n, exec);
 }
 
+int kmx_graph_begin(void)
+{
+	clear_error();
+	KMX_NOT_WHILE_CAPTURING("kmx_graph_begin");
+	if (!g_capture_stream) KMX_HIP(hipStreamCreateWithFlags(&g_capture_stream, hipStreamNonBlocking));
+	/* work already queued on the caller's stream stays ahead of whatever the graph will do: the graph is launched
+	 * on that stream; recording itself runs nothing */
+	KMX_HIP(hipStreamBeginCapture(g_capture_stream, hipStreamCaptureModeRelaxed));
+	g_capturing = true;
+	return KMX_OK;
+}
+
+int kmx_graph_end(void** graph)
+{
+	clear_error();
+	if (!g_capturing) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_graph_end: no recording in progress");
+	g_capturing = false;
+	hipGraph_t recorded = nullptr;
+	hipError_t e = hipStreamEndCapture(g_capture_stream, &recorded);
+	if (e != hipSuccess) {
+		(void)hipGetLastError(); /* a failed recording must not poison the launch checks that follow */
+		return fail(KMX_ERR_DEVICE, "hipStreamEndCapture failed: %s", hipGetErrorString(e));
+	}
+	if (!graph) {
+		(void)hipGraphDestroy(recorded);
+		return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_graph_end: null pointer");
+	}
+	hipGraphExec_t exec = nullptr;
+	e = hipGraphInstantiate(&exec, recorded, nullptr, nullptr, 0);
+	(void)hipGraphDestroy(recorded);
+	if (e != hipSuccess) {
+		(void)hipGetLastError();
+		return fail(KMX_ERR_DEVICE, "hipGraphInstantiate failed: %s", hipGetErrorString(e));
+	}
+	*graph = (void*)exec;
+	return KMX_OK;
+}
+
+int kmx_graph_launch(void* graph)
+{
+	clear_error();
+	KMX_NOT_WHILE_CAPTURING("kmx_graph_launch");
+	if (!graph) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_graph_launch: null graph");
+	KMX_HIP(hipGraphLaunch((hipGraphExec_t)graph, g_stream));
+	return KMX_OK;
+}
+
+int kmx_graph_destroy(void* graph)
+{
+	clear_error();
+	if (!graph) return KMX_OK;
+	KMX_HIP(hipGraphExecDestroy((hipGraphExec_t)graph));
+	return KMX_OK;
+}
+
 int kmx_set_profiling(int enabled)
 {
 	clear_error();
@@ -476,6 +553,7 @@ int kmx_event_destroy(void* event)
 int kmx_event_record(void* event)
 {
 	clear_error();
+	KMX_NOT_WHILE_CAPTURING("kmx_event_record");
 	if (!event) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_event_record: null event");
 	KMX_HIP(hipEventRecord((hipEvent_t)event, stream()));
 	return KMX_OK;
@@ -484,6 +562,7 @@ int kmx_event_record(void* event)
 int kmx_event_elapsed_ms(void* start, void* stop, float* ms)
 {
 	clear_error();
+	KMX_NOT_WHILE_CAPTURING("kmx_event_elapsed_ms");
 	if (!start || !stop || !ms) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_event_elapsed_ms: null argument");
 	KMX_HIP(hipEventSynchronize((hipEvent_t)stop));
 	KMX_HIP(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));

@@ -88,6 +88,7 @@ class HipKMeansAlgorithm : public IKMeansAlgorithm<F, IDX_T>
 	unsigned mLast = 0;
 	/* split timing (optional): events around the assignment and the update of every iteration */
 	bool mTimeSplit = false;
+	bool mUseGraph = false;
 	double mAssignMs = 0.0, mUpdateMs = 0.0;
 	std::uint64_t mRechecked = 0;
 
@@ -102,7 +103,9 @@ class HipKMeansAlgorithm : public IKMeansAlgorithm<F, IDX_T>
 	}
 
 public:
-	explicit HipKMeansAlgorithm(const HipExecParameters& exec, bool timeSplit = false) : mExecParams(exec), mTimeSplit(timeSplit) {}
+	/* useGraph: replay a recorded pair of iterations instead of launching every kernel (ignored with the timing split) */
+	explicit HipKMeansAlgorithm(const HipExecParameters& exec, bool timeSplit = false, bool useGraph = false)
+		: mExecParams(exec), mTimeSplit(timeSplit), mUseGraph(useGraph) {}
 
 	void initialize(std::size_t dim, std::size_t k, std::size_t n, std::size_t iters,
 		const std::vector<F>& data, const std::vector<F>& means) override
@@ -123,8 +126,50 @@ public:
 		KMX_CHECK(kmx_sync());
 	}
 
+private:
+	/* one iteration, launched kernel by kernel, without the optional timing */
+	void iterate()
+	{
+		const std::size_t copies = mExecParams.privatizedCopies ? mExecParams.privatizedCopies : 1;
+		const unsigned next = (mLast + 1) % 2;
+		AssignmentProblemInstance<F, IDX_T> assignment(*mDevData, *mDevMeans[mLast], *mDevAssignment[mLast],
+			*mDevAssignment[next], this->mDim, this->mK, this->mN);
+		ASGN_KERNEL::run(assignment, mExecParams);
+		runFillZeros<F>(*mDevMeans[next], meansSize() * copies);
+		runFillZeros<IDX_T>(*mDevClusterSizes, this->mK);
+		UpdateProblemInstance<F, IDX_T> update(*mDevData, *mDevAssignment[next], *mDevMeans[next], *mDevClusterSizes,
+			this->mDim, this->mK, this->mN);
+		UPDATE_KERNEL::run(update, mExecParams);
+		mLast = next;
+	}
+
+	/* the first iteration sizes the library's work space, then two ping-pong iterations are recorded once and replayed */
+	void runRecorded()
+	{
+		iterate();
+		const std::size_t pairs = (this->mIters - 1) / 2;
+		void* graph = nullptr;
+		KMX_CHECK(kmx_graph_begin());
+		try {
+			iterate();
+			iterate();
+		}
+		catch (...) {
+			kmx_graph_end(&graph);
+			kmx_graph_destroy(graph);
+			throw;
+		}
+		KMX_CHECK(kmx_graph_end(&graph));
+		for (std::size_t i = 0; i < pairs; ++i) KMX_CHECK(kmx_graph_launch(graph));
+		for (std::size_t done = 1 + 2 * pairs; done < this->mIters; ++done) iterate();
+		KMX_CHECK(kmx_sync());
+		KMX_CHECK(kmx_graph_destroy(graph));
+	}
+
+public:
 	void run() override
 	{
+		if (mUseGraph && !mTimeSplit && this->mIters >= 3) { runRecorded(); return; }
 		void* ev[3] = { nullptr, nullptr, nullptr };
 		if (mTimeSplit) for (auto& e : ev) KMX_CHECK(kmx_event_create(&e));
 		const std::size_t copies = mExecParams.privatizedCopies ? mExecParams.privatizedCopies : 1;

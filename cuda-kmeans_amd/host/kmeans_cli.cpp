@@ -156,6 +156,7 @@ void run_kmeans(const ProgramArguments& args, std::vector<F>& data, std::vector<
 	HipExecParameters exec;
 	getHipExecParameters(args, exec);
 
+	const bool graph = args.getBool("graph");
 	using Base = BaseAssignmentKernel<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC>;
 	using Best = BestCachedAssignmentKernel<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC>;
 	using Mfma = MfmaAssignmentKernel<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC>;
@@ -165,11 +166,11 @@ void run_kmeans(const ProgramArguments& args, std::vector<F>& data, std::vector<
 	using map_t = std::map<std::string, std::unique_ptr<IKMeansAlgorithm<F, IDX_T>>>;
 	map_t algorithms;
 	algorithms["serial"].reset(new SerialKMeansAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC>(threads));
-	algorithms["hip_base"].reset(new HipKMeansAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC, Base, Point>(exec, json));
-	algorithms["hip_base_shm"].reset(new HipKMeansAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC, Base, Shm>(exec, json));
-	algorithms["hip_mfma"].reset(new HipKMeansAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC, Mfma, Shm>(exec, json));
-	algorithms["hip_mfma_bf16"].reset(new HipKMeansAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC, MfmaBf16, Shm>(exec, json));
-	algorithms["hip_best"].reset(new HipKMeansAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC, Best, Shm>(exec, json));
+	algorithms["hip_base"].reset(new HipKMeansAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC, Base, Point>(exec, json, graph));
+	algorithms["hip_base_shm"].reset(new HipKMeansAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC, Base, Shm>(exec, json, graph));
+	algorithms["hip_mfma"].reset(new HipKMeansAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC, Mfma, Shm>(exec, json, graph));
+	algorithms["hip_mfma_bf16"].reset(new HipKMeansAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC, MfmaBf16, Shm>(exec, json, graph));
+	algorithms["hip_best"].reset(new HipKMeansAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC, Best, Shm>(exec, json, graph));
 	algorithms["hip_fused"].reset(new HipFusedKMeansAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC>(exec));
 
 	auto it = algorithms.find(algoName);
@@ -325,6 +326,7 @@ int main(int argc, char* argv[])
 		args.registerEnum("init", "Initial centroids: k shuffled points (reference) or the first k points.", "shuffle", { "shuffle", "first" });
 		args.registerInt("serialThreads", "Threads of the serial algorithm (results are bit-identical to 1 thread).", 1, 1, 1024);
 		args.registerBool("json", "Print a JSON report instead of the two-number line.");
+		args.registerBool("graph", "Record a pair of iterations as a HIP graph and replay it instead of launching every kernel (device algorithms; not with --json).");
 		args.registerString("dump", "Write the final centroids and assignment to <prefix>.means.f32 / <prefix>.assignment.u32.", "");
 		args.process(argc, argv);
 	}

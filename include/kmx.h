@@ -177,6 +177,21 @@ int kmx_event_record(void* event);
 int kmx_event_elapsed_ms(void* start, void* stop, float* ms); /* waits for `stop` */
 
 /*
+ * ---- recorded iterations (no counterpart in the reference, whose loop launches kernel by kernel,
+ *      cuda.hpp:70-88) ----
+ * Between kmx_graph_begin and kmx_graph_end the launching calls (kmx_assign_f32, kmx_update_f32, kmx_fused_f32,
+ * kmx_bucket_sum_f32, kmx_fill_zero_u32) run nothing: their kernels, with the arguments of that moment, are recorded into
+ * a HIP graph. kmx_graph_launch enqueues the whole recording on the library's stream as one unit, any number of times
+ * (the host driver records two ping-pong iterations once and replays them). Everything that allocates, copies or
+ * waits is refused while recording; a call whose work space would have to grow is refused too -- make the same
+ * calls once before recording. Per-kernel profiling events are not recorded.
+ */
+int kmx_graph_begin(void);
+int kmx_graph_end(void** graph);
+int kmx_graph_launch(void* graph);
+int kmx_graph_destroy(void* graph);
+
+/*
  * Per-kernel timing for roofline reports (no counterpart in the reference). While enabled, every
  * kmx_assign_f32 / kmx_update_f32 call brackets its dominant kernel (the sweep over the centroids /
  * the accumulation pass; not the small pack, recheck, merge and divide kernels around it) with a pair of

@@ -356,3 +356,67 @@ def test_full_size_properties(km, orc, gpu, cid):
     d_other = ((x - c[other]) ** 2).sum(1)
     assert np.all(d_own <= d_other * (1 + 1e-5) + 1e-12)
     assert rechecked < n // 10
+
+
+# ---------------------------------------------------------------- recorded iterations (HIP graph)
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("cid,n", [(2, 65536), (1, 65536), (5, 1 << 18)])
+def test_recorded_iterations_are_correct_iterations(km, orc, gpu, cid, n):
+    """Two ping-pong iterations recorded once and replayed. Two runs are not comparable bit for bit (the update's fp32
+    summation order is not fixed), so every replayed run is checked the way the call-by-call loop is: its last iteration
+    against the oracle fed with the centroids that iteration read (they are still in the other ping-pong buffer).
+    The recording is made and replayed in several runs, with call-by-call work and synchronisations in between."""
+    spec = km.baseline_config(cid)
+    dim, k = spec.dim, spec.k
+    data = km.generate_points(spec, n)
+    means0 = km.first_k_means(spec)
+    alg = km.HipKMeansAlgorithm(km.ASSIGN_BEST, km.UPDATE_ATOMIC_SHM)
+    alg.initialize(dim, k, n, 8, data, means0)
+    for iters in (7, 8, 3, 6):
+        alg.reset(means0)
+        alg.run(iters=iters, use_graph=True)
+        read_means = alg.cu_means[1 - alg.last].read(np.float32, alg.means_size)
+        ga, gm, gs = alg.getAssignment(), alg.getMeans(), alg.getClusterSizes()
+        oa = orc.assign(data, read_means, dim, k, n, threads=0, fast=True)
+        assert np.array_equal(ga, oa), "%d iterations: %d mismatches" % (iters, int((ga != oa).sum()))
+        om, osz = orc.update(data, ga, dim, k, n, threads=0)
+        assert np.array_equal(gs, osz)
+        assert rel_err(gm, om) < CENTROID_RTOL
+        alg.reset(means0)
+        alg.run(iters=2)                      # call-by-call work between the recordings
+    alg.cleanup()
+
+
+@pytest.mark.gpu
+def test_recording_refuses_what_cannot_be_recorded(km, gpu):
+    buf = km.DeviceBuffer(4096)
+    with pytest.raises(km.KmxError):
+        with km.Graph() as g:
+            buf.zero()
+            km.sync()                          # waiting is refused while recording
+    # the recording was closed by the context manager; the library is usable again
+    with km.Graph() as g:
+        buf.zero()
+    g.launch()
+    km.sync()
+    assert not buf.read(np.uint32, 1024).any()
+    g.destroy()
+    # a call that would have to grow the work space is refused while recording
+    dim, k, n = 16, 64, 4096
+    rng = np.random.default_rng(3)
+    d = km.DeviceBuffer(4 * n * dim); d.write(rng.normal(size=n * dim).astype(np.float32))
+    m = km.DeviceBuffer(4 * k * dim); m.write(rng.normal(size=k * dim).astype(np.float32))
+    a = km.DeviceBuffer(4 * n)
+    km.check(km.hip_lib().kmx_shutdown())      # releases the work space
+    with pytest.raises(km.KmxError):
+        with km.Graph() as g:
+            km.assign(km.ASSIGN_BEST, d, AOS, dim, m, AOS, dim, a, dim, k, n)
+    km.assign(km.ASSIGN_BEST, d, AOS, dim, m, AOS, dim, a, dim, k, n)   # sizes the work space
+    with km.Graph() as g:
+        km.assign(km.ASSIGN_BEST, d, AOS, dim, m, AOS, dim, a, dim, k, n)
+    g.launch()
+    km.sync()
+    g.destroy()
+    for b in (buf, d, m, a):
+        b.free()

@@ -115,3 +115,13 @@ def test_device_assignment_only_and_reference_dataset(harness, gpu):
         assert rc == 0 and "Verifying results ... OK" in err, err
     rc, out, err = run(harness, "--algorithm", "hip_lds_fma", "--assignmentOnly", "--dim", "100")
     assert rc == 2 and "not supported" in out
+
+
+@pytest.mark.gpu
+def test_recorded_iterations_verify(harness, gpu):
+    """--graph: the first iteration call by call, then a recorded pair of iterations replayed; one iteration cannot
+    diverge from the serial run, several are checked through the harness's own loose centroid rule."""
+    rc, out, err = run(harness, "--config", "1", "--algorithm", "hip_best", "--iterations", "5", "--graph")
+    assert rc == 0 and len(out.split()) == 2, out + err
+    rc, out, err = run(harness, "--algorithm", "hip_best", "--iterations", "4", "--graph", "--verify", "--N", "64k", "--k", "256", "--dim", "16")
+    assert rc == 0 and "Verifying results ..." in err, out + err
