@@ -79,7 +79,8 @@ bool bf16_supports(const AssignArgs& a, const DeviceInfo& dev)
 {
 	const uint32_t kb = pick_kb(a.dim);
 	if (kb == 0) return false;
-	return (size_t)(tile_floats(KBLOCK * kb + ROW_PAD) + NORM_TILE) * 4 + 8192 <= dev.lds_bytes;
+	/* two tiles (the double-buffered stream of the centroid block) plus the static flag lists must fit */
+	return (size_t)(tile_floats(KBLOCK * kb + ROW_PAD) + NORM_TILE) * 4 * 2 + 2 * FLAG_CAP * MFMA_WAVES * 4 + 1024 <= dev.lds_bytes;
 }
 
 #define KMX_DECLARE_BF16_LAUNCHER(W) \

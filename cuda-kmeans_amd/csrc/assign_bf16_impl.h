@@ -15,6 +15,7 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr uint32_t KBLOCK = 16; /* dimensions per v_mfma_f32_32x32x16_bf16 */
+constexpr int STAGE_VECS = 9;   /* 16-byte pieces of a streamed chunk per lane: a chunk holds at most 9 * 512 * 16 bytes of tiles */
 
 /* value = hi + mid + (at most 2^-18 |value|), both parts bf16 (round to nearest even) */
 __device__ __forceinline__ void split_bf16(float v, __bf16& hi, __bf16& mid)
@@ -173,22 +174,57 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 	for (uint32_t w = 0; w < MFMA_WAVES; ++w) cmax = max(cmax, wave_max[w]);
 	const float c2max = __uint_as_float(cmax);
 
-	float* lds_norms = lds + (size_t)(chunk_rows / TILE) * tile_floats(RS);
+	const uint32_t chunk_tiles = chunk_rows / TILE;
 	const uint32_t chunks = (kp + chunk_rows - 1) / chunk_rows;
+	/* STREAM: two LDS buffers of chunk_tiles packed tiles followed by their norms; `cur` is the one in use */
+	const uint32_t buf_floats = chunk_tiles * (tile_floats(RS) + NORM_TILE);
+	uint32_t cur = 0;
 
-	auto stage = [&](uint32_t row0, uint32_t rows) {
+	/* one chunk on its way from global memory to LDS: this lane's share, held in registers while the previous
+	 * chunk is being used (requested before, committed after the tile steps of that chunk) */
+	struct Staged {
+		f32x4 v[STAGE_VECS];
+		f32x4 nv;
+	};
+	auto request = [&](Staged& sg, uint32_t row0, uint32_t rows) {
 		const f32x4* src = (const f32x4*)(packed + packed_row(row0, RS));
-		f32x4* dst = (f32x4*)lds;
 		const uint32_t vecs = (rows / TILE) * tile_floats(RS) / 4;
-		for (uint32_t i = threadIdx.x; i < vecs; i += blockDim.x) dst[i] = src[i];
+#pragma unroll
+		for (int i = 0; i < STAGE_VECS; ++i) {
+			const uint32_t at = threadIdx.x + i * (MFMA_WAVES * WAVE);
+			if (at < vecs) sg.v[i] = src[at];
+		}
 		const f32x4* nsrc = (const f32x4*)(norms + (size_t)(row0 / TILE) * NORM_TILE);
-		f32x4* ndst = (f32x4*)lds_norms;
-		const uint32_t nvecs = (rows / TILE) * NORM_TILE / 4;
-		for (uint32_t i = threadIdx.x; i < nvecs; i += blockDim.x) ndst[i] = nsrc[i];
+		if (threadIdx.x < (rows / TILE) * NORM_TILE / 4) sg.nv = nsrc[threadIdx.x];
+	};
+	auto commit = [&](const Staged& sg, uint32_t buffer, uint32_t rows) {
+		f32x4* dst = (f32x4*)(lds + (size_t)buffer * buf_floats);
+		const uint32_t vecs = (rows / TILE) * tile_floats(RS) / 4;
+#pragma unroll
+		for (int i = 0; i < STAGE_VECS; ++i) {
+			const uint32_t at = threadIdx.x + i * (MFMA_WAVES * WAVE);
+			if (at < vecs) dst[at] = sg.v[i];
+		}
+		f32x4* ndst = (f32x4*)(lds + (size_t)buffer * buf_floats + (size_t)chunk_tiles * tile_floats(RS));
+		if (threadIdx.x < (rows / TILE) * NORM_TILE / 4) ndst[threadIdx.x] = sg.nv;
 	};
 
 	if (!STREAM) {
-		stage(0, kp);
+		/* everything resident: flat 16-byte copies of all packed tiles and norms */
+		const f32x4* src = (const f32x4*)packed;
+		f32x4* dst = (f32x4*)lds;
+		const uint32_t vecs = (kp / TILE) * tile_floats(RS) / 4;
+		for (uint32_t i = threadIdx.x; i < vecs; i += blockDim.x) dst[i] = src[i];
+		const f32x4* nsrc = (const f32x4*)norms;
+		f32x4* ndst = (f32x4*)(lds + (size_t)chunk_tiles * tile_floats(RS));
+		const uint32_t nvecs = (kp / TILE) * NORM_TILE / 4;
+		for (uint32_t i = threadIdx.x; i < nvecs; i += blockDim.x) ndst[i] = nsrc[i];
+		__syncthreads();
+	}
+	else {
+		Staged first;
+		request(first, 0, min(chunk_rows, kp));
+		commit(first, 0, min(chunk_rows, kp));
 		__syncthreads();
 	}
 
@@ -223,28 +259,37 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 		for (uint32_t chunk = 0; chunk < chunks; ++chunk) {
 			const uint32_t row0 = chunk * chunk_rows;
 			const uint32_t rows = min(chunk_rows, kp - row0);
-			if (STREAM) {
-				__syncthreads(); /* everyone is done with the previous chunk */
-				stage(row0, rows);
-				__syncthreads();
-			}
+			/* STREAM: while this chunk is used, the next one (after the last: the first one, for the next sweep) is on
+			 * its way; it is written to the other buffer once the tile steps are done */
+			const uint32_t next_row0 = chunk + 1 < chunks ? row0 + chunk_rows : 0;
+			const uint32_t next_rows = min(chunk_rows, kp - next_row0);
+			Staged incoming;
+			if (STREAM) request(incoming, next_row0, next_rows);
+			const float* lds_tiles = lds + (size_t)cur * buf_floats;
+			const float* lds_norms = lds_tiles + (size_t)chunk_tiles * tile_floats(RS);
 			const uint32_t tiles = rows / TILE;
 			const uint32_t tile0 = row0 / TILE;
-			tile_step_bf16<KB, P, false, COARSE>(lds, lds_norms, 0, col, h, b, acc0, acc1, 0, st, neg_inf);
+			tile_step_bf16<KB, P, false, COARSE>(lds_tiles, lds_norms, 0, col, h, b, acc0, acc1, 0, st, neg_inf);
 			uint32_t t = 0; /* acc0 holds tile t, not yet tracked */
 			while (t + 2 < tiles) {
-				tile_step_bf16<KB, P, true, COARSE>(lds, lds_norms, t + 1, col, h, b, acc1, acc0, tile0 + t, st, neg_inf);
-				tile_step_bf16<KB, P, true, COARSE>(lds, lds_norms, t + 2, col, h, b, acc0, acc1, tile0 + t + 1, st, neg_inf);
+				tile_step_bf16<KB, P, true, COARSE>(lds_tiles, lds_norms, t + 1, col, h, b, acc1, acc0, tile0 + t, st, neg_inf);
+				tile_step_bf16<KB, P, true, COARSE>(lds_tiles, lds_norms, t + 2, col, h, b, acc0, acc1, tile0 + t + 1, st, neg_inf);
 				t += 2;
 			}
 			if (t + 1 < tiles) {
-				tile_step_bf16<KB, P, true, COARSE>(lds, lds_norms, t + 1, col, h, b, acc1, acc0, tile0 + t, st, neg_inf);
+				tile_step_bf16<KB, P, true, COARSE>(lds_tiles, lds_norms, t + 1, col, h, b, acc1, acc0, tile0 + t, st, neg_inf);
 #pragma unroll
 				for (int p = 0; p < P; ++p) track_tile<COARSE>(acc1[p], st[p], tile0 + t + 1, neg_inf);
 			}
 			else {
 #pragma unroll
 				for (int p = 0; p < P; ++p) track_tile<COARSE>(acc0[p], st[p], tile0 + t, neg_inf);
+			}
+			if (STREAM) {
+				/* the other buffer was last read one chunk ago, before the barrier that ended that chunk */
+				commit(incoming, cur ^ 1u, next_rows);
+				__syncthreads();
+				cur ^= 1u;
 			}
 		}
 
@@ -263,7 +308,7 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 				const uint32_t wh = win ? h : 1u - h;
 				const float W = win ? fminf(o1, st[p].m2) : fminf(st[p].m1, o2);
 				const float* tile_base = STREAM ? packed + (size_t)ts * tile_floats(RS) : lds + (size_t)ts * tile_floats(RS);
-				const float* norm_base = STREAM ? norms + ts * NORM_TILE : lds_norms + ts * NORM_TILE;
+				const float* norm_base = STREAM ? norms + ts * NORM_TILE : lds + (size_t)chunk_tiles * tile_floats(RS) + ts * NORM_TILE;
 				float tot[16];
 #pragma unroll
 				for (int r = 0; r < 16; ++r)
@@ -358,10 +403,20 @@ static int launch_bf16_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 	const uint32_t static_bytes = (2 * FLAG_CAP * MFMA_WAVES + 64) * 4;
 	const uint32_t tile_bytes = (tile_floats(RS) + NORM_TILE) * 4;
 	if (budget < static_bytes + tile_bytes) return fail(KMX_ERR_UNSUPPORTED, "assign (split-bf16 MFMA): LDS budget of %u bytes is too small", budget);
-	const uint32_t chunk_rows = std::min<uint32_t>(kp, (budget - static_bytes) / tile_bytes * TILE);
-	const bool stream_mode = chunk_rows < kp;
+	/* everything resident if it fits (rows up to 64 dimensions only: the wider kernels always stream); otherwise two
+	 * buffers of as many tiles as fit, bounded by what a work-group carries in registers (STAGE_VECS) */
+	uint32_t chunk_rows = std::min<uint32_t>(kp, (budget - static_bytes) / tile_bytes * TILE);
+	const bool stream_mode = KB > 4 || chunk_rows < kp;
+	if (stream_mode) {
+		const uint32_t by_lds = (budget - static_bytes) / (2 * tile_bytes);
+		const uint32_t by_regs = (uint32_t)STAGE_VECS * MFMA_WAVES * WAVE * 16 / (tile_floats(RS) * 4);
+		const uint32_t by_norms = MFMA_WAVES * WAVE * 4 / NORM_TILE;
+		const uint32_t chunk_tiles = std::min({ by_lds, by_regs, by_norms, kp / TILE });
+		if (chunk_tiles == 0) return fail(KMX_ERR_UNSUPPORTED, "assign (split-bf16 MFMA): two tiles of %u-dimension rows do not fit the LDS budget of %u bytes", KBLOCK * KB, budget);
+		chunk_rows = chunk_tiles * TILE;
+	}
 	const bool coarse = kp / TILE >= COARSE_MIN_TILES && KB <= 4;
-	const uint32_t lds_bytes = chunk_rows / TILE * tile_bytes;
+	const uint32_t lds_bytes = (stream_mode ? 2u : 1u) * (chunk_rows / TILE) * tile_bytes;
 	const uint32_t unit_points = MFMA_WAVES * P * TILE;
 	const uint32_t units = (a.n + unit_points - 1) / unit_points;
 	void (*kernel)(const float*, size_t, const float*, const float*, uint32_t*, uint32_t*, uint32_t*,
