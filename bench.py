@@ -40,7 +40,7 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 PUBLISHED_MS = {2: 25.45}  # results/README.md:20 of the reference
 # HBM bytes per launch of the dominant kernels at configuration 2, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # scaled by the readings for a 256 MiB device copy (profiles/headline_cfg2_kernels.md); None where not measured
-MEASURED_TRAFFIC = {2: {"assign": 278.5e6, "update": 311.5e6}}
+MEASURED_TRAFFIC = {2: {"assign": 278.6e6, "update": 311.5e6}}
 
 
 def cpu_baseline(km, spec, n_sample, data, means0):
