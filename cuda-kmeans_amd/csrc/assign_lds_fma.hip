@@ -4,13 +4,18 @@
  * a[j] = |c_j|^2 - 2 c_j . x by plain v_fma_f32, exact (min, second min, argmin) tracking per lane, and the same
  * certification / recheck queue as the MFMA variant (see assign_mfma.hip for the error bound).
  *
+ * With a handful of centroids (the packed block within 8 KB: k = 16 at d = 16, k = 64 at d = 8) the rows are not staged
+ * in LDS at all: they are read with wave-uniform addresses, i.e. as scalar loads through the scalar cache, and feed
+ * the multiply-adds as scalar operands. That variant is the fastest sweep for k <= 32 (HBM-bound shapes; measured
+ * 0.26 ms against 0.32 ms for the MFMA sweep at N = 16.7 M, d = 16, k = 16).
+ *
  * This is the counterpart of the reference's shared-memory kernels (cachedFixedAssignmentKernel /
  * cachedRegsAssignmentKernel, reference kernels.cu:216-273,546-661): centroids cached on chip, distances
  * accumulated in registers. On gfx950 it is the SLOWER path at every shape that was measured: an fp32 MFMA
  * retires two multiply-adds per lane and cycle, a v_fma_f32 one (packed fp32 is not used), and the LDS
  * broadcast reads and the per-pair tracking come on top. It is kept as a selectable variant
- * (KMX_ASSIGN_LDS_FMA, `hip_lds_fma`) so that the choice can be measured; KMX_ASSIGN_BEST never picks it
- * where the MFMA variant applies.
+ * (KMX_ASSIGN_LDS_FMA, `hip_lds_fma`) so that the choice can be measured; KMX_ASSIGN_BEST picks it only for
+ * k <= 32 with the scalar-cache path.
  */
 #include "assign_mfma_impl.h"
 
@@ -18,11 +23,11 @@ namespace kmx {
 
 constexpr uint32_t FMA_WAVES = 4; /* wavefronts per work-group */
 
-template <int DP, int LD>
+template <int DP, int LD, bool SCALAR>
 __global__ void __launch_bounds__(FMA_WAVES * WAVE)
 assign_lds_fma_kernel(const float* __restrict__ data, size_t stride, const float* __restrict__ packed, const float* __restrict__ norms,
                       uint32_t* __restrict__ assignment, uint32_t* __restrict__ queue, uint32_t* __restrict__ counters,
-                      uint32_t dim, uint32_t k, uint32_t kp, uint32_t n, uint32_t chunk_rows, float kd)
+                      uint32_t dim, uint32_t k, uint32_t kp, uint32_t n, uint32_t chunk_rows, float kd, uint32_t vec4)
 {
 	constexpr uint32_t RS = DP + ROW_PAD;
 	extern __shared__ float lds[];
@@ -52,8 +57,12 @@ assign_lds_fma_kernel(const float* __restrict__ data, size_t stride, const float
 		const uint32_t nvecs = (rows / TILE) * NORM_TILE / 4;
 		for (uint32_t i = threadIdx.x; i < nvecs; i += blockDim.x) ndst[i] = nsrc[i];
 	};
-	const bool resident = chunks == 1;
-	if (resident) {
+	/* SCALAR: a handful of centroids. Their rows are read straight from memory with wave-uniform addresses, which the
+	 * compiler turns into scalar loads: the values arrive in scalar registers through the scalar cache and feed the
+	 * multiply-adds as scalar operands -- no LDS traffic at all, which is what bounds the LDS variant (one 128-bit
+	 * LDS read per four multiply-adds). */
+	const bool resident = chunks == 1 || SCALAR;
+	if (resident && !SCALAR) {
 		stage(0, kp);
 		__syncthreads();
 	}
@@ -78,14 +87,24 @@ assign_lds_fma_kernel(const float* __restrict__ data, size_t stride, const float
 		const bool valid = pt < n;
 		float x[DP];
 		float x2 = 0.0f;
+		if (LD == KMX_AOS && vec4) {
+			/* rows of whole, aligned 16-byte pieces */
 #pragma unroll
-		for (int q = 0; q < DP; ++q) {
-			x[q] = (valid && (uint32_t)q < dim) ? data[elem<LD>(stride, pt, q)] : 0.0f;
-			x2 += x[q] * x[q];
+			for (int q = 0; q < DP; q += 4) {
+				f32x4 v = { 0.0f, 0.0f, 0.0f, 0.0f };
+				if (valid && (uint32_t)q < dim) v = *(const f32x4*)(data + (size_t)pt * stride + q);
+				x[q] = v.x; x[q + 1] = v.y; x[q + 2] = v.z; x[q + 3] = v.w;
+			}
 		}
+		else {
+#pragma unroll
+			for (int q = 0; q < DP; ++q) x[q] = (valid && (uint32_t)q < dim) ? data[elem<LD>(stride, pt, q)] : 0.0f;
+		}
+#pragma unroll
+		for (int q = 0; q < DP; ++q) x2 += x[q] * x[q];
 		float m1 = __builtin_inff(), m2 = __builtin_inff();
 		uint32_t best = 0;
-		for (uint32_t chunk = 0; chunk < chunks; ++chunk) {
+		for (uint32_t chunk = 0; chunk < (SCALAR ? 1u : chunks); ++chunk) {
 			const uint32_t row0 = chunk * chunk_rows;
 			const uint32_t rows = min(chunk_rows, kp - row0);
 			if (!resident) {
@@ -93,9 +112,12 @@ assign_lds_fma_kernel(const float* __restrict__ data, size_t stride, const float
 				stage(row0, rows);
 				__syncthreads();
 			}
-			for (uint32_t r = 0; r < rows; ++r) {
-				const float* row = lds + packed_row(r, RS); /* uniform address: every lane reads the same words */
-				float a = lds_norms[norm_at(r)];
+			const uint32_t scan_rows = SCALAR ? k : rows; /* the scalar variant skips the padding rows */
+#pragma unroll 4
+			for (uint32_t r = 0; r < scan_rows; ++r) {
+				/* uniform address: every lane reads the same words */
+				const float* row = SCALAR ? packed + packed_row(r, RS) : lds + packed_row(r, RS);
+				float a = SCALAR ? norms[norm_at(r)] : lds_norms[norm_at(r)];
 #pragma unroll
 				for (int q = 0; q < DP; q += 4) {
 					const f32x4 c = *(const f32x4*)(row + q);
@@ -136,6 +158,20 @@ static uint32_t fma_dp(uint32_t dim)
 	return 0;
 }
 
+/* centroid blocks up to this size are read through the scalar cache instead of LDS */
+constexpr uint32_t SCALAR_BLOCK_BYTES = 8 * 1024;
+
+static bool scalar_block(uint32_t dp, uint32_t kp)
+{
+	return (size_t)(kp / TILE) * (tile_floats(dp + ROW_PAD) + NORM_TILE) * 4 <= SCALAR_BLOCK_BYTES;
+}
+
+bool lds_fma_reads_through_scalar_cache(const AssignArgs& a)
+{
+	const uint32_t dp = fma_dp(a.dim);
+	return dp != 0 && scalar_block(dp, round_up(a.k, TILE));
+}
+
 bool lds_fma_supports(const AssignArgs& a, const DeviceInfo& dev)
 {
 	const uint32_t dp = fma_dp(a.dim);
@@ -151,21 +187,23 @@ static int launch_fma_dp(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 	budget = std::min<uint32_t>(budget, 64 * 1024); /* leave room for several work-groups per CU */
 	const uint32_t static_bytes = (2 * FLAG_CAP * FMA_WAVES + 64) * 4;
 	const uint32_t tile_bytes = (tile_floats(RS) + NORM_TILE) * 4;
-	if (budget < static_bytes + tile_bytes) return fail(KMX_ERR_UNSUPPORTED, "assign (LDS/FMA): LDS budget of %u bytes is too small", budget);
-	const uint32_t chunk_rows = std::min<uint32_t>(kp, (budget - static_bytes) / tile_bytes * TILE);
-	const uint32_t lds_bytes = chunk_rows / TILE * tile_bytes;
+	const bool scalar = scalar_block(DP, kp);
+	if (!scalar && budget < static_bytes + tile_bytes) return fail(KMX_ERR_UNSUPPORTED, "assign (LDS/FMA): LDS budget of %u bytes is too small", budget);
+	const uint32_t chunk_rows = scalar ? kp : std::min<uint32_t>(kp, (budget - static_bytes) / tile_bytes * TILE);
+	const uint32_t lds_bytes = scalar ? 0 : chunk_rows / TILE * tile_bytes;
 	const uint32_t batches = (a.n + FMA_WAVES * WAVE - 1) / (FMA_WAVES * WAVE);
 	const uint32_t per_cu = std::max<uint32_t>(1, std::min<uint32_t>(8, dev.lds_bytes / (lds_bytes + static_bytes)));
 	const uint32_t grid = std::min(batches, dev.compute_units * per_cu);
 	exec->block_count = grid;
+	void (*kernel)(const float*, size_t, const float*, const float*, uint32_t*, uint32_t*, uint32_t*,
+	               uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, float, uint32_t) = nullptr;
+	const uint32_t vec4 = (a.layout == KMX_AOS && a.dim % 4 == 0 && a.stride % 4 == 0 && ((uintptr_t)a.data % 16) == 0) ? 1u : 0u;
+	if (a.layout == KMX_AOS) kernel = scalar ? assign_lds_fma_kernel<DP, KMX_AOS, true> : assign_lds_fma_kernel<DP, KMX_AOS, false>;
+	else kernel = scalar ? assign_lds_fma_kernel<DP, KMX_SOA, true> : assign_lds_fma_kernel<DP, KMX_SOA, false>;
 	int rc = profile_begin(0);
 	if (rc) return rc;
-	if (a.layout == KMX_AOS)
-		hipLaunchKernelGGL((assign_lds_fma_kernel<DP, KMX_AOS>), dim3(grid), dim3(FMA_WAVES * WAVE), lds_bytes, stream(),
-		                   a.data, a.stride, ws->packed_means, ws->norms, a.assignment, ws->queue, ws->counters, a.dim, a.k, kp, a.n, chunk_rows, kd);
-	else
-		hipLaunchKernelGGL((assign_lds_fma_kernel<DP, KMX_SOA>), dim3(grid), dim3(FMA_WAVES * WAVE), lds_bytes, stream(),
-		                   a.data, a.stride, ws->packed_means, ws->norms, a.assignment, ws->queue, ws->counters, a.dim, a.k, kp, a.n, chunk_rows, kd);
+	hipLaunchKernelGGL(kernel, dim3(grid), dim3(FMA_WAVES * WAVE), lds_bytes, stream(),
+	                   a.data, a.stride, ws->packed_means, ws->norms, a.assignment, ws->queue, ws->counters, a.dim, a.k, kp, a.n, chunk_rows, kd, vec4);
 	KMX_LAUNCH_CHECK("assign_lds_fma_kernel");
 	return profile_end(0);
 }

@@ -116,6 +116,7 @@ int launch_assign_mfma(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws
 bool bf16_supports(const AssignArgs& a, const DeviceInfo& dev);
 int launch_assign_bf16(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev);
 bool lds_fma_supports(const AssignArgs& a, const DeviceInfo& dev);
+bool lds_fma_reads_through_scalar_cache(const AssignArgs& a); /* a handful of centroids: no LDS staging */
 int launch_assign_lds_fma(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev);
 
 /* update.hip */

@@ -318,8 +318,10 @@ int kmx_assign_f32(int variant,
 		/* counterpart of BestCachedAssignmentKernel::run (reference kernels.cu:706-717): pick by shape.
 		 * Measured: the split-bf16 sweep is about twice as fast as the fp32 one wherever the sweep dominates; it hands
 		 * 2-3 times as many points to the exact pass, which costs more than it saves for very short rows and for
-		 * few centroids (HBM-bound shapes). The fp32 MFMA sweep beat the plain-VALU variant at every shape. */
-		if (bf16_supports(a, *dev) && dim >= 8 && k >= 64) variant = KMX_ASSIGN_MFMA_BF16X3;
+		 * few centroids (HBM-bound shapes). The fp32 MFMA sweep beat the plain-VALU variant at every shape except
+		 * a handful of centroids, where that variant reads them through the scalar cache. */
+		if (k <= 32 && lds_fma_supports(a, *dev) && lds_fma_reads_through_scalar_cache(a)) variant = KMX_ASSIGN_LDS_FMA;
+		else if (bf16_supports(a, *dev) && dim >= 8 && k >= 64) variant = KMX_ASSIGN_MFMA_BF16X3;
 		else if (mfma_supports(a, *dev)) variant = KMX_ASSIGN_MFMA;
 		else if (lds_fma_supports(a, *dev)) variant = KMX_ASSIGN_LDS_FMA;
 		else variant = KMX_ASSIGN_BASE;
