@@ -66,6 +66,50 @@ def cpu_baseline(km, spec, n_sample, data, means0):
     }
 
 
+def fused_main(km, args, spec, data, means0):
+    """--fused: the same protocol around HipFusedKMeansAlgorithm (mirror of CudaFusedKMeansAlgorithm, cuda.hpp:116-233)."""
+    n, dim, k = int(spec.n), spec.dim, spec.k
+    alg = km.HipFusedKMeansAlgorithm()
+    alg.initialize(dim, k, n, args.steps, data, means0)
+    alg.run(iters=args.warmup)
+    alg.cleanup()
+    alg.initialize(dim, k, n, args.steps, data, means0)
+    km.sync()
+    t0 = time.perf_counter()
+    alg.run(iters=args.steps)
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    assert int(alg.getClusterSizes().sum()) == n, "cluster counts do not sum to N"
+    km.set_profiling(True)
+    k_ms = 0.0
+    left_over = 0
+    for _ in range(args.steps):
+        alg.iteration()
+        k_ms += km.last_kernel_ms(0)
+        left_over += km.last_rechecked()
+    km.set_profiling(False)
+    k_ms /= args.steps
+    alg.cleanup()
+    one_pass = k <= 32 and dim <= 32
+    read_bytes = 4.0 * (n * dim + 2 * k * dim + k) if one_pass else 4.0 * (2 * n * dim + 2 * n + 2 * k * dim + k)
+    out = {
+        "metric": "ms per fused k-means iteration, benchmark configuration %d" % args.config,
+        "value": round(ms_per_step, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "benchmark configuration %d: N=%d d=%d k=%d, fused iteration (%s)"
+                               % (args.config, n, dim, k, "single pass over the points" if one_pass else "assignment + update behind one call"),
+                   "layout": "aos"},
+        "points_centroids_dims_per_s": round(float(n) * k * dim / (ms_per_step * 1e-3), 0),
+        "rechecked_points_per_iteration": round(left_over / args.steps, 1),
+    }
+    if one_pass:
+        gbs = read_bytes / (k_ms * 1e-3) / 1e9
+        out["roofline"] = {"kernel": "fused single-pass kernel", "bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS,
+                           "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None,
+                           "algorithmic_bytes": read_bytes, "avg_kernel_ms": round(k_ms, 4)}
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -75,6 +119,9 @@ def main():
     ap.add_argument("--cpu-sample", type=int, default=0, help="points in the CPU baseline sample (0 = about 12 s of work)")
     ap.add_argument("--assign-variant", default="best", choices=["base", "lds_fma", "mfma", "mfma_bf16x3", "best"])
     ap.add_argument("--update-variant", default="atomic_shm", choices=["atomic_point", "atomic_fine", "atomic_shm"])
+    ap.add_argument("--fused", action="store_true",
+                    help="time the fused iteration (kmx_fused_f32: one call per iteration, no assignment vector; a single "
+                         "pass over the points where k <= 32) instead of assignment + update")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--graph", action="store_true",
                     help="replay a recorded pair of iterations (HIP graph) instead of launching every kernel of the timed "
@@ -100,6 +147,8 @@ def main():
                       "best": km.ASSIGN_BEST}[args.assign_variant]
     update_variant = {"atomic_point": km.UPDATE_ATOMIC_POINT, "atomic_fine": km.UPDATE_ATOMIC_FINE,
                       "atomic_shm": km.UPDATE_ATOMIC_SHM}[args.update_variant]
+    if args.fused:
+        return fused_main(km, args, spec, data, means0)
     alg = km.HipKMeansAlgorithm(assign_variant, update_variant)
     alg.initialize(dim, k, n, args.steps, data, means0)
 

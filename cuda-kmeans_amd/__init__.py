@@ -21,7 +21,7 @@ HOST_LIB_PATH = os.path.join(_HERE, "host", "libkmx_host.so")
 
 AOS, SOA = 0, 1
 ASSIGN_BASE, ASSIGN_LDS_FMA, ASSIGN_MFMA, ASSIGN_BEST, ASSIGN_MFMA_BF16X3 = 0, 1, 2, 3, 4
-FUSED_TWO_PASS = 0
+FUSED_TWO_PASS, FUSED_ONE_PASS, FUSED_BEST = 0, 1, 2
 UPDATE_ATOMIC_POINT, UPDATE_ATOMIC_FINE, UPDATE_ATOMIC_SHM = 0, 1, 2
 
 KMX_OK, KMX_ERR_INVALID_ARGUMENT, KMX_ERR_UNSUPPORTED, KMX_ERR_DEVICE, KMX_ERR_NO_DEVICE = 0, 1, 2, 3, 4
@@ -452,7 +452,7 @@ class HipFusedKMeansAlgorithm:
     zero(means[next]) -> zero(sizes) -> fused(means[last] -> means[next]); getAssignment() is computed afterwards
     against the FINAL centroids (the reference does that on the host, cuda.hpp:199-221; here one more device pass)."""
 
-    def __init__(self, variant=FUSED_TWO_PASS, exec_params=None, layout=AOS, layout_means=AOS):
+    def __init__(self, variant=FUSED_BEST, exec_params=None, layout=AOS, layout_means=AOS):
         self.variant = variant
         self.exec = exec_params if exec_params is not None else ExecParams()
         self.layout, self.layout_means = layout, layout_means

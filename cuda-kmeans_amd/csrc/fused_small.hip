@@ -1,0 +1,331 @@
+/*
+ * One whole iteration in a single pass over the points, for a handful of centroids (k <= 32, rows up to 32
+ * floats): the shapes where the iteration is bound by HBM and reading the points twice (assignment, then
+ * update) costs the most. Role of the reference's fused kernels (kernels.cu:883-1190).
+ *
+ * One lane owns one point, its coordinates in registers.
+ *   1. Ranking a[j] = |c_j|^2 - 2 c_j.x with plain fused multiply-adds; the packed centroid rows are read with
+ *      wave-uniform addresses (scalar loads, scalar operands). The lane keeps the two smallest values with their
+ *      centroids and the third smallest value.
+ *   2. Exact result without a second kernel: if the runner-up is further than tau from the best, the best is the
+ *      serial result (same bound as the other fast variants, see assign_mfma.hip); if only the THIRD is further
+ *      than tau, the serial result is one of the two leaders, and the lane settles it with the serial arithmetic
+ *      on those two (every lane does that, no divergence: two exact distances cost a fifth of the scan). Only a
+ *      point with three or more centroids within tau, or with data the bound does not cover (NaN, overflow),
+ *      stays unresolved: it goes to the recheck queue and a fix-up kernel adds it to the sums afterwards.
+ *   3. Accumulation on the matrix cores: the sums of a wavefront's 64 points are the product of the k x 64 indicator
+ *      matrix (1 where the point belongs to the cluster) with the 64 x dim block of coordinates. The wavefront parks
+ *      its rows and results in LDS (that transposes them: the MFMA wants one lane per dimension) and issues
+ *      v_mfma_f32_16x16x4_f32 with the indicator as A and the coordinates as B; the accumulators stay in registers
+ *      for the whole kernel. 1.0 * x is exact, so only the summation order differs from the serial one. Rows of
+ *      unresolved points are parked as zeros (0 * NaN would poison every cluster). Counts are integer LDS atomics.
+ *      At the end the four wavefronts' accumulators meet in LDS: one global atomic per element and work-group.
+ *
+ * Floating-point contraction is off for the whole file (the serial arithmetic must not fuse); the ranking uses
+ * explicit fused multiply-adds.
+ */
+#include "assign_mfma_impl.h"
+
+#pragma clang fp contract(off)
+
+namespace kmx {
+
+constexpr uint32_t FUSED_WAVES = 4;
+constexpr uint32_t UNRESOLVED = 0xFFFFFFFFu;
+
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+
+template <int DP, int LD, int LM, int MT>
+__global__ void __launch_bounds__(FUSED_WAVES * WAVE)
+fused_small_kernel(const float* __restrict__ data, size_t stride, const float* __restrict__ packed, const float* __restrict__ norms,
+                   const float* __restrict__ means_in, size_t stride_means,
+                   float* __restrict__ means_out, uint32_t* __restrict__ sizes,
+                   uint32_t* __restrict__ queue, uint32_t* __restrict__ counters,
+                   uint32_t dim, uint32_t k, uint32_t n, float kd, uint32_t vec4)
+{
+	constexpr uint32_t RS = DP + ROW_PAD;
+	constexpr int NT = DP <= 16 ? 1 : 2;        /* tiles of 16 dimensions */
+	constexpr uint32_t PARK = NT * 16 + 1;      /* a parked row: coordinates padded with zeros to whole tiles, then the result */
+	constexpr uint32_t EX = DP + 1;             /* row stride of the exact centroid copy: odd, so that different rows start in different banks */
+	constexpr uint32_t SUM_ROWS = MT * 16, SUM_COLS = NT * 16;
+	extern __shared__ float lds[];
+	__shared__ uint32_t wave_max[FUSED_WAVES];
+	__shared__ uint32_t flag_list[FUSED_WAVES][2 * FLAG_CAP];
+	__shared__ uint32_t members[32];
+	const uint32_t lane = threadIdx.x & (WAVE - 1);
+	const uint32_t wave = threadIdx.x / WAVE;
+
+	/* LDS: [exact centroids k x EX][per wavefront: 64 parked rows, later its SUM_ROWS x SUM_COLS sums] */
+	constexpr uint32_t WAVE_FLOATS = WAVE * PARK > SUM_ROWS * SUM_COLS ? WAVE * PARK : SUM_ROWS * SUM_COLS;
+	float* exact = lds;
+	float* parked = exact + (size_t)k * EX + (size_t)wave * WAVE_FLOATS;
+	for (uint32_t i = threadIdx.x; i < k * EX; i += blockDim.x) {
+		const uint32_t j = i / EX, q = i - j * EX;
+		exact[i] = q < dim ? means_in[elem<LM>(stride_means, j, q)] : 0.0f;
+	}
+	for (uint32_t i = lane; i < WAVE * PARK; i += WAVE) parked[i] = 0.0f; /* the padding columns stay zero */
+	if (threadIdx.x < 32) members[threadIdx.x] = 0u;
+
+	uint32_t cmax = 0;
+	for (uint32_t j = threadIdx.x; j < k; j += blockDim.x) cmax = max(cmax, __float_as_uint(norms[norm_at(j)]));
+	for (int off = WAVE / 2; off > 0; off >>= 1) cmax = max(cmax, (uint32_t)__shfl_xor((int)cmax, off));
+	if (lane == 0) wave_max[wave] = cmax;
+	__syncthreads();
+	cmax = 0;
+	for (uint32_t w = 0; w < FUSED_WAVES; ++w) cmax = max(cmax, wave_max[w]);
+	const float c2max = __uint_as_float(cmax);
+
+	uint32_t flagged = 0; /* wave-uniform */
+	auto flush_flags = [&]() {
+		__builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+		__builtin_amdgcn_wave_barrier();
+		uint32_t slot = 0;
+		if (lane == 0) slot = atomicAdd(&counters[0], flagged);
+		slot = (uint32_t)__shfl((int)slot, 0);
+		for (uint32_t i = lane; i < 2 * flagged; i += WAVE) queue[2 * (size_t)slot + i] = flag_list[wave][i];
+		__builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+		__builtin_amdgcn_wave_barrier();
+		flagged = 0;
+	};
+
+	/* accumulators: MT x NT tiles of 16 clusters x 16 dimensions; this lane holds dimension lane % 16 of clusters
+	 * 4 * (lane / 16) + 0..3 of every tile */
+	f32x4v acc[MT][NT];
+#pragma unroll
+	for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+		for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = f32x4v{ 0.0f, 0.0f, 0.0f, 0.0f };
+	const uint32_t col = lane & 15, quad = lane >> 4;
+
+	const uint32_t batch_points = FUSED_WAVES * WAVE;
+	const uint32_t batches = (n + batch_points - 1) / batch_points;
+	for (uint32_t batch = blockIdx.x; batch < batches; batch += gridDim.x) {
+		const uint32_t pt = batch * batch_points + threadIdx.x;
+		const bool valid = pt < n;
+		float x[DP];
+		if (LD == KMX_AOS && vec4) {
+#pragma unroll
+			for (int q = 0; q < DP; q += 4) {
+				f32x4 v = { 0.0f, 0.0f, 0.0f, 0.0f };
+				if (valid && (uint32_t)q < dim) v = *(const f32x4*)(data + (size_t)pt * stride + q);
+				x[q] = v.x; x[q + 1] = v.y; x[q + 2] = v.z; x[q + 3] = v.w;
+			}
+		}
+		else {
+#pragma unroll
+			for (int q = 0; q < DP; ++q) x[q] = (valid && (uint32_t)q < dim) ? data[elem<LD>(stride, pt, q)] : 0.0f;
+		}
+		float x2 = 0.0f;
+#pragma unroll
+		for (int q = 0; q < DP; ++q) x2 = __builtin_fmaf(x[q], x[q], x2);
+
+		/* 1. ranking: two smallest values with their centroids, third smallest value */
+		float m1 = __builtin_inff(), m2 = __builtin_inff(), m3 = __builtin_inff();
+		uint32_t i1 = 0, i2 = 0;
+#pragma unroll 4
+		for (uint32_t r = 0; r < k; ++r) {
+			const float* row = packed + packed_row(r, RS); /* uniform address: scalar loads */
+			float a = norms[norm_at(r)];
+#pragma unroll
+			for (int q = 0; q < DP; ++q) a = __builtin_fmaf(row[q], x[q], a);
+			const bool lt1 = a < m1, lt2 = a < m2;
+			i2 = lt1 ? i1 : (lt2 ? r : i2);
+			i1 = lt1 ? r : i1;
+			m3 = __builtin_amdgcn_fmed3f(m2, m3, a); /* third smallest of {m1, m2, m3, a} as m1 <= m2 <= m3 */
+			m2 = __builtin_amdgcn_fmed3f(m1, m2, a);
+			m1 = lt1 ? a : m1;
+		}
+
+		/* 2. the serial arithmetic on the two leaders (rows of the exact copy in LDS, one row per lane) */
+		float d1, d2;
+		{
+			const float* c1 = exact + (size_t)i1 * EX;
+			const float* c2 = exact + (size_t)i2 * EX;
+			float s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+			for (int q = 0; q < DP; ++q) {
+				float e1 = x[q] - c1[q];
+				float e2 = x[q] - c2[q];
+				float q1 = e1 * e1;
+				float q2 = e2 * e2;
+				s1 = s1 + q1;
+				s2 = s2 + q2;
+			}
+			d1 = __builtin_sqrtf(s1);
+			d2 = __builtin_sqrtf(s2);
+		}
+		const float span = x2 + c2max;
+		const float tau = kd * span;
+		const bool covered = span > 1e-30f;
+		const bool decided = (m2 - m1 > tau) && covered;
+		const bool two = (m3 - m1 > tau) && covered;
+		const uint32_t of_two = (d2 < d1 || (d2 == d1 && i2 < i1)) ? i2 : i1;
+		uint32_t result = decided ? i1 : (two ? of_two : UNRESOLVED);
+		if (!valid) result = UNRESOLVED;
+
+		const bool flag = valid && result == UNRESOLVED;
+		const unsigned long long mask = __ballot(flag);
+		if (mask) {
+			const uint32_t add = (uint32_t)__builtin_popcountll(mask);
+			if (flagged + add > FLAG_CAP) flush_flags();
+			if (flag) {
+				const uint32_t at = 2 * (flagged + __builtin_popcountll(mask & ((1ull << lane) - 1ull)));
+				flag_list[wave][at] = pt;
+				flag_list[wave][at + 1] = screening_threshold(m1, tau);
+			}
+			flagged += add;
+		}
+
+		/* 3. park the rows (zeros for a point that is not accumulated here), then indicator x coordinates on the MFMA */
+		const bool counted = result != UNRESOLVED;
+		float* mine = parked + (size_t)lane * PARK;
+#pragma unroll
+		for (int q = 0; q < DP; ++q) mine[q] = counted ? x[q] : 0.0f;
+		mine[NT * 16] = __uint_as_float(result);
+		if (counted) atomicAdd(&members[result], 1u);
+		__builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+		__builtin_amdgcn_wave_barrier();
+#pragma unroll 4
+		for (uint32_t s = 0; s < WAVE / 4; ++s) {
+			/* this lane feeds point 4 s + quad: its membership of cluster col (A) and its coordinate col (B) */
+			const float* row = parked + (size_t)(4 * s + quad) * PARK;
+			const uint32_t t = __float_as_uint(row[NT * 16]);
+			float b[NT];
+#pragma unroll
+			for (int nt = 0; nt < NT; ++nt) b[nt] = row[nt * 16 + col];
+#pragma unroll
+			for (int mt = 0; mt < MT; ++mt) {
+				const float a = t == (uint32_t)(mt * 16) + col ? 1.0f : 0.0f;
+#pragma unroll
+				for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b[nt], acc[mt][nt], 0, 0, 0);
+			}
+		}
+		__builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+		__builtin_amdgcn_wave_barrier();
+	}
+	if (flagged) flush_flags();
+
+	/* the wavefront's sums to its LDS region (row = cluster, column = dimension), then one atomic per element */
+	__builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+	__builtin_amdgcn_wave_barrier();
+#pragma unroll
+	for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+		for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+			for (int r = 0; r < 4; ++r) parked[(size_t)(mt * 16 + 4 * quad + r) * SUM_COLS + nt * 16 + col] = acc[mt][nt][r];
+	__syncthreads();
+	const float* sums = exact + (size_t)k * EX;
+	for (uint32_t e = threadIdx.x; e < k * dim; e += blockDim.x) {
+		const uint32_t c = e / dim, d = e - c * dim;
+		float s = 0.0f;
+		for (uint32_t w = 0; w < FUSED_WAVES; ++w) s += sums[(size_t)w * WAVE_FLOATS + (size_t)c * SUM_COLS + d];
+		if (s != 0.0f) unsafeAtomicAdd(&means_out[elem<LM>(stride_means, c, d)], s);
+	}
+	if (threadIdx.x < k && members[threadIdx.x]) atomicAdd(&sizes[threadIdx.x], members[threadIdx.x]);
+}
+
+/* adds the points the exact pass has just resolved (the queue of the fused kernel) to the sums and counts: every
+ * work-group gathers its share in LDS first, so the few hundred result words see one global atomic per work-group */
+template <int LD, int LM>
+__global__ void __launch_bounds__(256)
+fused_fixup_kernel(const float* __restrict__ data, size_t stride, const uint32_t* __restrict__ assignment,
+                   float* __restrict__ means_out, size_t stride_means, uint32_t* __restrict__ sizes,
+                   const uint32_t* __restrict__ queue, const uint32_t* __restrict__ counters, uint32_t dim, uint32_t k)
+{
+	__shared__ float sums[32 * 32];
+	__shared__ uint32_t members[32];
+	const uint32_t count = counters[0];
+	if ((uint64_t)blockIdx.x * blockDim.x >= (uint64_t)count * dim) return; /* nothing for this work-group */
+	for (uint32_t i = threadIdx.x; i < k * dim; i += blockDim.x) sums[i] = 0.0f;
+	if (threadIdx.x < 32) members[threadIdx.x] = 0u;
+	__syncthreads();
+	const uint64_t total = (uint64_t)count * dim;
+	for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (uint64_t)gridDim.x * blockDim.x) {
+		const uint32_t entry = (uint32_t)(i / dim), d = (uint32_t)(i - (uint64_t)entry * dim);
+		const uint32_t pt = queue[2 * (size_t)entry];
+		const uint32_t t = assignment[pt];
+		unsafeAtomicAdd(&sums[t * dim + d], data[elem<LD>(stride, pt, d)]);
+		if (d == 0) atomicAdd(&members[t], 1u);
+	}
+	__syncthreads();
+	for (uint32_t e = threadIdx.x; e < k * dim; e += blockDim.x) {
+		const uint32_t c = e / dim, d = e - c * dim;
+		if (sums[e] != 0.0f) unsafeAtomicAdd(&means_out[elem<LM>(stride_means, c, d)], sums[e]);
+	}
+	if (threadIdx.x < k && members[threadIdx.x]) atomicAdd(&sizes[threadIdx.x], members[threadIdx.x]);
+}
+
+static uint32_t fused_dp(uint32_t dim)
+{
+	for (uint32_t o : { 4u, 8u, 16u, 24u, 32u })
+		if (dim <= o) return o;
+	return 0;
+}
+
+bool fused_small_supports(uint32_t dim, uint32_t k)
+{
+	return k <= 32 && fused_dp(dim) != 0;
+}
+
+template <int DP, int LD, int LM>
+static int launch_fused_t(const AssignArgs& a, float* means_out, uint32_t* sizes, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev, float kd)
+{
+	constexpr uint32_t NT = DP <= 16 ? 1 : 2;
+	const uint32_t mt = a.k <= 16 ? 1 : 2;
+	const uint32_t wave_floats = std::max<uint32_t>(WAVE * (NT * 16 + 1), mt * 16 * NT * 16);
+	const uint32_t lds_bytes = (a.k * (DP + 1) + FUSED_WAVES * wave_floats) * 4;
+	const uint32_t static_bytes = (2 * FLAG_CAP * FUSED_WAVES + 128) * 4;
+	if (lds_bytes + static_bytes > dev.lds_bytes) return fail(KMX_ERR_UNSUPPORTED, "fused iteration: %u bytes of LDS needed", lds_bytes + static_bytes);
+	void (*kernel)(const float*, size_t, const float*, const float*, const float*, size_t, float*, uint32_t*, uint32_t*, uint32_t*,
+	               uint32_t, uint32_t, uint32_t, float, uint32_t) = mt == 1 ? fused_small_kernel<DP, LD, LM, 1> : fused_small_kernel<DP, LD, LM, 2>;
+	const uint32_t batches = (a.n + FUSED_WAVES * WAVE - 1) / (FUSED_WAVES * WAVE);
+	const uint32_t per_cu = std::max<uint32_t>(1, std::min<uint32_t>(8, dev.lds_bytes / (lds_bytes + static_bytes)));
+	const uint32_t grid = std::min(batches, dev.compute_units * per_cu);
+	exec->block_count = grid;
+	const uint32_t vec4 = (a.layout == KMX_AOS && a.dim % 4 == 0 && a.stride % 4 == 0 && ((uintptr_t)a.data % 16) == 0) ? 1u : 0u;
+	int rc = profile_begin(0);
+	if (rc) return rc;
+	hipLaunchKernelGGL(kernel, dim3(grid), dim3(FUSED_WAVES * WAVE), lds_bytes, stream(),
+	                   a.data, a.stride, ws->packed_means, ws->norms, a.means, a.stride_means, means_out, sizes,
+	                   ws->queue, ws->counters, a.dim, a.k, a.n, kd, vec4);
+	KMX_LAUNCH_CHECK("fused_small_kernel");
+	return profile_end(0);
+}
+
+template <int LD, int LM>
+static int launch_fused_layouts(const AssignArgs& a, float* means_out, uint32_t* sizes, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev)
+{
+	const uint32_t dp = fused_dp(a.dim);
+	const uint32_t kp = round_up(a.k, TILE);
+	int rc = launch_pack_means(a, ws, dp, kp);
+	if (rc) return rc;
+	const float kd = (8.0f * (float)a.dim + 24.0f) * 1.1920929e-07f; /* the bound of the fp32 ranking, see assign_mfma.hip */
+	switch (dp) {
+	case 4: rc = launch_fused_t<4, LD, LM>(a, means_out, sizes, exec, ws, dev, kd); break;
+	case 8: rc = launch_fused_t<8, LD, LM>(a, means_out, sizes, exec, ws, dev, kd); break;
+	case 16: rc = launch_fused_t<16, LD, LM>(a, means_out, sizes, exec, ws, dev, kd); break;
+	case 24: rc = launch_fused_t<24, LD, LM>(a, means_out, sizes, exec, ws, dev, kd); break;
+	case 32: rc = launch_fused_t<32, LD, LM>(a, means_out, sizes, exec, ws, dev, kd); break;
+	default: return fail(KMX_ERR_UNSUPPORTED, "fused iteration: dim %u is not supported by the single-pass kernel", a.dim);
+	}
+	if (rc) return rc;
+	/* the unresolved points: exact pass into the work-space assignment vector, then their share of the sums */
+	rc = launch_recheck(a, ws, kp);
+	if (rc) return rc;
+	hipLaunchKernelGGL((fused_fixup_kernel<LD, LM>), dim3(64), dim3(256), 0, stream(),
+	                   a.data, a.stride, a.assignment, means_out, a.stride_means, sizes, ws->queue, ws->counters, a.dim, a.k);
+	KMX_LAUNCH_CHECK("fused_fixup_kernel");
+	return KMX_OK;
+}
+
+/* a.assignment must be the work-space vector of n entries; means_out and sizes are zero on entry; the caller divides */
+int launch_fused_small(const AssignArgs& a, float* means_out, uint32_t* sizes, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev)
+{
+	if (a.layout == KMX_AOS && a.layout_means == KMX_AOS) return launch_fused_layouts<KMX_AOS, KMX_AOS>(a, means_out, sizes, exec, ws, dev);
+	if (a.layout == KMX_AOS && a.layout_means == KMX_SOA) return launch_fused_layouts<KMX_AOS, KMX_SOA>(a, means_out, sizes, exec, ws, dev);
+	if (a.layout == KMX_SOA && a.layout_means == KMX_AOS) return launch_fused_layouts<KMX_SOA, KMX_AOS>(a, means_out, sizes, exec, ws, dev);
+	return launch_fused_layouts<KMX_SOA, KMX_SOA>(a, means_out, sizes, exec, ws, dev);
+}
+
+} // namespace kmx

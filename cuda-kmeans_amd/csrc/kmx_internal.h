@@ -121,6 +121,13 @@ int launch_assign_lds_fma(const AssignArgs& a, kmx_exec_params* exec, Workspace*
 
 /* update.hip */
 int launch_update(int variant, const UpdateArgs& u, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev);
+int launch_divide_means(const UpdateArgs& u);
+
+/* fused_small.hip: one pass over the points for a handful of centroids. a.assignment is a scratch vector of n entries
+ * (only the entries of the points left to the exact pass are written); means_out and sizes are zero on entry and hold
+ * sums and counts on return (the caller divides). */
+bool fused_small_supports(uint32_t dim, uint32_t k);
+int launch_fused_small(const AssignArgs& a, float* means_out, uint32_t* sizes, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev);
 
 } // namespace kmx
 

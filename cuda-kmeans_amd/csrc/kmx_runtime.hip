@@ -446,7 +446,7 @@ int kmx_fused_f32(int variant,
 {
 	clear_error();
 	if (!exec) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_fused_f32: exec is null");
-	if (variant != KMX_FUSED_TWO_PASS) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_fused_f32: unknown variant %d", variant);
+	if (variant < KMX_FUSED_TWO_PASS || variant > KMX_FUSED_BEST) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_fused_f32: unknown variant %d", variant);
 	if (!means_in || !means_out || !cluster_sizes) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_fused_f32: null device pointer");
 	if (means_in == means_out) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_fused_f32: means_in and means_out must differ");
 	Workspace* ws = nullptr;
@@ -454,6 +454,26 @@ int kmx_fused_f32(int variant,
 	if (rc) return rc;
 	rc = reserve_fused_assignment(ws, n);
 	if (rc) return rc;
+
+	const bool one_pass_fits = fused_small_supports(dim, k);
+	if (variant == KMX_FUSED_ONE_PASS && !one_pass_fits)
+		return fail(KMX_ERR_UNSUPPORTED, "kmx_fused_f32: shape dim=%u k=%u is not supported by the single-pass kernel", dim, k);
+	if (variant != KMX_FUSED_TWO_PASS && one_pass_fits && n > 0) {
+		if (dim == 0 || k == 0) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_fused_f32: dim and k must be positive");
+		if (!data) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_fused_f32: null device pointer");
+		rc = check_layout("kmx_fused_f32", "data", layout, stride, n, dim);
+		if (rc) return rc;
+		rc = check_layout("kmx_fused_f32", "means", layout_means, stride_means, k, dim);
+		if (rc) return rc;
+		const DeviceInfo* dev = nullptr;
+		rc = device_info(&dev);
+		if (rc) return rc;
+		AssignArgs a{ data, layout, stride, means_in, layout_means, stride_means, ws->fused_assignment, dim, k, n };
+		rc = launch_fused_small(a, means_out, cluster_sizes, exec, ws, *dev);
+		if (rc) return rc;
+		UpdateArgs u{ data, layout, stride, ws->fused_assignment, means_out, layout_means, stride_means, cluster_sizes, dim, k, n };
+		return launch_divide_means(u);
+	}
 	/* argument checks of the two halves apply unchanged (their messages name the half that objects) */
 	rc = kmx_assign_f32(KMX_ASSIGN_BEST, data, layout, stride, means_in, layout_means, stride_means, nullptr, ws->fused_assignment, dim, k, n, exec);
 	if (rc) return rc;

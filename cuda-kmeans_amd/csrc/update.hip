@@ -701,6 +701,19 @@ static int launch_update_t(int variant, const UpdateArgs& u, kmx_exec_params* ex
 	return KMX_OK;
 }
 
+/* means[c][d] /= count[c] for the non-empty clusters (divideMeansKernel of the reference, kernels.cu:149-171) */
+int launch_divide_means(const UpdateArgs& u)
+{
+	const uint32_t total = u.k * u.dim;
+	const uint32_t blocks = std::min<uint32_t>((total + 255) / 256, 1024);
+	if (u.layout_means == KMX_AOS)
+		hipLaunchKernelGGL((divide_means_kernel<KMX_AOS>), dim3(blocks), dim3(256), 0, stream(), u.means, u.stride_means, u.cluster_sizes, u.dim, u.k);
+	else
+		hipLaunchKernelGGL((divide_means_kernel<KMX_SOA>), dim3(blocks), dim3(256), 0, stream(), u.means, u.stride_means, u.cluster_sizes, u.dim, u.k);
+	KMX_LAUNCH_CHECK("divide_means_kernel");
+	return KMX_OK;
+}
+
 int launch_update(int variant, const UpdateArgs& u, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev)
 {
 	if (u.layout == KMX_AOS && u.layout_means == KMX_AOS) return launch_update_t<KMX_AOS, KMX_AOS>(variant, u, exec, ws, dev);

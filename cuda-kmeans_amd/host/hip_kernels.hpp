@@ -147,12 +147,17 @@ KMX_DEFINE_ASSIGNMENT_KERNEL(MfmaBf16AssignmentKernel, KMX_ASSIGN_MFMA_BF16X3) /
 KMX_DEFINE_ASSIGNMENT_KERNEL(BestCachedAssignmentKernel, KMX_ASSIGN_BEST) /* kernels.cu:706-717 */
 
 /* role of FusedCachedFixedKernel / FusedCachedRegsKernel (kernels.cu:883-1190): one call per iteration, no assignment buffer */
-template<typename F, typename IDX_T, class LAYOUT, class LAYOUT_MEANS, class METRIC>
-class FusedTwoPassKernel {
-public:
-	static void run(const FusedProblemInstance<F, IDX_T>& in, HipExecParameters& exec)
-	{ hip_detail::fused<F, IDX_T, LAYOUT, LAYOUT_MEANS>(KMX_FUSED_TWO_PASS, in, exec); }
+#define KMX_DEFINE_FUSED_KERNEL(NAME, VARIANT)\
+template<typename F, typename IDX_T, class LAYOUT, class LAYOUT_MEANS, class METRIC>\
+class NAME {\
+public:\
+	static void run(const FusedProblemInstance<F, IDX_T>& in, HipExecParameters& exec)\
+	{ hip_detail::fused<F, IDX_T, LAYOUT, LAYOUT_MEANS>(VARIANT, in, exec); }\
 };
+
+KMX_DEFINE_FUSED_KERNEL(FusedTwoPassKernel, KMX_FUSED_TWO_PASS) /* assignment sweep + update behind one call, any shape */
+KMX_DEFINE_FUSED_KERNEL(FusedOnePassKernel, KMX_FUSED_ONE_PASS) /* one kernel, a handful of centroids */
+KMX_DEFINE_FUSED_KERNEL(FusedBestKernel, KMX_FUSED_BEST)        /* one pass where it applies */
 
 #define KMX_DEFINE_UPDATE_KERNEL(NAME, VARIANT)\
 template<typename F, typename IDX_T, class LAYOUT, class LAYOUT_MEANS, int EMUL = false>\

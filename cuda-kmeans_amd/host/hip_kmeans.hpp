@@ -229,7 +229,7 @@ public:
  */
 template<typename F = float, typename IDX_T = std::uint32_t, class LAYOUT = AoSLayoutPolicy<>,
 	class LAYOUT_MEANS = LAYOUT, class METRIC = EuclideanMetricPolicy<F, LAYOUT, LAYOUT_MEANS>,
-	class KERNEL = FusedTwoPassKernel<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC>>
+	class KERNEL = FusedBestKernel<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC>>
 class HipFusedKMeansAlgorithm : public IKMeansAlgorithm<F, IDX_T>
 {
 	HipExecParameters mExecParams;

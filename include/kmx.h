@@ -159,8 +159,11 @@ int kmx_bucket_sum_f32(int variant,
  * are zero. The assignment lives in the library's work space (n words, grown on demand).
  */
 typedef enum kmx_fused_variant {
-	KMX_FUSED_TWO_PASS = 0 /* selector-chosen assignment sweep into the work space, then the tuned update (the points are
-	                          read twice; the reference's FusedCachedFixed / FusedCachedRegs read them once) */
+	KMX_FUSED_TWO_PASS = 0, /* selector-chosen assignment sweep into the work space, then the tuned update (any shape; the
+	                           points are read twice) */
+	KMX_FUSED_ONE_PASS = 1, /* a single kernel reads every point once, assigns it and accumulates it (k <= 32, dim <= 32:
+	                           the shapes bound by HBM; role of FusedCachedFixed / FusedCachedRegs) */
+	KMX_FUSED_BEST = 2      /* ONE_PASS where it applies, else TWO_PASS */
 } kmx_fused_variant;
 
 int kmx_fused_f32(int variant,

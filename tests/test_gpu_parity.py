@@ -273,7 +273,7 @@ def test_fused_iterations_match_oracle(km, orc, gpu, cid, n, iters, layout, layo
     dim, k = spec.dim, spec.k
     data = km.generate_points(spec, n, layout=layout)
     means0 = km.first_k_means(spec, layout_means)
-    alg = km.HipFusedKMeansAlgorithm(layout=layout, layout_means=layout_means)
+    alg = km.HipFusedKMeansAlgorithm(layout=layout, layout_means=layout_means)   # one pass for configuration 5, two otherwise
     alg.initialize(dim, k, n, iters, data, means0)
     for _ in range(iters):
         prev = alg.getMeans()
@@ -359,6 +359,86 @@ def test_full_size_properties(km, orc, gpu, cid):
 
 
 # ---------------------------------------------------------------- recorded iterations (HIP graph)
+
+def fused_step(km, variant, data, means, dim, k, n, layout=AOS, layout_means=AOS):
+    d = km.DeviceBuffer(data.nbytes); d.write(data)
+    mi = km.DeviceBuffer(means.nbytes); mi.write(means)
+    mo = km.DeviceBuffer(means.nbytes); mo.zero()
+    s = km.DeviceBuffer(4 * k); s.zero()
+    km.fused(variant, d, layout, km.layout_stride(layout, n, dim), mi, mo, layout_means, km.layout_stride(layout_means, k, dim),
+             s, dim, k, n)
+    km.sync()
+    out = mo.read(np.float32, means.size), s.read(np.uint32, k)
+    for b in (d, mi, mo, s):
+        b.free()
+    return out
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dim,k,n", [(16, 16, 100000), (3, 5, 257), (2, 2, 128), (8, 32, 5000), (20, 7, 3333), (32, 32, 4099),
+                                     (1, 3, 300), (31, 9, 1000)])
+@pytest.mark.parametrize("layout,layout_means", [(AOS, AOS), (SOA, SOA), (AOS, SOA), (SOA, AOS)])
+def test_single_pass_fused_kernel(km, orc, gpu, dim, k, n, layout, layout_means):
+    """KMX_FUSED_ONE_PASS: counts exactly those of the serial assignment, centroids within tolerance; the variants agree."""
+    rng = np.random.default_rng(dim * 131 + k)
+    centres = rng.normal(size=(k, dim)).astype(np.float32) * np.float32(2)
+    pts = (centres[rng.integers(0, k, size=n)] + rng.normal(size=(n, dim)).astype(np.float32)).astype(np.float32)
+    pts[: k] = centres                                   # points exactly on centroids
+    means = centres.copy()
+    if k > 2:
+        means[k - 1] = means[0]                              # a duplicated centroid: exact ties, lowest index must win
+    data = np.ascontiguousarray(pts if layout == AOS else pts.T).ravel()
+    mflat = np.ascontiguousarray(means if layout_means == AOS else means.T).ravel()
+    oa = orc.assign(data, mflat, dim, k, n, layout, layout_means, threads=0, fast=True)
+    om, osz = orc.update(data, oa, dim, k, n, layout, layout_means, threads=0)
+    for variant in (km.FUSED_ONE_PASS, km.FUSED_BEST, km.FUSED_TWO_PASS):
+        gm, gs = fused_step(km, variant, data, mflat, dim, k, n, layout, layout_means)
+        assert np.array_equal(gs, osz), "variant %d" % variant
+        assert rel_err(gm, om) < CENTROID_RTOL, "variant %d" % variant
+
+
+@pytest.mark.gpu
+def test_single_pass_fused_kernel_hard_inputs(km, orc, gpu):
+    """Near-ties of three centroids, coincident points, NaN / inf / huge / tiny values go through the exact pass and the
+    fix-up kernel; a shape the single-pass kernel does not take is refused by name."""
+    dim, k, n = 8, 16, 4096
+    rng = np.random.default_rng(77)
+    base = rng.normal(size=(n, dim)).astype(np.float32)
+    means = rng.normal(size=(k, dim)).astype(np.float32)
+    cases = {}
+    m = means.copy(); m[5] = m[3]; m[9] = m[3]
+    cases["three_equal_centroids"] = (base, m)
+    cases["all_centroids_identical"] = (base, np.repeat(means[:1], k, 0))
+    cases["all_points_identical"] = (np.repeat(base[:1], n, 0), means)
+    cases["grid_ties"] = (np.round(base * 2) / 2, np.round(means * 2) / 2)
+    cases["huge"] = (base * np.float32(1e18), means * np.float32(1e18))
+    cases["tiny"] = (base * np.float32(1e-25), means * np.float32(1e-25))
+    m = means.copy(); m[4, 1] = np.nan
+    cases["nan_centroid"] = (base, m)
+    m = means.copy(); m[0, 0] = np.nan
+    cases["nan_centroid_zero"] = (base, m)
+    d = base.copy(); d[5, 0] = np.nan; d[9, dim - 1] = np.inf
+    cases["nan_inf_points"] = (d, means)
+    for name, (d, m) in cases.items():
+        d = np.ascontiguousarray(d, dtype=np.float32).ravel()
+        m = np.ascontiguousarray(m, dtype=np.float32).ravel()
+        oa = orc.assign(d, m, dim, k, n, threads=0, fast=True)
+        om, osz = orc.update(d, oa, dim, k, n, threads=0)
+        gm, gs = fused_step(km, km.FUSED_ONE_PASS, d, m, dim, k, n)
+        assert np.array_equal(gs, osz), name
+        finite = np.isfinite(om)
+        assert np.array_equal(np.isfinite(gm), finite), name
+        # values against float64 means of the same assignment: the serial fp32 sum of thousands of equal rows (one
+        # of the cases) carries more rounding error than the tolerance, the tree-shaped device sum does not
+        sums = np.zeros((k, dim)); np.add.at(sums, oa, d.reshape(n, dim).astype(np.float64))
+        with np.errstate(invalid="ignore", divide="ignore"):
+            ref = np.where(osz[:, None] > 0, sums / np.maximum(osz, 1)[:, None], 0.0).ravel()
+        if finite.any():
+            scale = max(float(np.sqrt(np.mean(ref[finite] ** 2))), 1e-30)
+            assert float(np.abs(gm[finite] - ref[finite]).max()) / scale < CENTROID_RTOL, name
+    with pytest.raises(km.KmxError, match="single-pass"):
+        fused_step(km, km.FUSED_ONE_PASS, np.zeros(64 * 40, np.float32), np.zeros(40 * 40, np.float32), 40, 40, 64)
+
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("cid,n", [(2, 65536), (1, 65536), (5, 1 << 18)])
