@@ -13,7 +13,7 @@
  * Floating-point contraction is switched off for the whole file: a fused multiply-add here
  * would change low-order bits and with them the tie-breaks.
  */
-#include "kmx_internal.h"
+#include "assign_mfma_impl.h"
 
 #pragma clang fp contract(off)
 
@@ -302,6 +302,220 @@ recheck_reg_kernel(const float* __restrict__ data, size_t stride, const float* _
 	}
 }
 
+/*
+ * Exact pass with one lane per CENTROID and the queued points as scalar operands, for rows that fit the registers.
+ * A work-group of up to 16 wavefronts holds a chunk of up to 1024 centroids, one exact row per lane (read from the
+ * transposed exact copy, coalesced), and walks a batch of queue entries: the point of an entry is the same for
+ * every lane, so its coordinates and its threshold arrive as scalar loads (one cache fill serves all wavefronts)
+ * and feed the multiply-adds directly. A lane whose ranking value does not exceed the threshold evaluates the
+ * serial arithmetic for its centroid. The per-point minimum over all lanes and chunks is a 64-bit LDS atomic over
+ * (distance bits << 32 | centroid): for non-negative distances the bit pattern orders like the value, equal
+ * distances resolve to the smaller index, a NaN never beats a number, and key 0 encodes "NaN distance to
+ * centroid 0", which pins the point there as the serial scan does. The sweep's best centroid always passes the
+ * screen, so every point gets a key (a point without one -- only NaN coordinates do that -- goes to centroid 0).
+ * The batch size adapts to the queue length so that a short queue still spreads over the whole chip.
+ */
+/*
+ * The points of a batch are scattered rows of the input, and a scalar load that misses all the way to HBM stalls its
+ * wavefront for thousands of cycles, with nothing else in flight. Two measures keep those misses off the critical
+ * path: while a batch is worked on, the lanes touch the rows of the batch this work-group takes next with ordinary
+ * vector loads (one per 64 bytes of a row), which brings them into the L2; and every wavefront walks the points of
+ * a batch from a different starting point, so that the first access to each row is spread over the wavefronts
+ * instead of all of them waiting for the same row at the same time.
+ */
+template <int LD>
+static __device__ __forceinline__ float touch_rows(const float* __restrict__ data, size_t stride, uint32_t dim,
+                                                   const uint32_t* __restrict__ queue, uint32_t first, uint32_t points)
+{
+	const uint32_t parts = (dim + 15) / 16;
+	float touched = 0.0f;
+	for (uint32_t t = threadIdx.x; t < points * parts; t += blockDim.x)
+		touched += data[elem<LD>(stride, queue[2 * (size_t)(first + t / parts)], (t % parts) * 16)];
+	return touched;
+}
+
+constexpr uint32_t HIT_CAP = 1024;
+
+template <int LD>
+static __device__ __forceinline__ void evaluate_pair(const float* __restrict__ data, size_t stride, const float* __restrict__ means_t,
+                                                      uint32_t dim, uint32_t kp, uint32_t pt, uint32_t r, unsigned long long* key_slot)
+{
+	float sum = 0.0f;
+#pragma unroll 16
+	for (uint32_t q = 0; q < dim; ++q) {
+		float diff = data[elem<LD>(stride, pt, q)] - means_t[(size_t)q * kp + r];
+		float sq = diff * diff;
+		sum = sum + sq;
+	}
+	const float dist = __builtin_sqrtf(sum);
+	const unsigned long long key = (r == 0 && dist != dist) ? 0ull : (((unsigned long long)__float_as_uint(dist) << 32) | r);
+	atomicMin(key_slot, key);
+}
+
+constexpr uint32_t POINTS_BATCH = 64;
+
+template <int LD, int DPAD, bool FULL> /* FULL: dim == DPAD, no guards on the coordinate loads */
+__global__ void __launch_bounds__(1024)
+recheck_points_kernel(const float* __restrict__ data, size_t stride, const float* __restrict__ means_t, const float* __restrict__ norms,
+                      uint32_t* __restrict__ assignment, uint32_t dim, uint32_t k, uint32_t kp,
+                      const uint32_t* __restrict__ queue, const uint32_t* __restrict__ counters)
+{
+	__shared__ unsigned long long best_key[POINTS_BATCH];
+	__shared__ uint32_t hit_point[DPAD >= 16 ? HIT_CAP : 1], hit_centroid[DPAD >= 16 ? HIT_CAP : 1];
+	__shared__ uint32_t hit_count;
+	/* the wavefront number through readfirstlane: the compiler then knows that what depends on it is uniform */
+	const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE), waves = blockDim.x / WAVE;
+	const uint32_t count = counters[0];
+	const uint32_t slots = gridDim.x;
+	const uint32_t pb = count > slots * 32 ? 64 : count > slots * 16 ? 32 : 16;
+	const uint32_t batches = (count + pb - 1) / pb;
+
+	for (uint32_t batch = blockIdx.x; batch < batches; batch += gridDim.x) {
+		__syncthreads(); /* the previous batch has been written out */
+		if (threadIdx.x < POINTS_BATCH) best_key[threadIdx.x] = ~0ull;
+		if (threadIdx.x == 0) hit_count = 0;
+		__syncthreads();
+		const uint32_t first = batch * pb, here = min(pb, count - first);
+		const uint32_t next = (batch + gridDim.x) * pb;
+		const float touched = next < count ? touch_rows<LD>(data, stride, dim, queue, next, min(pb, count - next)) : 0.0f;
+		const uint32_t start = wave * here / waves;
+		for (uint32_t base = 0; base < k; base += blockDim.x) {
+			const uint32_t r = base + threadIdx.x, rr = min(r, k - 1); /* lanes past the end load a valid row, unconditionally, and never pass the screen */
+			float c[DPAD];
+#pragma unroll
+			for (int q = 0; q < DPAD; ++q) c[q] = (FULL || (uint32_t)q < dim) ? means_t[(size_t)q * kp + rr] : 0.0f;
+			const float c2 = r < k ? norms[norm_at(r)] : __builtin_inff();
+#pragma unroll 2
+			for (uint32_t step = 0; step < here; ++step) {
+				const uint32_t i = DPAD < 16 ? step : (start + step < here ? start + step : start + step - here); /* short rows: not worth the arithmetic */
+				const uint32_t pt = queue[2 * (size_t)(first + i)]; /* uniform: scalar loads */
+				const float thr = __uint_as_float(queue[2 * (size_t)(first + i) + 1]);
+				float x[DPAD];
+#pragma unroll
+				for (int q = 0; q < DPAD; ++q) x[q] = (FULL || (uint32_t)q < dim) ? data[elem<LD>(stride, pt, q)] : 0.0f;
+				float dot = 0.0f;
+#pragma unroll
+				for (int q = 0; q < DPAD; ++q) dot = __builtin_fmaf(x[q], c[q], dot);
+				if (r < k && !(__builtin_fmaf(-2.0f, dot, c2) > thr)) {
+					if constexpr (DPAD >= 16) { /* noted, and evaluated below by one lane per pair */
+						const uint32_t slot = atomicAdd(&hit_count, 1u);
+						if (slot < HIT_CAP) { hit_point[slot] = i; hit_centroid[slot] = r; }
+						else evaluate_pair<LD>(data, stride, means_t, dim, kp, pt, r, &best_key[i]);
+					} else { /* a short row is evaluated on the spot from the registers */
+						float sum = 0.0f;
+#pragma unroll
+						for (int q = 0; q < DPAD; ++q) { /* padding: (0-0)^2 = +0 leaves the sum unchanged */
+							float diff = x[q] - c[q];
+							float sq = diff * diff;
+							sum = sum + sq;
+						}
+						const float dist = __builtin_sqrtf(sum);
+						const unsigned long long key = (r == 0 && dist != dist) ? 0ull : (((unsigned long long)__float_as_uint(dist) << 32) | r);
+						atomicMin(&best_key[i], key);
+					}
+				}
+			}
+		}
+		asm volatile("" :: "v"(touched)); /* the touching loads are not dead code */
+		__syncthreads();
+		if constexpr (DPAD >= 16) {
+			const uint32_t noted = min(hit_count, HIT_CAP);
+			for (uint32_t t = threadIdx.x; t < noted; t += blockDim.x) {
+				const uint32_t i = hit_point[t];
+				evaluate_pair<LD>(data, stride, means_t, dim, kp, queue[2 * (size_t)(first + i)], hit_centroid[t], &best_key[i]);
+			}
+			__syncthreads();
+		}
+		if (threadIdx.x < here) {
+			const unsigned long long key = best_key[threadIdx.x];
+			assignment[queue[2 * (size_t)(first + threadIdx.x)]] = key == ~0ull ? 0u : (uint32_t)key;
+		}
+	}
+}
+
+/*
+ * The same scheme for rows too long for the registers: the dimensions go by in slices of 32. A lane keeps the
+ * running dot products of its centroid with the 16 points of the batch, loads one slice of its centroid and
+ * applies it to the 16 points in turn (their slices are scalar loads). Centroids that pass the screen of a point
+ * are noted in an LDS list, and when all centroids are through, one lane per noted (point, centroid) pair evaluates
+ * the serial arithmetic from memory: evaluating on the spot would leave 63 lanes of the wavefront waiting for
+ * every pair. Pairs beyond the list's capacity (many coincident centroids) are evaluated on the spot.
+ */
+constexpr int SLICE = 32;
+constexpr int SLICED_BATCH = 16;
+
+template <int LD, bool FULL> /* FULL: dim is a multiple of the slice, no guards on the coordinate loads */
+__global__ void __launch_bounds__(1024)
+recheck_sliced_kernel(const float* __restrict__ data, size_t stride, const float* __restrict__ means_t, const float* __restrict__ norms,
+                      uint32_t* __restrict__ assignment, uint32_t dim, uint32_t k, uint32_t kp,
+                      const uint32_t* __restrict__ queue, const uint32_t* __restrict__ counters)
+{
+	__shared__ unsigned long long best_key[SLICED_BATCH];
+	__shared__ uint32_t hit_point[HIT_CAP], hit_centroid[HIT_CAP];
+	__shared__ uint32_t hit_count;
+	const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+	const uint32_t count = counters[0];
+	const uint32_t batches = (count + SLICED_BATCH - 1) / SLICED_BATCH;
+
+	for (uint32_t batch = blockIdx.x; batch < batches; batch += gridDim.x) {
+		__syncthreads(); /* the previous batch has been written out */
+		if (threadIdx.x < SLICED_BATCH) best_key[threadIdx.x] = ~0ull;
+		if (threadIdx.x == 0) hit_count = 0;
+		__syncthreads();
+		const uint32_t first = batch * SLICED_BATCH, here = min((uint32_t)SLICED_BATCH, count - first);
+		const uint32_t next = (batch + gridDim.x) * SLICED_BATCH;
+		const float touched = next < count ? touch_rows<LD>(data, stride, dim, queue, next, min((uint32_t)SLICED_BATCH, count - next)) : 0.0f;
+		/* register i of this wavefront belongs to point at(i) of the batch: another rotation in every wavefront */
+		auto at = [&](int i) { return min((uint32_t)(i + wave) % SLICED_BATCH, here - 1); };
+		for (uint32_t base = 0; base < k; base += blockDim.x) {
+			const uint32_t r = base + threadIdx.x, rr = min(r, k - 1); /* lanes past the end load a valid row, unconditionally, and never pass the screen */
+			float dots[SLICED_BATCH];
+#pragma unroll
+			for (int i = 0; i < SLICED_BATCH; ++i) dots[i] = 0.0f;
+			for (uint32_t q0 = 0; q0 < dim; q0 += SLICE) {
+				float c[SLICE];
+#pragma unroll
+				for (int j = 0; j < SLICE; ++j) c[j] = (FULL || q0 + j < dim) ? means_t[(size_t)(q0 + j) * kp + rr] : 0.0f;
+#pragma unroll
+				for (int i = 0; i < SLICED_BATCH; ++i) {
+					const uint32_t pt = queue[2 * (size_t)(first + at(i))]; /* uniform: scalar loads */
+					float x[SLICE];
+#pragma unroll
+					for (int j = 0; j < SLICE; ++j) x[j] = (FULL || q0 + j < dim) ? data[elem<LD>(stride, pt, q0 + j)] : 0.0f;
+#pragma unroll
+					for (int j = 0; j < SLICE; ++j) dots[i] = __builtin_fmaf(x[j], c[j], dots[i]);
+				}
+			}
+			const float c2 = r < k ? norms[norm_at(r)] : __builtin_inff();
+#pragma unroll
+			for (int i = 0; i < SLICED_BATCH; ++i) {
+				const uint32_t point = at(i);
+				const size_t entry = 2 * (size_t)(first + point);
+				const float thr = __uint_as_float(queue[entry + 1]);
+				/* a batch that is not full has several registers on its last point: the first of them speaks for it */
+				const bool mine = (uint32_t)(i + wave) % SLICED_BATCH == point;
+				if (mine && r < k && !(__builtin_fmaf(-2.0f, dots[i], c2) > thr)) {
+					const uint32_t slot = atomicAdd(&hit_count, 1u);
+					if (slot < HIT_CAP) { hit_point[slot] = point; hit_centroid[slot] = r; }
+					else evaluate_pair<LD>(data, stride, means_t, dim, kp, queue[entry], r, &best_key[point]);
+				}
+			}
+		}
+		asm volatile("" :: "v"(touched)); /* the touching loads are not dead code */
+		__syncthreads();
+		const uint32_t noted = min(hit_count, HIT_CAP);
+		for (uint32_t t = threadIdx.x; t < noted; t += blockDim.x) {
+			const uint32_t i = hit_point[t];
+			evaluate_pair<LD>(data, stride, means_t, dim, kp, queue[2 * (size_t)(first + i)], hit_centroid[t], &best_key[i]);
+		}
+		__syncthreads();
+		if (threadIdx.x < here) {
+			const unsigned long long key = best_key[threadIdx.x];
+			assignment[queue[2 * (size_t)(first + threadIdx.x)]] = key == ~0ull ? 0u : (uint32_t)key;
+		}
+	}
+}
+
 template <int LD, int LM>
 static int launch_base_t(const AssignArgs& a, kmx_exec_params* exec, uint32_t* counters)
 {
@@ -359,9 +573,61 @@ static int launch_recheck_dpad(const AssignArgs& a, Workspace* ws, uint32_t kp)
 	return launch_recheck_reg<LD, L, 2, 64>(a, ws, kp);
 }
 
+template <int LD, int DPAD>
+static int launch_recheck_points(const AssignArgs& a, Workspace* ws, uint32_t kp)
+{
+	const uint32_t threads = std::min<uint32_t>(1024, round_up(a.k, WAVE));
+	const dim3 grid(DPAD <= 32 ? 512 : 256); /* two work-groups fit a compute unit while a row takes at most 32 registers */
+	if (a.dim == DPAD)
+		hipLaunchKernelGGL((recheck_points_kernel<LD, DPAD, true>), grid, dim3(threads), 0, stream(),
+		                   a.data, a.stride, ws->means_t, ws->norms, a.assignment, a.dim, a.k, kp, ws->queue, ws->counters);
+	else
+		hipLaunchKernelGGL((recheck_points_kernel<LD, DPAD, false>), grid, dim3(threads), 0, stream(),
+		                   a.data, a.stride, ws->means_t, ws->norms, a.assignment, a.dim, a.k, kp, ws->queue, ws->counters);
+	KMX_LAUNCH_CHECK("recheck_points_kernel");
+	return KMX_OK;
+}
+
+template <int LD>
+static int launch_recheck_sliced(const AssignArgs& a, Workspace* ws, uint32_t kp)
+{
+	const uint32_t threads = std::min<uint32_t>(1024, round_up(a.k, WAVE));
+	const dim3 grid(256);
+	if (a.dim % SLICE == 0)
+		hipLaunchKernelGGL((recheck_sliced_kernel<LD, true>), grid, dim3(threads), 0, stream(),
+		                   a.data, a.stride, ws->means_t, ws->norms, a.assignment, a.dim, a.k, kp, ws->queue, ws->counters);
+	else
+		hipLaunchKernelGGL((recheck_sliced_kernel<LD, false>), grid, dim3(threads), 0, stream(),
+		                   a.data, a.stride, ws->means_t, ws->norms, a.assignment, a.dim, a.k, kp, ws->queue, ws->counters);
+	KMX_LAUNCH_CHECK("recheck_sliced_kernel");
+	return KMX_OK;
+}
+
 template <int LD>
 static int launch_recheck_l(const AssignArgs& a, Workspace* ws, uint32_t kp)
 {
+	/* rows that fit the registers, many centroids: one lane per centroid, the points as scalar operands */
+	if (a.k >= 128 && a.dim <= 32) {
+		switch ((a.dim + 3) / 4) {
+		case 1: return launch_recheck_points<LD, 4>(a, ws, kp);
+		case 2: return launch_recheck_points<LD, 8>(a, ws, kp);
+		case 3: return launch_recheck_points<LD, 12>(a, ws, kp);
+		case 4: return launch_recheck_points<LD, 16>(a, ws, kp);
+		case 5: return launch_recheck_points<LD, 20>(a, ws, kp);
+		case 6: return launch_recheck_points<LD, 24>(a, ws, kp);
+		case 7: return launch_recheck_points<LD, 28>(a, ws, kp);
+		default: return launch_recheck_points<LD, 32>(a, ws, kp);
+		}
+	}
+	if (a.k >= 128 && a.dim > 64) return launch_recheck_sliced<LD>(a, ws, kp);
+	if (a.k >= 128 && a.dim <= 64) {
+		switch ((a.dim + 7) / 8) {
+		case 5: return launch_recheck_points<LD, 40>(a, ws, kp);
+		case 6: return launch_recheck_points<LD, 48>(a, ws, kp);
+		case 7: return launch_recheck_points<LD, 56>(a, ws, kp);
+		default: return launch_recheck_points<LD, 64>(a, ws, kp);
+		}
+	}
 	if (a.dim <= 64) {
 		if (a.k >= 48) return launch_recheck_dpad<LD, 64>(a, ws, kp);
 		if (a.k >= 24) return launch_recheck_dpad<LD, 32>(a, ws, kp);

@@ -106,6 +106,9 @@ SHAPES = [
     (130, 2000, 400),   # wide rows, centroids streamed through LDS in chunks
     (1, 7, 300),
     (5, 4100, 777),     # centroids do not fit one LDS chunk of the narrow layout
+    (48, 300, 3000),    # exact pass with one centroid row per lane, rows of 33..64 floats
+    (37, 2100, 2500),   # the same with a padded row and three chunks of centroids
+    (64, 1024, 6000),
 ]
 
 
@@ -123,7 +126,7 @@ def test_assignment_is_bit_exact(km, orc, gpu, dim, k, n, layout, layout_means):
         assert bad.size == 0, "variant %d: %d mismatches, first at %s" % (v, bad.size, bad[:5])
 
 
-@pytest.mark.parametrize("dim,k,n", [(8, 64, 4096), (32, 256, 3000), (4, 512, 2000)])
+@pytest.mark.parametrize("dim,k,n", [(8, 64, 4096), (32, 256, 3000), (4, 512, 2000), (48, 160, 2000), (21, 1500, 4000), (96, 200, 1500)])
 def test_hard_inputs(km, orc, gpu, dim, k, n):
     """Exact ties, duplicated centroids, coincident points, NaN / inf / huge / tiny values."""
     rng = np.random.default_rng(99 + dim)
