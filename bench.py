@@ -34,6 +34,7 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP32_TFLOPS = 157.3   # MI355X fp32 (vector or matrix), dense
 PEAK_BF16_TFLOPS = 2500.0  # MI355X bf16 matrix, dense
+PEAK_FP64_TFLOPS = 78.6    # MI355X fp64 (vector or matrix), dense
 VARIANT_NAMES = {0: "base", 1: "lds_fma", 2: "mfma", 4: "mfma_bf16x3"}
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # published full-iteration time for the headline shape on the reference's best hardware (V100 SXM2)
@@ -110,6 +111,55 @@ def fused_main(km, args, spec, data, means0):
     print(json.dumps(out))
 
 
+def double_main(km, args, spec, data, means0):
+    """--double: the same protocol on doubles (kmx_assign_f64 / kmx_update_f64, the reference's --double instantiation).
+    The points are the configuration's floats widened to doubles with full mantissas."""
+    import numpy as np
+    n, dim, k = int(spec.n), spec.dim, spec.k
+    data, means0 = km.widen_points(data), km.widen_points(means0)
+    alg = km.HipKMeansAlgorithm(dtype=np.float64)
+    alg.initialize(dim, k, n, args.steps, data, means0)
+    alg.run(iters=args.warmup)
+    alg.reset(means0)
+    km.sync()
+    t0 = time.perf_counter()
+    alg.run(iters=args.steps)
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    assert int(alg.getClusterSizes().sum()) == n, "cluster counts do not sum to N"
+    alg.reset(means0)
+    km.set_profiling(True)
+    k_assign = k_update = 0.0
+    for _ in range(args.steps):
+        nxt = alg.iteration()
+        alg.update_step(nxt)
+        k_assign += km.last_kernel_ms(0)
+        k_update += km.last_kernel_ms(1)
+    km.set_profiling(False)
+    k_assign /= args.steps; k_update /= args.steps
+    alg.cleanup()
+    executed = 3.0 * n * k * dim / (k_assign * 1e-3) / 1e12      # subtract, multiply, add per point x centroid x dim
+    update_bytes = 8.0 * (n * dim + k * dim) + 4.0 * (n + k)
+    update_gbs = update_bytes / (k_update * 1e-3) / 1e9
+    out = {
+        "metric": "ms per k-means iteration (assign+update) in double precision, benchmark configuration %d" % args.config,
+        "value": round(ms_per_step, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f64", "data": "synthetic",
+        "config": {"workload": "benchmark configuration %d: N=%d d=%d k=%d in doubles, initial centroids = first k points, seed %d"
+                               % (args.config, n, dim, k, spec.seed), "layout": "aos"},
+        "points_centroids_dims_per_s": round(float(n) * k * dim / (ms_per_step * 1e-3), 0),
+        "roofline": {"kernel": "assignment (serial arithmetic for every pair, fp64 vector instructions)", "bound": "fp64 vector",
+                     "achieved": round(executed, 2), "peak": PEAK_FP64_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(executed / PEAK_FP64_TFLOPS, 4), "traffic": None,
+                     "flops_counted": "executed: 3 per point x centroid x dim (no fused multiply-add: the serial code has none)",
+                     "avg_kernel_ms": round(k_assign, 4)},
+        "roofline_update": {"kernel": "update accumulation (fp64 atomics)", "bound": "hbm", "achieved": round(update_gbs, 1),
+                            "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(update_gbs / PEAK_HBM_GBS, 4), "traffic": None,
+                            "algorithmic_bytes": update_bytes, "avg_kernel_ms": round(k_update, 4)},
+    }
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -122,6 +172,8 @@ def main():
     ap.add_argument("--fused", action="store_true",
                     help="time the fused iteration (kmx_fused_f32: one call per iteration, no assignment vector; a single "
                          "pass over the points where k <= 32) instead of assignment + update")
+    ap.add_argument("--double", action="store_true",
+                    help="time the iteration on doubles (kmx_assign_f64 / kmx_update_f64) instead of floats")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--graph", action="store_true",
                     help="replay a recorded pair of iterations (HIP graph) instead of launching every kernel of the timed "
@@ -149,6 +201,8 @@ def main():
                       "atomic_shm": km.UPDATE_ATOMIC_SHM}[args.update_variant]
     if args.fused:
         return fused_main(km, args, spec, data, means0)
+    if args.double:
+        return double_main(km, args, spec, data, means0)
     alg = km.HipKMeansAlgorithm(assign_variant, update_variant)
     alg.initialize(dim, k, n, args.steps, data, means0)
 

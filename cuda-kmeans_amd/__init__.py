@@ -30,7 +30,8 @@ KMX_OK, KMX_ERR_INVALID_ARGUMENT, KMX_ERR_UNSUPPORTED, KMX_ERR_DEVICE, KMX_ERR_N
 ABI_SYMBOLS = [
     "kmx_device_count", "kmx_set_device", "kmx_device_props", "kmx_malloc", "kmx_free", "kmx_h2d", "kmx_d2h",
     "kmx_d2d", "kmx_sync", "kmx_set_stream", "kmx_shutdown", "kmx_fill_zero_u32", "kmx_assign_f32",
-    "kmx_assign_last_rechecked", "kmx_assign_last_variant", "kmx_update_f32", "kmx_bucket_sum_f32", "kmx_fused_f32", "kmx_graph_begin", "kmx_graph_end", "kmx_graph_launch", "kmx_graph_destroy", "kmx_event_create", "kmx_event_destroy", "kmx_event_record",
+    "kmx_assign_last_rechecked", "kmx_assign_last_variant", "kmx_update_f32", "kmx_bucket_sum_f32", "kmx_fused_f32", "kmx_assign_f64", "kmx_update_f64", "kmx_fused_f64",
+    "kmx_graph_begin", "kmx_graph_end", "kmx_graph_launch", "kmx_graph_destroy", "kmx_event_create", "kmx_event_destroy", "kmx_event_record",
     "kmx_event_elapsed_ms", "kmx_set_profiling", "kmx_last_kernel_ms", "kmx_last_error",
 ]
 
@@ -109,6 +110,9 @@ def hip_lib():
                                            ctypes.POINTER(ExecParams)]
         lib.kmx_fused_f32.argtypes = [ctypes.c_int, vp, ctypes.c_int, sz, vp, vp, ctypes.c_int, sz, vp, u32, u32, u32,
                                       ctypes.POINTER(ExecParams)]
+        lib.kmx_assign_f64.argtypes = lib.kmx_assign_f32.argtypes
+        lib.kmx_update_f64.argtypes = lib.kmx_update_f32.argtypes
+        lib.kmx_fused_f64.argtypes = lib.kmx_fused_f32.argtypes
         lib.kmx_graph_begin.argtypes = []
         lib.kmx_graph_end.argtypes = [ctypes.POINTER(vp)]
         lib.kmx_graph_launch.argtypes = [vp]
@@ -182,6 +186,14 @@ def first_k_means(spec, layout_means=AOS):
     if rc != 0:
         raise ValueError("kmx_gen_first_k_means rejected its arguments")
     return out
+
+
+def widen_points(values):
+    """float32 values as doubles that use the whole double mantissa: v * (1 + j * 2^-30) with j = (position % 7) - 3,
+    in IEEE double arithmetic (the same bits everywhere). Inputs of the double-precision tests and fixtures."""
+    v = np.ascontiguousarray(values, dtype=np.float32).astype(np.float64)
+    j = (np.arange(v.size, dtype=np.int64) % 7 - 3).astype(np.float64).reshape(v.shape)
+    return v * (1.0 + j * 2.0 ** -30)
 
 
 def fnv1a64(array):
@@ -267,20 +279,29 @@ class Event:
             pass
 
 
+def _is_double(dtype):
+    dtype = np.dtype(dtype)
+    if dtype not in (np.dtype(np.float32), np.dtype(np.float64)):
+        raise ValueError("element type must be float32 or float64")
+    return dtype == np.dtype(np.float64)
+
+
 def assign(variant, data_buf, layout, stride, means_buf, layout_means, stride_means, assignment_buf, dim, k, n,
-           exec_params=None):
-    """ASGN_KERNEL::run (kernels.cuh:81-93) through kmx_assign_f32; enqueues and returns."""
+           exec_params=None, dtype=np.float32):
+    """ASGN_KERNEL::run (kernels.cuh:81-93) through kmx_assign_f32 / kmx_assign_f64; enqueues and returns."""
     ex = exec_params if exec_params is not None else ExecParams()
-    check(hip_lib().kmx_assign_f32(variant, data_buf.ptr, layout, stride, means_buf.ptr, layout_means, stride_means,
+    fn = hip_lib().kmx_assign_f64 if _is_double(dtype) else hip_lib().kmx_assign_f32
+    check(fn(variant, data_buf.ptr, layout, stride, means_buf.ptr, layout_means, stride_means,
                                    None, assignment_buf.ptr, dim, k, n, ctypes.byref(ex)))
     return ex
 
 
 def update(variant, data_buf, layout, stride, assignment_buf, means_buf, layout_means, stride_means, sizes_buf, dim, k,
-           n, exec_params=None):
-    """UPDATE_KERNEL::run (kernels.cuh:96-105) through kmx_update_f32; enqueues and returns."""
+           n, exec_params=None, dtype=np.float32):
+    """UPDATE_KERNEL::run (kernels.cuh:96-105) through kmx_update_f32 / kmx_update_f64; enqueues and returns."""
     ex = exec_params if exec_params is not None else ExecParams()
-    check(hip_lib().kmx_update_f32(variant, data_buf.ptr, layout, stride, assignment_buf.ptr, means_buf.ptr,
+    fn = hip_lib().kmx_update_f64 if _is_double(dtype) else hip_lib().kmx_update_f32
+    check(fn(variant, data_buf.ptr, layout, stride, assignment_buf.ptr, means_buf.ptr,
                                    layout_means, stride_means, sizes_buf.ptr, dim, k, n, ctypes.byref(ex)))
     return ex
 
@@ -295,10 +316,11 @@ def bucket_sum(variant, data_buf, layout, stride, indices_buf, result_buf, layou
 
 
 def fused(variant, data_buf, layout, stride, means_in_buf, means_out_buf, layout_means, stride_means, sizes_buf, dim, k,
-          n, exec_params=None):
-    """FUSED_KERNEL::run (kernels.cuh:107-116) through kmx_fused_f32; enqueues and returns."""
+          n, exec_params=None, dtype=np.float32):
+    """FUSED_KERNEL::run (kernels.cuh:107-116) through kmx_fused_f32 / kmx_fused_f64; enqueues and returns."""
     ex = exec_params if exec_params is not None else ExecParams()
-    check(hip_lib().kmx_fused_f32(variant, data_buf.ptr, layout, stride, means_in_buf.ptr, means_out_buf.ptr,
+    fn = hip_lib().kmx_fused_f64 if _is_double(dtype) else hip_lib().kmx_fused_f32
+    check(fn(variant, data_buf.ptr, layout, stride, means_in_buf.ptr, means_out_buf.ptr,
                                   layout_means, stride_means, sizes_buf.ptr, dim, k, n, ctypes.byref(ex)))
     return ex
 
@@ -361,7 +383,9 @@ class HipKMeansAlgorithm:
     assign -> zero(means[next]) -> zero(sizes) -> update(+divide), one sync at the end of run()."""
 
     def __init__(self, assign_variant=ASSIGN_BEST, update_variant=UPDATE_ATOMIC_SHM, exec_params=None,
-                 layout=AOS, layout_means=AOS):
+                 layout=AOS, layout_means=AOS, dtype=np.float32):
+        self.dtype = np.dtype(dtype)  # float32, or float64 for the reference's --double instantiation
+        self.item = self.dtype.itemsize
         self.assign_variant = assign_variant
         self.update_variant = update_variant
         self.exec = exec_params if exec_params is not None else ExecParams()
@@ -378,9 +402,9 @@ class HipKMeansAlgorithm:
         self.stride_means = layout_stride(self.layout_means, self.k, self.dim)
         self.means_size = layout_size(self.layout_means, self.k, self.dim)
         copies = max(1, self.exec.privatized_copies)
-        self.cu_data = DeviceBuffer(4 * layout_size(self.layout, self.n, self.dim))
+        self.cu_data = DeviceBuffer(self.item * layout_size(self.layout, self.n, self.dim))
         self.cu_sizes = DeviceBuffer(4 * self.k)
-        self.cu_means = [DeviceBuffer(4 * self.means_size * copies) for _ in range(2)]
+        self.cu_means = [DeviceBuffer(self.item * self.means_size * copies) for _ in range(2)]
         self.cu_assignment = [DeviceBuffer(4 * self.n) for _ in range(2)]
         self._bufs = [self.cu_data, self.cu_sizes] + self.cu_means + self.cu_assignment
         self.cu_data.write(data)
@@ -397,14 +421,14 @@ class HipKMeansAlgorithm:
     def iteration(self):
         nxt = (self.last + 1) % 2
         assign(self.assign_variant, self.cu_data, self.layout, self.stride, self.cu_means[self.last], self.layout_means,
-               self.stride_means, self.cu_assignment[nxt], self.dim, self.k, self.n, self.exec)
+               self.stride_means, self.cu_assignment[nxt], self.dim, self.k, self.n, self.exec, self.dtype)
         return nxt
 
     def update_step(self, nxt):
         self.cu_means[nxt].zero()
         self.cu_sizes.zero()
         update(self.update_variant, self.cu_data, self.layout, self.stride, self.cu_assignment[nxt], self.cu_means[nxt],
-               self.layout_means, self.stride_means, self.cu_sizes, self.dim, self.k, self.n, self.exec)
+               self.layout_means, self.stride_means, self.cu_sizes, self.dim, self.k, self.n, self.exec, self.dtype)
         self.last = nxt
 
     def run(self, iters=None, collect_rechecked=False, use_graph=False):
@@ -433,7 +457,7 @@ class HipKMeansAlgorithm:
         sync()
 
     def getMeans(self):
-        return self.cu_means[self.last].read(np.float32, self.means_size)
+        return self.cu_means[self.last].read(self.dtype, self.means_size)
 
     def getAssignment(self):
         return self.cu_assignment[self.last].read(np.uint32, self.n)
@@ -452,7 +476,9 @@ class HipFusedKMeansAlgorithm:
     zero(means[next]) -> zero(sizes) -> fused(means[last] -> means[next]); getAssignment() is computed afterwards
     against the FINAL centroids (the reference does that on the host, cuda.hpp:199-221; here one more device pass)."""
 
-    def __init__(self, variant=FUSED_BEST, exec_params=None, layout=AOS, layout_means=AOS):
+    def __init__(self, variant=FUSED_BEST, exec_params=None, layout=AOS, layout_means=AOS, dtype=np.float32):
+        self.dtype = np.dtype(dtype)
+        self.item = self.dtype.itemsize
         self.variant = variant
         self.exec = exec_params if exec_params is not None else ExecParams()
         self.layout, self.layout_means = layout, layout_means
@@ -466,9 +492,9 @@ class HipFusedKMeansAlgorithm:
         self.stride = layout_stride(self.layout, self.n, self.dim)
         self.stride_means = layout_stride(self.layout_means, self.k, self.dim)
         self.means_size = layout_size(self.layout_means, self.k, self.dim)
-        self.cu_data = DeviceBuffer(4 * layout_size(self.layout, self.n, self.dim))
+        self.cu_data = DeviceBuffer(self.item * layout_size(self.layout, self.n, self.dim))
         self.cu_sizes = DeviceBuffer(4 * self.k)
-        self.cu_means = [DeviceBuffer(4 * self.means_size) for _ in range(2)]
+        self.cu_means = [DeviceBuffer(self.item * self.means_size) for _ in range(2)]
         self._bufs = [self.cu_data, self.cu_sizes] + self.cu_means
         self.cu_data.write(data)
         self.last = 0
@@ -481,7 +507,7 @@ class HipFusedKMeansAlgorithm:
         self.cu_means[nxt].zero()
         self.cu_sizes.zero()
         fused(self.variant, self.cu_data, self.layout, self.stride, self.cu_means[self.last], self.cu_means[nxt],
-              self.layout_means, self.stride_means, self.cu_sizes, self.dim, self.k, self.n, self.exec)
+              self.layout_means, self.stride_means, self.cu_sizes, self.dim, self.k, self.n, self.exec, self.dtype)
         self.last = nxt
 
     def run(self, iters=None):
@@ -490,7 +516,7 @@ class HipFusedKMeansAlgorithm:
         sync()
 
     def getMeans(self):
-        return self.cu_means[self.last].read(np.float32, self.means_size)
+        return self.cu_means[self.last].read(self.dtype, self.means_size)
 
     def getClusterSizes(self):
         return self.cu_sizes.read(np.uint32, self.k)
@@ -499,7 +525,7 @@ class HipFusedKMeansAlgorithm:
         out = DeviceBuffer(4 * max(self.n, 1))
         try:
             assign(ASSIGN_BEST, self.cu_data, self.layout, self.stride, self.cu_means[self.last], self.layout_means,
-                   self.stride_means, out, self.dim, self.k, self.n, self.exec)
+                   self.stride_means, out, self.dim, self.k, self.n, self.exec, self.dtype)
             sync()
             return out.read(np.uint32, self.n)
         finally:
@@ -514,7 +540,9 @@ class HipFusedKMeansAlgorithm:
 class HipAssignmentAlgorithm:
     """Mirror of CudaAssignmentAlgorithm (cuda.hpp:237-299): one assignment pass."""
 
-    def __init__(self, variant=ASSIGN_BEST, exec_params=None, layout=AOS, layout_means=AOS):
+    def __init__(self, variant=ASSIGN_BEST, exec_params=None, layout=AOS, layout_means=AOS, dtype=np.float32):
+        self.dtype = np.dtype(dtype)
+        self.item = self.dtype.itemsize
         self.variant = variant
         self.exec = exec_params if exec_params is not None else ExecParams()
         self.layout, self.layout_means = layout, layout_means
@@ -525,8 +553,8 @@ class HipAssignmentAlgorithm:
             raise KmxError(KMX_ERR_NO_DEVICE, "No HIP devices found!")
         check(hip_lib().kmx_set_device(0))
         self.dim, self.k, self.n = int(dim), int(k), int(n)
-        self.cu_data = DeviceBuffer(4 * layout_size(self.layout, self.n, self.dim))
-        self.cu_means = DeviceBuffer(4 * layout_size(self.layout_means, self.k, self.dim))
+        self.cu_data = DeviceBuffer(self.item * layout_size(self.layout, self.n, self.dim))
+        self.cu_means = DeviceBuffer(self.item * layout_size(self.layout_means, self.k, self.dim))
         self.cu_assignment = DeviceBuffer(4 * max(self.n, 1))
         self._bufs = [self.cu_data, self.cu_means, self.cu_assignment]
         self.cu_data.write(data)
@@ -536,7 +564,7 @@ class HipAssignmentAlgorithm:
     def run(self):
         assign(self.variant, self.cu_data, self.layout, layout_stride(self.layout, self.n, self.dim), self.cu_means,
                self.layout_means, layout_stride(self.layout_means, self.k, self.dim), self.cu_assignment, self.dim,
-               self.k, self.n, self.exec)
+               self.k, self.n, self.exec, self.dtype)
         sync()
 
     def getAssignment(self):

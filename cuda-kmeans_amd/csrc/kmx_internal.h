@@ -123,6 +123,11 @@ int launch_assign_lds_fma(const AssignArgs& a, kmx_exec_params* exec, Workspace*
 int launch_update(int variant, const UpdateArgs& u, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev);
 int launch_divide_means(const UpdateArgs& u);
 
+/* f64.hip: the double-precision calls keep their own transposed centroids; the runtime grows the buffer under the
+ * rules of the work space (not while a graph is recorded, after the stream has drained) and releases it on shutdown */
+int reserve_f64(double** ptr, size_t* cap, size_t doubles);
+int release_f64_workspace();
+
 /* fused_small.hip: one pass over the points for a handful of centroids. a.assignment is a scratch vector of n entries
  * (only the entries of the points left to the exact pass are written); means_out and sizes are zero on entry and hold
  * sums and counts on return (the caller divides). */

@@ -116,6 +116,7 @@ int reserve_packed(Workspace* ws, size_t packed_floats, size_t norm_floats, size
 int reserve_partials(Workspace* ws, size_t floats) { return grow(&ws->partials, &ws->partials_cap, floats); }
 int reserve_fused_assignment(Workspace* ws, size_t entries) { return grow(&ws->fused_assignment, &ws->fused_cap, entries); }
 int reserve_bucket_sizes(Workspace* ws, size_t entries) { return grow(&ws->bucket_sizes, &ws->bucket_cap, entries); }
+int reserve_f64(double** ptr, size_t* cap, size_t doubles) { return grow(ptr, cap, doubles); }
 
 static int release_workspace()
 {
@@ -128,7 +129,7 @@ static int release_workspace()
 	if (g_ws.fused_assignment) KMX_HIP(hipFree(g_ws.fused_assignment));
 	if (g_ws.bucket_sizes) KMX_HIP(hipFree(g_ws.bucket_sizes));
 	g_ws = Workspace();
-	return KMX_OK;
+	return release_f64_workspace();
 }
 
 /* counterpart of fillZeros (reference kernels.cu:12-17), grid-stride, 128-bit stores where aligned */

@@ -32,10 +32,11 @@
 template<typename F, class LAYOUT>
 void generate_benchmark_data(std::vector<F>& data, const kmx_dataset_spec& spec, std::size_t n)
 {
-	static_assert(sizeof(F) == 4, "the portable generator writes fp32");
-	data.assign(LAYOUT::size(n, spec.dim), F(0));
-	if (kmx_gen_points(&spec, 0, n, LAYOUT::ID, LAYOUT::precomputeConstants(n, spec.dim), data.data(), 0) != 0)
+	/* the portable generator writes fp32; for doubles the same values are widened (exactly) */
+	std::vector<float> raw(LAYOUT::size(n, spec.dim), 0.0f);
+	if (kmx_gen_points(&spec, 0, n, LAYOUT::ID, LAYOUT::precomputeConstants(n, spec.dim), raw.data(), 0) != 0)
 		throw std::runtime_error("data generator rejected its arguments");
+	data.assign(raw.begin(), raw.end());
 }
 
 /* initial centroids = the first k points ("--init first") */

@@ -7,7 +7,8 @@
  * rethrown as std::runtime_error, which is how the reference's runners report unsupported shapes
  * (kernels.cu:281-282,666,675,701) and how CUCH() reports device errors.
  *
- * Only F = float is built (the reference's --double path is not).
+ * F = float and F = double (the reference's --double) are built; the matrix-core and single-pass kernels are
+ * float-only and report that as an error for doubles.
  */
 #ifndef KMX_HOST_HIP_KERNELS_HPP
 #define KMX_HOST_HIP_KERNELS_HPP
@@ -92,17 +93,39 @@ static_assert(sizeof(HipExecParameters) == sizeof(kmx_exec_params), "HipExecPara
 template<typename T>
 void runFillZeros(T* data, std::size_t n)
 {
-	static_assert(sizeof(T) == 4, "only 32-bit element types are built");
-	KMX_CHECK(kmx_fill_zero_u32(data, n));
+	static_assert(sizeof(T) % 4 == 0, "element types are made of 32-bit words");
+	KMX_CHECK(kmx_fill_zero_u32(data, n * (sizeof(T) / 4)));
 }
 
 namespace hip_detail {
 
+/* the C ABI has one entry point per element type */
+inline int assign_call(int variant, const float* data, int ld, std::size_t stride, const float* means, int lm, std::size_t strideMeans,
+	const std::uint32_t* last, std::uint32_t* assignment, std::uint32_t dim, std::uint32_t k, std::uint32_t n, kmx_exec_params* exec)
+{ return kmx_assign_f32(variant, data, ld, stride, means, lm, strideMeans, last, assignment, dim, k, n, exec); }
+inline int assign_call(int variant, const double* data, int ld, std::size_t stride, const double* means, int lm, std::size_t strideMeans,
+	const std::uint32_t* last, std::uint32_t* assignment, std::uint32_t dim, std::uint32_t k, std::uint32_t n, kmx_exec_params* exec)
+{ return kmx_assign_f64(variant, data, ld, stride, means, lm, strideMeans, last, assignment, dim, k, n, exec); }
+
+inline int update_call(int variant, const float* data, int ld, std::size_t stride, const std::uint32_t* assignment, float* means, int lm,
+	std::size_t strideMeans, std::uint32_t* sizes, std::uint32_t dim, std::uint32_t k, std::uint32_t n, kmx_exec_params* exec)
+{ return kmx_update_f32(variant, data, ld, stride, assignment, means, lm, strideMeans, sizes, dim, k, n, exec); }
+inline int update_call(int variant, const double* data, int ld, std::size_t stride, const std::uint32_t* assignment, double* means, int lm,
+	std::size_t strideMeans, std::uint32_t* sizes, std::uint32_t dim, std::uint32_t k, std::uint32_t n, kmx_exec_params* exec)
+{ return kmx_update_f64(variant, data, ld, stride, assignment, means, lm, strideMeans, sizes, dim, k, n, exec); }
+
+inline int fused_call(int variant, const float* data, int ld, std::size_t stride, const float* meansIn, float* meansOut, int lm,
+	std::size_t strideMeans, std::uint32_t* sizes, std::uint32_t dim, std::uint32_t k, std::uint32_t n, kmx_exec_params* exec)
+{ return kmx_fused_f32(variant, data, ld, stride, meansIn, meansOut, lm, strideMeans, sizes, dim, k, n, exec); }
+inline int fused_call(int variant, const double* data, int ld, std::size_t stride, const double* meansIn, double* meansOut, int lm,
+	std::size_t strideMeans, std::uint32_t* sizes, std::uint32_t dim, std::uint32_t k, std::uint32_t n, kmx_exec_params* exec)
+{ return kmx_fused_f64(variant, data, ld, stride, meansIn, meansOut, lm, strideMeans, sizes, dim, k, n, exec); }
+
 template<typename F, typename IDX_T, class LAYOUT, class LAYOUT_MEANS>
 void assign(int variant, const AssignmentProblemInstance<F, IDX_T>& in, HipExecParameters& exec)
 {
-	static_assert(std::is_same<F, float>::value && sizeof(IDX_T) == 4, "built for float data and 32-bit indices");
-	KMX_CHECK(kmx_assign_f32(variant,
+	static_assert(sizeof(IDX_T) == 4, "built for 32-bit indices");
+	KMX_CHECK(assign_call(variant,
 		in.data, LAYOUT::ID, LAYOUT::precomputeConstants(in.n, in.dim),
 		in.means, LAYOUT_MEANS::ID, LAYOUT_MEANS::precomputeConstants(in.k, in.dim),
 		(const std::uint32_t*)in.lastAssignment, (std::uint32_t*)in.assignment,
@@ -112,8 +135,8 @@ void assign(int variant, const AssignmentProblemInstance<F, IDX_T>& in, HipExecP
 template<typename F, typename IDX_T, class LAYOUT, class LAYOUT_MEANS>
 void update(int variant, const UpdateProblemInstance<F, IDX_T>& in, HipExecParameters& exec)
 {
-	static_assert(std::is_same<F, float>::value && sizeof(IDX_T) == 4, "built for float data and 32-bit indices");
-	KMX_CHECK(kmx_update_f32(variant,
+	static_assert(sizeof(IDX_T) == 4, "built for 32-bit indices");
+	KMX_CHECK(update_call(variant,
 		in.data, LAYOUT::ID, LAYOUT::precomputeConstants(in.n, in.dim),
 		(const std::uint32_t*)in.assignment,
 		in.means, LAYOUT_MEANS::ID, LAYOUT_MEANS::precomputeConstants(in.k, in.dim),
@@ -123,8 +146,8 @@ void update(int variant, const UpdateProblemInstance<F, IDX_T>& in, HipExecParam
 template<typename F, typename IDX_T, class LAYOUT, class LAYOUT_MEANS>
 void fused(int variant, const FusedProblemInstance<F, IDX_T>& in, HipExecParameters& exec)
 {
-	static_assert(std::is_same<F, float>::value && sizeof(IDX_T) == 4, "built for float data and 32-bit indices");
-	KMX_CHECK(kmx_fused_f32(variant,
+	static_assert(sizeof(IDX_T) == 4, "built for 32-bit indices");
+	KMX_CHECK(fused_call(variant,
 		in.data, LAYOUT::ID, LAYOUT::precomputeConstants(in.n, in.dim),
 		in.meansIn, in.meansOut, LAYOUT_MEANS::ID, LAYOUT_MEANS::precomputeConstants(in.k, in.dim),
 		(std::uint32_t*)in.clusterSizes, in.dim, in.k, in.n, reinterpret_cast<kmx_exec_params*>(&exec)));

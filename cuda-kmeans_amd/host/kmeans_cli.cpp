@@ -39,7 +39,7 @@ public:
 	double getMiliseconds() const { return mMs; }
 };
 
-/* raw little-endian dump of a result vector (--dump): <prefix>.means.f32 / <prefix>.assignment.u32 */
+/* raw little-endian dump of a result vector (--dump): <prefix>.means.f32 (.f64 with --double) / <prefix>.assignment.u32 */
 template<typename T>
 void dumpVector(const std::string& path, const std::vector<T>& v)
 {
@@ -227,7 +227,7 @@ void run_kmeans(const ProgramArguments& args, std::vector<F>& data, std::vector<
 	}
 
 	if (args.isPresent("dump")) {
-		dumpVector(args.getString("dump") + ".means.f32", algorithm->getMeans());
+		dumpVector(args.getString("dump") + (sizeof(F) == 8 ? ".means.f64" : ".means.f32"), algorithm->getMeans());
 		dumpVector(args.getString("dump") + ".assignment.u32", algorithm->getAssignment());
 	}
 
@@ -309,7 +309,7 @@ int main(int argc, char* argv[])
 		args.registerString("algorithm", "Which algorithm is to be tested (serial, hip_base, hip_base_shm, hip_mfma, hip_mfma_bf16, hip_best, hip_fused; assignment only: hip_lds_fma).", "serial");
 		args.registerEnum("layout", "Type of data layout.", "aos", { "aos", "soa" });
 		args.registerEnum("layoutMeans", "Type of data layout (override for means only).", "aos", { "aos", "soa" });
-		args.registerBool("double", "Use doubles instead of floats (not built).");
+		args.registerBool("double", "Use doubles instead of floats.");
 		args.registerBool("verify", "Verify results against base (serial) algorithm.");
 		args.registerInt("privatizedCopies", "Number of privatized copies in global memory (relevant only to some algorithms).", 1, 1, 4096);
 		args.registerInt("itemsPerThread", "Number of computations performed per thread.", 1, 1, 4096);
@@ -327,7 +327,7 @@ int main(int argc, char* argv[])
 		args.registerInt("serialThreads", "Threads of the serial algorithm (results are bit-identical to 1 thread).", 1, 1, 1024);
 		args.registerBool("json", "Print a JSON report instead of the two-number line.");
 		args.registerBool("graph", "Record a pair of iterations as a HIP graph and replay it instead of launching every kernel (device algorithms; not with --json).");
-		args.registerString("dump", "Write the final centroids and assignment to <prefix>.means.f32 / <prefix>.assignment.u32.", "");
+		args.registerString("dump", "Write the final centroids and assignment to <prefix>.means.f32 (.f64 with --double) / <prefix>.assignment.u32.", "");
 		args.process(argc, argv);
 	}
 	catch (ArgumentException& e) {
@@ -337,7 +337,7 @@ int main(int argc, char* argv[])
 	}
 
 	try {
-		if (args.getBool("double")) throw std::runtime_error("The double-precision path is not built.");
+		const bool useDouble = args.getBool("double");
 		if (args.getInt("config") > 0) {
 			/* a benchmark configuration fixes the shape; explicit arguments may shrink N or the iteration count */
 			kmx_dataset_spec spec;
@@ -351,8 +351,10 @@ int main(int argc, char* argv[])
 			for (std::size_t i = 1; i < forced.size(); ++i) argv2.push_back(const_cast<char*>(forced[i].c_str()));
 			ProgramArguments again = args; /* same registrations, re-parse with the forced values appended */
 			again.process((int)argv2.size(), argv2.data());
-			select_layout_and_run<float>(again);
+			if (useDouble) select_layout_and_run<double>(again);
+			else select_layout_and_run<float>(again);
 		}
+		else if (useDouble) select_layout_and_run<double>(args);
 		else select_layout_and_run<float>(args);
 	}
 	catch (ArgumentException& e) {

@@ -172,6 +172,36 @@ int kmx_fused_f32(int variant,
                   uint32_t* cluster_sizes,
                   uint32_t dim, uint32_t k, uint32_t n, kmx_exec_params* exec);
 
+/*
+ * ---- the same runners instantiated with F = double: the reference's --double switch (k-means.cpp:341-342) selects
+ *      the <double> instantiations of every kernel (kernels.cu:1200-1261) ----
+ * Arguments as for the _f32 entry points, with doubles for data and centroids (strides in elements).
+ * kmx_assign_f64: variants KMX_ASSIGN_BASE (row re-read per group of centroids) and KMX_ASSIGN_BEST (rows of up to 32
+ *   doubles held in registers); both evaluate the serial arithmetic for every pair, so the result is the serial one.
+ *   The matrix-core variants are float-only: KMX_ERR_UNSUPPORTED.
+ * kmx_update_f64: every update variant; ATOMIC_SHM privatises the sums in LDS when k * dim doubles fit 32 KB, the
+ *   others (and larger k * dim) use fp64 atomics in global memory. privatized_copies > 1: KMX_ERR_UNSUPPORTED.
+ *   Precondition as for kmx_update_f32: means and cluster_sizes are zero (kmx_fill_zero_u32 with twice the count).
+ * kmx_fused_f64: KMX_FUSED_TWO_PASS / KMX_FUSED_BEST (assignment into the work space, then the update);
+ *   KMX_FUSED_ONE_PASS is float-only: KMX_ERR_UNSUPPORTED.
+ */
+int kmx_assign_f64(int variant,
+                   const double* data, int layout, size_t stride,
+                   const double* means, int layout_means, size_t stride_means,
+                   const uint32_t* last_assignment, uint32_t* assignment,
+                   uint32_t dim, uint32_t k, uint32_t n, kmx_exec_params* exec);
+int kmx_update_f64(int variant,
+                   const double* data, int layout, size_t stride,
+                   const uint32_t* assignment,
+                   double* means, int layout_means, size_t stride_means,
+                   uint32_t* cluster_sizes,
+                   uint32_t dim, uint32_t k, uint32_t n, kmx_exec_params* exec);
+int kmx_fused_f64(int variant,
+                  const double* data, int layout, size_t stride,
+                  const double* means_in, double* means_out, int layout_means, size_t stride_means,
+                  uint32_t* cluster_sizes,
+                  uint32_t dim, uint32_t k, uint32_t n, kmx_exec_params* exec);
+
 /* ---- events on the library's stream (for the assignment / update split; the reference only has
  *      a wall-clock Stopwatch around run(), k-means.cpp:155-158) ---- */
 int kmx_event_create(void** event);

@@ -12,6 +12,7 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _f32p = ctypes.POINTER(ctypes.c_float)
 _u32p = ctypes.POINTER(ctypes.c_uint32)
+_f64p = ctypes.POINTER(ctypes.c_double)
 
 AOS, SOA = 0, 1
 
@@ -59,6 +60,16 @@ def oracle_lib():
                                       ctypes.c_size_t, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32,
                                       _u32p, _u32p, ctypes.c_int, ctypes.c_int]
         lib.oracle_kmeans.restype = None
+        lib.oracle_assign_f64.argtypes = [_f64p, ctypes.c_int, ctypes.c_size_t, _f64p, ctypes.c_int, ctypes.c_size_t,
+                                          ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, _u32p, _f64p, _f64p, ctypes.c_int]
+        lib.oracle_assign_f64.restype = None
+        lib.oracle_update_f64.argtypes = [_f64p, ctypes.c_int, ctypes.c_size_t, _u32p, _f64p, ctypes.c_int, ctypes.c_size_t,
+                                          _u32p, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_int]
+        lib.oracle_update_f64.restype = None
+        lib.oracle_kmeans_f64.argtypes = [_f64p, ctypes.c_int, ctypes.c_size_t, _f64p, ctypes.c_int, ctypes.c_size_t,
+                                          ctypes.c_size_t, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32, ctypes.c_uint32,
+                                          _u32p, _u32p, ctypes.c_int]
+        lib.oracle_kmeans_f64.restype = None
         _oracle = lib
     return _oracle
 
@@ -77,12 +88,19 @@ def ref_lib():
         lib.ref_serial_assign.argtypes = [_f32p, ctypes.c_int, _f32p, ctypes.c_int, ctypes.c_size_t, ctypes.c_size_t,
                                           ctypes.c_size_t, _u32p]
         lib.ref_serial_assign.restype = ctypes.c_int
+        if hasattr(lib, "ref_serial_kmeans_f64"):
+            lib.ref_serial_kmeans_f64.argtypes = [_f64p, ctypes.c_int, _f64p, ctypes.c_int, ctypes.c_size_t, ctypes.c_size_t,
+                                                  ctypes.c_size_t, ctypes.c_size_t, _f64p, _u32p]
+            lib.ref_serial_kmeans_f64.restype = ctypes.c_int
+            lib.ref_serial_assign_f64.argtypes = [_f64p, ctypes.c_int, _f64p, ctypes.c_int, ctypes.c_size_t, ctypes.c_size_t,
+                                                  ctypes.c_size_t, _u32p]
+            lib.ref_serial_assign_f64.restype = ctypes.c_int
         _ref = lib
     return _ref
 
 
-def _check(data, means, layout, layout_means, dim, k, n):
-    assert data.dtype == np.float32 and means.dtype == np.float32
+def _check(data, means, layout, layout_means, dim, k, n, dtype=np.float32):
+    assert data.dtype == dtype and means.dtype == dtype
     assert data.flags.c_contiguous and means.flags.c_contiguous
     assert data.size >= layout_size(layout, n, dim) and means.size >= layout_size(layout_means, k, dim)
 
@@ -145,5 +163,68 @@ def ref_assign(data, means, dim, k, n, layout=AOS, layout_means=AOS):
     _check(data, means, layout, layout_means, dim, k, n)
     asg = np.empty(n, dtype=np.uint32)
     rc = lib.ref_serial_assign(_ptr(data, _f32p), layout, _ptr(means, _f32p), layout_means, dim, k, n, _ptr(asg, _u32p))
+    assert rc == 0
+    return asg
+
+
+# ---- F = double (the reference's --double instantiation) ----
+
+def assign_f64(data, means, dim, k, n, layout=AOS, layout_means=AOS, threads=1, detail=False):
+    """Oracle assignment on doubles. Returns assignment, or (assignment, best_dist, second_dist) with detail=True."""
+    _check(data, means, layout, layout_means, dim, k, n, np.float64)
+    asg = np.empty(n, dtype=np.uint32)
+    best = np.empty(n, dtype=np.float64) if detail else None
+    second = np.empty(n, dtype=np.float64) if detail else None
+    oracle_lib().oracle_assign_f64(_ptr(data, _f64p), layout, layout_stride(layout, n, dim), _ptr(means, _f64p), layout_means,
+                                   layout_stride(layout_means, k, dim), dim, k, n, _ptr(asg, _u32p), _ptr(best, _f64p),
+                                   _ptr(second, _f64p), threads)
+    return (asg, best, second) if detail else asg
+
+
+def update_f64(data, assignment, dim, k, n, layout=AOS, layout_means=AOS, threads=1):
+    """Oracle update on doubles. Returns (means, cluster_sizes)."""
+    assert data.dtype == np.float64 and assignment.dtype == np.uint32 and assignment.size >= n
+    means = np.zeros(layout_size(layout_means, k, dim), dtype=np.float64)
+    sizes = np.zeros(k, dtype=np.uint32)
+    oracle_lib().oracle_update_f64(_ptr(data, _f64p), layout, layout_stride(layout, n, dim), _ptr(assignment, _u32p),
+                                   _ptr(means, _f64p), layout_means, layout_stride(layout_means, k, dim), _ptr(sizes, _u32p),
+                                   dim, k, n, threads)
+    return means, sizes
+
+
+def kmeans_f64(data, means, dim, k, n, iters, layout=AOS, layout_means=AOS, threads=1):
+    """Oracle Lloyd iterations on doubles. Returns (means, assignment, cluster_sizes)."""
+    _check(data, means, layout, layout_means, dim, k, n, np.float64)
+    m = means.copy()
+    asg = np.zeros(n, dtype=np.uint32)
+    sizes = np.zeros(k, dtype=np.uint32)
+    oracle_lib().oracle_kmeans_f64(_ptr(data, _f64p), layout, layout_stride(layout, n, dim), _ptr(m, _f64p), layout_means,
+                                   layout_stride(layout_means, k, dim), m.size, dim, k, n, iters, _ptr(asg, _u32p),
+                                   _ptr(sizes, _u32p), threads)
+    return m, asg, sizes
+
+
+def ref_kmeans_f64(data, means, dim, k, n, iters, layout=AOS, layout_means=AOS):
+    """The reference's SerialKMeansAlgorithm<double, ...> (only where oracle/_ref was built). Returns (means, assignment)."""
+    lib = ref_lib()
+    if lib is None or not hasattr(lib, "ref_serial_kmeans_f64"):
+        raise RuntimeError("oracle/_ref/libref_serial.so is not built")
+    _check(data, means, layout, layout_means, dim, k, n, np.float64)
+    m = np.empty(layout_size(layout_means, k, dim), dtype=np.float64)
+    asg = np.empty(n, dtype=np.uint32)
+    rc = lib.ref_serial_kmeans_f64(_ptr(data, _f64p), layout, _ptr(means, _f64p), layout_means, dim, k, n, iters,
+                                   _ptr(m, _f64p), _ptr(asg, _u32p))
+    assert rc == 0
+    return m, asg
+
+
+def ref_assign_f64(data, means, dim, k, n, layout=AOS, layout_means=AOS):
+    """The reference's SerialAssignmentAlgorithm<double, ...> (only where oracle/_ref was built)."""
+    lib = ref_lib()
+    if lib is None or not hasattr(lib, "ref_serial_assign_f64"):
+        raise RuntimeError("oracle/_ref/libref_serial.so is not built")
+    _check(data, means, layout, layout_means, dim, k, n, np.float64)
+    asg = np.empty(n, dtype=np.uint32)
+    rc = lib.ref_serial_assign_f64(_ptr(data, _f64p), layout, _ptr(means, _f64p), layout_means, dim, k, n, _ptr(asg, _u32p))
     assert rc == 0
     return asg

@@ -66,6 +66,24 @@ void oracle_kmeans(const float* data, int layout, size_t stride,
                    uint32_t dim, uint32_t k, uint32_t n, uint32_t iters,
                    uint32_t* assignment, uint32_t* cluster_sizes, int threads, int fast);
 
+/*
+ * The same three functions for F = double, the reference's --double instantiation
+ * (k-means.cpp:341-342; serial.hpp and metric_policies.hpp are templates over F). Pinned like the
+ * float functions: golden vectors written by the reference's SerialKMeansAlgorithm<double, ...>,
+ * that build directly when oracle/_ref exists, brute force with extended precision on tiny inputs.
+ */
+void oracle_assign_f64(const double* data, int layout, size_t stride,
+                       const double* means, int layout_means, size_t stride_means,
+                       uint32_t dim, uint32_t k, uint32_t n,
+                       uint32_t* assignment, double* best_dist, double* second_dist, int threads);
+void oracle_update_f64(const double* data, int layout, size_t stride, const uint32_t* assignment,
+                       double* means, int layout_means, size_t stride_means, uint32_t* cluster_sizes,
+                       uint32_t dim, uint32_t k, uint32_t n, int threads);
+void oracle_kmeans_f64(const double* data, int layout, size_t stride,
+                       double* means, int layout_means, size_t stride_means, size_t means_size,
+                       uint32_t dim, uint32_t k, uint32_t n, uint32_t iters,
+                       uint32_t* assignment, uint32_t* cluster_sizes, int threads);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,199 @@
+"""Parity of the double-precision HIP path (kmx_assign_f64 / kmx_update_f64 / kmx_fused_f64, the counterpart of
+the reference's --double instantiation) with the CPU oracle's F = double functions, through the C ABI (-m gpu).
+
+Bar: assignment and counts bit-exact (the kernel evaluates the serial arithmetic itself for every pair);
+centroids within 1e-12 relative to the rms coordinate (the sums are accumulated by atomics in another order).
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+AOS, SOA = 0, 1
+CENTROID_RTOL = 1e-12
+
+
+def rel_err(got, want):
+    scale = float(np.sqrt(np.mean(want ** 2)))
+    return float(np.abs(got - want).max() / max(scale, 1e-300))
+
+
+def gpu_assign(km, variant, data, means, dim, k, n, layout=AOS, layout_means=AOS):
+    alg = km.HipAssignmentAlgorithm(variant, None, layout, layout_means, dtype=np.float64)
+    alg.initialize(dim, k, n, data, means)
+    alg.run()
+    out = alg.getAssignment()
+    alg.cleanup()
+    return out
+
+
+def gpu_update(km, variant, data, assignment, dim, k, n, layout=AOS, layout_means=AOS):
+    d = km.DeviceBuffer(8 * max(data.size, 1)); d.write(data)
+    a = km.DeviceBuffer(4 * max(n, 1)); a.write(assignment)
+    msize = km.layout_size(layout_means, k, dim)
+    m = km.DeviceBuffer(8 * msize); m.zero()
+    s = km.DeviceBuffer(4 * k); s.zero()
+    km.update(variant, d, layout, km.layout_stride(layout, n, dim), a, m, layout_means,
+              km.layout_stride(layout_means, k, dim), s, dim, k, n, dtype=np.float64)
+    km.sync()
+    means, sizes = m.read(np.float64, msize), s.read(np.uint32, k)
+    for b in (d, a, m, s):
+        b.free()
+    return means, sizes
+
+
+@pytest.fixture(scope="module")
+def golden():
+    with open(os.path.join(HERE, "golden", "golden_f64_index.json")) as f:
+        index = json.load(f)
+    return index, np.load(os.path.join(HERE, "golden", "golden_f64.npz"))
+
+
+@pytest.mark.parametrize("name", ["cfg1_f64", "cfg1_f64_soa_soa", "cfg1_f64_aos_soa", "cfg2_f64", "cfg3_f64", "cfg4_f64",
+                                  "cfg5_f64"])
+def test_first_pass_equals_reference_golden(km, gpu, golden, name):
+    """One assignment pass from the initial centroids against the REFERENCE's own double-precision output."""
+    index, arrays = golden
+    c = index[name]
+    spec = km.baseline_config(c["config"])
+    data = km.widen_points(km.generate_points(spec, c["n"], layout=c["layout"]))
+    means0 = km.widen_points(km.first_k_means(spec, c["layout_means"]))
+    want = arrays[name + "_assignment_first_pass"].astype(np.uint32)
+    for v in (km.ASSIGN_BASE, km.ASSIGN_BEST):
+        got = gpu_assign(km, v, data, means0, c["dim"], c["k"], c["n"], c["layout"], c["layout_means"])
+        assert np.array_equal(got, want), "variant %d: %d mismatches" % (v, int((got != want).sum()))
+
+
+SHAPES = [(20, 128, 10240), (3, 5, 257), (7, 33, 1000), (2, 2, 128), (16, 16, 5000), (32, 1000, 4099), (64, 96, 2048),
+          (100, 40, 1500), (256, 300, 700), (1, 7, 300), (5, 4100, 777), (9, 8, 64), (33, 9, 513)]
+
+
+@pytest.mark.parametrize("dim,k,n", SHAPES)
+@pytest.mark.parametrize("layout,layout_means", [(AOS, AOS), (SOA, SOA), (AOS, SOA), (SOA, AOS)])
+def test_assignment_is_bit_exact(km, orc, gpu, dim, k, n, layout, layout_means):
+    rng = np.random.default_rng(dim * 7919 + k)
+    data = rng.normal(size=n * dim) * 3.0
+    means = rng.normal(size=k * dim) * 3.0
+    want = orc.assign_f64(data, means, dim, k, n, layout, layout_means, threads=0)
+    for v in (km.ASSIGN_BASE, km.ASSIGN_BEST):
+        got = gpu_assign(km, v, data, means, dim, k, n, layout, layout_means)
+        bad = np.nonzero(got != want)[0]
+        assert bad.size == 0, "variant %d: %d mismatches, first at %s" % (v, bad.size, bad[:5])
+
+
+@pytest.mark.parametrize("dim,k,n", [(8, 64, 4096), (32, 256, 3000), (40, 70, 1000)])
+def test_hard_inputs(km, orc, gpu, dim, k, n):
+    """Exact ties, duplicated centroids, coincident points, NaN / inf / huge / tiny values, float-invisible gaps."""
+    rng = np.random.default_rng(99 + dim)
+    base = rng.normal(size=(n, dim))
+    means = rng.normal(size=(k, dim))
+    cases = {}
+    m = means.copy(); m[k // 2] = m[3]; m[k - 1] = m[3]; m[7] = m[5]
+    d = base.copy(); d[: k] = m
+    d[k: 2 * k] = (m + m[::-1]) / 2.0
+    cases["duplicates_and_midpoints"] = (d, m)
+    m = means.copy(); m[9] = m[2] * (1.0 + 2.0 ** -45)       # differs from centroid 2 far below float resolution
+    d = base.copy(); d[:50] = m[2] * 1.5
+    cases["gap_below_float_resolution"] = (d, m)
+    cases["all_points_identical"] = (np.repeat(base[:1], n, 0), means)
+    cases["all_centroids_identical"] = (base, np.repeat(means[:1], k, 0))
+    d = base.copy(); d[5, 0] = np.nan; d[9, dim - 1] = np.inf; d[11, 0] = -np.inf
+    cases["nan_inf_points"] = (d, means)
+    m = means.copy(); m[4, 1] = np.nan
+    cases["nan_centroid"] = (base, m)
+    m = means.copy(); m[0, 0] = np.nan
+    cases["nan_centroid_zero"] = (base, m)
+    cases["huge"] = (base * 1e160, means * 1e160)          # squares overflow to inf
+    cases["tiny"] = (base * 1e-170, means * 1e-170)        # squares underflow
+    cases["grid_ties"] = (np.round(base * 2) / 2, np.round(means * 2) / 2)
+    for name, (d, m) in cases.items():
+        d = np.ascontiguousarray(d).ravel()
+        m = np.ascontiguousarray(m).ravel()
+        want = orc.assign_f64(d, m, dim, k, n, threads=0)
+        for v in (km.ASSIGN_BASE, km.ASSIGN_BEST):
+            got = gpu_assign(km, v, d, m, dim, k, n)
+            bad = np.nonzero(got != want)[0]
+            assert bad.size == 0, "%s, variant %d: %d mismatches, first at %s (gpu %s, oracle %s)" % (
+                name, v, bad.size, bad[:5], got[bad[:5]], want[bad[:5]])
+
+
+UPDATE_SHAPES = [(8, 64, 65536), (20, 128, 10240), (3, 5, 257), (32, 1024, 50000), (4, 4096, 100000), (16, 16, 300000),
+                 (256, 1024, 4096), (33, 7, 1000)]
+
+
+@pytest.mark.parametrize("dim,k,n", UPDATE_SHAPES)
+@pytest.mark.parametrize("layout,layout_means", [(AOS, AOS), (SOA, SOA), (AOS, SOA), (SOA, AOS)])
+def test_update_matches_oracle(km, orc, gpu, dim, k, n, layout, layout_means):
+    rng = np.random.default_rng(dim + k + n)
+    data = rng.normal(size=n * dim) * 2.0 + 1.0
+    asg = rng.integers(0, k, size=n, dtype=np.uint32)
+    asg[asg == k // 2] = 0                                 # an empty cluster (k > 1)
+    want_m, want_s = orc.update_f64(data, asg, dim, k, n, layout, layout_means, threads=0)
+    for v in (km.UPDATE_ATOMIC_POINT, km.UPDATE_ATOMIC_FINE, km.UPDATE_ATOMIC_SHM):
+        got_m, got_s = gpu_update(km, v, data, asg, dim, k, n, layout, layout_means)
+        assert np.array_equal(got_s, want_s), v
+        assert rel_err(got_m, want_m) < CENTROID_RTOL, (v, rel_err(got_m, want_m))
+        if k > 1:
+            c = k // 2
+            empty = got_m.reshape(k, dim)[c] if layout_means == AOS else got_m.reshape(dim, k)[:, c]
+            assert np.array_equal(empty, np.zeros(dim)), "an empty cluster stays at the origin"
+
+
+@pytest.mark.parametrize("cid,n,iters", [(1, 65536, 6), (2, 32768, 3), (5, 200000, 4), (4, 4096, 2)])
+def test_every_iteration_matches_oracle(km, orc, gpu, cid, n, iters):
+    """Teacher-forced: every iteration's assignment against the oracle's on the centroids the GPU used (exact), every
+    update against the oracle's on that assignment (tolerance); then the free-running result."""
+    spec = km.baseline_config(cid)
+    data = km.widen_points(km.generate_points(spec, n))
+    means0 = km.widen_points(km.first_k_means(spec))
+    alg = km.HipKMeansAlgorithm(dtype=np.float64)
+    alg.initialize(spec.dim, spec.k, n, iters, data, means0)
+    prev = means0
+    for it in range(iters):
+        nxt = alg.iteration()
+        km.sync()
+        got_a = alg.cu_assignment[nxt].read(np.uint32, n)
+        want_a = orc.assign_f64(data, prev, spec.dim, spec.k, n, threads=0)
+        assert np.array_equal(got_a, want_a), "iteration %d: %d mismatches" % (it, int((got_a != want_a).sum()))
+        alg.update_step(nxt)
+        km.sync()
+        got_m, got_s = alg.getMeans(), alg.getClusterSizes()
+        want_m, want_s = orc.update_f64(data, want_a, spec.dim, spec.k, n, threads=0)
+        assert np.array_equal(got_s, want_s)
+        assert rel_err(got_m, want_m) < CENTROID_RTOL
+        prev = got_m
+    alg.cleanup()
+
+
+def test_fused_call_and_argument_errors(km, orc, gpu):
+    spec = km.baseline_config(1)
+    n = 20000
+    data = km.widen_points(km.generate_points(spec, n))
+    means0 = km.widen_points(km.first_k_means(spec))
+    alg = km.HipFusedKMeansAlgorithm(dtype=np.float64)
+    alg.initialize(spec.dim, spec.k, n, 1, data, means0)
+    alg.run()
+    want_a = orc.assign_f64(data, means0, spec.dim, spec.k, n, threads=0)
+    want_m, want_s = orc.update_f64(data, want_a, spec.dim, spec.k, n, threads=0)
+    assert np.array_equal(alg.getClusterSizes(), want_s)
+    assert rel_err(alg.getMeans(), want_m) < CENTROID_RTOL
+    alg.cleanup()
+    # the float-only variants say so instead of running something else
+    for bad in (km.ASSIGN_MFMA, km.ASSIGN_MFMA_BF16X3, km.ASSIGN_LDS_FMA):
+        with pytest.raises(km.KmxError) as e:
+            gpu_assign(km, bad, data[:100 * spec.dim], means0, spec.dim, spec.k, 100)
+        assert e.value.code == km.KMX_ERR_UNSUPPORTED
+    with pytest.raises(km.KmxError) as e:
+        a = km.HipFusedKMeansAlgorithm(km.FUSED_ONE_PASS, dtype=np.float64)
+        a.initialize(spec.dim, spec.k, 100, 1, data[:100 * spec.dim], means0)
+        try:
+            a.run()
+        finally:
+            a.cleanup()
+    assert e.value.code == km.KMX_ERR_UNSUPPORTED
+    # empty input: nothing to do
+    assert gpu_assign(km, km.ASSIGN_BEST, np.zeros(0), means0, spec.dim, spec.k, 0).size == 0

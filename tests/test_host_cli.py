@@ -50,8 +50,6 @@ def test_argument_errors_exit_1(harness):
 def test_runtime_errors_exit_2(harness):
     rc, out, err = run(harness, "--algorithm", "nope")
     assert rc == 2 and "Error: Unkown algorithm 'nope'." in out
-    rc, out, err = run(harness, "--double")
-    assert rc == 2 and "not built" in out
     rc, out, err = run(harness, "--N", "128", "--k", "1k")
     assert rc == 2
 
@@ -81,6 +79,21 @@ def test_serial_matches_oracle_and_threads_do_not_change_bits(harness, km, orc, 
         got = np.fromfile(prefix + ".means.f32", dtype=np.float32)
         got = got.reshape(spec.k, spec.dim) if lm == km.AOS else got.reshape(spec.dim, spec.k).T
         assert np.array_equal(got, want_m.reshape(spec.k, spec.dim))
+
+
+def test_double_serial_matches_oracle(harness, km, orc, tmp_path):
+    """--double: the harness's serial algorithm instantiated with doubles against the oracle's F = double functions
+    (the benchmark generator's floats widened exactly)."""
+    spec = km.baseline_config(1)
+    n, iters = 4096, 3
+    data = km.generate_points(spec, n).astype(np.float64)
+    means0 = km.first_k_means(spec).astype(np.float64)
+    want_m, want_a, _ = orc.kmeans_f64(data, means0, spec.dim, spec.k, n, iters)
+    prefix = str(tmp_path / "out")
+    rc, out, err = run(harness, "--config", "1", "--N", str(n), "--iterations", str(iters), "--double", "--json", "--dump", prefix)
+    assert rc == 0, out
+    assert np.array_equal(np.fromfile(prefix + ".assignment.u32", dtype=np.uint32), want_a)
+    assert np.array_equal(np.fromfile(prefix + ".means.f64", dtype=np.uint64), want_m.view(np.uint64))
 
 
 def test_no_device_is_an_error_not_a_fallback(harness, km):
@@ -115,6 +128,22 @@ def test_device_assignment_only_and_reference_dataset(harness, gpu):
         assert rc == 0 and "Verifying results ... OK" in err, err
     rc, out, err = run(harness, "--algorithm", "hip_lds_fma", "--assignmentOnly", "--dim", "100")
     assert rc == 2 and "not supported" in out
+
+
+@pytest.mark.gpu
+def test_device_algorithms_verify_in_double(harness, gpu):
+    for algo in ("hip_best", "hip_base", "hip_base_shm", "hip_fused", "cuda_best"):
+        rc, out, err = run(harness, "--config", "1", "--double", "--algorithm", algo, "--iterations", "1", "--verify",
+                           "--serialThreads", "8", "--json")
+        assert rc == 0, out + err
+        rep = json.loads(out)
+        assert rep["verify_errors"] == 0 and rep["assignment_mismatches"] == 0 and rep["centroid_error"] < 1e-10
+    rc, out, err = run(harness, "--double", "--assignmentOnly", "--algorithm", "hip_best", "--N", "64k", "--k", "256", "--dim", "16",
+                       "--verify", "--serialThreads", "8")
+    assert rc == 0 and "Verifying results ... OK" in err, err
+    # the matrix-core sweeps are float-only and say so
+    rc, out, err = run(harness, "--double", "--algorithm", "hip_mfma", "--iterations", "1")
+    assert rc == 2 and "built for doubles" in out
 
 
 @pytest.mark.gpu
