@@ -107,7 +107,7 @@ int launch_assign_bf16(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws
 	KMX_LAUNCH_CHECK("pack_means_bf16_kernel");
 
 	/* tau = kd (|x|^2 + max|c|^2), kd = (14 d + 224) 2^-23 (see the bound at the top of the file) */
-	const float kd = (14.0f * (float)a.dim + 224.0f) * 1.1920929e-07f;
+	const float kd = (14.0f * (float)a.dim + 224.0f) * 1.1920929e-07f + a.kd_extra;
 	switch (kb) {
 	case 1: rc = launch_bf16_1(a, exec, ws, dev, kp, kd); break;
 	case 2: rc = launch_bf16_2(a, exec, ws, dev, kp, kd); break;
@@ -118,6 +118,7 @@ int launch_assign_bf16(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws
 	default: return fail(KMX_ERR_UNSUPPORTED, "assign (split-bf16 MFMA): dim %u is not supported", a.dim);
 	}
 	if (rc) return rc;
+	if (a.ranking_only) return KMX_OK; /* the caller resolves the queued points */
 	return launch_recheck(a, ws, kp);
 }
 

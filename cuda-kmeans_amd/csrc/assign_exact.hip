@@ -354,7 +354,7 @@ static __device__ __forceinline__ void evaluate_pair(const float* __restrict__ d
 
 constexpr uint32_t POINTS_BATCH = 64;
 
-template <int LD, int DPAD, bool FULL> /* FULL: dim == DPAD, no guards on the coordinate loads */
+template <int LD, int DPAD, bool FULL, int CPL> /* FULL: dim == DPAD, no guards on the coordinate loads; CPL: centroids per lane */
 __global__ void __launch_bounds__(1024)
 recheck_points_kernel(const float* __restrict__ data, size_t stride, const float* __restrict__ means_t, const float* __restrict__ norms,
                       uint32_t* __restrict__ assignment, uint32_t dim, uint32_t k, uint32_t kp,
@@ -379,12 +379,20 @@ recheck_points_kernel(const float* __restrict__ data, size_t stride, const float
 		const uint32_t next = (batch + gridDim.x) * pb;
 		const float touched = next < count ? touch_rows<LD>(data, stride, dim, queue, next, min(pb, count - next)) : 0.0f;
 		const uint32_t start = wave * here / waves;
-		for (uint32_t base = 0; base < k; base += blockDim.x) {
-			const uint32_t r = base + threadIdx.x, rr = min(r, k - 1); /* lanes past the end load a valid row, unconditionally, and never pass the screen */
-			float c[DPAD];
+		for (uint32_t base = 0; base < k; base += blockDim.x * CPL) {
+			/* The scalar cache delivers about one dword per cycle to the compute units that share it, which is half of
+			 * what their SIMDs consume when every multiply-add takes a fresh scalar operand: with two centroids per lane
+			 * every coordinate of a point is used twice. */
+			uint32_t r[CPL];
+			float c[CPL][DPAD], c2[CPL];
 #pragma unroll
-			for (int q = 0; q < DPAD; ++q) c[q] = (FULL || (uint32_t)q < dim) ? means_t[(size_t)q * kp + rr] : 0.0f;
-			const float c2 = r < k ? norms[norm_at(r)] : __builtin_inff();
+			for (int u = 0; u < CPL; ++u) {
+				r[u] = base + u * blockDim.x + threadIdx.x;
+				const uint32_t rr = min(r[u], k - 1); /* lanes past the end load a valid row, unconditionally, and never pass the screen */
+#pragma unroll
+				for (int q = 0; q < DPAD; ++q) c[u][q] = (FULL || (uint32_t)q < dim) ? means_t[(size_t)q * kp + rr] : 0.0f;
+				c2[u] = r[u] < k ? norms[norm_at(r[u])] : __builtin_inff();
+			}
 #pragma unroll 2
 			for (uint32_t step = 0; step < here; ++step) {
 				const uint32_t i = DPAD < 16 ? step : (start + step < here ? start + step : start + step - here); /* short rows: not worth the arithmetic */
@@ -393,25 +401,33 @@ recheck_points_kernel(const float* __restrict__ data, size_t stride, const float
 				float x[DPAD];
 #pragma unroll
 				for (int q = 0; q < DPAD; ++q) x[q] = (FULL || (uint32_t)q < dim) ? data[elem<LD>(stride, pt, q)] : 0.0f;
-				float dot = 0.0f;
+				float dot[CPL];
 #pragma unroll
-				for (int q = 0; q < DPAD; ++q) dot = __builtin_fmaf(x[q], c[q], dot);
-				if (r < k && !(__builtin_fmaf(-2.0f, dot, c2) > thr)) {
-					if constexpr (DPAD >= 16) { /* noted, and evaluated below by one lane per pair */
-						const uint32_t slot = atomicAdd(&hit_count, 1u);
-						if (slot < HIT_CAP) { hit_point[slot] = i; hit_centroid[slot] = r; }
-						else evaluate_pair<LD>(data, stride, means_t, dim, kp, pt, r, &best_key[i]);
-					} else { /* a short row is evaluated on the spot from the registers */
-						float sum = 0.0f;
+				for (int u = 0; u < CPL; ++u) dot[u] = 0.0f;
 #pragma unroll
-						for (int q = 0; q < DPAD; ++q) { /* padding: (0-0)^2 = +0 leaves the sum unchanged */
-							float diff = x[q] - c[q];
-							float sq = diff * diff;
-							sum = sum + sq;
+				for (int q = 0; q < DPAD; ++q) {
+#pragma unroll
+					for (int u = 0; u < CPL; ++u) dot[u] = __builtin_fmaf(x[q], c[u][q], dot[u]);
+				}
+#pragma unroll
+				for (int u = 0; u < CPL; ++u) {
+					if (r[u] < k && !(__builtin_fmaf(-2.0f, dot[u], c2[u]) > thr)) {
+						if constexpr (DPAD >= 16) { /* noted, and evaluated below by one lane per pair */
+							const uint32_t slot = atomicAdd(&hit_count, 1u);
+							if (slot < HIT_CAP) { hit_point[slot] = i; hit_centroid[slot] = r[u]; }
+							else evaluate_pair<LD>(data, stride, means_t, dim, kp, pt, r[u], &best_key[i]);
+						} else { /* a short row is evaluated on the spot from the registers */
+							float sum = 0.0f;
+#pragma unroll
+							for (int q = 0; q < DPAD; ++q) { /* padding: (0-0)^2 = +0 leaves the sum unchanged */
+								float diff = x[q] - c[u][q];
+								float sq = diff * diff;
+								sum = sum + sq;
+							}
+							const float dist = __builtin_sqrtf(sum);
+							const unsigned long long key = (r[u] == 0 && dist != dist) ? 0ull : (((unsigned long long)__float_as_uint(dist) << 32) | r[u]);
+							atomicMin(&best_key[i], key);
 						}
-						const float dist = __builtin_sqrtf(sum);
-						const unsigned long long key = (r == 0 && dist != dist) ? 0ull : (((unsigned long long)__float_as_uint(dist) << 32) | r);
-						atomicMin(&best_key[i], key);
 					}
 				}
 			}
@@ -576,14 +592,17 @@ static int launch_recheck_dpad(const AssignArgs& a, Workspace* ws, uint32_t kp)
 template <int LD, int DPAD>
 static int launch_recheck_points(const AssignArgs& a, Workspace* ws, uint32_t kp)
 {
-	const uint32_t threads = std::min<uint32_t>(1024, round_up(a.k, WAVE));
-	const dim3 grid(DPAD <= 32 ? 512 : 256); /* two work-groups fit a compute unit while a row takes at most 32 registers */
-	if (a.dim == DPAD)
-		hipLaunchKernelGGL((recheck_points_kernel<LD, DPAD, true>), grid, dim3(threads), 0, stream(),
-		                   a.data, a.stride, ws->means_t, ws->norms, a.assignment, a.dim, a.k, kp, ws->queue, ws->counters);
-	else
-		hipLaunchKernelGGL((recheck_points_kernel<LD, DPAD, false>), grid, dim3(threads), 0, stream(),
-		                   a.data, a.stride, ws->means_t, ws->norms, a.assignment, a.dim, a.k, kp, ws->queue, ws->counters);
+	/* two centroids per lane while their rows fit the registers and the work-group stays large */
+	constexpr int CPL = DPAD <= 32 ? 2 : 1;
+	const bool two = CPL == 2 && a.k > 512;
+	const uint32_t threads = std::min<uint32_t>(1024, round_up(two ? (a.k + 1) / 2 : a.k, WAVE));
+	const dim3 grid(DPAD <= 32 ? 512 : 256); /* two work-groups fit a compute unit while the rows of a lane take at most 64 registers */
+#define KMX_RECHECK_POINTS(FULL, C) \
+	hipLaunchKernelGGL((recheck_points_kernel<LD, DPAD, FULL, C>), grid, dim3(threads), 0, stream(), \
+	                   a.data, a.stride, ws->means_t, ws->norms, a.assignment, a.dim, a.k, kp, ws->queue, ws->counters)
+	if (a.dim == DPAD) { if (two) KMX_RECHECK_POINTS(true, CPL); else KMX_RECHECK_POINTS(true, 1); }
+	else { if (two) KMX_RECHECK_POINTS(false, CPL); else KMX_RECHECK_POINTS(false, 1); }
+#undef KMX_RECHECK_POINTS
 	KMX_LAUNCH_CHECK("recheck_points_kernel");
 	return KMX_OK;
 }

@@ -214,7 +214,7 @@ int launch_assign_lds_fma(const AssignArgs& a, kmx_exec_params* exec, Workspace*
 	const uint32_t kp = round_up(a.k, TILE);
 	int rc = launch_pack_means(a, ws, dp, kp);
 	if (rc) return rc;
-	const float kd = (8.0f * (float)a.dim + 24.0f) * 1.1920929e-07f;
+	const float kd = (8.0f * (float)a.dim + 24.0f) * 1.1920929e-07f + a.kd_extra;
 	switch (dp) {
 	case 4: rc = launch_fma_dp<4>(a, exec, ws, dev, kp, kd); break;
 	case 8: rc = launch_fma_dp<8>(a, exec, ws, dev, kp, kd); break;
@@ -226,6 +226,7 @@ int launch_assign_lds_fma(const AssignArgs& a, kmx_exec_params* exec, Workspace*
 	default: return fail(KMX_ERR_UNSUPPORTED, "assign (LDS/FMA): dim %u is not supported", a.dim);
 	}
 	if (rc) return rc;
+	if (a.ranking_only) return KMX_OK; /* the caller resolves the queued points */
 	return launch_recheck(a, ws, kp);
 }
 

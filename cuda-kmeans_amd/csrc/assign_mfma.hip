@@ -120,7 +120,7 @@ int launch_assign_mfma(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws
 	if (rc) return rc;
 
 	/* tau = kd (|x|^2 + max|c|^2), kd = (8 d + 24) 2^-23 (see the bound at the top of the file) */
-	const float kd = (8.0f * (float)a.dim + 24.0f) * 1.1920929e-07f;
+	const float kd = (8.0f * (float)a.dim + 24.0f) * 1.1920929e-07f + a.kd_extra;
 	switch (dph) {
 	case 2: rc = launch_mfma_2(a, exec, ws, dev, kp, kd); break;
 	case 4: rc = launch_mfma_4(a, exec, ws, dev, kp, kd); break;
@@ -134,6 +134,7 @@ int launch_assign_mfma(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws
 	default: return fail(KMX_ERR_UNSUPPORTED, "assign (MFMA): dim %u is not supported", a.dim);
 	}
 	if (rc) return rc;
+	if (a.ranking_only) return KMX_OK; /* the caller resolves the queued points */
 	return launch_recheck(a, ws, kp);
 }
 

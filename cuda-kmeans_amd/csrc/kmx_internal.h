@@ -90,6 +90,11 @@ struct AssignArgs {
 	const float* means; int layout_means; size_t stride_means;
 	uint32_t* assignment;
 	uint32_t dim, k, n;
+	/* The double-precision entry point runs the float sweeps on rounded copies of its inputs as a ranking stage:
+	 * kd_extra widens the certificate by the effect of that rounding, and ranking_only leaves the queue of
+	 * uncertified points (pairs of point number and threshold, length in counters[0]) to the caller. */
+	float kd_extra = 0.0f;
+	bool ranking_only = false;
 };
 
 struct UpdateArgs {
@@ -100,6 +105,9 @@ struct UpdateArgs {
 	uint32_t dim, k, n;
 	bool divide = true; /* false: leave the member sums in `means` (the update micro-benchmark) */
 };
+
+/* kmx_runtime.hip: runs one assignment variant (KMX_ASSIGN_BEST: chosen by shape); *chosen receives the concrete variant */
+int dispatch_assign(int variant, const AssignArgs& a, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev, int* chosen);
 
 /* assign_exact.hip */
 int launch_assign_base(const AssignArgs& a, kmx_exec_params* exec);

@@ -144,6 +144,48 @@ __global__ void fill_zero_kernel(uint32_t* __restrict__ p, size_t count)
 
 using namespace kmx;
 
+static int g_last_assign_variant = -1; /* concrete variant of the last assignment sweep (kmx_assign_f32, or the ranking stage of kmx_assign_f64) */
+
+namespace kmx {
+
+int dispatch_assign(int variant, const AssignArgs& a, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev, int* chosen)
+{
+	if (variant == KMX_ASSIGN_BEST) {
+		/* counterpart of BestCachedAssignmentKernel::run (reference kernels.cu:706-717): pick by shape.
+		 * Measured: the split-bf16 sweep is about twice as fast as the fp32 one wherever the sweep dominates; it hands
+		 * 2-3 times as many points to the exact pass, which costs more than it saves for very short rows and for
+		 * few centroids (HBM-bound shapes). The fp32 MFMA sweep beat the plain-VALU variant at every shape except
+		 * a handful of centroids, where that variant reads them through the scalar cache. */
+		if (a.k <= 32 && lds_fma_supports(a, dev) && lds_fma_reads_through_scalar_cache(a)) variant = KMX_ASSIGN_LDS_FMA;
+		else if (bf16_supports(a, dev) && a.dim >= 8 && a.k >= 64) variant = KMX_ASSIGN_MFMA_BF16X3;
+		else if (mfma_supports(a, dev)) variant = KMX_ASSIGN_MFMA;
+		else if (lds_fma_supports(a, dev)) variant = KMX_ASSIGN_LDS_FMA;
+		else variant = KMX_ASSIGN_BASE;
+	}
+	g_last_assign_variant = variant;
+	if (chosen) *chosen = variant;
+	switch (variant) {
+	case KMX_ASSIGN_BASE:
+		return launch_assign_base(a, exec);
+	case KMX_ASSIGN_LDS_FMA:
+		if (!lds_fma_supports(a, dev))
+			return fail(KMX_ERR_UNSUPPORTED, "kmx_assign_f32: shape dim=%u k=%u is not supported by the LDS/FMA variant", a.dim, a.k);
+		return launch_assign_lds_fma(a, exec, ws, dev);
+	case KMX_ASSIGN_MFMA:
+		if (!mfma_supports(a, dev))
+			return fail(KMX_ERR_UNSUPPORTED, "kmx_assign_f32: shape dim=%u k=%u is not supported by the MFMA variant", a.dim, a.k);
+		return launch_assign_mfma(a, exec, ws, dev);
+	case KMX_ASSIGN_MFMA_BF16X3:
+		if (!bf16_supports(a, dev))
+			return fail(KMX_ERR_UNSUPPORTED, "kmx_assign_f32: shape dim=%u k=%u is not supported by the split-bf16 MFMA variant", a.dim, a.k);
+		return launch_assign_bf16(a, exec, ws, dev);
+	default:
+		return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_assign_f32: unknown variant %d", variant);
+	}
+}
+
+} // namespace kmx
+
 extern "C" {
 
 const char* kmx_last_error(void) { return g_error; }
@@ -280,7 +322,6 @@ int kmx_fill_zero_u32(void* dptr, size_t count)
 	return KMX_OK;
 }
 
-static int g_last_assign_variant = -1; /* concrete variant of the last kmx_assign_f32 call */
 
 static int check_layout(const char* who, const char* what, int layout, size_t stride, uint32_t count, uint32_t dim)
 {
@@ -315,37 +356,7 @@ int kmx_assign_f32(int variant,
 	if (rc) return rc;
 
 	AssignArgs a{ data, layout, stride, means, layout_means, stride_means, assignment, dim, k, n };
-	if (variant == KMX_ASSIGN_BEST) {
-		/* counterpart of BestCachedAssignmentKernel::run (reference kernels.cu:706-717): pick by shape.
-		 * Measured: the split-bf16 sweep is about twice as fast as the fp32 one wherever the sweep dominates; it hands
-		 * 2-3 times as many points to the exact pass, which costs more than it saves for very short rows and for
-		 * few centroids (HBM-bound shapes). The fp32 MFMA sweep beat the plain-VALU variant at every shape except
-		 * a handful of centroids, where that variant reads them through the scalar cache. */
-		if (k <= 32 && lds_fma_supports(a, *dev) && lds_fma_reads_through_scalar_cache(a)) variant = KMX_ASSIGN_LDS_FMA;
-		else if (bf16_supports(a, *dev) && dim >= 8 && k >= 64) variant = KMX_ASSIGN_MFMA_BF16X3;
-		else if (mfma_supports(a, *dev)) variant = KMX_ASSIGN_MFMA;
-		else if (lds_fma_supports(a, *dev)) variant = KMX_ASSIGN_LDS_FMA;
-		else variant = KMX_ASSIGN_BASE;
-	}
-	g_last_assign_variant = variant;
-	switch (variant) {
-	case KMX_ASSIGN_BASE:
-		return launch_assign_base(a, exec);
-	case KMX_ASSIGN_LDS_FMA:
-		if (!lds_fma_supports(a, *dev))
-			return fail(KMX_ERR_UNSUPPORTED, "kmx_assign_f32: shape dim=%u k=%u is not supported by the LDS/FMA variant", dim, k);
-		return launch_assign_lds_fma(a, exec, ws, *dev);
-	case KMX_ASSIGN_MFMA:
-		if (!mfma_supports(a, *dev))
-			return fail(KMX_ERR_UNSUPPORTED, "kmx_assign_f32: shape dim=%u k=%u is not supported by the MFMA variant", dim, k);
-		return launch_assign_mfma(a, exec, ws, *dev);
-	case KMX_ASSIGN_MFMA_BF16X3:
-		if (!bf16_supports(a, *dev))
-			return fail(KMX_ERR_UNSUPPORTED, "kmx_assign_f32: shape dim=%u k=%u is not supported by the split-bf16 MFMA variant", dim, k);
-		return launch_assign_bf16(a, exec, ws, *dev);
-	default:
-		return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_assign_f32: unknown variant %d", variant);
-	}
+	return dispatch_assign(variant, a, exec, ws, *dev, nullptr);
 }
 
 int kmx_assign_last_variant(int* variant)

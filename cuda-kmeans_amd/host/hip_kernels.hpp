@@ -7,8 +7,8 @@
  * rethrown as std::runtime_error, which is how the reference's runners report unsupported shapes
  * (kernels.cu:281-282,666,675,701) and how CUCH() reports device errors.
  *
- * F = float and F = double (the reference's --double) are built; the matrix-core and single-pass kernels are
- * float-only and report that as an error for doubles.
+ * F = float and F = double (the reference's --double) are built; the single-pass fused kernel is float-only and
+ * reports that as an error for doubles.
  */
 #ifndef KMX_HOST_HIP_KERNELS_HPP
 #define KMX_HOST_HIP_KERNELS_HPP

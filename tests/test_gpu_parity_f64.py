@@ -1,7 +1,8 @@
 """Parity of the double-precision HIP path (kmx_assign_f64 / kmx_update_f64 / kmx_fused_f64, the counterpart of
 the reference's --double instantiation) with the CPU oracle's F = double functions, through the C ABI (-m gpu).
 
-Bar: assignment and counts bit-exact (the kernel evaluates the serial arithmetic itself for every pair);
+Bar: assignment and counts bit-exact (KMX_ASSIGN_BASE evaluates the serial arithmetic itself for every pair; the ranking
+sweeps behind the other variants certify their result or hand the point to that arithmetic);
 centroids within 1e-12 relative to the rms coordinate (the sums are accumulated by atomics in another order).
 """
 import json
@@ -15,6 +16,12 @@ pytestmark = pytest.mark.gpu
 HERE = os.path.dirname(os.path.abspath(__file__))
 AOS, SOA = 0, 1
 CENTROID_RTOL = 1e-12
+
+
+def F64_VARIANTS(km):
+    """BASE: serial arithmetic for every pair; LDS_FMA: fp64 FMA ranking; MFMA, MFMA_BF16X3, BEST: the float sweeps rank
+    rounded copies. All hand what they cannot certify to the serial arithmetic on the doubles."""
+    return (km.ASSIGN_BASE, km.ASSIGN_LDS_FMA, km.ASSIGN_MFMA, km.ASSIGN_MFMA_BF16X3, km.ASSIGN_BEST)
 
 
 def rel_err(got, want):
@@ -63,7 +70,7 @@ def test_first_pass_equals_reference_golden(km, gpu, golden, name):
     data = km.widen_points(km.generate_points(spec, c["n"], layout=c["layout"]))
     means0 = km.widen_points(km.first_k_means(spec, c["layout_means"]))
     want = arrays[name + "_assignment_first_pass"].astype(np.uint32)
-    for v in (km.ASSIGN_BASE, km.ASSIGN_BEST):
+    for v in F64_VARIANTS(km):
         got = gpu_assign(km, v, data, means0, c["dim"], c["k"], c["n"], c["layout"], c["layout_means"])
         assert np.array_equal(got, want), "variant %d: %d mismatches" % (v, int((got != want).sum()))
 
@@ -79,7 +86,7 @@ def test_assignment_is_bit_exact(km, orc, gpu, dim, k, n, layout, layout_means):
     data = rng.normal(size=n * dim) * 3.0
     means = rng.normal(size=k * dim) * 3.0
     want = orc.assign_f64(data, means, dim, k, n, layout, layout_means, threads=0)
-    for v in (km.ASSIGN_BASE, km.ASSIGN_BEST):
+    for v in F64_VARIANTS(km):
         got = gpu_assign(km, v, data, means, dim, k, n, layout, layout_means)
         bad = np.nonzero(got != want)[0]
         assert bad.size == 0, "variant %d: %d mismatches, first at %s" % (v, bad.size, bad[:5])
@@ -114,7 +121,7 @@ def test_hard_inputs(km, orc, gpu, dim, k, n):
         d = np.ascontiguousarray(d).ravel()
         m = np.ascontiguousarray(m).ravel()
         want = orc.assign_f64(d, m, dim, k, n, threads=0)
-        for v in (km.ASSIGN_BASE, km.ASSIGN_BEST):
+        for v in F64_VARIANTS(km):
             got = gpu_assign(km, v, d, m, dim, k, n)
             bad = np.nonzero(got != want)[0]
             assert bad.size == 0, "%s, variant %d: %d mismatches, first at %s (gpu %s, oracle %s)" % (
@@ -182,11 +189,10 @@ def test_fused_call_and_argument_errors(km, orc, gpu):
     assert np.array_equal(alg.getClusterSizes(), want_s)
     assert rel_err(alg.getMeans(), want_m) < CENTROID_RTOL
     alg.cleanup()
-    # the float-only variants say so instead of running something else
-    for bad in (km.ASSIGN_MFMA, km.ASSIGN_MFMA_BF16X3, km.ASSIGN_LDS_FMA):
-        with pytest.raises(km.KmxError) as e:
-            gpu_assign(km, bad, data[:100 * spec.dim], means0, spec.dim, spec.k, 100)
-        assert e.value.code == km.KMX_ERR_UNSUPPORTED
+    with pytest.raises(km.KmxError) as e:
+        gpu_assign(km, 17, data[:100 * spec.dim], means0, spec.dim, spec.k, 100)
+    assert e.value.code == km.KMX_ERR_INVALID_ARGUMENT
+    # the single-pass fused kernel is float-only and says so instead of running something else
     with pytest.raises(km.KmxError) as e:
         a = km.HipFusedKMeansAlgorithm(km.FUSED_ONE_PASS, dtype=np.float64)
         a.initialize(spec.dim, spec.k, 100, 1, data[:100 * spec.dim], means0)

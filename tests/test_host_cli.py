@@ -141,9 +141,11 @@ def test_device_algorithms_verify_in_double(harness, gpu):
     rc, out, err = run(harness, "--double", "--assignmentOnly", "--algorithm", "hip_best", "--N", "64k", "--k", "256", "--dim", "16",
                        "--verify", "--serialThreads", "8")
     assert rc == 0 and "Verifying results ... OK" in err, err
-    # the matrix-core sweeps are float-only and say so
-    rc, out, err = run(harness, "--double", "--algorithm", "hip_mfma", "--iterations", "1")
-    assert rc == 2 and "built for doubles" in out
+    # the matrix-core sweeps rank float copies and leave the rest to the double arithmetic
+    for algo in ("hip_mfma", "hip_mfma_bf16"):
+        rc, out, err = run(harness, "--config", "2", "--N", "64k", "--double", "--algorithm", algo, "--iterations", "1", "--verify",
+                           "--serialThreads", "8", "--json")
+        assert rc == 0 and json.loads(out)["assignment_mismatches"] == 0, out + err
 
 
 @pytest.mark.gpu
