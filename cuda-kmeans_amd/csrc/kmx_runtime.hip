@@ -323,6 +323,15 @@ int kmx_fill_zero_u32(void* dptr, size_t count)
 }
 
 
+static int check_update_variant(const char* who, int variant)
+{
+	const int base = variant & ~KMX_UPDATE_EMULATED_ATOMICS;
+	if (base < KMX_UPDATE_ATOMIC_POINT || base > KMX_UPDATE_ATOMIC_WARP) return fail(KMX_ERR_INVALID_ARGUMENT, "%s: unknown variant %d", who, variant);
+	if ((variant & KMX_UPDATE_EMULATED_ATOMICS) && (base == KMX_UPDATE_ATOMIC_SHM || base == KMX_UPDATE_BASE))
+		return fail(KMX_ERR_UNSUPPORTED, "%s: emulated atomics exist for the point, fine and wavefront variants only", who);
+	return KMX_OK;
+}
+
 static int check_layout(const char* who, const char* what, int layout, size_t stride, uint32_t count, uint32_t dim)
 {
 	if (layout != KMX_AOS && layout != KMX_SOA) return fail(KMX_ERR_INVALID_ARGUMENT, "%s: unknown %s layout %d", who, what, layout);
@@ -399,8 +408,8 @@ int kmx_update_f32(int variant,
 	if (rc) return rc;
 	rc = check_layout("kmx_update_f32", "means", layout_means, stride_means, k, dim);
 	if (rc) return rc;
-	if (variant < KMX_UPDATE_ATOMIC_POINT || variant > KMX_UPDATE_ATOMIC_SHM)
-		return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_update_f32: unknown variant %d", variant);
+	rc = check_update_variant("kmx_update_f32", variant);
+	if (rc) return rc;
 	if (exec->privatized_copies == 0) exec->privatized_copies = 1;
 
 	const DeviceInfo* dev = nullptr;
@@ -429,8 +438,8 @@ int kmx_bucket_sum_f32(int variant,
 	if (rc) return rc;
 	rc = check_layout("kmx_bucket_sum_f32", "result", layout_result, stride_result, k, dim);
 	if (rc) return rc;
-	if (variant < KMX_UPDATE_ATOMIC_POINT || variant > KMX_UPDATE_ATOMIC_SHM)
-		return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_bucket_sum_f32: unknown variant %d", variant);
+	rc = check_update_variant("kmx_bucket_sum_f32", variant);
+	if (rc) return rc;
 	if (exec->privatized_copies == 0) exec->privatized_copies = 1;
 
 	const DeviceInfo* dev = nullptr;

@@ -36,6 +36,20 @@ namespace kmx {
 /* hardware fp32 atomic add without return value (global_atomic_add_f32 / ds_add_f32) */
 __device__ __forceinline__ void atomic_add_f32(float* addr, float v) { unsafeAtomicAdd(addr, v); }
 
+/* EMUL: the addition as a compare-and-swap loop (atomicAddEmul of the update micro-benchmark, reference
+ * bucketing-cuda/kernels/kernels.cu:46-57), for measuring what the hardware atomic is worth */
+template <bool EMUL>
+__device__ __forceinline__ void atomic_add_global(float* addr, float v)
+{
+	if (!EMUL) { unsafeAtomicAdd(addr, v); return; }
+	unsigned int* word = (unsigned int*)addr;
+	unsigned int old = *word, assumed;
+	do {
+		assumed = old;
+		old = atomicCAS(word, assumed, __float_as_uint(v + __uint_as_float(assumed)));
+	} while (assumed != old);
+}
+
 template <int LM>
 __device__ __forceinline__ float* privatized(float* means, size_t copy_floats, uint32_t copies)
 {
@@ -44,7 +58,7 @@ __device__ __forceinline__ float* privatized(float* means, size_t copy_floats, u
 	return means;
 }
 
-template <int LD, int LM>
+template <int LD, int LM, bool EMUL>
 __global__ void __launch_bounds__(1024)
 update_point_kernel(const float* __restrict__ data, size_t stride, const uint32_t* __restrict__ assignment,
                     float* __restrict__ means, size_t stride_means, uint32_t* __restrict__ sizes,
@@ -56,12 +70,55 @@ update_point_kernel(const float* __restrict__ data, size_t stride, const uint32_
 	for (uint32_t idx = threadIdx.x + blockIdx.x * blockDim.x; idx < n; idx += threads) {
 		uint32_t target = assignment[idx];
 		for (uint32_t d = 0; d < dim; ++d)
-			atomic_add_f32(&means[elem<LM>(stride_means, target, d)], data[elem<LD>(stride, idx, d)]);
+			atomic_add_global<EMUL>(&means[elem<LM>(stride_means, target, d)], data[elem<LD>(stride, idx, d)]);
 		atomicAdd(&sizes[target], 1u);
 	}
 }
 
+/* one wavefront per point, the lanes stride over its dimensions (atomicWarpKernel of the update micro-benchmark,
+ * reference bucketing-cuda/kernels/kernels.cu:234-251, with 64 lanes instead of 32) */
+template <int LD, int LM, bool EMUL>
+__global__ void __launch_bounds__(1024)
+update_warp_kernel(const float* __restrict__ data, size_t stride, const uint32_t* __restrict__ assignment,
+                   float* __restrict__ means, size_t stride_means, uint32_t* __restrict__ sizes,
+                   uint32_t dim, uint32_t k, uint32_t n, size_t copy_floats, uint32_t copies)
+{
+	(void)k;
+	means = privatized<LM>(means, copy_floats, copies);
+	const uint32_t waves = blockDim.x * gridDim.x / WAVE;
+	const uint32_t lane = threadIdx.x % WAVE;
+	for (uint32_t idx = (threadIdx.x + blockIdx.x * blockDim.x) / WAVE; idx < n; idx += waves) {
+		const uint32_t target = assignment[idx];
+		for (uint32_t d = lane; d < dim; d += WAVE)
+			atomic_add_global<EMUL>(&means[elem<LM>(stride_means, target, d)], data[elem<LD>(stride, idx, d)]);
+		if (lane == 0) atomicAdd(&sizes[target], 1u);
+	}
+}
+
+/* no atomics at all: one lane per element of the result walks all points and adds those of its cluster, in point
+ * order (baseKernel of the update micro-benchmark, reference bucketing-cuda/kernels/kernels.cu:163-178); the sums
+ * therefore have the bits of the serial loop. O(n k dim): a baseline for small inputs. */
 template <int LD, int LM>
+__global__ void __launch_bounds__(256)
+update_base_kernel(const float* __restrict__ data, size_t stride, const uint32_t* __restrict__ assignment,
+                   float* __restrict__ means, size_t stride_means, uint32_t* __restrict__ sizes,
+                   uint32_t dim, uint32_t k, uint32_t n)
+{
+	const uint32_t e = threadIdx.x + blockIdx.x * blockDim.x;
+	const uint32_t d = e % dim, c = e / dim;
+	if (c >= k) return;
+	float sum = 0.0f;
+	uint32_t members = 0;
+	for (uint32_t i = 0; i < n; ++i) {
+		if (assignment[i] != c) continue;
+		sum += data[elem<LD>(stride, i, d)];
+		++members;
+	}
+	means[elem<LM>(stride_means, c, d)] = sum;
+	if (d == 0) sizes[c] = members;
+}
+
+template <int LD, int LM, bool EMUL>
 __global__ void __launch_bounds__(1024)
 update_fine_kernel(const float* __restrict__ data, size_t stride, const uint32_t* __restrict__ assignment,
                    float* __restrict__ means, size_t stride_means, uint32_t* __restrict__ sizes,
@@ -75,7 +132,7 @@ update_fine_kernel(const float* __restrict__ data, size_t stride, const uint32_t
 		uint32_t d = (uint32_t)(i % dim);
 		uint32_t idx = (uint32_t)(i / dim);
 		uint32_t target = assignment[idx];
-		atomic_add_f32(&means[elem<LM>(stride_means, target, d)], data[elem<LD>(stride, idx, d)]);
+		atomic_add_global<EMUL>(&means[elem<LM>(stride_means, target, d)], data[elem<LD>(stride, idx, d)]);
 		if (d == 0) atomicAdd(&sizes[target], 1u);
 	}
 }
@@ -655,6 +712,8 @@ static int launch_update_t(int variant, const UpdateArgs& u, kmx_exec_params* ex
 	const uint32_t ipt = exec->items_per_thread ? exec->items_per_thread : 1;
 	const size_t copy_floats = copy_floats_of(u);
 	uint32_t copies = exec->privatized_copies;
+	const bool emulated = (variant & KMX_UPDATE_EMULATED_ATOMICS) != 0;
+	variant &= ~KMX_UPDATE_EMULATED_ATOMICS;
 
 	int rc = KMX_OK;
 	if (u.n > 0) {
@@ -670,21 +729,38 @@ static int launch_update_t(int variant, const UpdateArgs& u, kmx_exec_params* ex
 				copies = 1;
 			}
 		}
+#define KMX_UPDATE_LAUNCH(KERNEL, NAME) \
+	do { \
+		if (emulated) hipLaunchKernelGGL((KERNEL<LD, LM, true>), dim3(exec->block_count), dim3(block), 0, stream(), u.data, u.stride, u.assignment, \
+		                                 u.means, u.stride_means, u.cluster_sizes, u.dim, u.k, u.n, copy_floats, copies); \
+		else hipLaunchKernelGGL((KERNEL<LD, LM, false>), dim3(exec->block_count), dim3(block), 0, stream(), u.data, u.stride, u.assignment, \
+		                        u.means, u.stride_means, u.cluster_sizes, u.dim, u.k, u.n, copy_floats, copies); \
+		KMX_LAUNCH_CHECK(NAME); \
+	} while (0)
 		if (variant == KMX_UPDATE_ATOMIC_POINT) {
 			uint32_t threads = (u.n + ipt - 1) / ipt;
 			exec->block_count = (threads + block - 1) / block;
-			hipLaunchKernelGGL((update_point_kernel<LD, LM>), dim3(exec->block_count), dim3(block), 0, stream(),
-			                   u.data, u.stride, u.assignment, u.means, u.stride_means, u.cluster_sizes, u.dim, u.k, u.n, copy_floats, copies);
-			KMX_LAUNCH_CHECK("update_point_kernel");
+			KMX_UPDATE_LAUNCH(update_point_kernel, "update_point_kernel");
+		}
+		else if (variant == KMX_UPDATE_ATOMIC_WARP) {
+			size_t threads = ((size_t)u.n * WAVE + ipt - 1) / ipt;
+			exec->block_count = (uint32_t)std::min<size_t>((threads + block - 1) / block, 1u << 20);
+			KMX_UPDATE_LAUNCH(update_warp_kernel, "update_warp_kernel");
 		}
 		else if (variant == KMX_UPDATE_ATOMIC_FINE) {
 			size_t threads = ((size_t)u.n * u.dim + ipt - 1) / ipt;
 			size_t blocks = (threads + block - 1) / block;
 			exec->block_count = (uint32_t)std::min<size_t>(blocks, 1u << 20);
-			hipLaunchKernelGGL((update_fine_kernel<LD, LM>), dim3(exec->block_count), dim3(block), 0, stream(),
-			                   u.data, u.stride, u.assignment, u.means, u.stride_means, u.cluster_sizes, u.dim, u.k, u.n, copy_floats, copies);
-			KMX_LAUNCH_CHECK("update_fine_kernel");
+			KMX_UPDATE_LAUNCH(update_fine_kernel, "update_fine_kernel");
 		}
+		else if (variant == KMX_UPDATE_BASE) {
+			exec->block_count = (u.k * u.dim + 255) / 256;
+			copies = 1; /* no replicas: every element of the result has one owner */
+			hipLaunchKernelGGL((update_base_kernel<LD, LM>), dim3(exec->block_count), dim3(256), 0, stream(),
+			                   u.data, u.stride, u.assignment, u.means, u.stride_means, u.cluster_sizes, u.dim, u.k, u.n);
+			KMX_LAUNCH_CHECK("update_base_kernel");
+		}
+#undef KMX_UPDATE_LAUNCH
 		if ((rc = profile_end(1))) return rc;
 	}
 

@@ -116,24 +116,26 @@ struct BucketingProblemInstance {
 };
 
 /* kernel policy classes of the micro-benchmark (bucketing-cuda/headers/kernels.cuh:44-63): one static run() each */
-#define KMX_DEFINE_BUCKETING_KERNEL(NAME, VARIANT)\
+#define KMX_DEFINE_BUCKETING_KERNEL(NAME, VARIANT, CAN_EMULATE)\
 template<typename F, class LAYOUT, int EMUL = false>\
 class NAME {\
 public:\
 	static void run(const BucketingProblemInstance<F>& in, HipExecParameters& exec)\
 	{\
 		static_assert(std::is_same<F, float>::value, "built for float data");\
-		static_assert(!EMUL, "CAS-emulated atomics are not built: gfx950 has native fp32 atomics");\
-		KMX_CHECK(kmx_bucket_sum_f32(VARIANT,\
+		/* EMUL: additions as compare-and-swap loops; kernels without global fp32 atomics ignore it, as in the reference */\
+		KMX_CHECK(kmx_bucket_sum_f32((EMUL && CAN_EMULATE) ? (VARIANT | KMX_UPDATE_EMULATED_ATOMICS) : VARIANT,\
 			in.data, LAYOUT::ID, LAYOUT::precomputeConstants(in.n, in.dim), in.indices,\
 			in.result, LAYOUT::ID, LAYOUT::precomputeConstants(in.k, in.dim),\
 			in.dim, in.k, in.n, reinterpret_cast<kmx_exec_params*>(&exec)));\
 	}\
 };
 
-KMX_DEFINE_BUCKETING_KERNEL(AtomicPointKernel, KMX_UPDATE_ATOMIC_POINT) /* bucketing-cuda/kernels/kernels.cu: atomic_point */
-KMX_DEFINE_BUCKETING_KERNEL(AtomicFineKernel, KMX_UPDATE_ATOMIC_FINE)   /* atomic_fine */
-KMX_DEFINE_BUCKETING_KERNEL(AtomicShmKernel, KMX_UPDATE_ATOMIC_SHM)     /* atomic_shm: here the tuned LDS kernels */
+KMX_DEFINE_BUCKETING_KERNEL(BaseKernel, KMX_UPDATE_BASE, false)                /* bucketing-cuda/kernels/kernels.cu:163-188 base */
+KMX_DEFINE_BUCKETING_KERNEL(AtomicPointKernel, KMX_UPDATE_ATOMIC_POINT, true)  /* :195-226 atomic_point */
+KMX_DEFINE_BUCKETING_KERNEL(AtomicWarpKernel, KMX_UPDATE_ATOMIC_WARP, true)    /* :234-266 atomic_warp, with 64-lane wavefronts */
+KMX_DEFINE_BUCKETING_KERNEL(AtomicFineKernel, KMX_UPDATE_ATOMIC_FINE, true)    /* :275-307 atomic_fine */
+KMX_DEFINE_BUCKETING_KERNEL(AtomicShmKernel, KMX_UPDATE_ATOMIC_SHM, false)     /* :317-372 atomic_shm (and the role of atomic_shm2, :381-447): here the tuned LDS kernels */
 
 /* = CudaBucketingAlgorithm (bucketing-cuda/headers/cuda.hpp:13-86): one buffer set per batch, one kernel call per batch */
 template<typename F = float, class LAYOUT = AoSLayoutPolicy<>, class KERNEL = AtomicShmKernel<F, LAYOUT>>

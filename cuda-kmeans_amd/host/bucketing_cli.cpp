@@ -5,8 +5,10 @@
  * relative tolerance of 5e-5 :104-142). Inputs: data uniform in [0,1), indices uniform in [0,k), from mt19937(seed)
  * as in the reference (:177-178).
  *
- * Algorithms: serial, hip_atomic_point, hip_atomic_fine, hip_atomic_shm (the reference's cuda_atomic_* names are
- * accepted). Not built: cuda_base, cuda_atomic_warp, cuda_atomic_shm2, the two "fake" kernels, --emul, --double.
+ * Algorithms: serial, hip_base, hip_atomic_point, hip_atomic_warp, hip_atomic_fine, hip_atomic_shm (the reference's
+ * cuda_* names are accepted; cuda_atomic_shm2 runs the same tuned LDS kernels as cuda_atomic_shm), --emul.
+ * Not built: the two "fake" kernels (non-atomic additions that race on purpose: their results are wrong by design
+ * and cannot be verified) and --double.
  */
 #include "bucketing.hpp"
 #include "cli_args.hpp"
@@ -44,7 +46,9 @@ void generate_random(std::vector<T>& data, DIST distribution, std::size_t seed)
 std::string canonicalAlgorithm(const std::string& name)
 {
 	static const std::map<std::string, std::string> aliases = {
-		{ "cuda_atomic_point", "hip_atomic_point" }, { "cuda_atomic_fine", "hip_atomic_fine" }, { "cuda_atomic_shm", "hip_atomic_shm" },
+		{ "cuda_base", "hip_base" }, { "cuda_atomic_point", "hip_atomic_point" }, { "cuda_atomic_warp", "hip_atomic_warp" },
+		{ "cuda_atomic_fine", "hip_atomic_fine" }, { "cuda_atomic_shm", "hip_atomic_shm" }, { "cuda_atomic_shm2", "hip_atomic_shm" },
+		{ "hip_atomic_shm2", "hip_atomic_shm" },
 	};
 	auto it = aliases.find(name);
 	return it == aliases.end() ? name : it->second;
@@ -107,14 +111,25 @@ void run(const ProgramArguments& args)
 	generate_random(indices, std::uniform_int_distribution<std::uint32_t>(0, (std::uint32_t)k - 1), seed);
 
 	const std::string algoName = canonicalAlgorithm(args.getString("algorithm"));
-	if (args.getBool("emul")) throw std::runtime_error("CAS-emulated atomic additions are not built (gfx950 has native fp32 atomics).");
+	if (algoName == "cuda_fake" || algoName == "cuda_fake_shm" || algoName == "hip_fake" || algoName == "hip_fake_shm")
+		throw std::runtime_error("The 'fake' kernels (non-atomic additions that race on purpose) are not built.");
 	HipExecParameters exec;
 	getHipExecParameters(args, exec);
 	std::map<std::string, std::unique_ptr<IBucketingAlgorithm<F>>> algorithms;
 	algorithms["serial"].reset(new SerialBucketingAlgorithm<F, LAYOUT>());
-	algorithms["hip_atomic_point"].reset(new HipBucketingAlgorithm<F, LAYOUT, AtomicPointKernel<F, LAYOUT>>(exec));
-	algorithms["hip_atomic_fine"].reset(new HipBucketingAlgorithm<F, LAYOUT, AtomicFineKernel<F, LAYOUT>>(exec));
-	algorithms["hip_atomic_shm"].reset(new HipBucketingAlgorithm<F, LAYOUT, AtomicShmKernel<F, LAYOUT>>(exec));
+	algorithms["hip_base"].reset(new HipBucketingAlgorithm<F, LAYOUT, BaseKernel<F, LAYOUT>>(exec));
+	if (args.getBool("emul")) {
+		algorithms["hip_atomic_point"].reset(new HipBucketingAlgorithm<F, LAYOUT, AtomicPointKernel<F, LAYOUT, true>>(exec));
+		algorithms["hip_atomic_warp"].reset(new HipBucketingAlgorithm<F, LAYOUT, AtomicWarpKernel<F, LAYOUT, true>>(exec));
+		algorithms["hip_atomic_fine"].reset(new HipBucketingAlgorithm<F, LAYOUT, AtomicFineKernel<F, LAYOUT, true>>(exec));
+		algorithms["hip_atomic_shm"].reset(new HipBucketingAlgorithm<F, LAYOUT, AtomicShmKernel<F, LAYOUT, true>>(exec));
+	}
+	else {
+		algorithms["hip_atomic_point"].reset(new HipBucketingAlgorithm<F, LAYOUT, AtomicPointKernel<F, LAYOUT>>(exec));
+		algorithms["hip_atomic_warp"].reset(new HipBucketingAlgorithm<F, LAYOUT, AtomicWarpKernel<F, LAYOUT>>(exec));
+		algorithms["hip_atomic_fine"].reset(new HipBucketingAlgorithm<F, LAYOUT, AtomicFineKernel<F, LAYOUT>>(exec));
+		algorithms["hip_atomic_shm"].reset(new HipBucketingAlgorithm<F, LAYOUT, AtomicShmKernel<F, LAYOUT>>(exec));
+	}
 	auto it = algorithms.find(algoName);
 	if (it == algorithms.end()) throw std::runtime_error("Unkown algorithm '" + algoName + "'.");
 	std::cerr << "Selected algorithm: " << algoName << std::endl;
@@ -174,8 +189,8 @@ int main(int argc, char* argv[])
 		args.registerInt("N", "Number of vectors in a batch.", 10240, 128);
 		args.registerInt("iterations", "Iterations to be performed (i.e., number of batches).", 1, 1);
 		args.registerInt("seed", "Random generator seed.", 42, 0);
-		args.registerString("algorithm", "Which algorithm is to be tested (serial, hip_atomic_point, hip_atomic_fine, hip_atomic_shm).", "serial");
-		args.registerBool("emul", "Emulate atomic additions with atomic CAS operations (not built).");
+		args.registerString("algorithm", "Which algorithm is to be tested (serial, hip_base, hip_atomic_point, hip_atomic_warp, hip_atomic_fine, hip_atomic_shm).", "serial");
+		args.registerBool("emul", "Emulate atomic additions with atomic CAS operations (point, warp and fine algorithms).");
 		args.registerEnum("layout", "Type of data layout and alignment.", "aos", { "aos", "soa", "aos32", "soa32" });
 		args.registerBool("double", "Use doubles instead of floats (not built).");
 		args.registerBool("verify", "Verify results against base (serial) algorithm.");

@@ -68,7 +68,14 @@ typedef enum kmx_assign_variant {
 typedef enum kmx_update_variant {
 	KMX_UPDATE_ATOMIC_POINT = 0, /* UpdateAtomicPointKernel: one lane per point, global atomics      */
 	KMX_UPDATE_ATOMIC_FINE = 1,  /* UpdateAtomicFineKernel: one lane per (point, dim) element        */
-	KMX_UPDATE_ATOMIC_SHM = 2    /* UpdateAtomicShmKernel: LDS-privatised partial sums, wave-aggregated flush */
+	KMX_UPDATE_ATOMIC_SHM = 2,   /* UpdateAtomicShmKernel: LDS-privatised partial sums, wave-aggregated flush */
+	/* the remaining variants of the update micro-benchmark (bucketing-cuda/headers/kernels.cuh:44-63) */
+	KMX_UPDATE_BASE = 3,         /* BaseKernel: no atomics, one lane per element of the result walks all points (sums in
+	                                point order, i.e. with the bits of the serial loop); O(n k dim), for small inputs */
+	KMX_UPDATE_ATOMIC_WARP = 4,  /* AtomicWarpKernel: one wavefront per point, lanes stride over the dimensions */
+	/* flag, or-ed to ATOMIC_POINT / ATOMIC_FINE / ATOMIC_WARP: additions as compare-and-swap loops instead of the hardware
+	 * atomic (the micro-benchmark's --emul, AtomicEmulTrait, bucketing-cuda/kernels/kernels.cu:83-91) */
+	KMX_UPDATE_EMULATED_ATOMICS = 0x100
 } kmx_update_variant;
 
 typedef struct kmx_props {
@@ -141,7 +148,7 @@ int kmx_update_f32(int variant,
  *      CudaBucketingAlgorithm::run, bucketing-cuda/headers/cuda.hpp:56-63) ----
  * result[b][d] = sum of data[i][d] over the vectors with indices[i] == b: the accumulation of kmx_update_f32 without
  * counts and without the divide, same variants (enum kmx_update_variant). Precondition as in the reference
- * (cuda.hpp:48): result (k x dim, times privatized_copies for variants 0 and 1) is zero. The sums of the replicas
+ * (cuda.hpp:48): result (k x dim, times privatized_copies for ATOMIC_POINT / _FINE / _WARP) is zero. The sums of the replicas
  * are merged into replica 0.
  */
 int kmx_bucket_sum_f32(int variant,

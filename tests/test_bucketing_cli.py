@@ -56,16 +56,37 @@ def test_errors(harness):
     assert rc == 2 and "Error: Unkown algorithm 'nope'." in out
     rc, out, err = run(harness, "--double")
     assert rc == 2 and "not built" in out
+    rc, out, err = run(harness, "--algorithm", "cuda_fake_shm")
+    assert rc == 2 and "not built" in out
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("algo", ["hip_atomic_shm", "hip_atomic_fine", "hip_atomic_point", "cuda_atomic_shm"])
+@pytest.mark.parametrize("algo", ["hip_atomic_shm", "hip_atomic_fine", "hip_atomic_point", "hip_atomic_warp", "cuda_atomic_shm",
+                                  "cuda_atomic_shm2"])
 @pytest.mark.parametrize("layout", ["aos", "soa", "aos32", "soa32"])
 def test_device_algorithms_verify(harness, gpu, algo, layout):
     rc, out, err = run(harness, "--algorithm", algo, "--layout", layout, "--N", "64k", "--k", "512", "--dim", "20",
                        "--iterations", "2", "--verify")
     assert rc == 0 and "Verifying results ... OK" in err, out + err
     assert len(out.split()) == 2
+
+
+@pytest.mark.gpu
+def test_base_and_emulated_atomics(harness, gpu, tmp_path):
+    """hip_base has no atomics and adds in point order: its sums have the bits of the serial algorithm's. --emul swaps
+    the hardware atomic for a compare-and-swap loop in the point, warp and fine algorithms."""
+    common = ["--N", "8k", "--k", "64", "--dim", "12", "--iterations", "2", "--seed", "3"]
+    a, b = str(tmp_path / "serial.txt"), str(tmp_path / "base.txt")
+    rc, out, err = run(harness, "--algorithm", "serial", "--out", a, *common)
+    assert rc == 0
+    rc, out, err = run(harness, "--algorithm", "cuda_base", "--verify", "--out", b, *common)
+    assert rc == 0 and "Verifying results ... OK" in err, out + err
+    assert open(a).read() == open(b).read()
+    for algo in ("hip_atomic_point", "hip_atomic_warp", "hip_atomic_fine", "hip_atomic_shm"):
+        rc, out, err = run(harness, "--algorithm", algo, "--emul", "--verify", "--privatizedCopies", "2", *common)
+        assert rc == 0 and "Verifying results ... OK" in err, algo + out + err
+    rc, out, err = run(harness, "--algorithm", "cuda_fake")
+    assert rc == 2 and "not built" in out
 
 
 @pytest.mark.gpu
@@ -89,7 +110,8 @@ def test_bucket_sum_entry_point_matches_numpy(km, gpu):
         np.add.at(want, idx, data.reshape(n, dim).astype(np.float64))
         d = km.DeviceBuffer(data.nbytes); d.write(data)
         i = km.DeviceBuffer(idx.nbytes); i.write(idx)
-        for variant in (km.UPDATE_ATOMIC_SHM, km.UPDATE_ATOMIC_FINE, km.UPDATE_ATOMIC_POINT):
+        for variant in (km.UPDATE_ATOMIC_SHM, km.UPDATE_ATOMIC_FINE, km.UPDATE_ATOMIC_POINT, km.UPDATE_ATOMIC_WARP,
+                        km.UPDATE_ATOMIC_FINE | km.UPDATE_EMULATED_ATOMICS, km.UPDATE_ATOMIC_WARP | km.UPDATE_EMULATED_ATOMICS):
             r = km.DeviceBuffer(4 * k * dim); r.zero()
             km.bucket_sum(variant, d, km.AOS, dim, i, r, km.AOS, dim, dim, k, n)
             km.sync()

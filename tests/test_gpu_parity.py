@@ -210,13 +210,22 @@ def test_update_matches_oracle(km, orc, gpu, dim, k, n, layout, layout_means):
     if k > 2:
         asg[asg == 1] = 0
     want_means, want_sizes = orc.update(data, asg, dim, k, n, layout, layout_means, threads=0)
-    for variant, ex in [(km.UPDATE_ATOMIC_POINT, km.ExecParams()), (km.UPDATE_ATOMIC_FINE, km.ExecParams()),
-                        (km.UPDATE_ATOMIC_SHM, km.ExecParams()),
-                        (km.UPDATE_ATOMIC_FINE, km.ExecParams(privatized_copies=3, items_per_thread=4)),
-                        (km.UPDATE_ATOMIC_SHM, km.ExecParams(shared_mem_bytes=48 * 1024))]:
+    cases = [(km.UPDATE_ATOMIC_POINT, km.ExecParams()), (km.UPDATE_ATOMIC_FINE, km.ExecParams()),
+             (km.UPDATE_ATOMIC_SHM, km.ExecParams()),
+             (km.UPDATE_ATOMIC_FINE, km.ExecParams(privatized_copies=3, items_per_thread=4)),
+             (km.UPDATE_ATOMIC_SHM, km.ExecParams(shared_mem_bytes=48 * 1024)),
+             (km.UPDATE_ATOMIC_WARP, km.ExecParams())]
+    if n <= 70000:   # the micro-benchmark's baselines: compare-and-swap loops and the O(n k dim) kernel without atomics
+        cases += [(km.UPDATE_ATOMIC_WARP | km.UPDATE_EMULATED_ATOMICS, km.ExecParams(privatized_copies=2)),
+                  (km.UPDATE_ATOMIC_POINT | km.UPDATE_EMULATED_ATOMICS, km.ExecParams()),
+                  (km.UPDATE_ATOMIC_FINE | km.UPDATE_EMULATED_ATOMICS, km.ExecParams()),
+                  (km.UPDATE_BASE, km.ExecParams())]
+    for variant, ex in cases:
         means, sizes = gpu_update(km, variant, data, asg, dim, k, n, layout, layout_means, ex)
         assert np.array_equal(sizes, want_sizes), "variant %d: counts differ" % variant
         assert rel_err(means, want_means) < CENTROID_RTOL, "variant %d" % variant
+        if variant == km.UPDATE_BASE:   # no atomics, sums in point order: the serial loop's bits
+            assert np.array_equal(means.view(np.uint32), want_means.view(np.uint32))
         if k > 2:
             lm = means.reshape(k, dim) if layout_means == AOS else means.reshape(dim, k).T
             assert np.all(lm[1] == 0), "empty cluster must stay at the origin"
