@@ -78,6 +78,9 @@ __device__ __forceinline__ bf16x8 row_unit(const float* row, uint32_t unit) { re
  * Packed row layout, in 16-byte units: block kb, half-wave h -> unit 4 kb + 2 h holds the hi parts of the
  * 8 dimensions, unit 4 kb + 2 h + 1 the mid parts.
  */
+/* rows of at least 32 dimensions: the refinement is worth halving (see track_tile) */
+template <int KB> constexpr bool fine8_bf16() { return KB >= 2; }
+
 template <int KB, int P, bool TRACK, bool COARSE>
 __device__ __forceinline__ void tile_step_bf16(const float* __restrict__ lds, const float* __restrict__ lds_norms, uint32_t tile_new,
                                                uint32_t col, uint32_t h, const SplitPoints<KB> (&b)[P],
@@ -114,9 +117,9 @@ __device__ __forceinline__ void tile_step_bf16(const float* __restrict__ lds, co
 	}
 	if (TRACK) {
 #pragma unroll
-		for (int p = 0; p < P; ++p) track_tile<COARSE>(acc_old[p], st[p], tile_old, neg_inf);
+		for (int p = 0; p < P; ++p) track_tile<COARSE, fine8_bf16<KB>()>(acc_old[p], st[p], tile_old, neg_inf);
 		constexpr int MFMAS = 3 * KB * P;
-		constexpr int VALU = (COARSE ? 16 : 67) * P;
+		constexpr int VALU = (COARSE ? (fine8_bf16<KB>() ? 20 : 16) : 67) * P;
 		if (KB <= 4) {
 			__builtin_amdgcn_sched_group_barrier(0x008, MFMAS, 0);
 			__builtin_amdgcn_sched_group_barrier(0x002, VALU, 0);
@@ -279,11 +282,11 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 			if (t + 1 < tiles) {
 				tile_step_bf16<KB, P, true, COARSE>(lds_tiles, lds_norms, t + 1, col, h, b, acc1, acc0, tile0 + t, st, neg_inf);
 #pragma unroll
-				for (int p = 0; p < P; ++p) track_tile<COARSE>(acc1[p], st[p], tile0 + t + 1, neg_inf);
+				for (int p = 0; p < P; ++p) track_tile<COARSE, fine8_bf16<KB>()>(acc1[p], st[p], tile0 + t + 1, neg_inf);
 			}
 			else {
 #pragma unroll
-				for (int p = 0; p < P; ++p) track_tile<COARSE>(acc0[p], st[p], tile0 + t, neg_inf);
+				for (int p = 0; p < P; ++p) track_tile<COARSE, fine8_bf16<KB>()>(acc0[p], st[p], tile0 + t, neg_inf);
 			}
 			if (STREAM) {
 				/* the other buffer was last read one chunk ago, before the barrier that ended that chunk */
@@ -302,22 +305,26 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 			uint32_t idx;
 			float first, second;
 			if (COARSE) {
-				/* refinement of the winning 16-row subset (see assign_mfma_impl.h); the rows are re-evaluated with
+				/* refinement of the winning group of 8 or 16 rows (see assign_mfma_impl.h); the rows are re-evaluated with
 				 * v_dot2c_f32_bf16 on the same three products, so the error bound of the MFMA results covers them */
-				const uint32_t ts = win ? st[p].tile : ot;
+				constexpr bool FINE8 = fine8_bf16<KB>();
+				constexpr int ROWS = FINE8 ? 8 : 16;
+				const uint32_t code = win ? st[p].tile : ot;
+				const uint32_t ts = FINE8 ? code >> 1 : code;      /* tile */
+				const uint32_t sub = FINE8 ? 2 * (code & 1u) : 0u; /* first group of 4 rows of the tracked group */
 				const uint32_t wh = win ? h : 1u - h;
 				const float W = win ? fminf(o1, st[p].m2) : fminf(st[p].m1, o2);
 				const float* tile_base = STREAM ? packed + (size_t)ts * tile_floats(RS) : lds + (size_t)ts * tile_floats(RS);
 				const float* norm_base = STREAM ? norms + ts * NORM_TILE : lds + (size_t)chunk_tiles * tile_floats(RS) + ts * NORM_TILE;
-				float tot[16];
+				float tot[ROWS];
 #pragma unroll
-				for (int r = 0; r < 16; ++r)
-					tot[r] = row_dot_bf16<KB>(tile_base + (size_t)(8 * (r / 4) + 4 * wh + (r % 4)) * RS, h, b[p]);
+				for (int r = 0; r < ROWS; ++r)
+					tot[r] = row_dot_bf16<KB>(tile_base + (size_t)(8 * (sub + r / 4) + 4 * wh + (r % 4)) * RS, h, b[p]);
 				float v1 = __builtin_inff(), v2 = __builtin_inff();
 				uint32_t rbest = 0;
 #pragma unroll
-				for (int g = 0; g < 4; ++g) {
-					const f32x4 c2 = *(const f32x4*)(norm_base + 8 * g + 4 * wh);
+				for (int g = 0; g < ROWS / 4; ++g) {
+					const f32x4 c2 = *(const f32x4*)(norm_base + 8 * (sub + g) + 4 * wh);
 #pragma unroll
 					for (int q = 0; q < 4; ++q) {
 						const int r = 4 * g + q;
@@ -328,7 +335,7 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 						v1 = lt ? v : v1;
 					}
 				}
-				idx = ts * TILE + 8 * (rbest / 4) + 4 * wh + (rbest % 4);
+				idx = ts * TILE + 8 * (sub + rbest / 4) + 4 * wh + (rbest % 4);
 				first = v1;
 				second = fminf(v2, W);
 			}

@@ -90,7 +90,7 @@ __device__ __forceinline__ float min2_raw(float a, float b, float neg_inf) { ret
 /* per-lane tracking state of one point: smallest value, a lower bound for all others, where the smallest was seen */
 struct Track {
 	float m1, m2;
-	uint32_t tile; /* tile of m1 */
+	uint32_t tile; /* tile of m1; with FINE8: 2 * tile + (0: results 0..7, 1: results 8..15) */
 	uint32_t loc;  /* fine mode only: row of m1 inside the tile, without the half-wave's +4 */
 };
 
@@ -98,25 +98,42 @@ struct Track {
  * COARSE = true, 16 VALU operations per tile and point: the minimum t of the lane's 16 results (a min tree),
  * then over the tiles the smallest t (m1, with its tile) and the second smallest t (m2). Which of the 16
  * rows attained m1, and how close the runner-up inside that tile is, is settled once per sweep by the
- * refinement in the kernel.
+ * refinement in the kernel, which recomputes those rows.
+ * COARSE and FINE8, 20 operations: the same for the lane's results 0..7 and 8..15 separately (`tile` then holds
+ * 2 * tile + group), so that the refinement recomputes 8 rows instead of 16: worth it when a row is long enough
+ * for the refinement to cost more than four operations per tile.
  * COARSE = false, 66 operations: exact smallest / second smallest / row over all results; used when the
  * sweep has too few tiles to pay for the refinement.
  */
-template <bool COARSE>
+template <bool COARSE, bool FINE8>
 __device__ __forceinline__ void track_tile(const f32x16& acc, Track& s, uint32_t tile, float neg_inf)
 {
 	if (COARSE) {
 		float e[8];
 #pragma unroll
 		for (int i = 0; i < 8; ++i) e[i] = min2_raw(acc[2 * i], acc[2 * i + 1], neg_inf);
-		const float f0 = fminf(fminf(e[0], e[1]), e[2]);
-		const float f1 = fminf(fminf(e[3], e[4]), e[5]);
-		const float f2 = fminf(fminf(e[6], e[7]), f0);
-		const float t = fminf(f1, f2);
-		s.m2 = __builtin_amdgcn_fmed3f(s.m1, s.m2, t); /* second smallest of {m1, m2, t} as m1 <= m2 */
-		const bool lt = t < s.m1;
-		s.tile = lt ? tile : s.tile;
-		s.m1 = lt ? t : s.m1;
+		if (FINE8) {
+			const float ta = fminf(fminf(fminf(e[0], e[1]), e[2]), e[3]); /* results 0..7 */
+			const float tb = fminf(fminf(fminf(e[4], e[5]), e[6]), e[7]); /* results 8..15 */
+			s.m2 = __builtin_amdgcn_fmed3f(s.m1, s.m2, ta); /* second smallest of {m1, m2, ta} as m1 <= m2 */
+			const bool lta = ta < s.m1;
+			s.tile = lta ? 2 * tile : s.tile;
+			s.m1 = lta ? ta : s.m1;
+			s.m2 = __builtin_amdgcn_fmed3f(s.m1, s.m2, tb);
+			const bool ltb = tb < s.m1;
+			s.tile = ltb ? 2 * tile + 1 : s.tile;
+			s.m1 = ltb ? tb : s.m1;
+		}
+		else {
+			const float f0 = fminf(fminf(e[0], e[1]), e[2]);
+			const float f1 = fminf(fminf(e[3], e[4]), e[5]);
+			const float f2 = fminf(fminf(e[6], e[7]), f0);
+			const float t = fminf(f1, f2);
+			s.m2 = __builtin_amdgcn_fmed3f(s.m1, s.m2, t); /* second smallest of {m1, m2, t} as m1 <= m2 */
+			const bool lt = t < s.m1;
+			s.tile = lt ? tile : s.tile;
+			s.m1 = lt ? t : s.m1;
+		}
 	}
 	else {
 		const float start = s.m1;
@@ -137,6 +154,9 @@ __device__ __forceinline__ void track_tile(const f32x16& acc, Track& s, uint32_t
  * tracking of the previous tile's results in acc_old, which are complete by then: no wavefront ever waits
  * for an MFMA result. sched_group_barrier keeps the MFMAs and the VALU work in GROUPS large runs.
  */
+/* rows of at least 16 dimensions: the refinement is worth halving */
+template <int DPH> constexpr bool fine8() { return DPH >= 8; }
+
 template <int DPH, int P, bool TRACK, bool COARSE>
 __device__ __forceinline__ void tile_step(const float* __restrict__ lds, const float* __restrict__ lds_norms, uint32_t tile_new,
                                           uint32_t col, uint32_t h, const float (&b)[P][DPH],
@@ -177,10 +197,10 @@ __device__ __forceinline__ void tile_step(const float* __restrict__ lds, const f
 	}
 	if (TRACK) {
 #pragma unroll
-		for (int p = 0; p < P; ++p) track_tile<COARSE>(acc_old[p], st[p], tile_old, neg_inf);
+		for (int p = 0; p < P; ++p) track_tile<COARSE, fine8<DPH>()>(acc_old[p], st[p], tile_old, neg_inf);
 		constexpr int MFMAS = DPH * P;
 		constexpr int GROUPS = COARSE ? 1 : (MFMAS >= 4 ? 4 : 1);
-		constexpr int VALU_PER_GROUP = ((COARSE ? 16 : 67) * P + GROUPS - 1) / GROUPS;
+		constexpr int VALU_PER_GROUP = ((COARSE ? (fine8<DPH>() ? 20 : 16) : 67) * P + GROUPS - 1) / GROUPS;
 		if (DPH <= 32) { /* wider rows: the tracking is a few per cent of the step, the default schedule will do */
 #pragma unroll
 			for (int i = 0; i < GROUPS; ++i) {
@@ -292,11 +312,11 @@ assign_mfma_kernel(const float* __restrict__ data, size_t stride, const float* _
 			if (t + 1 < tiles) {
 				tile_step<DPH, P, true, COARSE>(lds, lds_norms, t + 1, col, h, b, acc1, acc0, tile0 + t, st, neg_inf);
 #pragma unroll
-				for (int p = 0; p < P; ++p) track_tile<COARSE>(acc1[p], st[p], tile0 + t + 1, neg_inf);
+				for (int p = 0; p < P; ++p) track_tile<COARSE, fine8<DPH>()>(acc1[p], st[p], tile0 + t + 1, neg_inf);
 			}
 			else {
 #pragma unroll
-				for (int p = 0; p < P; ++p) track_tile<COARSE>(acc0[p], st[p], tile0 + t, neg_inf);
+				for (int p = 0; p < P; ++p) track_tile<COARSE, fine8<DPH>()>(acc0[p], st[p], tile0 + t, neg_inf);
 			}
 		}
 
@@ -311,22 +331,27 @@ assign_mfma_kernel(const float* __restrict__ data, size_t stride, const float* _
 			float first, second;
 			if (COARSE) {
 				/*
-				 * Refinement. The two half-waves hold disjoint 16-row subsets of every tile. The subset with the
-				 * smaller m1 (half wh, tile ts) contains the winner; everything outside it is bounded below by
-				 * W = min(the other half's m1, the winning half's m2). The 16 values of the winning subset are
+				 * Refinement. The two half-waves hold disjoint 16-row subsets of every tile, tracked whole or (FINE8)
+				 * as two groups of 8 rows. The tracked group with the smallest m1 (half wh, tile ts) contains the
+				 * winner; everything outside it is bounded below by W = min(the other half's m1, the winning
+				 * half's m2). The values of the winning group are
 				 * recomputed with plain fused multiply-adds (both half-waves contribute their half of the
 				 * dimensions), which yields the winner's row and the runner-up inside the subset. The
 				 * recomputed values obey the same rounding-error bound as the MFMA results, so tau covers them.
 				 */
-				const uint32_t ts = win ? st[p].tile : ot;
+				constexpr bool FINE8 = fine8<DPH>();
+				constexpr int ROWS = FINE8 ? 8 : 16;
+				const uint32_t code = win ? st[p].tile : ot;
+				const uint32_t ts = FINE8 ? code >> 1 : code;      /* tile */
+				const uint32_t sub = FINE8 ? 2 * (code & 1u) : 0u; /* first group of 4 rows of the tracked group */
 				const uint32_t wh = win ? h : 1u - h;
 				const float W = win ? fminf(o1, st[p].m2) : fminf(st[p].m1, o2);
 				const float* tile_base = STREAM ? packed + (size_t)ts * tile_floats(RS) : lds + (size_t)ts * tile_floats(RS);
 				const float* norm_base = STREAM ? norms + ts * NORM_TILE : lds_norms + ts * NORM_TILE;
-				float tot[16];
+				float tot[ROWS];
 #pragma unroll
-				for (int r = 0; r < 16; ++r) {
-					const float* ar = tile_base + (size_t)(8 * (r / 4) + 4 * wh + (r % 4)) * RS + h * DPH;
+				for (int r = 0; r < ROWS; ++r) {
+					const float* ar = tile_base + (size_t)(8 * (sub + r / 4) + 4 * wh + (r % 4)) * RS + h * DPH;
 					float part = 0.0f;
 					if (DPH % 4 == 0) {
 #pragma unroll
@@ -351,8 +376,8 @@ assign_mfma_kernel(const float* __restrict__ data, size_t stride, const float* _
 				float v1 = __builtin_inff(), v2 = __builtin_inff();
 				uint32_t rbest = 0;
 #pragma unroll
-				for (int g = 0; g < 4; ++g) {
-					const f32x4 c2 = *(const f32x4*)(norm_base + 8 * g + 4 * wh);
+				for (int g = 0; g < ROWS / 4; ++g) {
+					const f32x4 c2 = *(const f32x4*)(norm_base + 8 * (sub + g) + 4 * wh);
 #pragma unroll
 					for (int q = 0; q < 4; ++q) {
 						const int r = 4 * g + q;
@@ -363,7 +388,7 @@ assign_mfma_kernel(const float* __restrict__ data, size_t stride, const float* _
 						v1 = lt ? v : v1;
 					}
 				}
-				idx = ts * TILE + 8 * (rbest / 4) + 4 * wh + (rbest % 4);
+				idx = ts * TILE + 8 * (sub + rbest / 4) + 4 * wh + (rbest % 4);
 				first = v1;
 				second = fminf(v2, W);
 			}
