@@ -269,16 +269,16 @@ requeued_f64_kernel(const double* __restrict__ data, size_t stride, const double
  */
 constexpr int BATCH = 16;
 
-template <int LD>
+template <int LD, bool SCREEN>
 __global__ void __launch_bounds__(1024)
-requeued_batch_f64_kernel(const double* __restrict__ data, size_t stride, const double* __restrict__ means_t,
+requeued_batch_f64_kernel(const double* __restrict__ data, size_t stride, const double* __restrict__ means_t, const double* __restrict__ norms,
                           uint32_t* __restrict__ assignment, uint32_t dim, uint32_t k, uint32_t kp,
                           const uint32_t* __restrict__ queue, uint32_t queue_stride, const uint32_t* __restrict__ queue_length)
 {
 	extern __shared__ double rows[]; /* BATCH x dim */
 	__shared__ unsigned long long chunk_min[BATCH];
 	__shared__ uint32_t chunk_arg[BATCH];
-	__shared__ double best_dist[BATCH];
+	__shared__ double best_dist[BATCH], threshold[BATCH];
 	__shared__ uint32_t best_arg[BATCH], pinned[BATCH], point_of[BATCH];
 	constexpr uint32_t NONE = 0xffffffffu;
 	const uint32_t total = *queue_length;
@@ -286,7 +286,12 @@ requeued_batch_f64_kernel(const double* __restrict__ data, size_t stride, const 
 		const uint32_t here = min((uint32_t)BATCH, total - first);
 		__syncthreads(); /* the previous batch is written out */
 		if (threadIdx.x < BATCH) {
-			point_of[threadIdx.x] = queue[(size_t)(first + min(threadIdx.x, here - 1)) * queue_stride];
+			const size_t entry = (size_t)(first + min(threadIdx.x, here - 1)) * queue_stride;
+			point_of[threadIdx.x] = queue[entry];
+			/* SCREEN: the queue holds (point, threshold) pairs of a float sweep: only a centroid whose ranking value
+			 * c^2 - 2 c.x does not exceed the threshold can be the serial choice (the threshold is the sweep's best
+			 * value plus its certificate, which covers the sweep's errors; the double ranking value is more accurate) */
+			threshold[threadIdx.x] = SCREEN ? (double)__uint_as_float(queue[entry + 1]) : __builtin_inf();
 			best_dist[threadIdx.x] = __builtin_inf();
 			best_arg[threadIdx.x] = NONE;
 			pinned[threadIdx.x] = 0;
@@ -297,36 +302,65 @@ requeued_batch_f64_kernel(const double* __restrict__ data, size_t stride, const 
 			__syncthreads(); /* rows are in place; the previous chunk is merged */
 			if (threadIdx.x < BATCH) { chunk_min[threadIdx.x] = ~0ull; chunk_arg[threadIdx.x] = NONE; }
 			const uint32_t j = base + threadIdx.x, jj = min(j, kp - 1);
-			double sum[BATCH];
+			double dist[BATCH];
+			uint32_t takes_part = 0; /* bit b: this lane's centroid is evaluated for point b */
+			if (SCREEN) {
+				double dot[BATCH];
 #pragma unroll
-			for (int b = 0; b < BATCH; ++b) sum[b] = 0.0;
+				for (int b = 0; b < BATCH; ++b) dot[b] = 0.0;
 #pragma unroll 2
-			for (uint32_t q = 0; q < dim; ++q) {
-				const double c = means_t[(size_t)q * kp + jj];
+				for (uint32_t q = 0; q < dim; ++q) {
+					const double c = means_t[(size_t)q * kp + jj];
+#pragma unroll
+					for (int b = 0; b < BATCH; ++b) dot[b] = __builtin_fma(rows[b * dim + q], c, dot[b]);
+				}
+				const double c2 = norms[jj];
 #pragma unroll
 				for (int b = 0; b < BATCH; ++b) {
-					double diff = rows[b * dim + q] - c;
-					double sq = diff * diff;
-					sum[b] = sum[b] + sq;
+					dist[b] = 0.0;
+					if (j < k && !(__builtin_fma(-2.0, dot[b], c2) > threshold[b])) { /* rare */
+						double sum = 0.0;
+#pragma unroll 8
+						for (uint32_t q = 0; q < dim; ++q) {
+							double diff = rows[b * dim + q] - means_t[(size_t)q * kp + jj];
+							double sq = diff * diff;
+							sum = sum + sq;
+						}
+						dist[b] = __builtin_sqrt(sum);
+						takes_part |= 1u << b;
+					}
 				}
 			}
-			double dist[BATCH];
+			else {
+				double sum[BATCH];
 #pragma unroll
-			for (int b = 0; b < BATCH; ++b) dist[b] = __builtin_sqrt(sum[b]);
+				for (int b = 0; b < BATCH; ++b) sum[b] = 0.0;
+#pragma unroll 2
+				for (uint32_t q = 0; q < dim; ++q) {
+					const double c = means_t[(size_t)q * kp + jj];
+#pragma unroll
+					for (int b = 0; b < BATCH; ++b) {
+						double diff = rows[b * dim + q] - c;
+						double sq = diff * diff;
+						sum[b] = sum[b] + sq;
+					}
+				}
+#pragma unroll
+				for (int b = 0; b < BATCH; ++b) dist[b] = __builtin_sqrt(sum[b]);
+				takes_part = j < k ? 0xffffu : 0u;
+			}
 			__syncthreads(); /* chunk_min is reset */
-			if (j < k) {
 #pragma unroll
-				for (int b = 0; b < BATCH; ++b) {
+			for (int b = 0; b < BATCH; ++b) {
+				if (takes_part & (1u << b)) {
 					if (dist[b] == dist[b]) atomicMin(&chunk_min[b], (unsigned long long)__double_as_longlong(dist[b]));
 					else if (j == 0) pinned[b] = 1;
 				}
 			}
 			__syncthreads();
-			if (j < k) {
 #pragma unroll
-				for (int b = 0; b < BATCH; ++b)
-					if ((unsigned long long)__double_as_longlong(dist[b]) == chunk_min[b] && dist[b] == dist[b]) atomicMin(&chunk_arg[b], j);
-			}
+			for (int b = 0; b < BATCH; ++b)
+				if ((takes_part & (1u << b)) && dist[b] == dist[b] && (unsigned long long)__double_as_longlong(dist[b]) == chunk_min[b]) atomicMin(&chunk_arg[b], j);
 			__syncthreads();
 			if (threadIdx.x < BATCH && chunk_arg[threadIdx.x] != NONE) {
 				const double d = __longlong_as_double((long long)chunk_min[threadIdx.x]);
@@ -590,9 +624,12 @@ int launch_assign_f64_ld(int variant, const double* data, size_t stride, uint32_
 	} while (0)
 #define KMX_F64_REQUEUED_BY_DIM() \
 	do { \
-		if (batched) \
-			hipLaunchKernelGGL((requeued_batch_f64_kernel<LD>), bgrid, dim3(batch_threads), (size_t)BATCH * dim * sizeof(double), stream(), \
-			                   data, stride, g_means_t, assignment, dim, k, kp, exact_queue, exact_stride, exact_length); \
+		if (batched && float_queue) \
+			hipLaunchKernelGGL((requeued_batch_f64_kernel<LD, true>), bgrid, dim3(batch_threads), (size_t)BATCH * dim * sizeof(double), stream(), \
+			                   data, stride, g_means_t, g_norms, assignment, dim, k, kp, exact_queue, exact_stride, exact_length); \
+		else if (batched) \
+			hipLaunchKernelGGL((requeued_batch_f64_kernel<LD, false>), bgrid, dim3(batch_threads), (size_t)BATCH * dim * sizeof(double), stream(), \
+			                   data, stride, g_means_t, g_norms, assignment, dim, k, kp, exact_queue, exact_stride, exact_length); \
 		else if (dim > 32) KMX_F64_REQUEUED(0); \
 		else if (dim <= 8) KMX_F64_REQUEUED(8); \
 		else if (dim <= 16) KMX_F64_REQUEUED(16); \
