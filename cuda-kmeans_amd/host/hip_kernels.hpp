@@ -182,19 +182,21 @@ KMX_DEFINE_FUSED_KERNEL(FusedTwoPassKernel, KMX_FUSED_TWO_PASS) /* assignment sw
 KMX_DEFINE_FUSED_KERNEL(FusedOnePassKernel, KMX_FUSED_ONE_PASS) /* one kernel, a handful of centroids */
 KMX_DEFINE_FUSED_KERNEL(FusedBestKernel, KMX_FUSED_BEST)        /* one pass where it applies */
 
-#define KMX_DEFINE_UPDATE_KERNEL(NAME, VARIANT)\
+/* EMUL (the reference's template argument, kernels.cuh:96-105): additions as compare-and-swap loops; built for the float
+ * point and fine kernels (KMX_UPDATE_EMULATED_ATOMICS), ignored by the LDS kernels, which have no global fp32 atomics to emulate */
+#define KMX_DEFINE_UPDATE_KERNEL(NAME, VARIANT, CAN_EMULATE)\
 template<typename F, typename IDX_T, class LAYOUT, class LAYOUT_MEANS, int EMUL = false>\
 class NAME {\
 public:\
 	static void run(const UpdateProblemInstance<F, IDX_T>& in, HipExecParameters& exec)\
 	{\
-		static_assert(!EMUL, "CAS-emulated atomics are not built: gfx950 has native fp32 atomics");\
-		hip_detail::update<F, IDX_T, LAYOUT, LAYOUT_MEANS>(VARIANT, in, exec);\
+		static_assert(!(EMUL && CAN_EMULATE) || std::is_same<F, float>::value, "emulated atomics are built for floats");\
+		hip_detail::update<F, IDX_T, LAYOUT, LAYOUT_MEANS>((EMUL && CAN_EMULATE) ? (VARIANT | KMX_UPDATE_EMULATED_ATOMICS) : VARIANT, in, exec);\
 	}\
 };
 
-KMX_DEFINE_UPDATE_KERNEL(UpdateAtomicPointKernel, KMX_UPDATE_ATOMIC_POINT) /* kernels.cu:726-761 */
-KMX_DEFINE_UPDATE_KERNEL(UpdateAtomicFineKernel, KMX_UPDATE_ATOMIC_FINE)   /* kernels.cu:770-809 */
-KMX_DEFINE_UPDATE_KERNEL(UpdateAtomicShmKernel, KMX_UPDATE_ATOMIC_SHM)     /* kernels.cu:817-878 */
+KMX_DEFINE_UPDATE_KERNEL(UpdateAtomicPointKernel, KMX_UPDATE_ATOMIC_POINT, true) /* kernels.cu:726-761 */
+KMX_DEFINE_UPDATE_KERNEL(UpdateAtomicFineKernel, KMX_UPDATE_ATOMIC_FINE, true)   /* kernels.cu:770-809 */
+KMX_DEFINE_UPDATE_KERNEL(UpdateAtomicShmKernel, KMX_UPDATE_ATOMIC_SHM, false)    /* kernels.cu:817-878 */
 
 #endif
