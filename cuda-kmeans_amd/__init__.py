@@ -31,7 +31,7 @@ KMX_OK, KMX_ERR_INVALID_ARGUMENT, KMX_ERR_UNSUPPORTED, KMX_ERR_DEVICE, KMX_ERR_N
 ABI_SYMBOLS = [
     "kmx_device_count", "kmx_set_device", "kmx_device_props", "kmx_malloc", "kmx_free", "kmx_h2d", "kmx_d2h",
     "kmx_d2d", "kmx_sync", "kmx_set_stream", "kmx_shutdown", "kmx_fill_zero_u32", "kmx_assign_f32",
-    "kmx_assign_last_rechecked", "kmx_assign_last_variant", "kmx_update_f32", "kmx_bucket_sum_f32", "kmx_fused_f32", "kmx_assign_f64", "kmx_update_f64", "kmx_fused_f64",
+    "kmx_assign_last_rechecked", "kmx_assign_last_variant", "kmx_update_f32", "kmx_bucket_sum_f32", "kmx_fused_f32", "kmx_assign_f64", "kmx_update_f64", "kmx_fused_f64", "kmx_bucket_sum_f64",
     "kmx_graph_begin", "kmx_graph_end", "kmx_graph_launch", "kmx_graph_destroy", "kmx_event_create", "kmx_event_destroy", "kmx_event_record",
     "kmx_event_elapsed_ms", "kmx_set_profiling", "kmx_last_kernel_ms", "kmx_last_error",
 ]
@@ -114,6 +114,7 @@ def hip_lib():
         lib.kmx_assign_f64.argtypes = lib.kmx_assign_f32.argtypes
         lib.kmx_update_f64.argtypes = lib.kmx_update_f32.argtypes
         lib.kmx_fused_f64.argtypes = lib.kmx_fused_f32.argtypes
+        lib.kmx_bucket_sum_f64.argtypes = lib.kmx_bucket_sum_f32.argtypes
         lib.kmx_graph_begin.argtypes = []
         lib.kmx_graph_end.argtypes = [ctypes.POINTER(vp)]
         lib.kmx_graph_launch.argtypes = [vp]
@@ -308,10 +309,11 @@ def update(variant, data_buf, layout, stride, assignment_buf, means_buf, layout_
 
 
 def bucket_sum(variant, data_buf, layout, stride, indices_buf, result_buf, layout_result, stride_result, dim, k, n,
-               exec_params=None):
-    """KERNEL::run of the update micro-benchmark (bucketing-cuda/headers/kernels.cuh:44-63) through kmx_bucket_sum_f32."""
+               exec_params=None, dtype=np.float32):
+    """KERNEL::run of the update micro-benchmark (bucketing-cuda/headers/kernels.cuh:44-63) through kmx_bucket_sum_f32 / _f64."""
     ex = exec_params if exec_params is not None else ExecParams()
-    check(hip_lib().kmx_bucket_sum_f32(variant, data_buf.ptr, layout, stride, indices_buf.ptr, result_buf.ptr,
+    fn = hip_lib().kmx_bucket_sum_f64 if _is_double(dtype) else hip_lib().kmx_bucket_sum_f32
+    check(fn(variant, data_buf.ptr, layout, stride, indices_buf.ptr, result_buf.ptr,
                                        layout_result, stride_result, dim, k, n, ctypes.byref(ex)))
     return ex
 

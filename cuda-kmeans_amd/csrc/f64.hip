@@ -669,7 +669,7 @@ int launch_assign_f64_ld(int variant, const double* data, size_t stride, uint32_
 
 template <int LD, int LM>
 int launch_update_f64_t(int variant, const double* data, size_t stride, const uint32_t* assignment, double* means, size_t stride_means,
-                        uint32_t* sizes, uint32_t dim, uint32_t k, uint32_t n, kmx_exec_params* exec, const DeviceInfo& dev)
+                        uint32_t* sizes, uint32_t dim, uint32_t k, uint32_t n, kmx_exec_params* exec, const DeviceInfo& dev, bool divide)
 {
 	const size_t private_bytes = ((size_t)k * dim) * sizeof(double) + (size_t)k * sizeof(uint32_t);
 	const bool use_private = variant == KMX_UPDATE_ATOMIC_SHM && private_bytes <= 32 * 1024;
@@ -709,6 +709,7 @@ int launch_update_f64_t(int variant, const double* data, size_t stride, const ui
 			                   data, stride, assignment, means, stride_means, sizes, dim, k, n);
 		KMX_LAUNCH_CHECK("update_f64_kernel");
 	}
+	if (!divide) return KMX_OK; /* the update micro-benchmark wants the sums */
 	hipLaunchKernelGGL((divide_means_f64_kernel<LM>), dim3((k * dim + 255) / 256), dim3(256), 0, stream(), means, stride_means, sizes, dim, k);
 	KMX_LAUNCH_CHECK("divide_means_f64_kernel");
 	return KMX_OK;
@@ -816,6 +817,41 @@ extern "C" int kmx_assign_f64(int variant,
 	return float_queue ? KMX_OK : profile_end(0);
 }
 
+static int update_f64_call(const char* who, bool divide, int variant,
+                           const double* data, int layout, size_t stride,
+                           const uint32_t* assignment,
+                           double* means, int layout_means, size_t stride_means,
+                           uint32_t* cluster_sizes,
+                           uint32_t dim, uint32_t k, uint32_t n, kmx_exec_params* exec)
+{
+	if (!exec) return fail(KMX_ERR_INVALID_ARGUMENT, "%s: exec is null", who);
+	if (dim == 0 || k == 0) return fail(KMX_ERR_INVALID_ARGUMENT, "%s: dim and k must be positive", who);
+	if (!means || !cluster_sizes) return fail(KMX_ERR_INVALID_ARGUMENT, "%s: null device pointer", who);
+	if (n > 0 && (!data || !assignment)) return fail(KMX_ERR_INVALID_ARGUMENT, "%s: null device pointer", who);
+	int rc = check_layout_f64(who, "data", layout, stride, n, dim);
+	if (rc) return rc;
+	rc = check_layout_f64(who, "means", layout_means, stride_means, k, dim);
+	if (rc) return rc;
+	if (variant < KMX_UPDATE_ATOMIC_POINT || variant > KMX_UPDATE_ATOMIC_SHM)
+		return fail(KMX_ERR_INVALID_ARGUMENT, "%s: unknown variant %d (doubles: ATOMIC_POINT, ATOMIC_FINE, ATOMIC_SHM)", who, variant);
+	if (exec->privatized_copies > 1)
+		return fail(KMX_ERR_UNSUPPORTED, "%s: privatized copies in global memory are not built for doubles", who);
+	if ((uint64_t)k * dim > 0xffffffffull) return fail(KMX_ERR_UNSUPPORTED, "%s: k * dim does not fit 32 bits", who);
+	const DeviceInfo* dev = nullptr;
+	rc = device_info(&dev);
+	if (rc) return rc;
+
+	rc = profile_begin(1);
+	if (rc) return rc;
+#define KMX_F64_UPDATE(LD, LM) \
+	launch_update_f64_t<LD, LM>(variant, data, stride, assignment, means, stride_means, cluster_sizes, dim, k, n, exec, *dev, divide)
+	if (layout == KMX_AOS) rc = layout_means == KMX_AOS ? KMX_F64_UPDATE(KMX_AOS, KMX_AOS) : KMX_F64_UPDATE(KMX_AOS, KMX_SOA);
+	else rc = layout_means == KMX_AOS ? KMX_F64_UPDATE(KMX_SOA, KMX_AOS) : KMX_F64_UPDATE(KMX_SOA, KMX_SOA);
+#undef KMX_F64_UPDATE
+	if (rc) return rc;
+	return profile_end(1);
+}
+
 extern "C" int kmx_update_f64(int variant,
                               const double* data, int layout, size_t stride,
                               const uint32_t* assignment,
@@ -824,32 +860,28 @@ extern "C" int kmx_update_f64(int variant,
                               uint32_t dim, uint32_t k, uint32_t n, kmx_exec_params* exec)
 {
 	clear_error();
-	if (!exec) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_update_f64: exec is null");
-	if (dim == 0 || k == 0) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_update_f64: dim and k must be positive");
-	if (!means || !cluster_sizes) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_update_f64: null device pointer");
-	if (n > 0 && (!data || !assignment)) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_update_f64: null device pointer");
-	int rc = check_layout_f64("kmx_update_f64", "data", layout, stride, n, dim);
-	if (rc) return rc;
-	rc = check_layout_f64("kmx_update_f64", "means", layout_means, stride_means, k, dim);
-	if (rc) return rc;
-	if (variant < KMX_UPDATE_ATOMIC_POINT || variant > KMX_UPDATE_ATOMIC_SHM)
-		return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_update_f64: unknown variant %d", variant);
-	if (exec->privatized_copies > 1)
-		return fail(KMX_ERR_UNSUPPORTED, "kmx_update_f64: privatized copies in global memory are not built for doubles");
-	if ((uint64_t)k * dim > 0xffffffffull) return fail(KMX_ERR_UNSUPPORTED, "kmx_update_f64: k * dim does not fit 32 bits");
-	const DeviceInfo* dev = nullptr;
-	rc = device_info(&dev);
-	if (rc) return rc;
+	return update_f64_call("kmx_update_f64", true, variant, data, layout, stride, assignment, means, layout_means, stride_means, cluster_sizes,
+	                       dim, k, n, exec);
+}
 
-	rc = profile_begin(1);
+extern "C" int kmx_bucket_sum_f64(int variant,
+                                  const double* data, int layout, size_t stride,
+                                  const uint32_t* indices,
+                                  double* result, int layout_result, size_t stride_result,
+                                  uint32_t dim, uint32_t k, uint32_t n, kmx_exec_params* exec)
+{
+	clear_error();
+	if (k == 0) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_bucket_sum_f64: dim and k must be positive");
+	Workspace* ws = nullptr;
+	int rc = workspace(&ws);
 	if (rc) return rc;
-#define KMX_F64_UPDATE(LD, LM) \
-	launch_update_f64_t<LD, LM>(variant, data, stride, assignment, means, stride_means, cluster_sizes, dim, k, n, exec, *dev)
-	if (layout == KMX_AOS) rc = layout_means == KMX_AOS ? KMX_F64_UPDATE(KMX_AOS, KMX_AOS) : KMX_F64_UPDATE(KMX_AOS, KMX_SOA);
-	else rc = layout_means == KMX_AOS ? KMX_F64_UPDATE(KMX_SOA, KMX_AOS) : KMX_F64_UPDATE(KMX_SOA, KMX_SOA);
-#undef KMX_F64_UPDATE
+	/* the kernels count members as they go; the counts land in a scratch array */
+	rc = reserve_bucket_sizes(ws, k);
 	if (rc) return rc;
-	return profile_end(1);
+	rc = kmx_fill_zero_u32(ws->bucket_sizes, k);
+	if (rc) return rc;
+	return update_f64_call("kmx_bucket_sum_f64", false, variant, data, layout, stride, indices, result, layout_result, stride_result,
+	                       ws->bucket_sizes, dim, k, n, exec);
 }
 
 extern "C" int kmx_fused_f64(int variant,

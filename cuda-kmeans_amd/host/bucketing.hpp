@@ -115,6 +115,14 @@ struct BucketingProblemInstance {
 		: data(_data), indices(_indices), result(_result), dim((std::uint32_t)_dim), k((std::uint32_t)_k), n((std::uint32_t)_n) {}
 };
 
+/* the C ABI has one entry point per element type (doubles: the atomic point, fine and shm kernels) */
+inline int bucket_sum_call(int variant, const float* data, int layout, std::size_t stride, const std::uint32_t* indices, float* result,
+	int layoutResult, std::size_t strideResult, std::uint32_t dim, std::uint32_t k, std::uint32_t n, kmx_exec_params* exec)
+{ return kmx_bucket_sum_f32(variant, data, layout, stride, indices, result, layoutResult, strideResult, dim, k, n, exec); }
+inline int bucket_sum_call(int variant, const double* data, int layout, std::size_t stride, const std::uint32_t* indices, double* result,
+	int layoutResult, std::size_t strideResult, std::uint32_t dim, std::uint32_t k, std::uint32_t n, kmx_exec_params* exec)
+{ return kmx_bucket_sum_f64(variant, data, layout, stride, indices, result, layoutResult, strideResult, dim, k, n, exec); }
+
 /* kernel policy classes of the micro-benchmark (bucketing-cuda/headers/kernels.cuh:44-63): one static run() each */
 #define KMX_DEFINE_BUCKETING_KERNEL(NAME, VARIANT, CAN_EMULATE)\
 template<typename F, class LAYOUT, int EMUL = false>\
@@ -122,9 +130,8 @@ class NAME {\
 public:\
 	static void run(const BucketingProblemInstance<F>& in, HipExecParameters& exec)\
 	{\
-		static_assert(std::is_same<F, float>::value, "built for float data");\
 		/* EMUL: additions as compare-and-swap loops; kernels without global fp32 atomics ignore it, as in the reference */\
-		KMX_CHECK(kmx_bucket_sum_f32((EMUL && CAN_EMULATE) ? (VARIANT | KMX_UPDATE_EMULATED_ATOMICS) : VARIANT,\
+		KMX_CHECK(bucket_sum_call((EMUL && CAN_EMULATE) ? (VARIANT | KMX_UPDATE_EMULATED_ATOMICS) : VARIANT,\
 			in.data, LAYOUT::ID, LAYOUT::precomputeConstants(in.n, in.dim), in.indices,\
 			in.result, LAYOUT::ID, LAYOUT::precomputeConstants(in.k, in.dim),\
 			in.dim, in.k, in.n, reinterpret_cast<kmx_exec_params*>(&exec)));\

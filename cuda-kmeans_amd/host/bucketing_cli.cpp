@@ -8,7 +8,7 @@
  * Algorithms: serial, hip_base, hip_atomic_point, hip_atomic_warp, hip_atomic_fine, hip_atomic_shm (the reference's
  * cuda_* names are accepted; cuda_atomic_shm2 runs the same tuned LDS kernels as cuda_atomic_shm), --emul.
  * Not built: the two "fake" kernels (non-atomic additions that race on purpose: their results are wrong by design
- * and cannot be verified) and --double.
+ * and cannot be verified). --double: the serial algorithm and the atomic point, fine and shm kernels.
  */
 #include "bucketing.hpp"
 #include "cli_args.hpp"
@@ -192,7 +192,7 @@ int main(int argc, char* argv[])
 		args.registerString("algorithm", "Which algorithm is to be tested (serial, hip_base, hip_atomic_point, hip_atomic_warp, hip_atomic_fine, hip_atomic_shm).", "serial");
 		args.registerBool("emul", "Emulate atomic additions with atomic CAS operations (point, warp and fine algorithms).");
 		args.registerEnum("layout", "Type of data layout and alignment.", "aos", { "aos", "soa", "aos32", "soa32" });
-		args.registerBool("double", "Use doubles instead of floats (not built).");
+		args.registerBool("double", "Use doubles instead of floats (serial, hip_atomic_point, hip_atomic_fine, hip_atomic_shm).");
 		args.registerBool("verify", "Verify results against base (serial) algorithm.");
 		args.registerString("out", "Path to a file where the results are saved.", "");
 		args.registerInt("privatizedCopies", "Number of privatized copies in global memory (relevant only to some algorithms).", 1, 1, 4096);
@@ -212,8 +212,8 @@ int main(int argc, char* argv[])
 	}
 
 	try {
-		if (args.getBool("double")) throw std::runtime_error("The double-precision variant is not built.");
-		select_layout_and_run<float>(args);
+		if (args.getBool("double")) select_layout_and_run<double>(args);
+		else select_layout_and_run<float>(args);
 	}
 	catch (std::exception& e) {
 		std::cout << "Error: " << e.what() << std::endl << std::endl;

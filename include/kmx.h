@@ -204,6 +204,12 @@ int kmx_update_f64(int variant,
                    double* means, int layout_means, size_t stride_means,
                    uint32_t* cluster_sizes,
                    uint32_t dim, uint32_t k, uint32_t n, kmx_exec_params* exec);
+/* kmx_bucket_sum_f32 on doubles (the micro-benchmark's --double): variants ATOMIC_POINT, ATOMIC_FINE, ATOMIC_SHM */
+int kmx_bucket_sum_f64(int variant,
+                       const double* data, int layout, size_t stride,
+                       const uint32_t* indices,
+                       double* result, int layout_result, size_t stride_result,
+                       uint32_t dim, uint32_t k, uint32_t n, kmx_exec_params* exec);
 int kmx_fused_f64(int variant,
                   const double* data, int layout, size_t stride,
                   const double* means_in, double* means_out, int layout_means, size_t stride_means,

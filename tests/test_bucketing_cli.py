@@ -54,8 +54,8 @@ def test_errors(harness):
     assert rc == 1 and out.startswith("Invalid arguments:") and "default 20" in out
     rc, out, err = run(harness, "--algorithm", "nope")
     assert rc == 2 and "Error: Unkown algorithm 'nope'." in out
-    rc, out, err = run(harness, "--double")
-    assert rc == 2 and "not built" in out
+    rc, out, err = run(harness, "--double", "--N", "1k", "--k", "8", "--dim", "3")   # the serial algorithm on doubles
+    assert rc == 0 and len(out.split()) == 2
     rc, out, err = run(harness, "--algorithm", "cuda_fake_shm")
     assert rc == 2 and "not built" in out
 
@@ -87,6 +87,16 @@ def test_base_and_emulated_atomics(harness, gpu, tmp_path):
         assert rc == 0 and "Verifying results ... OK" in err, algo + out + err
     rc, out, err = run(harness, "--algorithm", "cuda_fake")
     assert rc == 2 and "not built" in out
+
+
+@pytest.mark.gpu
+def test_double_precision(harness, gpu):
+    for algo in ("hip_atomic_shm", "hip_atomic_fine", "hip_atomic_point", "cuda_atomic_shm2"):
+        for extra in (["--k", "512", "--dim", "20"], ["--k", "16", "--dim", "16", "--layout", "soa"], ["--k", "2048", "--dim", "32"]):
+            rc, out, err = run(harness, "--double", "--algorithm", algo, "--N", "64k", "--iterations", "2", "--verify", *extra)
+            assert rc == 0 and "Verifying results ... OK" in err, algo + " ".join(extra) + out + err
+    rc, out, err = run(harness, "--double", "--algorithm", "hip_base")   # the baselines of the micro-benchmark are float-only
+    assert rc == 2 and "doubles" in out
 
 
 @pytest.mark.gpu
