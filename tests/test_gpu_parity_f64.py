@@ -76,7 +76,7 @@ def test_first_pass_equals_reference_golden(km, gpu, golden, name):
 
 
 SHAPES = [(20, 128, 10240), (3, 5, 257), (7, 33, 1000), (2, 2, 128), (16, 16, 5000), (32, 1000, 4099), (64, 96, 2048),
-          (100, 40, 1500), (256, 300, 700), (1, 7, 300), (5, 4100, 777), (9, 8, 64), (33, 9, 513)]
+          (100, 40, 1500), (256, 300, 700), (1, 7, 300), (5, 4100, 777), (9, 8, 64), (33, 9, 513), (4, 1, 100), (3, 5, 1), (40, 1, 1)]
 
 
 @pytest.mark.parametrize("dim,k,n", SHAPES)
