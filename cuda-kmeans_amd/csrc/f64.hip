@@ -34,8 +34,8 @@
  * Update. One lane per element of the input (coalesced in either layout), as in the reference's updateAtomicFineKernel
  * (kernels.cu:770-809), with fp64 atomics, which gfx950 has natively in LDS and in L2: a work-group first adds into a
  * private copy of the sums in LDS when k * d doubles fit 32 KB and flushes it with one global atomic per element;
- * larger sums are split into ranges of clusters that fit, one work-group per (slice of the points, range); beyond 8 ranges,
- * and for the POINT / FINE variants, the lanes add to global memory directly. Counts are
+ * larger sums are split into ranges of clusters that fit, one work-group per (slice of the points, range); beyond 256
+ * ranges, and for the POINT / FINE variants, the lanes add to global memory directly. Counts are
  * integer atomics issued by the lane of dimension 0.
  * The order of the additions is not the serial one (it is not in the reference's kernels either).
  */
@@ -516,48 +516,54 @@ update_f64_kernel(const double* __restrict__ data, size_t stride, const uint32_t
 }
 
 /*
- * Sums that do not fit one private copy: the clusters are split into ranges whose sums do (range_size clusters),
- * and work-group (slice, range) walks its slice of the points and adds only those assigned to its range, so every
- * addition still is an LDS atomic and every row still is read from HBM once (the assignment vector is read once per
- * range). BY_POINT (rows of at least 64 doubles): a wavefront takes whole points, the test for the range is uniform;
- * else one lane per element.
+ * Sums that do not fit one private copy: the clusters are split into ranges whose sums fit 32 KB of LDS, and work-group
+ * (slice, range) walks its slice of the points in pieces of 8192: first it scans the piece's assignments (4 bytes per
+ * point, coalesced) and lists the points of its range in LDS, then all lanes add the listed rows, one lane per
+ * element, with LDS atomics. Every row is read from HBM once, by the work-group of its cluster's range; only the
+ * assignment vector is read once per range. Listing first keeps all lanes busy in the second step and makes its loads
+ * independent of each other (testing the assignment in the adding loop left most lanes idle behind a dependent load).
  */
-template <int LD, int LM, bool BY_POINT>
+constexpr uint32_t RANGE_BYTES = 32 * 1024;  /* private sums of one range */
+constexpr uint32_t PIECE_POINTS = 8192;      /* listed per step: 13 bits of position, the rest of the word for the cluster */
+
+template <int LD, int LM>
 __global__ void __launch_bounds__(1024)
 update_ranges_f64_kernel(const double* __restrict__ data, size_t stride, const uint32_t* __restrict__ assignment,
                          double* __restrict__ means, size_t stride_means, uint32_t* __restrict__ sizes,
                          uint32_t dim, uint32_t k, uint32_t n, uint32_t range_size, uint32_t slices)
 {
-	extern __shared__ double sums[]; /* range_size * dim doubles, then range_size counts */
+	extern __shared__ double sums[]; /* range_size * dim doubles, range_size counts, PIECE_POINTS list entries */
+	__shared__ uint32_t listed;
 	uint32_t* counts = (uint32_t*)(sums + (size_t)range_size * dim);
+	uint32_t* list = counts + range_size;
 	const uint32_t slice = blockIdx.x % slices, range = blockIdx.x / slices;
 	const uint32_t c0 = range * range_size, cn = min(range_size, k - c0);
 	for (uint32_t e = threadIdx.x; e < cn * dim; e += blockDim.x) sums[e] = 0.0;
 	for (uint32_t e = threadIdx.x; e < cn; e += blockDim.x) counts[e] = 0;
-	__syncthreads();
-	if (BY_POINT) {
-		const uint32_t lane = threadIdx.x & (WAVE - 1);
-		const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE), waves = blockDim.x / WAVE;
-#pragma unroll 4
-		for (uint32_t i = slice * waves + wave; i < n; i += slices * waves) {
-			const uint32_t c = assignment[i] - c0; /* uniform */
-			if (c < cn) {
-				for (uint32_t q = lane; q < dim; q += WAVE) unsafeAtomicAdd(&sums[(size_t)c * dim + q], data[elem<LD>(stride, i, q)]);
-				if (lane == 0) atomicAdd(&counts[c], 1u);
-			}
-		}
-	}
-	else {
-		const size_t total = (size_t)n * dim;
-#pragma unroll 4
-		for (size_t e = (size_t)slice * blockDim.x + threadIdx.x; e < total; e += (size_t)slices * blockDim.x) {
-			const uint32_t i = LD == KMX_AOS ? (uint32_t)(e / dim) : (uint32_t)(e % n);
-			const uint32_t q = LD == KMX_AOS ? (uint32_t)(e % dim) : (uint32_t)(e / n);
+	const uint32_t per_slice = (n + slices - 1) / slices;
+	const uint32_t s0 = min(slice * per_slice, n), s1 = min(s0 + per_slice, n);
+	for (uint32_t p0 = s0; p0 < s1; p0 += PIECE_POINTS) {
+		__syncthreads(); /* sums are zero / the previous piece is added */
+		if (threadIdx.x == 0) listed = 0;
+		__syncthreads();
+		const uint32_t p1 = min(p0 + PIECE_POINTS, s1);
+		for (uint32_t i = p0 + threadIdx.x; i < p1; i += blockDim.x) {
 			const uint32_t c = assignment[i] - c0;
 			if (c < cn) {
-				unsafeAtomicAdd(&sums[(size_t)c * dim + q], data[elem<LD>(stride, i, q)]);
-				if (q == 0) atomicAdd(&counts[c], 1u);
+				list[atomicAdd(&listed, 1u)] = (i - p0) | (c << 13);
+				atomicAdd(&counts[c], 1u);
 			}
+		}
+		__syncthreads();
+		const uint32_t members = listed;
+		const uint32_t total = members * dim;
+#pragma unroll 4
+		for (uint32_t e = threadIdx.x; e < total; e += blockDim.x) {
+			/* consecutive lanes: consecutive dimensions of a row (AoS) / consecutive listed points of a dimension (SoA) */
+			const uint32_t m = LD == KMX_AOS ? e / dim : e % members;
+			const uint32_t q = LD == KMX_AOS ? e % dim : e / members;
+			const uint32_t entry = list[m];
+			unsafeAtomicAdd(&sums[(size_t)(entry >> 13) * dim + q], data[elem<LD>(stride, p0 + (entry & (PIECE_POINTS - 1)), q)]);
 		}
 	}
 	__syncthreads();
@@ -673,11 +679,11 @@ int launch_update_f64_t(int variant, const double* data, size_t stride, const ui
 {
 	const size_t private_bytes = ((size_t)k * dim) * sizeof(double) + (size_t)k * sizeof(uint32_t);
 	const bool use_private = variant == KMX_UPDATE_ATOMIC_SHM && private_bytes <= 32 * 1024;
-	/* ranges of clusters whose sums fit 64 KB of LDS; rows beyond that (dim > 8000) go to global atomics */
-	const uint32_t range_size = (uint32_t)std::min<size_t>(k, (64 * 1024) / ((size_t)dim * sizeof(double) + sizeof(uint32_t)));
+	/* ranges of clusters whose sums fit RANGE_BYTES of LDS (the cluster number must fit the list entry's 19 bits, which it
+	 * does: at most RANGE_BYTES / 12 clusters); rows beyond that (dim > 4000) go to global atomics */
+	const uint32_t range_size = (uint32_t)std::min<size_t>(k, RANGE_BYTES / ((size_t)dim * sizeof(double) + sizeof(uint32_t)));
 	const uint32_t ranges = range_size ? (k + range_size - 1) / range_size : 0;
-	const bool by_point = dim >= 64;
-	const bool use_ranges = variant == KMX_UPDATE_ATOMIC_SHM && !use_private && range_size > 0 && ranges <= 8; /* measured: with 32 ranges (d = 256, k = 1024) the global atomics win */
+	const bool use_ranges = variant == KMX_UPDATE_ATOMIC_SHM && !use_private && range_size > 0 && ranges <= 256;
 	const dim3 block(256);
 	const size_t total = (size_t)n * dim;
 	/* a work-group with private sums should add at least 16 times as many elements as it has sums to clear and flush */
@@ -687,17 +693,13 @@ int launch_update_f64_t(int variant, const double* data, size_t stride, const ui
 	exec->block_size = block.x;
 	exec->block_count = grid.x;
 	if (n > 0 && use_ranges) {
-		const size_t range_bytes = (size_t)range_size * dim * sizeof(double) + (size_t)range_size * sizeof(uint32_t);
-		const dim3 wide(1024); /* the ranges take the whole LDS budget of a work-group: make it a large one */
+		const size_t range_bytes = (size_t)range_size * dim * sizeof(double) + (size_t)range_size * sizeof(uint32_t) + PIECE_POINTS * sizeof(uint32_t);
+		const dim3 wide(1024);
 		const size_t per_slice = std::max<size_t>(1024, 16 * (size_t)range_size * dim);
 		const uint32_t slices = (uint32_t)std::max<size_t>(1, std::min<size_t>((total + per_slice - 1) / per_slice, std::max<size_t>(1, (size_t)dev.compute_units * 2 / ranges)));
 		exec->block_count = slices * ranges;
-		if (by_point)
-			hipLaunchKernelGGL((update_ranges_f64_kernel<LD, LM, true>), dim3(slices * ranges), wide, range_bytes, stream(),
-			                   data, stride, assignment, means, stride_means, sizes, dim, k, n, range_size, slices);
-		else
-			hipLaunchKernelGGL((update_ranges_f64_kernel<LD, LM, false>), dim3(slices * ranges), wide, range_bytes, stream(),
-			                   data, stride, assignment, means, stride_means, sizes, dim, k, n, range_size, slices);
+		hipLaunchKernelGGL((update_ranges_f64_kernel<LD, LM>), dim3(slices * ranges), wide, range_bytes, stream(),
+		                   data, stride, assignment, means, stride_means, sizes, dim, k, n, range_size, slices);
 		KMX_LAUNCH_CHECK("update_ranges_f64_kernel");
 	}
 	else if (n > 0) {
