@@ -72,11 +72,20 @@ __global__ void reset_f64_kernel(unsigned long long* __restrict__ misc)
 	if (threadIdx.x < 2) misc[threadIdx.x] = 0;
 }
 
-/* round-to-nearest float copy; values beyond the float range become infinities, tiny ones zeros or subnormals */
+/* round-to-nearest float copy; values beyond the float range become infinities, tiny ones zeros or subnormals.
+ * Four elements per lane and step (two 16-byte loads, one 16-byte store); both buffers are 16-byte aligned. */
+typedef double f64x2 __attribute__((ext_vector_type(2)));
+
 __global__ void __launch_bounds__(256)
 round_to_float_kernel(const double* __restrict__ in, float* __restrict__ out, size_t count)
 {
-	for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < count; e += (size_t)gridDim.x * blockDim.x) out[e] = (float)in[e];
+	const size_t quads = count / 4;
+	for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < quads; e += (size_t)gridDim.x * blockDim.x) {
+		const f64x2 a = ((const f64x2*)in)[2 * e], b = ((const f64x2*)in)[2 * e + 1];
+		const f32x4 r = { (float)a.x, (float)a.y, (float)b.x, (float)b.y };
+		((f32x4*)out)[e] = r;
+	}
+	if (blockIdx.x == 0 && threadIdx.x < count % 4) out[4 * quads + threadIdx.x] = (float)in[4 * quads + threadIdx.x];
 }
 
 /* one lane per (padded) centroid: transposed copy, |c|^2, and the largest |c|^2 as the maximum of the bit patterns
@@ -787,9 +796,9 @@ extern "C" int kmx_assign_f64(int variant,
 		if (rc) return rc;
 		rc = reserve_f64(&g_means32, &g_means32_cap, means_extent / 2 + 1);
 		if (rc) return rc;
-		hipLaunchKernelGGL(round_to_float_kernel, dim3((uint32_t)std::min<size_t>((data_extent + 255) / 256, (size_t)dev->compute_units * 16)), dim3(256), 0,
+		hipLaunchKernelGGL(round_to_float_kernel, dim3((uint32_t)std::min<size_t>((data_extent + 1023) / 1024, (size_t)dev->compute_units * 32)), dim3(256), 0,
 		                   stream(), data, (float*)g_data32, data_extent);
-		hipLaunchKernelGGL(round_to_float_kernel, dim3((uint32_t)std::min<size_t>((means_extent + 255) / 256, (size_t)dev->compute_units * 16)), dim3(256), 0,
+		hipLaunchKernelGGL(round_to_float_kernel, dim3((uint32_t)std::min<size_t>((means_extent + 1023) / 1024, (size_t)dev->compute_units * 32)), dim3(256), 0,
 		                   stream(), means, (float*)g_means32, means_extent);
 		KMX_LAUNCH_CHECK("round_to_float_kernel");
 		Workspace* ws = nullptr;

@@ -187,8 +187,8 @@ int kmx_fused_f32(int variant,
  *   KMX_ASSIGN_LDS_FMA ranks with fp64 FMAs; KMX_ASSIGN_MFMA, _MFMA_BF16X3 and _BEST rank float copies of the inputs with the
  *   float sweeps (work space: n * dim + k * dim floats); all hand the points they cannot certify to the serial arithmetic
  *   on the doubles.
- * kmx_update_f64: every update variant; ATOMIC_SHM privatises the sums in LDS (whole when k * dim doubles fit 32 KB, in up
- *   to 8 ranges of clusters beyond), the others (and larger k * dim) use fp64 atomics in global memory. privatized_copies > 1: KMX_ERR_UNSUPPORTED.
+ * kmx_update_f64: ATOMIC_POINT / _FINE / _SHM; ATOMIC_SHM privatises the sums in LDS (whole when k * dim doubles fit 32 KB,
+ *   in ranges of clusters of that size beyond), the others (and more than 256 ranges) use fp64 atomics in global memory. privatized_copies > 1: KMX_ERR_UNSUPPORTED.
  *   Precondition as for kmx_update_f32: means and cluster_sizes are zero (kmx_fill_zero_u32 with twice the count).
  * kmx_fused_f64: KMX_FUSED_TWO_PASS / KMX_FUSED_BEST (assignment into the work space, then the update);
  *   KMX_FUSED_ONE_PASS is float-only: KMX_ERR_UNSUPPORTED.
