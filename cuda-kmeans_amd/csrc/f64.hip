@@ -532,7 +532,7 @@ update_f64_kernel(const double* __restrict__ data, size_t stride, const uint32_t
  * assignment vector is read once per range. Listing first keeps all lanes busy in the second step and makes its loads
  * independent of each other (testing the assignment in the adding loop left most lanes idle behind a dependent load).
  */
-constexpr uint32_t RANGE_BYTES = 32 * 1024;  /* private sums of one range */
+constexpr uint32_t RANGE_BYTES = 32 * 1024 - 64; /* private sums of one range (with the list: just below 64 KB) */
 constexpr uint32_t PIECE_POINTS = 8192;      /* listed per step: 13 bits of position, the rest of the word for the cluster */
 
 template <int LD, int LM>
@@ -625,7 +625,7 @@ int launch_assign_f64_ld(int variant, const double* data, size_t stride, uint32_
 	hipLaunchKernelGGL((assign_f64_kernel<LD, DPAD, G>), grid, block, 0, stream(), data, stride, g_means_t, assignment, dim, k, kp, n)
 	/* queued points: many centroids and rows long enough to pay for the work-group-wide minimum -> batches of points
 	 * against one lane per centroid; else 16 lanes (2 for few centroids) share a point */
-	const bool batched = k >= 256 && dim >= 16 && (size_t)BATCH * dim * sizeof(double) <= 64 * 1024;
+	const bool batched = k >= 256 && dim >= 16 && (size_t)BATCH * dim * sizeof(double) <= 48 * 1024; /* dynamic + static LDS stay below 64 KB */
 	const uint32_t batch_threads = std::min<uint32_t>(1024, (k + WAVE - 1) / WAVE * WAVE);
 	const dim3 bgrid(std::min<uint32_t>((n + BATCH - 1) / BATCH, dev.compute_units * 2));
 	const bool many = k >= 256;
