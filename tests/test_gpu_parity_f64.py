@@ -76,7 +76,7 @@ def test_first_pass_equals_reference_golden(km, gpu, golden, name):
 
 
 SHAPES = [(20, 128, 10240), (3, 5, 257), (7, 33, 1000), (2, 2, 128), (16, 16, 5000), (32, 1000, 4099), (64, 96, 2048),
-          (100, 40, 1500), (256, 300, 700), (1, 7, 300), (5, 4100, 777), (9, 8, 64), (33, 9, 513), (4, 1, 100), (3, 5, 1), (40, 1, 1)]
+          (100, 40, 1500), (256, 300, 700), (1, 7, 300), (5, 4100, 777), (9, 8, 64), (33, 9, 513), (4, 1, 100), (3, 5, 1), (40, 1, 1), (300, 260, 300), (400, 256, 200)]
 
 
 @pytest.mark.parametrize("dim,k,n", SHAPES)
@@ -87,6 +87,10 @@ def test_assignment_is_bit_exact(km, orc, gpu, dim, k, n, layout, layout_means):
     means = rng.normal(size=k * dim) * 3.0
     want = orc.assign_f64(data, means, dim, k, n, layout, layout_means, threads=0)
     for v in F64_VARIANTS(km):
+        if dim > 256 and v in (km.ASSIGN_MFMA, km.ASSIGN_MFMA_BF16X3):
+            with pytest.raises(km.KmxError):   # the matrix-core sweeps take rows of up to 256 dimensions, for either element type
+                gpu_assign(km, v, data, means, dim, k, n, layout, layout_means)
+            continue
         got = gpu_assign(km, v, data, means, dim, k, n, layout, layout_means)
         bad = np.nonzero(got != want)[0]
         assert bad.size == 0, "variant %d: %d mismatches, first at %s" % (v, bad.size, bad[:5])
@@ -129,7 +133,7 @@ def test_hard_inputs(km, orc, gpu, dim, k, n):
 
 
 UPDATE_SHAPES = [(8, 64, 65536), (20, 128, 10240), (3, 5, 257), (32, 1024, 50000), (4, 4096, 100000), (16, 16, 300000),
-                 (256, 1024, 4096), (33, 7, 1000)]
+                 (256, 1024, 4096), (33, 7, 1000), (300, 260, 3000), (5000, 3, 64)]
 
 
 @pytest.mark.parametrize("dim,k,n", UPDATE_SHAPES)
