@@ -119,7 +119,7 @@ __device__ __forceinline__ void tile_step_bf16(const float* __restrict__ lds, co
 #pragma unroll
 		for (int p = 0; p < P; ++p) track_tile<COARSE, fine8_bf16<KB>()>(acc_old[p], st[p], tile_old, neg_inf);
 		constexpr int MFMAS = 3 * KB * P;
-		constexpr int VALU = (COARSE ? (fine8_bf16<KB>() ? 20 : 16) : 67) * P;
+		constexpr int VALU = (COARSE ? (fine8_bf16<KB>() ? 16 : 12) : 67) * P;
 		if (KB <= 4) {
 			__builtin_amdgcn_sched_group_barrier(0x008, MFMAS, 0);
 			__builtin_amdgcn_sched_group_barrier(0x002, VALU, 0);

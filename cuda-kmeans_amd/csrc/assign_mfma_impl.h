@@ -95,11 +95,11 @@ struct Track {
 };
 
 /*
- * COARSE = true, 16 VALU operations per tile and point: the minimum t of the lane's 16 results (a min tree),
+ * COARSE = true, 12 VALU operations per tile and point: the minimum t of the lane's 16 results (a min tree),
  * then over the tiles the smallest t (m1, with its tile) and the second smallest t (m2). Which of the 16
  * rows attained m1, and how close the runner-up inside that tile is, is settled once per sweep by the
  * refinement in the kernel, which recomputes those rows.
- * COARSE and FINE8, 20 operations: the same for the lane's results 0..7 and 8..15 separately (`tile` then holds
+ * COARSE and FINE8, 16 operations: the same for the lane's results 0..7 and 8..15 separately (`tile` then holds
  * 2 * tile + group), so that the refinement recomputes 8 rows instead of 16: worth it when a row is long enough
  * for the refinement to cost more than four operations per tile.
  * COARSE = false, 66 operations: exact smallest / second smallest / row over all results; used when the
@@ -109,12 +109,14 @@ template <bool COARSE, bool FINE8>
 __device__ __forceinline__ void track_tile(const f32x16& acc, Track& s, uint32_t tile, float neg_inf)
 {
 	if (COARSE) {
-		float e[8];
-#pragma unroll
-		for (int i = 0; i < 8; ++i) e[i] = min2_raw(acc[2 * i], acc[2 * i + 1], neg_inf);
+		/* Minimum trees in v_minimum3_f32 (two values per instruction; unlike fminf() it needs no canonicalised operands,
+		 * so it works on the raw MFMA results). It propagates NaN: a group that contains a NaN result has a NaN minimum,
+		 * which is never smaller than m1 and makes the median below return m1, so m2 = m1 and the point is not
+		 * certified -- the exact pass then decides it, as it must. */
+		auto lowest = [](float a, float b) { return __builtin_elementwise_minimum(a, b); };
 		if (FINE8) {
-			const float ta = fminf(fminf(fminf(e[0], e[1]), e[2]), e[3]); /* results 0..7 */
-			const float tb = fminf(fminf(fminf(e[4], e[5]), e[6]), e[7]); /* results 8..15 */
+			const float ta = lowest(lowest(lowest(lowest(lowest(lowest(lowest(acc[0], acc[1]), acc[2]), acc[3]), acc[4]), acc[5]), acc[6]), acc[7]); /* results 0..7 */
+			const float tb = lowest(lowest(lowest(lowest(lowest(lowest(lowest(acc[8], acc[9]), acc[10]), acc[11]), acc[12]), acc[13]), acc[14]), acc[15]); /* results 8..15 */
 			s.m2 = __builtin_amdgcn_fmed3f(s.m1, s.m2, ta); /* second smallest of {m1, m2, ta} as m1 <= m2 */
 			const bool lta = ta < s.m1;
 			s.tile = lta ? 2 * tile : s.tile;
@@ -125,10 +127,9 @@ __device__ __forceinline__ void track_tile(const f32x16& acc, Track& s, uint32_t
 			s.m1 = ltb ? tb : s.m1;
 		}
 		else {
-			const float f0 = fminf(fminf(e[0], e[1]), e[2]);
-			const float f1 = fminf(fminf(e[3], e[4]), e[5]);
-			const float f2 = fminf(fminf(e[6], e[7]), f0);
-			const float t = fminf(f1, f2);
+			float t = acc[0];
+#pragma unroll
+			for (int i = 1; i < 16; ++i) t = lowest(t, acc[i]);
 			s.m2 = __builtin_amdgcn_fmed3f(s.m1, s.m2, t); /* second smallest of {m1, m2, t} as m1 <= m2 */
 			const bool lt = t < s.m1;
 			s.tile = lt ? tile : s.tile;
@@ -200,7 +201,7 @@ __device__ __forceinline__ void tile_step(const float* __restrict__ lds, const f
 		for (int p = 0; p < P; ++p) track_tile<COARSE, fine8<DPH>()>(acc_old[p], st[p], tile_old, neg_inf);
 		constexpr int MFMAS = DPH * P;
 		constexpr int GROUPS = COARSE ? 1 : (MFMAS >= 4 ? 4 : 1);
-		constexpr int VALU_PER_GROUP = ((COARSE ? (fine8<DPH>() ? 20 : 16) : 67) * P + GROUPS - 1) / GROUPS;
+		constexpr int VALU_PER_GROUP = ((COARSE ? (fine8<DPH>() ? 16 : 12) : 67) * P + GROUPS - 1) / GROUPS;
 		if (DPH <= 32) { /* wider rows: the tracking is a few per cent of the step, the default schedule will do */
 #pragma unroll
 			for (int i = 0; i < GROUPS; ++i) {
