@@ -149,7 +149,7 @@ update_fine_kernel(const float* __restrict__ data, size_t stride, const uint32_t
  * Replica = point slot % replicas: for small k the slots of one wavefront then add to different
  * copies, which removes the same-address serialisation of hot clusters.
  */
-constexpr int UPDATE_UNROLL = 8;
+constexpr int UPDATE_UNROLL = 16;
 
 template <int LD, int LM>
 __global__ void __launch_bounds__(1024)
