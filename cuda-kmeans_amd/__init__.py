@@ -31,7 +31,7 @@ KMX_OK, KMX_ERR_INVALID_ARGUMENT, KMX_ERR_UNSUPPORTED, KMX_ERR_DEVICE, KMX_ERR_N
 ABI_SYMBOLS = [
     "kmx_device_count", "kmx_set_device", "kmx_device_props", "kmx_malloc", "kmx_free", "kmx_h2d", "kmx_d2h",
     "kmx_d2d", "kmx_sync", "kmx_set_stream", "kmx_shutdown", "kmx_fill_zero_u32", "kmx_assign_f32",
-    "kmx_assign_last_rechecked", "kmx_assign_last_variant", "kmx_update_f32", "kmx_bucket_sum_f32", "kmx_fused_f32", "kmx_assign_f64", "kmx_update_f64", "kmx_fused_f64", "kmx_bucket_sum_f64",
+    "kmx_assign_last_rechecked", "kmx_assign_last_variant", "kmx_update_f32", "kmx_bucket_sum_f32", "kmx_fused_f32", "kmx_assign_f64", "kmx_update_f64", "kmx_fused_f64", "kmx_bucket_sum_f64", "kmx_set_queued_rows_limit",
     "kmx_graph_begin", "kmx_graph_end", "kmx_graph_launch", "kmx_graph_destroy", "kmx_event_create", "kmx_event_destroy", "kmx_event_record",
     "kmx_event_elapsed_ms", "kmx_set_profiling", "kmx_last_kernel_ms", "kmx_last_error",
 ]
@@ -124,6 +124,7 @@ def hip_lib():
         lib.kmx_event_record.argtypes = [vp]
         lib.kmx_event_elapsed_ms.argtypes = [vp, vp, ctypes.POINTER(ctypes.c_float)]
         lib.kmx_set_profiling.argtypes = [ctypes.c_int]
+        lib.kmx_set_queued_rows_limit.argtypes = [ctypes.c_size_t]
         lib.kmx_last_kernel_ms.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_float)]
         _hip = lib
     return _hip
@@ -353,6 +354,11 @@ class Graph:
         if self._g:
             check(hip_lib().kmx_graph_destroy(self._g))
             self._g = ctypes.c_void_p()
+
+
+def set_queued_rows_limit(nbytes):
+    """Bound of the block of copied rows the exact pass keeps for SoA points (kmx_set_queued_rows_limit)."""
+    check(hip_lib().kmx_set_queued_rows_limit(ctypes.c_size_t(nbytes)))
 
 
 def set_profiling(enabled):

@@ -75,9 +75,15 @@ __device__ __forceinline__ void load_points(float (&b)[P][DPH], const float* __r
 			}
 		}
 		else {
+			/* wide rows: the address advances from load to load and the loads are issued in groups of 16, so that
+			 * no more than 16 addresses are alive at a time (128 independent 64-bit addresses do not fit the registers) */
+			const float* src = data + (size_t)(h * DPH) * stride + pt;
 #pragma unroll
-			for (int s = 0; s < DPH; ++s)
-				b[p][s] = (valid && h * DPH + s < dim) ? data[(size_t)(h * DPH + s) * stride + pt] : 0.0f;
+			for (int s = 0; s < DPH; ++s) {
+				b[p][s] = (valid && h * DPH + s < dim) ? *src : 0.0f;
+				src += stride;
+				if (DPH > 64 && s % 16 == 15) __builtin_amdgcn_sched_barrier(0);
+			}
 		}
 	}
 }

@@ -72,6 +72,12 @@ __global__ void reset_f64_kernel(unsigned long long* __restrict__ misc)
 	if (threadIdx.x < 2) misc[threadIdx.x] = 0;
 }
 
+/* the count kmx_assign_last_rechecked() reports, for the variants that do not go through the float sweeps */
+__global__ void publish_queue_length_kernel(const unsigned long long* __restrict__ misc, uint32_t* __restrict__ counters, bool queued)
+{
+	if (threadIdx.x == 0) counters[0] = queued ? (uint32_t)misc[0] : 0u;
+}
+
 /* round-to-nearest float copy; values beyond the float range become infinities, tiny ones zeros or subnormals.
  * Four elements per lane and step (two 16-byte loads, one 16-byte store); both buffers are 16-byte aligned. */
 typedef double f64x2 __attribute__((ext_vector_type(2)));
@@ -825,7 +831,15 @@ extern "C" int kmx_assign_f64(int variant,
 	rc = layout == KMX_AOS ? launch_assign_f64_ld<KMX_AOS>(variant, data, stride, assignment, dim, k, kp, n, exec, *dev, float_queue, float_queue_length)
 	                       : launch_assign_f64_ld<KMX_SOA>(variant, data, stride, assignment, dim, k, kp, n, exec, *dev, float_queue, float_queue_length);
 	if (rc) return rc;
-	return float_queue ? KMX_OK : profile_end(0);
+	if (float_queue) return KMX_OK;
+	rc = profile_end(0);
+	if (rc) return rc;
+	Workspace* ws = nullptr;
+	rc = workspace(&ws);
+	if (rc) return rc;
+	hipLaunchKernelGGL(publish_queue_length_kernel, dim3(1), dim3(64), 0, stream(), misc, ws->counters, variant == KMX_ASSIGN_LDS_FMA);
+	KMX_LAUNCH_CHECK("publish_queue_length_kernel");
+	return KMX_OK;
 }
 
 static int update_f64_call(const char* who, bool divide, int variant,

@@ -117,6 +117,12 @@ int reserve_partials(Workspace* ws, size_t floats) { return grow(&ws->partials, 
 int reserve_fused_assignment(Workspace* ws, size_t entries) { return grow(&ws->fused_assignment, &ws->fused_cap, entries); }
 int reserve_bucket_sizes(Workspace* ws, size_t entries) { return grow(&ws->bucket_sizes, &ws->bucket_cap, entries); }
 int reserve_f64(double** ptr, size_t* cap, size_t doubles) { return grow(ptr, cap, doubles); }
+int reserve_queued_rows(Workspace* ws, size_t rows, size_t dim)
+{
+	int rc = grow(&ws->queued_rows, &ws->queued_rows_cap, rows * dim);
+	if (rc) return rc;
+	return grow(&ws->queued_index, &ws->queued_index_cap, 3 * rows);
+}
 
 static int release_workspace()
 {
@@ -128,6 +134,8 @@ static int release_workspace()
 	if (g_ws.partials) KMX_HIP(hipFree(g_ws.partials));
 	if (g_ws.fused_assignment) KMX_HIP(hipFree(g_ws.fused_assignment));
 	if (g_ws.bucket_sizes) KMX_HIP(hipFree(g_ws.bucket_sizes));
+	if (g_ws.queued_rows) KMX_HIP(hipFree(g_ws.queued_rows));
+	if (g_ws.queued_index) KMX_HIP(hipFree(g_ws.queued_index));
 	g_ws = Workspace();
 	return release_f64_workspace();
 }
@@ -554,6 +562,13 @@ int kmx_graph_destroy(void* graph)
 	clear_error();
 	if (!graph) return KMX_OK;
 	KMX_HIP(hipGraphExecDestroy((hipGraphExec_t)graph));
+	return KMX_OK;
+}
+
+int kmx_set_queued_rows_limit(size_t bytes)
+{
+	clear_error();
+	set_queued_rows_limit(bytes);
 	return KMX_OK;
 }
 

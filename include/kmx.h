@@ -248,6 +248,14 @@ int kmx_graph_destroy(void* graph);
 int kmx_set_profiling(int enabled);
 int kmx_last_kernel_ms(int which, float* ms);
 
+/*
+ * Work-space bound (no counterpart in the reference: its kernels evaluate every point directly). With SoA points the
+ * exact pass of the tuned assignment variants copies the rows of the points it has to re-evaluate into a compact
+ * block in the library's work space; `bytes` bounds that block (default 1 GiB, at least 1024 rows are always kept).
+ * Points beyond the bound are still re-evaluated, reading the SoA data directly (slower, same results).
+ */
+int kmx_set_queued_rows_limit(size_t bytes);
+
 /* Message of the last failed call on this thread ("" if none). */
 const char* kmx_last_error(void);
 

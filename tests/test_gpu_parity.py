@@ -165,6 +165,35 @@ def test_hard_inputs(km, orc, gpu, dim, k, n):
                 name, v, bad.size, bad[:5], got[bad[:5]], want[bad[:5]])
 
 
+@pytest.mark.parametrize("dim,k,n", [(32, 256, 3000), (21, 1500, 4000), (96, 200, 1500), (4, 512, 5000)])
+def test_soa_points_in_the_exact_pass(km, orc, gpu, dim, k, n):
+    """SoA points: the exact pass copies the rows of the queued points into a compact block. Inputs that queue every point
+    (identical centroids, ties on a grid), with the default bound and with a bound of 1024 rows, which leaves most of
+    the queue to the kernels that read the SoA data directly."""
+    rng = np.random.default_rng(7 + dim)
+    base = rng.normal(size=(n, dim)).astype(np.float32)
+    means = rng.normal(size=(k, dim)).astype(np.float32)
+    cases = {
+        "all_centroids_identical": (base, np.repeat(means[:1], k, 0)),
+        "grid_ties": (np.round(base * 2) / 2, np.round(means * 2) / 2),
+        "plain": (base, means),
+    }
+    try:
+        for limit in (1 << 30, 4096):
+            km.set_queued_rows_limit(limit)
+            for name, (d, m) in cases.items():
+                want = orc.assign(np.ascontiguousarray(d).ravel(), np.ascontiguousarray(m).ravel(), dim, k, n, threads=0, fast=True)
+                for layout_means in (km.AOS, km.SOA):
+                    dd = np.ascontiguousarray(d.T).ravel()
+                    mm = np.ascontiguousarray(m if layout_means == km.AOS else m.T).ravel()
+                    for v in variants(km, dim):
+                        got, _ = gpu_assign(km, v, dd, mm, dim, k, n, km.SOA, layout_means)
+                        bad = np.nonzero(got != want)[0]
+                        assert bad.size == 0, "%s, limit %d, variant %d: %d mismatches, first at %s" % (name, limit, v, bad.size, bad[:5])
+    finally:
+        km.set_queued_rows_limit(1 << 30)
+
+
 def test_sqrt_is_correctly_rounded_on_device(km, orc, gpu):
     """The exact pass compares sqrt values: a 1-ulp device sqrt would flip ties. d = 1, k = n centroids such
     that point i's nearest candidates have adjacent squared distances; also a direct sweep through BASE."""
