@@ -52,6 +52,17 @@ __device__ __forceinline__ void load_split_points(SplitPoints<KB> (&b)[P], float
 				v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w;
 				v[4] = up.x; v[5] = up.y; v[6] = up.z; v[7] = up.w;
 			}
+			else if (LD == KMX_SOA) {
+				/* the address advances from load to load; long rows are loaded 16 coordinates at a time, so that only a few
+				 * of their 64-bit addresses are alive at once */
+				const float* src = data + (size_t)d0 * stride + pt;
+#pragma unroll
+				for (int j = 0; j < 8; ++j) {
+					v[j] = (valid && d0 + j < dim) ? *src : 0.0f;
+					src += stride;
+				}
+				if (KB > 4 && kb % 2 == 1) __builtin_amdgcn_sched_barrier(0);
+			}
 			else {
 #pragma unroll
 				for (int j = 0; j < 8; ++j) v[j] = (valid && d0 + j < dim) ? data[elem<LD>(stride, pt, d0 + j)] : 0.0f;
@@ -397,7 +408,7 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 /* point tiles per wavefront and sweep, and whether the next sweep's points are prefetched: bounded by the register file */
 template <int KB> struct SplitSweepShape {
 	static constexpr int P = KB <= 4 ? 2 : 1;
-	static constexpr bool PREFETCH = KB <= 8;
+	static constexpr bool PREFETCH = KB <= 2;
 };
 
 template <int KB, int LD, bool VEC>
