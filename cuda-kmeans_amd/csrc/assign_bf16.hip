@@ -88,6 +88,28 @@ bool bf16_supports(const AssignArgs& a, const DeviceInfo& dev)
 KMX_DECLARE_BF16_LAUNCHER(1) KMX_DECLARE_BF16_LAUNCHER(2) KMX_DECLARE_BF16_LAUNCHER(3) KMX_DECLARE_BF16_LAUNCHER(4)
 KMX_DECLARE_BF16_LAUNCHER(8) KMX_DECLARE_BF16_LAUNCHER(16)
 
+#define KMX_DECLARE_BF16_SCREEN(W) \
+	int launch_screen_bf16_##W(const float* rows, const Workspace* ws, const uint32_t* row_queue, const uint32_t* row_count, \
+	                           uint32_t* pairs, uint32_t* item_pairs, unsigned long long* keys, uint32_t dim, uint32_t k, uint32_t kp, \
+	                           const DeviceInfo& dev, uint32_t* waves);
+KMX_DECLARE_BF16_SCREEN(1) KMX_DECLARE_BF16_SCREEN(2) KMX_DECLARE_BF16_SCREEN(3) KMX_DECLARE_BF16_SCREEN(4)
+KMX_DECLARE_BF16_SCREEN(8) KMX_DECLARE_BF16_SCREEN(16)
+
+/* rows per work item of the screen: two tiles of 32 while the operands of two tiles fit the registers */
+uint32_t screen_unit_rows(uint32_t dim) { return pick_kb(dim) <= 4 ? 2 * TILE : TILE; }
+
+int launch_screen_bf16(const float* rows, const Workspace* ws, const uint32_t* row_queue, const uint32_t* row_count,
+                       uint32_t* pairs, uint32_t* item_pairs, unsigned long long* keys, uint32_t dim, uint32_t k, uint32_t kp,
+                       const DeviceInfo& dev, uint32_t* waves)
+{
+#define KMX_SCREEN_CASE(W) case W: return launch_screen_bf16_##W(rows, ws, row_queue, row_count, pairs, item_pairs, keys, dim, k, kp, dev, waves)
+	switch (pick_kb(dim)) {
+	KMX_SCREEN_CASE(1); KMX_SCREEN_CASE(2); KMX_SCREEN_CASE(3); KMX_SCREEN_CASE(4); KMX_SCREEN_CASE(8); KMX_SCREEN_CASE(16);
+	default: return fail(KMX_ERR_UNSUPPORTED, "assign (split-bf16 MFMA): dim %u is not supported", dim);
+	}
+#undef KMX_SCREEN_CASE
+}
+
 int launch_assign_bf16(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev)
 {
 	const uint32_t kb = pick_kb(a.dim);
@@ -119,7 +141,9 @@ int launch_assign_bf16(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws
 	}
 	if (rc) return rc;
 	if (a.ranking_only) return KMX_OK; /* the caller resolves the queued points */
-	return launch_recheck(a, ws, kp);
+	/* wide rows and many centroids: a second sweep screens the queued points (narrow rows fit the registers of the
+	 * lane-per-centroid kernels, which then need fewer launches) */
+	return a.k >= 128 && a.dim > 32 ? launch_recheck_screened(a, ws, kp, dev) : launch_recheck(a, ws, kp);
 }
 
 } // namespace kmx

@@ -8,6 +8,8 @@
 
 #include "assign_mfma_impl.h"
 
+#include <type_traits>
+
 namespace kmx {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -403,6 +405,203 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 		}
 	}
 	if (flagged) flush_flags();
+}
+
+/*
+ * The screen of the exact pass: a second sweep over the queued points only. Their rows lie in a compact AoS block
+ * (row e of the block = entry e of the queue, `dim` floats apart) with the threshold the first sweep gave them
+ * (its best ranking value + tau). The same MFMAs on the same operands reproduce the ranking values a[j] of the first
+ * sweep, and every centroid with a[j] <= threshold -- the only ones that can win or tie the serial comparison, two
+ * or three of k -- is noted as a (row, centroid) pair for the kernel that evaluates the serial arithmetic. A NaN
+ * a[j] and an infinite threshold (values the sweep could not cover) pass the screen. Per tile the lane only takes
+ * the minimum of its 16 results and compares it with the threshold; the pairs are picked out on the rare hit.
+ * Every work item has a slice of the pair list to itself (no atomics); pairs beyond it (many coincident centroids)
+ * are evaluated when the wavefront hands its pairs over.
+ * The centroid operands are read from global memory (they stay in the caches; this kernel sees a small share of
+ * the points), one wavefront per P tiles of 32 rows.
+ */
+/* the rare pair beyond its slice's capacity; not inlined, so that the sweep's registers are not sized for it */
+static __device__ __attribute__((noinline)) void evaluate_pair_of_row(const float* __restrict__ rows, uint32_t dim, const float* __restrict__ means_t,
+                                                                      uint32_t kp, uint32_t row, uint32_t j, unsigned long long* __restrict__ keys)
+{
+	evaluate_pair<KMX_AOS>(rows, dim, means_t, dim, kp, row, j, &keys[row]);
+}
+
+template <int KB, int P>
+__global__ void __launch_bounds__(SCREEN_WAVES * WAVE)
+screen_bf16_kernel(const float* __restrict__ rows, const float* __restrict__ packed, const float* __restrict__ norms,
+                   const float* __restrict__ means_t, const uint32_t* __restrict__ row_queue, const uint32_t* __restrict__ row_count,
+                   uint32_t* __restrict__ pairs, uint32_t* __restrict__ item_pairs,
+                   unsigned long long* __restrict__ keys, uint32_t dim, uint32_t k, uint32_t kp)
+{
+	constexpr uint32_t RS = KBLOCK * KB + ROW_PAD;
+	constexpr int G = KB < 4 ? KB : 4; /* blocks of 16 dimensions whose centroid operands travel together */
+	constexpr int GROUPS = KB / G;     /* 1, 2 or 4 */
+	static_assert(KB % G == 0 && (GROUPS == 1 || GROUPS % 2 == 0), "operand groups");
+	constexpr uint32_t unit_rows = P * TILE;
+	constexpr uint32_t SLICE = SCREEN_SLICE_PER_ROW * unit_rows; /* pairs an item can note */
+	const uint32_t lane = threadIdx.x & (WAVE - 1);
+	const uint32_t col = lane & 31, h = lane >> 5;
+	const uint32_t count = row_count[0];
+	const uint32_t tiles = kp / TILE;
+	const uint32_t waves = gridDim.x * SCREEN_WAVES;
+	const ScreenItems work = screen_items(count, unit_rows, tiles, waves);
+
+	struct Operands { bf16x8 hi[G], mid[G]; };
+
+	/* the pairs a wavefront notes wait in LDS and go to the item's slice of the list a few hundred at a time; pairs
+	 * beyond the slice are evaluated then and there */
+	constexpr uint32_t HIT_LIST = 256;
+	__shared__ uint32_t hit_list[SCREEN_WAVES][2 * HIT_LIST];
+	const uint32_t wave = threadIdx.x / WAVE;
+	uint32_t listed = 0, written = 0; /* wave-uniform: pairs in LDS, pairs of the current item handed over */
+	uint32_t* slice = pairs;
+	auto flush = [&]() {
+		__builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+		__builtin_amdgcn_wave_barrier();
+		for (uint32_t i = lane; i < listed; i += WAVE) {
+			const uint32_t row = hit_list[wave][2 * i], j = hit_list[wave][2 * i + 1];
+			if (written + i < SLICE) { slice[2 * (written + i)] = row; slice[2 * (written + i) + 1] = j; }
+			else evaluate_pair_of_row(rows, dim, means_t, kp, row, j, keys);
+		}
+		__builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+		__builtin_amdgcn_wave_barrier();
+		written += listed;
+		listed = 0;
+	};
+
+	for (uint32_t item = blockIdx.x * SCREEN_WAVES + threadIdx.x / WAVE; item < work.items; item += waves) {
+		const uint32_t base = (item / work.parts) * unit_rows;
+		const uint32_t tile_begin = (item % work.parts) * work.part_tiles, tile_end = min(tiles, tile_begin + work.part_tiles);
+		slice = pairs + 2 * (size_t)item * SLICE;
+		written = 0;
+		SplitPoints<KB> b[P];
+		float xx[P];
+		load_split_points<KB, P, KMX_AOS, false>(b, xx, rows, dim, base, col, h, dim, count);
+		float thr[P];
+		bool valid[P];
+#pragma unroll
+		for (int p = 0; p < P; ++p) {
+			const uint32_t row = base + p * TILE + col;
+			valid[p] = row < count;
+			thr[p] = valid[p] ? __uint_as_float(row_queue[2 * (size_t)row + 1]) : 0.0f;
+		}
+
+		auto fetch = [&](Operands& o, uint32_t tile, int group) {
+			const float* arow = packed + (size_t)tile * tile_floats(RS) + (size_t)col * RS;
+#pragma unroll
+			for (int i = 0; i < G; ++i) {
+				o.hi[i] = row_unit(arow, 4 * (group * G + i) + 2 * h);
+				o.mid[i] = row_unit(arow, 4 * (group * G + i) + 2 * h + 1);
+			}
+		};
+		auto fetch_norms = [&](f32x16& c, uint32_t tile) { /* |c|^2 of the 16 rows this lane receives */
+#pragma unroll
+			for (int g = 0; g < 4; ++g) {
+				const f32x4 v = *(const f32x4*)(norms + tile * NORM_TILE + 8 * g + 4 * h);
+				c[4 * g] = v.x; c[4 * g + 1] = v.y; c[4 * g + 2] = v.z; c[4 * g + 3] = v.w;
+			}
+		};
+		auto screen = [&](const f32x16& a, int p, uint32_t tile) {
+			float t = a[0]; /* NaN-propagating minimum of the lane's 16 results */
+#pragma unroll
+			for (int r = 1; r < 16; ++r) t = __builtin_elementwise_minimum(t, a[r]);
+			const bool near = valid[p] && !(t > thr[p]);
+			if (__builtin_amdgcn_ballot_w64(near) == 0) return;
+			const uint32_t row = base + p * TILE + col;
+#pragma unroll
+			for (int r = 0; r < 16; ++r) {
+				const uint32_t j = tile * TILE + 8 * (r / 4) + 4 * h + (r % 4);
+				const bool hit = near && j < k && !(a[r] > thr[p]);
+				const unsigned long long mask = __builtin_amdgcn_ballot_w64(hit);
+				if (mask == 0) continue;
+				const uint32_t more = (uint32_t)__popcll(mask);
+				if (listed + more > HIT_LIST) flush();
+				if (hit) {
+					const uint32_t slot = listed + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
+					hit_list[wave][2 * slot] = row;
+					hit_list[wave][2 * slot + 1] = j;
+				}
+				listed += more;
+			}
+		};
+
+		f32x16 acc[P], norms_next;
+		fetch_norms(norms_next, tile_begin);
+		/* the MFMAs of one operand group (the order of tile_step_bf16: hi*mid, mid*hi, hi*hi per block) */
+		auto compute = [&](const Operands& o, uint32_t tile, auto group_c) {
+			constexpr int group = decltype(group_c)::value;
+			if (group == 0) {
+#pragma unroll
+				for (int p = 0; p < P; ++p) acc[p] = norms_next;
+				if (tile + 1 < tile_end) fetch_norms(norms_next, tile + 1);
+			}
+#pragma unroll
+			for (int i = 0; i < G; ++i) {
+#pragma unroll
+				for (int p = 0; p < P; ++p) acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(o.hi[i], b[p].mid[group * G + i], acc[p], 0, 0, 0);
+#pragma unroll
+				for (int p = 0; p < P; ++p) acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(o.mid[i], b[p].hi[group * G + i], acc[p], 0, 0, 0);
+#pragma unroll
+				for (int p = 0; p < P; ++p) acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(o.hi[i], b[p].hi[group * G + i], acc[p], 0, 0, 0);
+			}
+			if (group == GROUPS - 1) {
+#pragma unroll
+				for (int p = 0; p < P; ++p) screen(acc[p], p, tile);
+			}
+		};
+
+		/* two operand buffers: while one feeds the MFMAs the other one is on its way from the caches */
+		Operands o0, o1;
+		fetch(o0, tile_begin, 0);
+		if constexpr (GROUPS == 1) {
+			for (uint32_t tile = tile_begin; tile < tile_end; tile += 2) {
+				if (tile + 1 < tile_end) fetch(o1, tile + 1, 0);
+				compute(o0, tile, std::integral_constant<int, 0>());
+				if (tile + 2 < tile_end) fetch(o0, tile + 2, 0);
+				if (tile + 1 < tile_end) compute(o1, tile + 1, std::integral_constant<int, 0>());
+			}
+		}
+		else {
+			for (uint32_t tile = tile_begin; tile < tile_end; ++tile) {
+				fetch(o1, tile, 1);
+				compute(o0, tile, std::integral_constant<int, 0>());
+				if constexpr (GROUPS == 2) {
+					if (tile + 1 < tile_end) fetch(o0, tile + 1, 0);
+					compute(o1, tile, std::integral_constant<int, 1>());
+				}
+				else {
+					fetch(o0, tile, 2);
+					compute(o1, tile, std::integral_constant<int, 1>());
+					fetch(o1, tile, 3);
+					compute(o0, tile, std::integral_constant<int, 2>());
+					if (tile + 1 < tile_end) fetch(o0, tile + 1, 0);
+					compute(o1, tile, std::integral_constant<int, 3>());
+				}
+			}
+		}
+		flush();
+		if (lane == 0) item_pairs[item] = min(written, SLICE);
+	}
+}
+
+template <int KB> struct ScreenShape { static constexpr int P = KB <= 4 ? 2 : 1; };
+
+template <int KB>
+static int launch_screen_bf16_kb(const float* rows, const Workspace* ws, const uint32_t* row_queue, const uint32_t* row_count,
+                                 uint32_t* pairs, uint32_t* item_pairs, unsigned long long* keys, uint32_t dim, uint32_t k, uint32_t kp,
+                                 const DeviceInfo& dev, uint32_t* waves)
+{
+	auto kernel = screen_bf16_kernel<KB, ScreenShape<KB>::P>;
+	/* as many wavefronts as the device holds at once: the partition of the work counts on all of them running together */
+	int per_cu = 1;
+	KMX_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)kernel, (int)(SCREEN_WAVES * WAVE), 0));
+	const uint32_t grid = std::min<uint32_t>(dev.compute_units * (uint32_t)std::max(1, per_cu), SCREEN_MAX_WAVES / SCREEN_WAVES);
+	*waves = grid * SCREEN_WAVES;
+	hipLaunchKernelGGL(kernel, dim3(grid), dim3(SCREEN_WAVES * WAVE), 0, stream(),
+	                   rows, ws->packed_means, ws->norms, ws->means_t, row_queue, row_count, pairs, item_pairs, keys, dim, k, kp);
+	KMX_LAUNCH_CHECK("screen_bf16_kernel");
+	return KMX_OK;
 }
 
 /* point tiles per wavefront and sweep, and whether the next sweep's points are prefetched: bounded by the register file */

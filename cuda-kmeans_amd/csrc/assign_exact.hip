@@ -336,22 +336,6 @@ static __device__ __forceinline__ float touch_rows(const float* __restrict__ dat
 
 constexpr uint32_t HIT_CAP = 1024;
 
-template <int LD>
-static __device__ __forceinline__ void evaluate_pair(const float* __restrict__ data, size_t stride, const float* __restrict__ means_t,
-                                                      uint32_t dim, uint32_t kp, uint32_t pt, uint32_t r, unsigned long long* key_slot)
-{
-	float sum = 0.0f;
-#pragma unroll 16
-	for (uint32_t q = 0; q < dim; ++q) {
-		float diff = data[elem<LD>(stride, pt, q)] - means_t[(size_t)q * kp + r];
-		float sq = diff * diff;
-		sum = sum + sq;
-	}
-	const float dist = __builtin_sqrtf(sum);
-	const unsigned long long key = (r == 0 && dist != dist) ? 0ull : (((unsigned long long)__float_as_uint(dist) << 32) | r);
-	atomicMin(key_slot, key);
-}
-
 constexpr uint32_t POINTS_BATCH = 64;
 
 template <int LD, int DPAD, bool FULL, int CPL> /* FULL: dim == DPAD, no guards on the coordinate loads; CPL: centroids per lane */
@@ -668,19 +652,27 @@ static size_t g_queued_rows_bytes = (size_t)1 << 30; /* upper bound of the block
 
 void set_queued_rows_limit(size_t bytes) { g_queued_rows_bytes = bytes; }
 
+/* a group of `1 << group_shift` lanes (the smallest power of two that covers the row, at most a wavefront) copies one row */
+template <int LD>
 __global__ void __launch_bounds__(256)
 gather_queued_rows_kernel(const float* __restrict__ data, size_t stride, uint32_t dim, const uint32_t* __restrict__ queue,
-                          uint32_t* __restrict__ counters, float* __restrict__ rows, uint32_t* __restrict__ row_queue, uint32_t cap)
+                          uint32_t* __restrict__ counters, float* __restrict__ rows, uint32_t* __restrict__ row_queue,
+                          unsigned long long* __restrict__ keys, uint32_t cap, uint32_t group_shift)
 {
 	const uint32_t count = counters[0];
 	const uint32_t taken = min(count, cap);
 	if (blockIdx.x == 0 && threadIdx.x == 0) { counters[1] = taken; counters[2] = count - taken; }
-	const size_t total = (size_t)taken * dim;
-	for (size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (size_t)gridDim.x * blockDim.x) {
-		const size_t e = t / dim;
-		const uint32_t q = (uint32_t)(t - e * dim);
-		rows[t] = data[(size_t)q * stride + queue[2 * e]];
-		if (q == 0) { row_queue[2 * e] = (uint32_t)e; row_queue[2 * e + 1] = queue[2 * e + 1]; }
+	const uint32_t group = 1u << group_shift;
+	const uint32_t q0 = threadIdx.x & (group - 1);
+	const uint32_t groups = (gridDim.x * blockDim.x) >> group_shift;
+	for (uint32_t e = (blockIdx.x * blockDim.x + threadIdx.x) >> group_shift; e < taken; e += groups) {
+		const uint32_t pt = queue[2 * (size_t)e];
+		for (uint32_t q = q0; q < dim; q += group) rows[(size_t)e * dim + q] = data[elem<LD>(stride, pt, q)];
+		if (q0 == 0) {
+			row_queue[2 * (size_t)e] = e;
+			row_queue[2 * (size_t)e + 1] = queue[2 * (size_t)e + 1];
+			if (keys) keys[e] = ~0ull; /* no centroid evaluated yet */
+		}
 	}
 }
 
@@ -693,6 +685,85 @@ scatter_row_results_kernel(const uint32_t* __restrict__ queue, const uint32_t* _
 		assignment[queue[2 * (size_t)e]] = row_assignment[e];
 }
 
+/* the pairs the screen noted: a wavefront per work item of the screen (same partition), a lane per pair */
+__global__ void __launch_bounds__(256)
+evaluate_pairs_kernel(const float* __restrict__ rows, uint32_t dim, const float* __restrict__ means_t, uint32_t kp,
+                      const uint32_t* __restrict__ pairs, const uint32_t* __restrict__ item_pairs, const uint32_t* __restrict__ row_count,
+                      uint32_t unit_rows, uint32_t screen_waves, unsigned long long* __restrict__ keys)
+{
+	const ScreenItems work = screen_items(row_count[0], unit_rows, kp / TILE, screen_waves);
+	const uint32_t slice = SCREEN_SLICE_PER_ROW * unit_rows;
+	const uint32_t lane = threadIdx.x & (WAVE - 1);
+	const uint32_t waves = gridDim.x * (blockDim.x / WAVE);
+	for (uint32_t item = (blockIdx.x * blockDim.x + threadIdx.x) / WAVE; item < work.items; item += waves) {
+		const uint32_t noted = item_pairs[item];
+		const uint32_t* mine = pairs + 2 * (size_t)item * slice;
+		for (uint32_t t = lane; t < noted; t += WAVE) {
+			const uint32_t row = mine[2 * t];
+			evaluate_pair<KMX_AOS>(rows, dim, means_t, dim, kp, row, mine[2 * t + 1], &keys[row]);
+		}
+	}
+}
+
+/* a row no centroid was evaluated for (every distance a NaN, or nothing within the threshold, which only values the
+ * sweep does not cover produce) stays where the serial scan leaves it: at centroid 0 */
+__global__ void __launch_bounds__(256)
+scatter_row_keys_kernel(const uint32_t* __restrict__ queue, const uint32_t* __restrict__ counters,
+                        const unsigned long long* __restrict__ keys, uint32_t* __restrict__ assignment)
+{
+	const uint32_t taken = counters[1];
+	for (uint32_t e = blockIdx.x * blockDim.x + threadIdx.x; e < taken; e += gridDim.x * blockDim.x) {
+		const unsigned long long key = keys[e];
+		assignment[queue[2 * (size_t)e]] = key == ~0ull ? 0u : (uint32_t)key;
+	}
+}
+
+static uint32_t row_group_shift(uint32_t dim)
+{
+	uint32_t shift = 0;
+	while (shift < 6 && (1u << shift) < dim) ++shift;
+	return shift;
+}
+
+static uint32_t queued_rows_cap(const AssignArgs& a)
+{
+	return (uint32_t)std::min<size_t>(a.n, std::max<size_t>(1024, g_queued_rows_bytes / ((size_t)a.dim * sizeof(float))));
+}
+
+int launch_recheck_screened(const AssignArgs& a, Workspace* ws, uint32_t kp, const DeviceInfo& dev)
+{
+	const uint32_t cap = std::min<uint32_t>(queued_rows_cap(a), 4u << 20); /* the pair list takes 32 bytes per row */
+	const uint32_t unit_rows = screen_unit_rows(a.dim);
+	const uint32_t items_max = screen_items_max(cap, unit_rows);
+	const size_t slice_words = 2 * (size_t)SCREEN_SLICE_PER_ROW * unit_rows;
+	int rc = reserve_queued_rows(ws, cap, a.dim, items_max + items_max * slice_words);
+	if (rc) return rc;
+	const uint32_t group_shift = row_group_shift(a.dim);
+	uint32_t* row_queue = ws->queued_index;
+	unsigned long long* keys = (unsigned long long*)(ws->queued_index + 2 * (size_t)cap);
+	uint32_t* item_pairs = ws->queued_index + 4 * (size_t)cap;
+	uint32_t* pairs = item_pairs + items_max;
+	if (a.layout == KMX_AOS)
+		hipLaunchKernelGGL((gather_queued_rows_kernel<KMX_AOS>), dim3(1024), dim3(256), 0, stream(),
+		                   a.data, a.stride, a.dim, ws->queue, ws->counters, ws->queued_rows, row_queue, keys, cap, group_shift);
+	else
+		hipLaunchKernelGGL((gather_queued_rows_kernel<KMX_SOA>), dim3(1024), dim3(256), 0, stream(),
+		                   a.data, a.stride, a.dim, ws->queue, ws->counters, ws->queued_rows, row_queue, keys, cap, group_shift);
+	KMX_LAUNCH_CHECK("gather_queued_rows_kernel");
+	uint32_t screen_waves = 0;
+	rc = launch_screen_bf16(ws->queued_rows, ws, row_queue, ws->counters + 1, pairs, item_pairs, keys, a.dim, a.k, kp, dev, &screen_waves);
+	if (rc) return rc;
+	hipLaunchKernelGGL(evaluate_pairs_kernel, dim3(1024), dim3(256), 0, stream(),
+	                   ws->queued_rows, a.dim, ws->means_t, kp, pairs, item_pairs, ws->counters + 1, unit_rows, screen_waves, keys);
+	KMX_LAUNCH_CHECK("evaluate_pairs_kernel");
+	hipLaunchKernelGGL(scatter_row_keys_kernel, dim3(512), dim3(256), 0, stream(), ws->queue, ws->counters, keys, a.assignment);
+	KMX_LAUNCH_CHECK("scatter_row_keys_kernel");
+	if (cap == a.n) return KMX_OK; /* every point has a row: nothing can be left over */
+	Workspace rest = *ws; /* the launchers only read the pointers */
+	rest.queue = ws->queue + 2 * (size_t)cap; rest.counters = ws->counters + 2;
+	return a.layout == KMX_AOS ? launch_recheck_l<KMX_AOS>(a, &rest, kp) : launch_recheck_l<KMX_SOA>(a, &rest, kp);
+}
+
 int launch_recheck(const AssignArgs& a, Workspace* ws, uint32_t kp)
 {
 	if ((size_t)a.dim * sizeof(float) * 16 > 160 * 1024)
@@ -700,13 +771,14 @@ int launch_recheck(const AssignArgs& a, Workspace* ws, uint32_t kp)
 	if (a.layout == KMX_AOS) return launch_recheck_l<KMX_AOS>(a, ws, kp);
 	if (a.k < 128) return launch_recheck_l<KMX_SOA>(a, ws, kp); /* these kernels stage the points in LDS with vector loads */
 
-	const uint32_t cap = (uint32_t)std::min<size_t>(a.n, std::max<size_t>(1024, g_queued_rows_bytes / ((size_t)a.dim * sizeof(float))));
-	int rc = reserve_queued_rows(ws, cap, a.dim);
+	const uint32_t cap = queued_rows_cap(a);
+	int rc = reserve_queued_rows(ws, cap, a.dim, 0);
 	if (rc) return rc;
+	const uint32_t group_shift = row_group_shift(a.dim);
 	uint32_t* row_queue = ws->queued_index;
 	uint32_t* row_assignment = ws->queued_index + 2 * (size_t)cap;
-	hipLaunchKernelGGL(gather_queued_rows_kernel, dim3(2048), dim3(256), 0, stream(),
-	                   a.data, a.stride, a.dim, ws->queue, ws->counters, ws->queued_rows, row_queue, cap);
+	hipLaunchKernelGGL((gather_queued_rows_kernel<KMX_SOA>), dim3(2048), dim3(256), 0, stream(),
+	                   a.data, a.stride, a.dim, ws->queue, ws->counters, ws->queued_rows, row_queue, (unsigned long long*)nullptr, cap, group_shift);
 	KMX_LAUNCH_CHECK("gather_queued_rows_kernel");
 	AssignArgs rows = a;
 	rows.data = ws->queued_rows; rows.layout = KMX_AOS; rows.stride = a.dim; rows.assignment = row_assignment; rows.n = cap;

@@ -42,6 +42,59 @@ __host__ __device__ constexpr uint32_t tile_floats(uint32_t rs) { return TILE * 
 __host__ __device__ __forceinline__ size_t packed_row(uint32_t row, uint32_t rs) { return (size_t)(row / TILE) * tile_floats(rs) + (size_t)(row % TILE) * rs; }
 __host__ __device__ __forceinline__ uint32_t norm_at(uint32_t row) { return (row / TILE) * NORM_TILE + (row % TILE); }
 
+/*
+ * The serial distance of one (point, centroid) pair -- subtract, multiply, add, every operation rounded separately, in
+ * ascending dimension, then the correctly rounded square root (reference metric_policies.hpp:23-28,40-44) -- merged
+ * into the point's 64-bit key (distance bits << 32 | centroid) by an atomic minimum: the smallest key is what the
+ * serial scan returns (lower index on equal distances; a NaN distance has the largest bit patterns and never wins,
+ * except at centroid 0, where the scan starts: key 0). Contraction is off inside this function whatever the
+ * translation unit's setting.
+ */
+template <int LD>
+static __device__ __forceinline__ void evaluate_pair(const float* __restrict__ data, size_t stride, const float* __restrict__ means_t,
+                                                      uint32_t dim, uint32_t kp, uint32_t pt, uint32_t r, unsigned long long* key_slot)
+{
+#pragma clang fp contract(off)
+	float sum = 0.0f;
+#pragma unroll 16
+	for (uint32_t q = 0; q < dim; ++q) {
+		float diff = data[elem<LD>(stride, pt, q)] - means_t[(size_t)q * kp + r];
+		float sq = diff * diff;
+		sum = sum + sq;
+	}
+	const float dist = __builtin_sqrtf(sum);
+	const unsigned long long key = (r == 0 && dist != dist) ? 0ull : (((unsigned long long)__float_as_uint(dist) << 32) | r);
+	atomicMin(key_slot, key);
+}
+
+/*
+ * Work items of the screen of the exact pass (screen_bf16_kernel) and of the kernel that evaluates what it notes: a
+ * unit of `unit_rows` queued rows, and, when there are fewer units than wavefronts in the launch (as many as the
+ * device holds at once), a share of the centroid tiles.
+ * Every item owns a slice of SCREEN_SLICE_PER_ROW * unit_rows (row, centroid) pairs of the list and a counter.
+ */
+constexpr uint32_t SCREEN_WAVES = 4;          /* wavefronts per work-group */
+constexpr uint32_t SCREEN_MAX_WAVES = 16384;  /* upper bound of the wavefronts of a launch (as many as are resident at once) */
+constexpr uint32_t SCREEN_SLICE_PER_ROW = 4;
+struct ScreenItems { uint32_t units, parts, part_tiles, items; };
+__host__ __device__ __forceinline__ ScreenItems screen_items(uint32_t rows, uint32_t unit_rows, uint32_t tiles, uint32_t waves)
+{
+	ScreenItems w;
+	w.units = (rows + unit_rows - 1) / unit_rows;
+	uint32_t want = w.units ? waves / w.units : 1u;
+	want = want < 1u ? 1u : (want > tiles ? tiles : want);
+	w.part_tiles = (tiles + want - 1) / want;
+	w.parts = (tiles + w.part_tiles - 1) / w.part_tiles;
+	w.items = w.units * w.parts;
+	return w;
+}
+/* upper bound of the number of items for up to `cap` rows */
+__host__ __forceinline__ uint32_t screen_items_max(uint32_t cap, uint32_t unit_rows)
+{
+	const uint32_t units = (cap + unit_rows - 1) / unit_rows;
+	return units > SCREEN_MAX_WAVES ? units : SCREEN_MAX_WAVES;
+}
+
 /* points of one sweep unit (P tiles of 32 points) -> registers as MFMA B operands; rows beyond n read as zero */
 template <int DPH, int P, int LD, bool VEC>
 __device__ __forceinline__ void load_points(float (&b)[P][DPH], const float* __restrict__ data, size_t stride,

@@ -45,8 +45,9 @@ int device_info(const DeviceInfo** out);
  *   packed means  : centroids re-laid-out (scaled by -2, padded) for the fast assignment kernels
  *   norms         : |c|^2 per (padded) centroid followed by max_j |c_j|^2
  *   partials      : per-work-group partial sums/counts of the update kernels that need them
- *   queued rows   : SoA points only: the rows of the queued points as a compact AoS block for the exact pass, with a
- *                   queue and an assignment vector of their own (counters[1] = rows taken, counters[2] = entries left over)
+ *   queued rows   : the rows of the queued points as a compact AoS block for the exact pass, with a
+ *                   queue and an assignment vector of their own (counters[1] = rows taken, counters[2] = entries left
+ *                   over); the split-bf16 sweep uses the block for every layout
  */
 struct Workspace {
 	uint32_t* queue = nullptr;      size_t queue_cap = 0;      /* entries */
@@ -58,7 +59,7 @@ struct Workspace {
 	uint32_t* fused_assignment = nullptr; size_t fused_cap = 0; /* entries: assignment vector of kmx_fused_f32 */
 	uint32_t* bucket_sizes = nullptr;     size_t bucket_cap = 0; /* entries: member counts nobody asked for (kmx_bucket_sum_f32) */
 	float* queued_rows = nullptr;         size_t queued_rows_cap = 0;   /* floats */
-	uint32_t* queued_index = nullptr;     size_t queued_index_cap = 0;  /* entries: 2 per row (queue) + 1 per row (assignment) */
+	uint32_t* queued_index = nullptr;     size_t queued_index_cap = 0;  /* words: per row 2 (queue) + 2 (assignment or 64-bit key), then the screen's pair counters and pairs */
 };
 int workspace(Workspace** ws);
 int reserve_queue(Workspace* ws, size_t entries);
@@ -66,7 +67,7 @@ int reserve_packed(Workspace* ws, size_t packed_floats, size_t norm_floats, size
 int reserve_partials(Workspace* ws, size_t floats);
 int reserve_fused_assignment(Workspace* ws, size_t entries);
 int reserve_bucket_sizes(Workspace* ws, size_t entries);
-int reserve_queued_rows(Workspace* ws, size_t rows, size_t dim);
+int reserve_queued_rows(Workspace* ws, size_t rows, size_t dim, size_t extra_words);
 
 #define KMX_HIP(call)                                                                                         \
 	do {                                                                                                      \
@@ -119,7 +120,15 @@ int launch_assign_base(const AssignArgs& a, kmx_exec_params* exec);
 /* Re-evaluates the points listed in ws->queue[0 .. counters[0]) with the serial arithmetic, reading the
  * exact transposed centroids ws->means_t ([dim][kp]) that pack_means wrote for this call. */
 int launch_recheck(const AssignArgs& a, Workspace* ws, uint32_t kp);
-void set_queued_rows_limit(size_t bytes); /* bound of the block of copied rows (SoA points) */
+void set_queued_rows_limit(size_t bytes); /* bound of the block of copied rows */
+/* The exact pass behind the split-bf16 sweep for k >= 128 and rows of more than 32 dimensions: the queued rows are copied into a compact block, a second
+ * split-bf16 sweep over them notes the (row, centroid) pairs within the threshold (assign_bf16.hip), and one lane
+ * per pair evaluates the serial arithmetic. */
+int launch_recheck_screened(const AssignArgs& a, Workspace* ws, uint32_t kp, const DeviceInfo& dev);
+int launch_screen_bf16(const float* rows, const Workspace* ws, const uint32_t* row_queue, const uint32_t* row_count,
+                       uint32_t* pairs, uint32_t* item_pairs, unsigned long long* keys, uint32_t dim, uint32_t k, uint32_t kp,
+                       const DeviceInfo& dev, uint32_t* waves);
+uint32_t screen_unit_rows(uint32_t dim);
 
 /* assign_mfma.hip / assign_lds_fma.hip: return KMX_ERR_UNSUPPORTED (without message side effects
  * beyond kmx_last_error) when the shape does not fit the variant. */

@@ -117,11 +117,11 @@ int reserve_partials(Workspace* ws, size_t floats) { return grow(&ws->partials, 
 int reserve_fused_assignment(Workspace* ws, size_t entries) { return grow(&ws->fused_assignment, &ws->fused_cap, entries); }
 int reserve_bucket_sizes(Workspace* ws, size_t entries) { return grow(&ws->bucket_sizes, &ws->bucket_cap, entries); }
 int reserve_f64(double** ptr, size_t* cap, size_t doubles) { return grow(ptr, cap, doubles); }
-int reserve_queued_rows(Workspace* ws, size_t rows, size_t dim)
+int reserve_queued_rows(Workspace* ws, size_t rows, size_t dim, size_t extra_words)
 {
 	int rc = grow(&ws->queued_rows, &ws->queued_rows_cap, rows * dim);
 	if (rc) return rc;
-	return grow(&ws->queued_index, &ws->queued_index_cap, 3 * rows);
+	return grow(&ws->queued_index, &ws->queued_index_cap, 4 * rows + extra_words);
 }
 
 static int release_workspace()
