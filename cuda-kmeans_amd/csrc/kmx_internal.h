@@ -58,6 +58,7 @@ struct Workspace {
 	float* partials = nullptr;      size_t partials_cap = 0;   /* floats  */
 	uint32_t* fused_assignment = nullptr; size_t fused_cap = 0; /* entries: assignment vector of kmx_fused_f32 */
 	uint32_t* bucket_sizes = nullptr;     size_t bucket_cap = 0; /* entries: member counts nobody asked for (kmx_bucket_sum_f32) */
+	float* rows_copy = nullptr;           size_t rows_copy_cap = 0;     /* floats: AoS copy of SoA points for the tuned update */
 	float* queued_rows = nullptr;         size_t queued_rows_cap = 0;   /* floats */
 	uint32_t* queued_index = nullptr;     size_t queued_index_cap = 0;  /* words: per row 2 (queue) + 2 (assignment or 64-bit key), then the screen's pair counters and pairs */
 };
@@ -67,6 +68,7 @@ int reserve_packed(Workspace* ws, size_t packed_floats, size_t norm_floats, size
 int reserve_partials(Workspace* ws, size_t floats);
 int reserve_fused_assignment(Workspace* ws, size_t entries);
 int reserve_bucket_sizes(Workspace* ws, size_t entries);
+int reserve_rows_copy(Workspace* ws, size_t floats);
 int reserve_queued_rows(Workspace* ws, size_t rows, size_t dim, size_t extra_words);
 
 #define KMX_HIP(call)                                                                                         \

@@ -117,6 +117,7 @@ int reserve_partials(Workspace* ws, size_t floats) { return grow(&ws->partials, 
 int reserve_fused_assignment(Workspace* ws, size_t entries) { return grow(&ws->fused_assignment, &ws->fused_cap, entries); }
 int reserve_bucket_sizes(Workspace* ws, size_t entries) { return grow(&ws->bucket_sizes, &ws->bucket_cap, entries); }
 int reserve_f64(double** ptr, size_t* cap, size_t doubles) { return grow(ptr, cap, doubles); }
+int reserve_rows_copy(Workspace* ws, size_t floats) { return grow(&ws->rows_copy, &ws->rows_copy_cap, floats); }
 int reserve_queued_rows(Workspace* ws, size_t rows, size_t dim, size_t extra_words)
 {
 	int rc = grow(&ws->queued_rows, &ws->queued_rows_cap, rows * dim);
@@ -134,6 +135,7 @@ static int release_workspace()
 	if (g_ws.partials) KMX_HIP(hipFree(g_ws.partials));
 	if (g_ws.fused_assignment) KMX_HIP(hipFree(g_ws.fused_assignment));
 	if (g_ws.bucket_sizes) KMX_HIP(hipFree(g_ws.bucket_sizes));
+	if (g_ws.rows_copy) KMX_HIP(hipFree(g_ws.rows_copy));
 	if (g_ws.queued_rows) KMX_HIP(hipFree(g_ws.queued_rows));
 	if (g_ws.queued_index) KMX_HIP(hipFree(g_ws.queued_index));
 	g_ws = Workspace();

@@ -790,8 +790,51 @@ int launch_divide_means(const UpdateArgs& u)
 	return KMX_OK;
 }
 
+/*
+ * SoA points and the tuned variant: the kernels that read whole rows (sorted chunks, private copies) are 5 to 10 times
+ * faster than anything that adds element by element (measured at N = 2M, d = 32, k = 1024: 0.07 ms against 0.68 ms for the
+ * LDS atomics), more than a transposition costs. The points are therefore copied into AoS rows first: tiles of
+ * 64 points x 32 dimensions through LDS, reads contiguous along the points, writes contiguous along the dimensions.
+ * Rows of fewer than 8 dimensions stay with the element-wise kernel (0.11 ms against 0.15 ms at N = 4M, d = 4, k = 4096).
+ */
+constexpr size_t ROWS_COPY_MAX_BYTES = (size_t)4 << 30; /* larger inputs keep the element-wise kernel */
+
+__global__ void __launch_bounds__(256)
+rows_from_soa_kernel(const float* __restrict__ data, size_t stride, float* __restrict__ rows, uint32_t dim, uint32_t n)
+{
+	__shared__ float tile[32][65];
+	const uint32_t tiles_q = (dim + 31) / 32;
+	const size_t tiles = (size_t)((n + 63) / 64) * tiles_q;
+	for (size_t t = blockIdx.x; t < tiles; t += gridDim.x) {
+		const uint32_t p0 = (uint32_t)(t / tiles_q) * 64, q0 = (uint32_t)(t % tiles_q) * 32;
+		__syncthreads(); /* the previous tile has been written out */
+		for (uint32_t q = threadIdx.x / 64; q < 32; q += 4) {
+			const uint32_t p = threadIdx.x % 64;
+			if (q0 + q < dim && p0 + p < n) tile[q][p] = data[(size_t)(q0 + q) * stride + p0 + p];
+		}
+		__syncthreads();
+		for (uint32_t p = threadIdx.x / 32; p < 64; p += 8) {
+			const uint32_t q = threadIdx.x % 32;
+			if (q0 + q < dim && p0 + p < n) rows[(size_t)(p0 + p) * dim + q0 + q] = tile[q][p];
+		}
+	}
+}
+
 int launch_update(int variant, const UpdateArgs& u, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev)
 {
+	if (u.layout == KMX_SOA && (variant & ~KMX_UPDATE_EMULATED_ATOMICS) == KMX_UPDATE_ATOMIC_SHM && u.n > 0 && u.dim >= 8 &&
+	    (size_t)u.n * u.dim * sizeof(float) <= ROWS_COPY_MAX_BYTES) {
+		int rc = reserve_rows_copy(ws, (size_t)u.n * u.dim);
+		if (rc) return rc;
+		const size_t tiles = (size_t)((u.n + 63) / 64) * ((u.dim + 31) / 32);
+		hipLaunchKernelGGL(rows_from_soa_kernel, dim3((uint32_t)std::min<size_t>(tiles, (size_t)dev.compute_units * 32)), dim3(256), 0, stream(),
+		                   u.data, u.stride, ws->rows_copy, u.dim, u.n);
+		KMX_LAUNCH_CHECK("rows_from_soa_kernel");
+		UpdateArgs rows = u;
+		rows.data = ws->rows_copy; rows.layout = KMX_AOS; rows.stride = u.dim;
+		return u.layout_means == KMX_AOS ? launch_update_t<KMX_AOS, KMX_AOS>(variant, rows, exec, ws, dev)
+		                                 : launch_update_t<KMX_AOS, KMX_SOA>(variant, rows, exec, ws, dev);
+	}
 	if (u.layout == KMX_AOS && u.layout_means == KMX_AOS) return launch_update_t<KMX_AOS, KMX_AOS>(variant, u, exec, ws, dev);
 	if (u.layout == KMX_AOS && u.layout_means == KMX_SOA) return launch_update_t<KMX_AOS, KMX_SOA>(variant, u, exec, ws, dev);
 	if (u.layout == KMX_SOA && u.layout_means == KMX_AOS) return launch_update_t<KMX_SOA, KMX_AOS>(variant, u, exec, ws, dev);
