@@ -260,6 +260,90 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 	const uint32_t unit_points = MFMA_WAVES * P * TILE;
 	const uint32_t units = (n + unit_points - 1) / unit_points;
 
+	/*
+	 * Rows of more than 64 dimensions (always streamed, one point tile per wavefront, whose split operands take half of the
+	 * register file). Per centroid tile: one chain of 3 KB MFMAs into a single accumulator that starts from the norms;
+	 * the centroid operands of block kb + 2 are requested from LDS before the MFMAs of block kb are issued
+	 * (sched_group_barrier pins that order: left to itself the scheduler reads each block right before its MFMAs and the
+	 * matrix pipe waits out an LDS round trip per block). The next chunk travels in pieces, one per tile step: requested
+	 * from global memory before the step's MFMAs, written to the other LDS buffer after them (a few registers instead of a
+	 * whole chunk's share). Lanes beyond the end of the chunk repeat its last piece, so the step has no branches.
+	 */
+	constexpr int AHEAD = 2; /* blocks of centroid operands requested before the first MFMA of a step (one in flight behind the one in use; a deeper pipeline measured no faster) */
+	constexpr uint32_t PIECE_VECS = (tile_floats(RS) / 4 + MFMA_WAVES * WAVE - 1) / (MFMA_WAVES * WAVE); /* 16-byte pieces per lane that cover one tile */
+	auto wide_sweep = [&](const SplitPoints<KB>& x, Track& st) {
+		for (uint32_t chunk = 0; chunk < chunks; ++chunk) {
+			const uint32_t row0 = chunk * chunk_rows;
+			const uint32_t rows = min(chunk_rows, kp - row0);
+			const uint32_t next_row0 = chunk + 1 < chunks ? row0 + chunk_rows : 0;
+			const uint32_t next_rows = min(chunk_rows, kp - next_row0);
+			const float* lds_tiles = lds + (size_t)cur * buf_floats;
+			const float* lds_norms = lds_tiles + (size_t)chunk_tiles * tile_floats(RS);
+			const uint32_t tiles = rows / TILE;
+			const uint32_t tile0 = row0 / TILE;
+			const f32x4* src = (const f32x4*)(packed + packed_row(next_row0, RS));
+			const f32x4* nsrc = (const f32x4*)(norms + (size_t)(next_row0 / TILE) * NORM_TILE);
+			f32x4* dst = (f32x4*)(lds + (size_t)(cur ^ 1u) * buf_floats);
+			f32x4* ndst = (f32x4*)(lds + (size_t)(cur ^ 1u) * buf_floats + (size_t)chunk_tiles * tile_floats(RS));
+			const uint32_t last_vec = (next_rows / TILE) * tile_floats(RS) / 4 - 1;
+			const uint32_t norm_vec = min((uint32_t)threadIdx.x, (next_rows / TILE) * NORM_TILE / 4 - 1);
+			uint32_t piece = threadIdx.x; /* first 16-byte piece of this lane in the current step */
+			for (uint32_t t = 0; t < tiles; ++t) {
+				f32x4 pv[PIECE_VECS];
+#pragma unroll
+				for (uint32_t i = 0; i < PIECE_VECS; ++i) pv[i] = src[min(piece + i * (MFMA_WAVES * WAVE), last_vec)];
+				const f32x4 nv = nsrc[norm_vec];
+				const float* arow = lds_tiles + (size_t)t * tile_floats(RS) + (size_t)col * RS;
+				f32x16 acc;
+#pragma unroll
+				for (int g = 0; g < 4; ++g) {
+					f32x4 v = *(const f32x4*)(lds_norms + t * NORM_TILE + 8 * g + 4 * h);
+					acc[4 * g] = v.x; acc[4 * g + 1] = v.y; acc[4 * g + 2] = v.z; acc[4 * g + 3] = v.w;
+				}
+				bf16x8 chi[KB], cmid[KB];
+#pragma unroll
+				for (int kb = 0; kb < AHEAD; ++kb) {
+					chi[kb] = row_unit(arow, 4 * kb + 2 * h);
+					cmid[kb] = row_unit(arow, 4 * kb + 2 * h + 1);
+				}
+#pragma unroll
+				for (int kb = 0; kb < KB; ++kb) {
+					if (kb + AHEAD < KB) {
+						chi[kb + AHEAD] = row_unit(arow, 4 * (kb + AHEAD) + 2 * h);
+						cmid[kb + AHEAD] = row_unit(arow, 4 * (kb + AHEAD) + 2 * h + 1);
+					}
+					acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(chi[kb], x.mid[kb], acc, 0, 0, 0);
+					acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cmid[kb], x.hi[kb], acc, 0, 0, 0);
+					acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(chi[kb], x.hi[kb], acc, 0, 0, 0);
+				}
+				track_tile<false, false>(acc, st, tile0 + t, neg_inf);
+#pragma unroll
+				for (uint32_t i = 0; i < PIECE_VECS; ++i) dst[min(piece + i * (MFMA_WAVES * WAVE), last_vec)] = pv[i];
+				ndst[norm_vec] = nv;
+				piece += PIECE_VECS * (MFMA_WAVES * WAVE);
+				/* the order of the step: global requests; norms and AHEAD blocks of operands; then per block its MFMAs
+				 * and the request for the block AHEAD blocks on; tracking and the LDS writes come last by their dependences */
+				__builtin_amdgcn_sched_group_barrier(0x020, PIECE_VECS + 1, 0);
+				__builtin_amdgcn_sched_group_barrier(0x100, 4 + 2 * AHEAD, 0);
+#pragma unroll
+				for (int kb = 0; kb < KB; ++kb) {
+					__builtin_amdgcn_sched_group_barrier(0x008, 3, 0);
+					if (kb + AHEAD < KB) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+				}
+			}
+			/* a short chunk (the last one) has fewer steps than the next chunk has tiles: the remaining pieces */
+			for (; piece - threadIdx.x <= last_vec; piece += PIECE_VECS * (MFMA_WAVES * WAVE)) {
+#pragma unroll
+				for (uint32_t i = 0; i < PIECE_VECS; ++i) {
+					const uint32_t at = min(piece + i * (MFMA_WAVES * WAVE), last_vec);
+					dst[at] = src[at];
+				}
+			}
+			__syncthreads();
+			cur ^= 1u;
+		}
+	};
+
 	auto sweep = [&](const SplitPoints<KB> (&b)[P], const float (&xx)[P], uint32_t base) {
 		float x2[P];
 		Track st[P];
@@ -272,6 +356,10 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 			st[p].loc = 0;
 		}
 		f32x16 acc0[P], acc1[P];
+		if constexpr (KB > 4) {
+			wide_sweep(b[0], st[0]);
+		}
+		else
 		for (uint32_t chunk = 0; chunk < chunks; ++chunk) {
 			const uint32_t row0 = chunk * chunk_rows;
 			const uint32_t rows = min(chunk_rows, kp - row0);
