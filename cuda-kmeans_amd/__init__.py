@@ -434,8 +434,10 @@ class HipKMeansAlgorithm:
         return nxt
 
     def update_step(self, nxt):
-        self.cu_means[nxt].zero()
-        self.cu_sizes.zero()
+        # the tuned float update clears or overwrites its outputs itself (kmx_update_f32, KMX_UPDATE_ATOMIC_SHM)
+        if not (self.update_variant == UPDATE_ATOMIC_SHM and np.dtype(self.dtype) == np.float32):
+            self.cu_means[nxt].zero()
+            self.cu_sizes.zero()
         update(self.update_variant, self.cu_data, self.layout, self.stride, self.cu_assignment[nxt], self.cu_means[nxt],
                self.layout_means, self.stride_means, self.cu_sizes, self.dim, self.k, self.n, self.exec, self.dtype)
         self.last = nxt

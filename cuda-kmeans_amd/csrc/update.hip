@@ -310,8 +310,8 @@ update_private_kernel(const float* __restrict__ data, size_t stride, const uint3
  *      (groups of GW lanes, lane = dimension), balanced by entry count; a group walks its range in batches
  *      of 8 entries (8 row loads in flight), adds in a register and stores a cluster's row of sums when the
  *      cluster changes -- zero rows for clusters without members, so the partial buffer needs no clearing.
- * Per-chunk counts go to cluster_sizes with integer global atomics (dimension slice 0 only).
- * partial layout: [chunk][cluster][dim].
+ * Per-chunk counts go to a second partial array (dimension slice 0 only), so that nothing has to be zero beforehand.
+ * partial layouts: [chunk][cluster][dim] and [chunk][cluster].
  */
 constexpr uint32_t SORT_SHIFT = 15; /* local point index bits: chunk_points <= 32768 */
 constexpr int SORT_UNROLL = 8;      /* row loads per batch and lane group in the segment-sum phase (two batches in flight) */
@@ -349,7 +349,7 @@ __device__ __forceinline__ void store_part(float* p, const RowPart<VEC>& r)
 template <int ITEMS, int GW, int VEC>
 __global__ void __launch_bounds__(1024)
 update_sorted_kernel(const float* __restrict__ data, size_t stride, const uint32_t* __restrict__ assignment,
-                     float* __restrict__ partial, uint32_t* __restrict__ sizes,
+                     float* __restrict__ partial, uint32_t* __restrict__ partial_counts,
                      uint32_t dim, uint32_t k, uint32_t n, uint32_t chunk_points)
 {
 	extern __shared__ uint32_t sm[];
@@ -380,12 +380,9 @@ update_sorted_kernel(const float* __restrict__ data, size_t stride, const uint32
 	}
 	__syncthreads();
 
-	/* counts of this chunk */
+	/* counts of this chunk: a row of the count partials, every entry written */
 	if (blockIdx.y == 0)
-		for (uint32_t c = tid; c < k; c += 1024) {
-			const uint32_t s = offsets[c];
-			if (s) atomicAdd(&sizes[c], s);
-		}
+		for (uint32_t c = tid; c < k; c += 1024) partial_counts[(size_t)blockIdx.x * k + c] = offsets[c];
 
 	/* 2. exclusive scan of offsets[0..k) in place; offsets[k] = number of entries */
 	const uint32_t per = (k + 1023) / 1024;
@@ -509,17 +506,28 @@ constexpr uint32_t REDUCE_SHARES = 16;
 
 template <int LM>
 __global__ void __launch_bounds__(64 * REDUCE_SHARES)
-reduce_partials_kernel(const float* __restrict__ partial, float* __restrict__ means, size_t stride_means,
-                       const uint32_t* __restrict__ sizes, uint32_t dim, uint32_t k, uint32_t chunks, uint32_t divide)
+reduce_partials_kernel(const float* __restrict__ partial, const uint32_t* __restrict__ partial_counts, float* __restrict__ means, size_t stride_means,
+                       uint32_t* __restrict__ sizes, uint32_t dim, uint32_t k, uint32_t chunks, uint32_t divide)
 {
 	__shared__ float part[REDUCE_SHARES][64];
+	__shared__ uint32_t part_count[REDUCE_SHARES][64];
 	const uint32_t col = threadIdx.x & 63, share = threadIdx.x >> 6;
 	const uint32_t e = blockIdx.x * 64 + col;
 	const size_t kd = (size_t)k * dim;
+	const uint32_t per = (chunks + REDUCE_SHARES - 1) / REDUCE_SHARES;
+	const uint32_t c0 = min(share * per, chunks), c1 = min(c0 + per, chunks);
+	/* the clusters the 64 elements of this work-group belong to (at most 64): lane `col` counts cluster cl_lo + col */
+	const uint32_t cl_lo = (uint32_t)(((size_t)blockIdx.x * 64) / dim);
+	const uint32_t cl_hi = (uint32_t)min((size_t)k - 1, ((size_t)blockIdx.x * 64 + 63) / dim);
+	/* the count partials of this lane's cluster are requested first and added up after the sums, so that both sets of
+	 * loads are in flight together */
+	const bool counting = cl_lo + col <= cl_hi;
+	const uint32_t* pc = partial_counts + cl_lo + (counting ? col : 0);
+	uint32_t cv[16];
+#pragma unroll
+	for (int u = 0; u < 16; ++u) cv[u] = (counting && c0 + u < c1) ? pc[(size_t)(c0 + u) * k] : 0u;
 	float s = 0.0f;
 	if (e < kd) {
-		const uint32_t per = (chunks + REDUCE_SHARES - 1) / REDUCE_SHARES;
-		const uint32_t c0 = min(share * per, chunks), c1 = min(c0 + per, chunks);
 		uint32_t c = c0;
 		for (; c + 16 <= c1; c += 16) {
 			float v[16];
@@ -530,6 +538,12 @@ reduce_partials_kernel(const float* __restrict__ partial, float* __restrict__ me
 		}
 		for (; c < c1; ++c) s += partial[(size_t)c * kd + e];
 	}
+	uint32_t members = 0;
+#pragma unroll
+	for (int u = 0; u < 16; ++u) members += cv[u];
+	if (counting)
+		for (uint32_t c = c0 + 16; c < c1; ++c) members += pc[(size_t)c * k];
+	part_count[share][col] = members;
 	part[share][col] = s;
 	__syncthreads();
 	if (share == 0 && e < kd) {
@@ -537,8 +551,22 @@ reduce_partials_kernel(const float* __restrict__ partial, float* __restrict__ me
 #pragma unroll
 		for (uint32_t i = 0; i < REDUCE_SHARES; ++i) s += part[i][col];
 		const uint32_t cl = e / dim, d = e - cl * dim;
-		const uint32_t count = sizes[cl];
+		uint32_t count = 0;
+#pragma unroll
+		for (uint32_t i = 0; i < REDUCE_SHARES; ++i) count += part_count[i][cl - cl_lo];
+		if (d == 0) sizes[cl] = count; /* the work-group that holds the cluster's first element publishes its size */
 		means[elem<LM>(stride_means, cl, d)] = !divide ? s : (count ? s / (float)count : 0.0f);
+	}
+}
+
+/* means (replica 0) and cluster sizes := 0 in one launch, for the kernels that accumulate into them */
+__global__ void __launch_bounds__(256)
+clear_outputs_kernel(uint32_t* __restrict__ means_words, size_t words, uint32_t* __restrict__ sizes, uint32_t k)
+{
+	const size_t threads = (size_t)blockDim.x * gridDim.x;
+	for (size_t i = threadIdx.x + (size_t)blockIdx.x * blockDim.x; i < words + k; i += threads) {
+		if (i < words) means_words[i] = 0u;
+		else sizes[i - words] = 0u;
 	}
 }
 
@@ -577,6 +605,16 @@ static size_t copy_floats_of(const UpdateArgs& u)
 	return u.layout_means == KMX_AOS ? (size_t)u.k * u.stride_means : (size_t)u.dim * u.stride_means;
 }
 
+/* The tuned variant does not ask for zeroed outputs: the kernels that accumulate into them start with this. */
+static int clear_outputs(const UpdateArgs& u)
+{
+	const size_t words = copy_floats_of(u);
+	const uint32_t blocks = (uint32_t)std::min<size_t>((words + u.k + 255) / 256, 1024);
+	hipLaunchKernelGGL(clear_outputs_kernel, dim3(std::max(blocks, 1u)), dim3(256), 0, stream(), (uint32_t*)u.means, words, u.cluster_sizes, u.k);
+	KMX_LAUNCH_CHECK("clear_outputs_kernel");
+	return KMX_OK;
+}
+
 static uint32_t pow2_at_least(uint32_t v)
 {
 	uint32_t p = 1;
@@ -588,6 +626,7 @@ template <int ITEMS, int LM>
 static int launch_sorted(const UpdateArgs& u, Workspace* ws, uint32_t chunks, uint32_t slices, uint32_t chunk_points, uint32_t gw, uint32_t vec, uint32_t lds_bytes)
 {
 	void (*kernel)(const float*, size_t, const uint32_t*, float*, uint32_t*, uint32_t, uint32_t, uint32_t, uint32_t) = nullptr;
+	uint32_t* partial_counts = (uint32_t*)(ws->partials + (size_t)chunks * u.k * u.dim);
 	if (vec == 4) {
 		switch (gw) {
 		case 1: kernel = update_sorted_kernel<ITEMS, 1, 4>; break;
@@ -605,11 +644,11 @@ static int launch_sorted(const UpdateArgs& u, Workspace* ws, uint32_t chunks, ui
 	}
 	KMX_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
 	hipLaunchKernelGGL(kernel, dim3(chunks, slices), dim3(1024), lds_bytes, stream(),
-	                   u.data, u.stride, u.assignment, ws->partials, u.cluster_sizes, u.dim, u.k, u.n, chunk_points);
+	                   u.data, u.stride, u.assignment, ws->partials, partial_counts, u.dim, u.k, u.n, chunk_points);
 	KMX_LAUNCH_CHECK("update_sorted_kernel");
 	const uint32_t total = u.k * u.dim;
 	hipLaunchKernelGGL((reduce_partials_kernel<LM>), dim3((total + 63) / 64), dim3(64 * REDUCE_SHARES), 0, stream(),
-	                   ws->partials, u.means, u.stride_means, u.cluster_sizes, u.dim, u.k, chunks, u.divide ? 1u : 0u);
+	                   ws->partials, partial_counts, u.means, u.stride_means, u.cluster_sizes, u.dim, u.k, chunks, u.divide ? 1u : 0u);
 	KMX_LAUNCH_CHECK("reduce_partials_kernel");
 	return KMX_OK;
 }
@@ -637,6 +676,8 @@ static int launch_update_tuned(const UpdateArgs& u, kmx_exec_params* exec, Works
 			chunk_points = (chunk_points + quantum - 1) / quantum * quantum;
 			chunks = (u.n + chunk_points - 1) / chunk_points;
 			exec->block_count = chunks;
+			int rc = clear_outputs(u);
+			if (rc) return rc;
 			hipLaunchKernelGGL((update_private_kernel<LM>), dim3(chunks), dim3(256), (uint32_t)lds_bytes, stream(),
 			                   u.data, u.stride, u.assignment, u.means, u.stride_means, u.cluster_sizes,
 			                   u.dim, u.k, u.n, gw, (uint32_t)copy_stride, chunk_points);
@@ -656,7 +697,7 @@ static int launch_update_tuned(const UpdateArgs& u, kmx_exec_params* exec, Works
 		chunk_points = std::min(max_points, (chunk_points + 1023) / 1024 * 1024);
 		chunks = (u.n + chunk_points - 1) / chunk_points;
 		const uint32_t lds_bytes = (u.k + 33 + chunk_points) * 4;
-		int rc = reserve_partials(ws, (size_t)chunks * u.k * u.dim);
+		int rc = reserve_partials(ws, (size_t)chunks * u.k * u.dim + (size_t)chunks * u.k); /* sums, then counts */
 		if (rc) return rc;
 		exec->block_count = chunks * slices;
 		*state = 2;
@@ -677,6 +718,8 @@ static int launch_update_tuned(const UpdateArgs& u, kmx_exec_params* exec, Works
 		for (uint32_t nice : { 32u, 16u, 8u, 4u })
 			if (slice >= nice) { slice = slice / nice * nice; break; }
 	}
+	int rc = clear_outputs(u);
+	if (rc) return rc;
 	if (slice == 0) {
 		*state = 0;
 		return KMX_OK;
@@ -762,6 +805,9 @@ static int launch_update_t(int variant, const UpdateArgs& u, kmx_exec_params* ex
 		}
 #undef KMX_UPDATE_LAUNCH
 		if ((rc = profile_end(1))) return rc;
+	}
+	else if (variant == KMX_UPDATE_ATOMIC_SHM) {
+		if ((rc = clear_outputs(u))) return rc; /* no points: every cluster is empty */
 	}
 
 	const uint32_t total = u.k * u.dim;

@@ -184,10 +184,12 @@ KMX_DEFINE_FUSED_KERNEL(FusedBestKernel, KMX_FUSED_BEST)        /* one pass wher
 
 /* EMUL (the reference's template argument, kernels.cuh:96-105): additions as compare-and-swap loops; built for the float
  * point and fine kernels (KMX_UPDATE_EMULATED_ATOMICS), ignored by the LDS kernels, which have no global fp32 atomics to emulate */
-#define KMX_DEFINE_UPDATE_KERNEL(NAME, VARIANT, CAN_EMULATE)\
+#define KMX_DEFINE_UPDATE_KERNEL(NAME, VARIANT, CAN_EMULATE, SELF_CLEARING)\
 template<typename F, typename IDX_T, class LAYOUT, class LAYOUT_MEANS, int EMUL = false>\
 class NAME {\
 public:\
+	/* false: the runner clears or overwrites its outputs itself, the driver may leave out the two runFillZeros calls */\
+	static constexpr bool needsZeroedOutput = !(SELF_CLEARING && std::is_same<F, float>::value);\
 	static void run(const UpdateProblemInstance<F, IDX_T>& in, HipExecParameters& exec)\
 	{\
 		static_assert(!(EMUL && CAN_EMULATE) || std::is_same<F, float>::value, "emulated atomics are built for floats");\
@@ -195,8 +197,8 @@ public:\
 	}\
 };
 
-KMX_DEFINE_UPDATE_KERNEL(UpdateAtomicPointKernel, KMX_UPDATE_ATOMIC_POINT, true) /* kernels.cu:726-761 */
-KMX_DEFINE_UPDATE_KERNEL(UpdateAtomicFineKernel, KMX_UPDATE_ATOMIC_FINE, true)   /* kernels.cu:770-809 */
-KMX_DEFINE_UPDATE_KERNEL(UpdateAtomicShmKernel, KMX_UPDATE_ATOMIC_SHM, false)    /* kernels.cu:817-878 */
+KMX_DEFINE_UPDATE_KERNEL(UpdateAtomicPointKernel, KMX_UPDATE_ATOMIC_POINT, true, false) /* kernels.cu:726-761 */
+KMX_DEFINE_UPDATE_KERNEL(UpdateAtomicFineKernel, KMX_UPDATE_ATOMIC_FINE, true, false)   /* kernels.cu:770-809 */
+KMX_DEFINE_UPDATE_KERNEL(UpdateAtomicShmKernel, KMX_UPDATE_ATOMIC_SHM, false, true)    /* kernels.cu:817-878 */
 
 #endif

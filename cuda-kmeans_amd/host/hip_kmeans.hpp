@@ -135,8 +135,10 @@ private:
 		AssignmentProblemInstance<F, IDX_T> assignment(*mDevData, *mDevMeans[mLast], *mDevAssignment[mLast],
 			*mDevAssignment[next], this->mDim, this->mK, this->mN);
 		ASGN_KERNEL::run(assignment, mExecParams);
-		runFillZeros<F>(*mDevMeans[next], meansSize() * copies);
-		runFillZeros<IDX_T>(*mDevClusterSizes, this->mK);
+		if (UPDATE_KERNEL::needsZeroedOutput) {
+			runFillZeros<F>(*mDevMeans[next], meansSize() * copies);
+			runFillZeros<IDX_T>(*mDevClusterSizes, this->mK);
+		}
 		UpdateProblemInstance<F, IDX_T> update(*mDevData, *mDevAssignment[next], *mDevMeans[next], *mDevClusterSizes,
 			this->mDim, this->mK, this->mN);
 		UPDATE_KERNEL::run(update, mExecParams);
@@ -181,8 +183,10 @@ public:
 			ASGN_KERNEL::run(assignment, mExecParams);
 			if (mTimeSplit) KMX_CHECK(kmx_event_record(ev[1]));
 
-			runFillZeros<F>(*mDevMeans[next], meansSize() * copies);
-			runFillZeros<IDX_T>(*mDevClusterSizes, this->mK);
+			if (UPDATE_KERNEL::needsZeroedOutput) {
+				runFillZeros<F>(*mDevMeans[next], meansSize() * copies);
+				runFillZeros<IDX_T>(*mDevClusterSizes, this->mK);
+			}
 			UpdateProblemInstance<F, IDX_T> update(*mDevData, *mDevAssignment[next], *mDevMeans[next], *mDevClusterSizes,
 				this->mDim, this->mK, this->mN);
 			UPDATE_KERNEL::run(update, mExecParams);

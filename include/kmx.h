@@ -134,6 +134,9 @@ int kmx_assign_last_variant(int* variant);
  * variants 0 and 1) and cluster_sizes (k) are zero. Accumulates member sums and counts, merges
  * the privatised replicas and divides every non-empty cluster by its count; empty clusters stay
  * at zero (kernels.cu:149-163, serial.hpp:66-67).
+ * KMX_UPDATE_ATOMIC_SHM has no precondition: it overwrites means (replica 0) and cluster_sizes, or
+ * clears them itself where its kernel accumulates into them, so a driver may leave out the two
+ * runFillZeros calls of cuda.hpp:78-79 (zeroing anyway is harmless).
  */
 int kmx_update_f32(int variant,
                    const float* data, int layout, size_t stride,

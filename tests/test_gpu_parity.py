@@ -45,14 +45,18 @@ def gpu_assign(km, variant, data, means, dim, k, n, layout=AOS, layout_means=AOS
     return out, rechecked
 
 
-def gpu_update(km, variant, data, assignment, dim, k, n, layout=AOS, layout_means=AOS, exec_params=None):
+def gpu_update(km, variant, data, assignment, dim, k, n, layout=AOS, layout_means=AOS, exec_params=None, dirty=False):
     ex = exec_params if exec_params is not None else km.ExecParams()
     copies = max(1, ex.privatized_copies)
     d = km.DeviceBuffer(4 * max(data.size, 1)); d.write(data)
     a = km.DeviceBuffer(4 * max(n, 1)); a.write(assignment)
     msize = km.layout_size(layout_means, k, dim)
-    m = km.DeviceBuffer(4 * msize * copies); m.zero()
-    s = km.DeviceBuffer(4 * k); s.zero()
+    m = km.DeviceBuffer(4 * msize * copies)
+    s = km.DeviceBuffer(4 * k)
+    if dirty:   # outputs full of leftovers (NaN bit patterns and large counts) instead of zeros
+        m.write(np.full(msize * copies, 0x7FC12345, np.uint32)); s.write(np.full(k, 0xDEADBEEF, np.uint32))
+    else:
+        m.zero(); s.zero()
     km.update(variant, d, layout, km.layout_stride(layout, n, dim), a, m, layout_means,
               km.layout_stride(layout_means, k, dim), s, dim, k, n, ex)
     km.sync()
@@ -261,6 +265,25 @@ def test_update_matches_oracle(km, orc, gpu, dim, k, n, layout, layout_means):
         if k > 2:
             lm = means.reshape(k, dim) if layout_means == AOS else means.reshape(dim, k).T
             assert np.all(lm[1] == 0), "empty cluster must stay at the origin"
+
+
+@pytest.mark.parametrize("dim,k,n", UPDATE_SHAPES + [(8, 64, 0), (32, 1024, 0)])
+@pytest.mark.parametrize("layout,layout_means", [(AOS, AOS), (SOA, SOA), (AOS, SOA), (SOA, AOS)])
+def test_tuned_update_needs_no_zeroed_outputs(km, orc, gpu, dim, k, n, layout, layout_means):
+    """KMX_UPDATE_ATOMIC_SHM overwrites or clears its outputs itself: leftovers in them change nothing."""
+    rng = np.random.default_rng(3 * k + dim)
+    data = rng.normal(size=n * dim).astype(np.float32) * np.float32(5) + np.float32(2)
+    asg = np.minimum((rng.exponential(scale=k / 4, size=n)).astype(np.uint32), k - 1).astype(np.uint32)
+    if k > 2:
+        asg[asg == 1] = 0
+    want_means, want_sizes = orc.update(data, asg, dim, k, n, layout, layout_means, threads=0)
+    for ex in (km.ExecParams(), km.ExecParams(shared_mem_bytes=48 * 1024)):
+        means, sizes = gpu_update(km, km.UPDATE_ATOMIC_SHM, data, asg, dim, k, n, layout, layout_means, ex, dirty=True)
+        assert np.array_equal(sizes, want_sizes)
+        assert rel_err(means, want_means) < CENTROID_RTOL
+        if k > 2:
+            lm = means.reshape(k, dim) if layout_means == AOS else means.reshape(dim, k).T
+            assert np.all(lm[1] == 0), "empty cluster must end at the origin"
 
 
 # ---------------------------------------------------------------- the Lloyd loop
