@@ -60,11 +60,21 @@ def cpu_baseline(km, spec, n_sample, data, means0):
         orc.kmeans(sample, means0, dim, k, n_sample, 1, threads=1, fast=False)
         dt = time.perf_counter() - t0
     scaled_ms = dt * 1e3 * (int(spec.n) / n_sample)
-    return {
+    out = {
         "value": round(scaled_ms, 1), "unit": "ms/iteration", "cores": 1, "kind": kind,
         "sample": "1 iteration over the first %d of %d points x all %d centroids took %.2f s on 1 core; scaled by N/sample"
                   % (n_sample, int(spec.n), k, dt),
     }
+    # the same iteration with the restatement's OpenMP mode (results bit-identical to one thread): what the host cores
+    # of this box deliver together; the reference itself has no multi-threaded CPU path
+    cores = int(os.environ.get("OMP_NUM_THREADS") or 0) or min(os.cpu_count() or 1, 16)
+    if cores > 1:
+        t0 = time.perf_counter()
+        orc.kmeans(sample, means0, dim, k, n_sample, 1, threads=cores, fast=False)
+        dt_all = time.perf_counter() - t0
+        out["all_cores"] = {"value": round(dt_all * 1e3 * (int(spec.n) / n_sample), 1), "unit": "ms/iteration", "cores": cores,
+                            "kind": "port", "sample": "same sample, %d OpenMP threads: %.2f s" % (cores, dt_all)}
+    return out
 
 
 def fused_main(km, args, spec, data, means0):
