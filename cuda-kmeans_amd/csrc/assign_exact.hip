@@ -351,7 +351,7 @@ recheck_points_kernel(const float* __restrict__ data, size_t stride, const float
 	const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE), waves = blockDim.x / WAVE;
 	const uint32_t count = counters[0];
 	const uint32_t slots = gridDim.x;
-	const uint32_t pb = count > slots * 32 ? 64 : count > slots * 16 ? 32 : 16;
+	const uint32_t pb = min(POINTS_BATCH, max(16u, (count + slots - 1) / slots)); /* one batch per work-group while 64 points suffice for that */
 	const uint32_t batches = (count + pb - 1) / pb;
 
 	for (uint32_t batch = blockIdx.x; batch < batches; batch += gridDim.x) {
