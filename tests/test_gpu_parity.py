@@ -267,7 +267,7 @@ def test_update_matches_oracle(km, orc, gpu, dim, k, n, layout, layout_means):
             assert np.all(lm[1] == 0), "empty cluster must stay at the origin"
 
 
-@pytest.mark.parametrize("dim,k,n", UPDATE_SHAPES + [(8, 64, 0), (32, 1024, 0)])
+@pytest.mark.parametrize("dim,k,n", UPDATE_SHAPES + [(8, 64, 0), (32, 1024, 0), (8, 1024, 9000000)])   # the last: more than 256 chunks of sorted points
 @pytest.mark.parametrize("layout,layout_means", [(AOS, AOS), (SOA, SOA), (AOS, SOA), (SOA, AOS)])
 def test_tuned_update_needs_no_zeroed_outputs(km, orc, gpu, dim, k, n, layout, layout_means):
     """KMX_UPDATE_ATOMIC_SHM overwrites or clears its outputs itself: leftovers in them change nothing."""
