@@ -512,9 +512,10 @@ reduce_partials_kernel(const float* __restrict__ partial, const uint32_t* __rest
 	__shared__ float part[REDUCE_SHARES][64];
 	__shared__ uint32_t part_count[REDUCE_SHARES][64];
 	const uint32_t col = threadIdx.x & 63, share = threadIdx.x >> 6;
+	const uint32_t shares = blockDim.x >> 6; /* 1 to REDUCE_SHARES: the launcher gives every share at least 8 chunks */
 	const uint32_t e = blockIdx.x * 64 + col;
 	const size_t kd = (size_t)k * dim;
-	const uint32_t per = (chunks + REDUCE_SHARES - 1) / REDUCE_SHARES;
+	const uint32_t per = (chunks + shares - 1) / shares;
 	const uint32_t c0 = min(share * per, chunks), c1 = min(c0 + per, chunks);
 	/* the clusters the 64 elements of this work-group belong to (at most 64): lane `col` counts cluster cl_lo + col */
 	const uint32_t cl_lo = (uint32_t)(((size_t)blockIdx.x * 64) / dim);
@@ -548,12 +549,10 @@ reduce_partials_kernel(const float* __restrict__ partial, const uint32_t* __rest
 	__syncthreads();
 	if (share == 0 && e < kd) {
 		s = 0.0f;
-#pragma unroll
-		for (uint32_t i = 0; i < REDUCE_SHARES; ++i) s += part[i][col];
+		for (uint32_t i = 0; i < shares; ++i) s += part[i][col];
 		const uint32_t cl = e / dim, d = e - cl * dim;
 		uint32_t count = 0;
-#pragma unroll
-		for (uint32_t i = 0; i < REDUCE_SHARES; ++i) count += part_count[i][cl - cl_lo];
+		for (uint32_t i = 0; i < shares; ++i) count += part_count[i][cl - cl_lo];
 		if (d == 0) sizes[cl] = count; /* the work-group that holds the cluster's first element publishes its size */
 		means[elem<LM>(stride_means, cl, d)] = !divide ? s : (count ? s / (float)count : 0.0f);
 	}
@@ -647,7 +646,8 @@ static int launch_sorted(const UpdateArgs& u, Workspace* ws, uint32_t chunks, ui
 	                   u.data, u.stride, u.assignment, ws->partials, partial_counts, u.dim, u.k, u.n, chunk_points);
 	KMX_LAUNCH_CHECK("update_sorted_kernel");
 	const uint32_t total = u.k * u.dim;
-	hipLaunchKernelGGL((reduce_partials_kernel<LM>), dim3((total + 63) / 64), dim3(64 * REDUCE_SHARES), 0, stream(),
+	const uint32_t shares = std::max<uint32_t>(1, std::min<uint32_t>(REDUCE_SHARES, chunks / 8));
+	hipLaunchKernelGGL((reduce_partials_kernel<LM>), dim3((total + 63) / 64), dim3(64 * shares), 0, stream(),
 	                   ws->partials, partial_counts, u.means, u.stride_means, u.cluster_sizes, u.dim, u.k, chunks, u.divide ? 1u : 0u);
 	KMX_LAUNCH_CHECK("reduce_partials_kernel");
 	return KMX_OK;
