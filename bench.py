@@ -1,16 +1,18 @@
 #!/usr/bin/env python3
 """Benchmark of the Lloyd iteration on one MI355X.
 
-    python bench.py [--gpus 1] [--steps 20] [--warmup 5] [--config 2]
+    python bench.py [--gpus 1] [--steps 20] [--warmup 100] [--config 2]
 
-A "step" is one full k-means iteration (assignment + zero-fill + update + divide) over the whole
+A "step" is one full k-means iteration (assignment + update + divide) over the whole
 synthetic data set of the chosen benchmark configuration (default: the headline, N = 2,097,152,
 d = 32, k = 1024, fp32, seeded Gaussian mixture, initial centroids = first k points), with the points
 and the initial centroids already resident in HBM when the clock starts -- the reference's protocol
 (k-means.cpp:155-169: wall clock around run(), transfers excluded). Prints ONE JSON line.
 
 Legs:
-  1. warm-up iterations, then state reset;
+  1. warm-up: the configuration's own run (20 iterations from the initial centroids at the headline) repeated until
+     --warmup iterations are done, each followed by a state reset: the first 50 or so iterations after an idle period
+     run up to 15 % slower than the following ones;
   2. the timed region: K iterations back to back on the library's stream, one sync on each side,
      wall clock -> value / ms_per_step; every kernel is launched call by call (--graph: the first iteration call by
      call, the others as replays of a recorded pair of iterations, a HIP graph);
@@ -77,14 +79,24 @@ def cpu_baseline(km, spec, n_sample, data, means0):
     return out
 
 
+def warm_up(alg, args, spec, means0, **run_args):
+    """The untimed iterations: the configuration's own run (its iteration count, from the initial centroids) as often
+    as --warmup asks for, so that the timed run starts from the same state on a device at its working clocks (the
+    first 50 or so iterations after an idle period run up to 15 % slower)."""
+    left = args.warmup
+    while left > 0:
+        it = min(left, max(1, int(spec.iterations)))
+        alg.run(iters=it, **run_args)
+        alg.reset(means0)
+        left -= it
+
+
 def fused_main(km, args, spec, data, means0):
     """--fused: the same protocol around HipFusedKMeansAlgorithm (mirror of CudaFusedKMeansAlgorithm, cuda.hpp:116-233)."""
     n, dim, k = int(spec.n), spec.dim, spec.k
     alg = km.HipFusedKMeansAlgorithm()
     alg.initialize(dim, k, n, args.steps, data, means0)
-    alg.run(iters=args.warmup)
-    alg.cleanup()
-    alg.initialize(dim, k, n, args.steps, data, means0)
+    warm_up(alg, args, spec, means0)
     km.sync()
     t0 = time.perf_counter()
     alg.run(iters=args.steps)
@@ -129,8 +141,7 @@ def double_main(km, args, spec, data, means0):
     data, means0 = km.widen_points(data), km.widen_points(means0)
     alg = km.HipKMeansAlgorithm(dtype=np.float64)
     alg.initialize(dim, k, n, args.steps, data, means0)
-    alg.run(iters=args.warmup)
-    alg.reset(means0)
+    warm_up(alg, args, spec, means0)
     km.sync()
     t0 = time.perf_counter()
     alg.run(iters=args.steps)
@@ -185,7 +196,8 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=100,
+                    help="untimed iterations before the timed ones, run as repetitions of the configuration's own run")
     ap.add_argument("--config", type=int, default=2, help="benchmark configuration 1..5 (2 = headline)")
     ap.add_argument("--cpu-sample", type=int, default=0, help="points in the CPU baseline sample (0 = about 12 s of work)")
     ap.add_argument("--assign-variant", default="best", choices=["base", "lds_fma", "mfma", "mfma_bf16x3", "best"])
@@ -234,8 +246,7 @@ def main():
         scratch.free()
 
     # 1. warm-up
-    alg.run(iters=args.warmup, use_graph=args.graph)
-    alg.reset(means0)
+    warm_up(alg, args, spec, means0, use_graph=args.graph)
 
     # 2. timed region
     km.sync()

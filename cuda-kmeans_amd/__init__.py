@@ -513,6 +513,13 @@ class HipFusedKMeansAlgorithm:
         self.cu_sizes.zero()
         sync()
 
+    def reset(self, means):
+        """Back to the state right after initialize() (initial centroids)."""
+        self.last = 0
+        self.cu_means[0].write(means)
+        self.cu_sizes.zero()
+        sync()
+
     def iteration(self):
         nxt = (self.last + 1) % 2
         self.cu_means[nxt].zero()
