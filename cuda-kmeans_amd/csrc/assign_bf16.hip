@@ -23,6 +23,13 @@
  * The refinement (winning row inside the winning tile) re-evaluates rows with v_dot2c_f32_bf16 on the same
  * three products, so the same bound covers it.
  *
+ * Rows of at most 4 dimensions (PACKED): a block of 16 MFMA slots holds ALL FOUR hi/mid products of every dimension
+ * (4 d <= 16), so a tile costs one MFMA instead of three and nothing of (hi + mid)(hi + mid) is dropped:
+ *   - operands cut to hi + mid:   |c'_i x_i - (four products)| <= (2^-18 + 2^-18 + 2^-36) |c'_i||x_i|  -> 2.0001 * 2^-18 S  (= 64.01 u' S)
+ *   - accumulation of 4d products and |c|^2 in fp32                                              -> (4d + 2) u' * 2 S
+ *   - serial margin as above                                                                          -> (2d + 12) u' S
+ * tau > (128.02 + 16d + 8 + 2d + 12) u' S:   tau = (18 d + 149) 2^-23 (|x|^2 + max_j |c_j|^2).
+ *
  * Data flow, tiling, tracking, flag buffering and the recheck hand-over are those of the fp32 kernel
  * (assign_mfma.hip); the packed centroid row holds hi and mid parts of -2c, 4 bytes per dimension as before.
  */
@@ -47,7 +54,8 @@ static uint32_t pick_kb(uint32_t dim)
 template <int LM>
 __global__ void __launch_bounds__(256)
 pack_means_bf16_kernel(const float* __restrict__ means, size_t stride_means, float* __restrict__ packed, float* __restrict__ norms,
-                       float* __restrict__ means_t, uint32_t dim, uint32_t k, uint32_t kp, uint32_t dp, uint32_t* __restrict__ counters)
+                       float* __restrict__ means_t, uint32_t dim, uint32_t k, uint32_t kp, uint32_t dp, uint32_t packed_slots,
+                       uint32_t* __restrict__ counters)
 {
 	const uint32_t lane = threadIdx.x & (WAVE - 1);
 	const uint32_t j = (blockIdx.x * blockDim.x + threadIdx.x) / WAVE;
@@ -57,6 +65,25 @@ pack_means_bf16_kernel(const float* __restrict__ means, size_t stride_means, flo
 	float* row = packed + packed_row(j, rs);
 	__bf16* parts = (__bf16*)row;
 	float c2 = 0.0f;
+	if (packed_slots) {
+		/* rows of at most 4 dimensions: slots 0..3 = hi, 4..7 = mid, 8..11 = hi, 12..15 = mid of -2c, the slots of a
+		 * half-wave in the row's "hi" unit (units 0 and 2); the "mid" units stay zero (load_packed_points has the
+		 * matching order of the point's parts) */
+		if (lane < KBLOCK) {
+			const uint32_t q = lane % 4;
+			const float v = (j < k && q < dim) ? means[elem<LM>(stride_means, j, q)] : 0.0f;
+			__bf16 hi, mid;
+			split_bf16(-2.0f * v, hi, mid);
+			const uint32_t unit = 2 * (lane / 8);
+			parts[8 * unit + lane % 8] = (lane / 4) % 2 == 1 ? mid : hi;
+			parts[8 * (unit + 1) + lane % 8] = (__bf16)0.0f;
+			if (lane < 4) {
+				c2 = v * v;
+				if (q < dim) means_t[(size_t)q * kp + j] = v; /* exact copy for the recheck pass */
+			}
+		}
+	}
+	else
 	for (uint32_t q = lane; q < dp; q += WAVE) {
 		const float v = (j < k && q < dim) ? means[elem<LM>(stride_means, j, q)] : 0.0f;
 		c2 += v * v;
@@ -122,14 +149,15 @@ int launch_assign_bf16(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws
 	const uint32_t pack_blocks = (kp * WAVE + 255) / 256;
 	if (a.layout_means == KMX_AOS)
 		hipLaunchKernelGGL((pack_means_bf16_kernel<KMX_AOS>), dim3(pack_blocks), dim3(256), 0, stream(),
-		                   a.means, a.stride_means, ws->packed_means, ws->norms, ws->means_t, a.dim, a.k, kp, dp, ws->counters);
+		                   a.means, a.stride_means, ws->packed_means, ws->norms, ws->means_t, a.dim, a.k, kp, dp, packed_rows(a.dim) ? 1u : 0u, ws->counters);
 	else
 		hipLaunchKernelGGL((pack_means_bf16_kernel<KMX_SOA>), dim3(pack_blocks), dim3(256), 0, stream(),
-		                   a.means, a.stride_means, ws->packed_means, ws->norms, ws->means_t, a.dim, a.k, kp, dp, ws->counters);
+		                   a.means, a.stride_means, ws->packed_means, ws->norms, ws->means_t, a.dim, a.k, kp, dp, packed_rows(a.dim) ? 1u : 0u, ws->counters);
 	KMX_LAUNCH_CHECK("pack_means_bf16_kernel");
 
-	/* tau = kd (|x|^2 + max|c|^2), kd = (14 d + 224) 2^-23 (see the bound at the top of the file) */
-	const float kd = (14.0f * (float)a.dim + 224.0f) * 1.1920929e-07f + a.kd_extra;
+	/* tau = kd (|x|^2 + max|c|^2), kd = (14 d + 224) 2^-23, or (18 d + 149) 2^-23 for the packed rows, which keep all
+	 * four products (see the bounds at the top of the file) */
+	const float kd = (packed_rows(a.dim) ? 18.0f * (float)a.dim + 149.0f : 14.0f * (float)a.dim + 224.0f) * 1.1920929e-07f + a.kd_extra;
 	switch (kb) {
 	case 1: rc = launch_bf16_1(a, exec, ws, dev, kp, kd); break;
 	case 2: rc = launch_bf16_2(a, exec, ws, dev, kp, kd); break;

@@ -33,6 +33,47 @@ template <int KB> struct SplitPoints {
 };
 
 /* points of one sweep unit -> split B operands; xx = this lane's share of |x|^2; rows beyond n read as zero */
+/*
+ * Rows of at most 4 dimensions, PACKED form: the four hi/mid products of all dimensions share ONE block of 16 MFMA slots,
+ *      slot      0..3       4..7       8..11     12..15
+ *      centroid  c'hi       c'mid      c'hi      c'mid
+ *      point     x_mid      x_hi       x_hi      x_mid
+ * so a tile costs one MFMA instead of three and the mid * mid product is kept (bound at the top of assign_bf16.hip).
+ * The lane holds the 8 slots of its half-wave in b.hi[0]; b.mid stays unused.
+ */
+template <int P, int LD, bool VEC>
+__device__ __forceinline__ void load_packed_points(SplitPoints<1> (&b)[P], float (&xx)[P], const float* __restrict__ data, size_t stride,
+                                                   uint32_t base, uint32_t col, uint32_t h, uint32_t dim, uint32_t n)
+{
+#pragma unroll
+	for (int p = 0; p < P; ++p) {
+		const uint32_t pt = base + p * TILE + col;
+		const bool valid = pt < n;
+		float v[4];
+		if (LD == KMX_AOS && VEC) { /* dim == 4, aligned rows */
+			f32x4 t = { 0.0f, 0.0f, 0.0f, 0.0f };
+			if (valid) t = *(const f32x4*)(data + (size_t)pt * stride);
+			v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+		}
+		else {
+#pragma unroll
+			for (int j = 0; j < 4; ++j) v[j] = (valid && (uint32_t)j < dim) ? data[elem<LD>(stride, pt, j)] : 0.0f;
+		}
+		float part = 0.0f;
+#pragma unroll
+		for (int j = 0; j < 4; ++j) {
+			part += v[j] * v[j];
+			__bf16 hi, mid;
+			split_bf16(v[j], hi, mid);
+			b[p].hi[0][j] = h == 0 ? mid : hi;      /* slots 0..3: x_mid,  slots 8..11: x_hi   */
+			b[p].hi[0][4 + j] = h == 0 ? hi : mid;  /* slots 4..7: x_hi,   slots 12..15: x_mid */
+			b[p].mid[0][j] = (__bf16)0.0f;
+			b[p].mid[0][4 + j] = (__bf16)0.0f;
+		}
+		xx[p] = h == 0 ? part : 0.0f; /* the two half-waves hold the same point: |x|^2 once */
+	}
+}
+
 template <int KB, int P, int LD, bool VEC>
 __device__ __forceinline__ void load_split_points(SplitPoints<KB> (&b)[P], float (&xx)[P], const float* __restrict__ data, size_t stride,
                                                   uint32_t base, uint32_t col, uint32_t h, uint32_t dim, uint32_t n)
@@ -94,7 +135,7 @@ __device__ __forceinline__ bf16x8 row_unit(const float* row, uint32_t unit) { re
 /* rows of at least 32 dimensions: the refinement is worth halving (see track_tile) */
 template <int KB> constexpr bool fine8_bf16() { return KB >= 2; }
 
-template <int KB, int P, bool TRACK, bool COARSE>
+template <int KB, int P, bool TRACK, bool COARSE, bool PACKED = false>
 __device__ __forceinline__ void tile_step_bf16(const float* __restrict__ lds, const float* __restrict__ lds_norms, uint32_t tile_new,
                                                uint32_t col, uint32_t h, const SplitPoints<KB> (&b)[P],
                                                f32x16 (&acc_new)[P], const f32x16 (&acc_old)[P], uint32_t tile_old,
@@ -114,6 +155,18 @@ __device__ __forceinline__ void tile_step_bf16(const float* __restrict__ lds, co
 	for (int g = 0; g < 4; ++g) {
 		f32x4 v = *(const f32x4*)(lds_norms + tile_new * NORM_TILE + 8 * g + 4 * h);
 		cinit[4 * g] = v.x; cinit[4 * g + 1] = v.y; cinit[4 * g + 2] = v.z; cinit[4 * g + 3] = v.w;
+	}
+	if constexpr (PACKED) {
+		/* one MFMA per tile: the row's unit 2 h holds the half-wave's 8 slots, b.hi[0] the point's */
+#pragma unroll
+		for (int p = 0; p < P; ++p) acc_new[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(chi[0], b[p].hi[0], cinit, 0, 0, 0);
+		if (TRACK) {
+#pragma unroll
+			for (int p = 0; p < P; ++p) track_tile<COARSE, false>(acc_old[p], st[p], tile_old, neg_inf);
+			__builtin_amdgcn_sched_group_barrier(0x008, P, 0);
+			__builtin_amdgcn_sched_group_barrier(0x002, (COARSE ? 12 : 67) * P, 0);
+		}
+		return;
 	}
 #pragma unroll
 	for (int p = 0; p < P; ++p) acc_new[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(chi[0], b[p].mid[0], cinit, 0, 0, 0);
@@ -146,10 +199,17 @@ __device__ __forceinline__ void tile_step_bf16(const float* __restrict__ lds, co
 	__builtin_amdgcn_fdot2_f32_bf16(__builtin_shufflevector(a, a, 2 * (i), 2 * (i) + 1), __builtin_shufflevector(b, b, 2 * (i), 2 * (i) + 1), acc, false)
 
 /* this half-wave's share of the three-product dot of one packed row with one point (the same terms the MFMAs add) */
-template <int KB>
+template <int KB, bool PACKED = false>
 __device__ __forceinline__ float row_dot_bf16(const float* row, uint32_t h, const SplitPoints<KB>& x)
 {
 	float part = 0.0f;
+	if constexpr (PACKED) { /* the half-wave's 8 slots of the packed row against the point's */
+		const bf16x8 ch = row_unit(row, 2 * h);
+		const bf16x8 xh = x.hi[0];
+		part = KMX_DOT2_PAIR(part, ch, xh, 0); part = KMX_DOT2_PAIR(part, ch, xh, 1);
+		part = KMX_DOT2_PAIR(part, ch, xh, 2); part = KMX_DOT2_PAIR(part, ch, xh, 3);
+		return part;
+	}
 #pragma unroll
 	for (int kb = 0; kb < KB; ++kb) {
 		const bf16x8 ch = row_unit(row, 4 * kb + 2 * h);
@@ -164,7 +224,7 @@ __device__ __forceinline__ float row_dot_bf16(const float* row, uint32_t h, cons
 	return part;
 }
 
-template <int KB, int P, int LD, bool VEC, bool STREAM, bool COARSE, bool PREFETCH>
+template <int KB, int P, int LD, bool VEC, bool STREAM, bool COARSE, bool PREFETCH, bool PACKED = false>
 __global__ void __launch_bounds__(MFMA_WAVES * WAVE)
 assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* __restrict__ packed, const float* __restrict__ norms,
                    uint32_t* __restrict__ assignment, uint32_t* __restrict__ queue, uint32_t* __restrict__ counters,
@@ -373,15 +433,15 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 			const float* lds_norms = lds_tiles + (size_t)chunk_tiles * tile_floats(RS);
 			const uint32_t tiles = rows / TILE;
 			const uint32_t tile0 = row0 / TILE;
-			tile_step_bf16<KB, P, false, COARSE>(lds_tiles, lds_norms, 0, col, h, b, acc0, acc1, 0, st, neg_inf);
+			tile_step_bf16<KB, P, false, COARSE, PACKED>(lds_tiles, lds_norms, 0, col, h, b, acc0, acc1, 0, st, neg_inf);
 			uint32_t t = 0; /* acc0 holds tile t, not yet tracked */
 			while (t + 2 < tiles) {
-				tile_step_bf16<KB, P, true, COARSE>(lds_tiles, lds_norms, t + 1, col, h, b, acc1, acc0, tile0 + t, st, neg_inf);
-				tile_step_bf16<KB, P, true, COARSE>(lds_tiles, lds_norms, t + 2, col, h, b, acc0, acc1, tile0 + t + 1, st, neg_inf);
+				tile_step_bf16<KB, P, true, COARSE, PACKED>(lds_tiles, lds_norms, t + 1, col, h, b, acc1, acc0, tile0 + t, st, neg_inf);
+				tile_step_bf16<KB, P, true, COARSE, PACKED>(lds_tiles, lds_norms, t + 2, col, h, b, acc0, acc1, tile0 + t + 1, st, neg_inf);
 				t += 2;
 			}
 			if (t + 1 < tiles) {
-				tile_step_bf16<KB, P, true, COARSE>(lds_tiles, lds_norms, t + 1, col, h, b, acc1, acc0, tile0 + t, st, neg_inf);
+				tile_step_bf16<KB, P, true, COARSE, PACKED>(lds_tiles, lds_norms, t + 1, col, h, b, acc1, acc0, tile0 + t, st, neg_inf);
 #pragma unroll
 				for (int p = 0; p < P; ++p) track_tile<COARSE, fine8_bf16<KB>()>(acc1[p], st[p], tile0 + t + 1, neg_inf);
 			}
@@ -420,7 +480,7 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 				float tot[ROWS];
 #pragma unroll
 				for (int r = 0; r < ROWS; ++r)
-					tot[r] = row_dot_bf16<KB>(tile_base + (size_t)(8 * (sub + r / 4) + 4 * wh + (r % 4)) * RS, h, b[p]);
+					tot[r] = row_dot_bf16<KB, PACKED>(tile_base + (size_t)(8 * (sub + r / 4) + 4 * wh + (r % 4)) * RS, h, b[p]);
 				float v1 = __builtin_inff(), v2 = __builtin_inff();
 				uint32_t rbest = 0;
 #pragma unroll
@@ -467,19 +527,25 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 		}
 	};
 
+	static_assert(!PACKED || KB == 1, "the packed form is one block of 16 slots");
+	auto load_points = [&](SplitPoints<KB> (&bb)[P], float (&xs)[P], uint32_t first) {
+		if constexpr (PACKED) load_packed_points<P, LD, VEC>(bb, xs, data, stride, first, col, h, dim, n);
+		else load_split_points<KB, P, LD, VEC>(bb, xs, data, stride, first, col, h, dim, n);
+	};
+
 	if (PREFETCH) {
 		SplitPoints<KB> b0[P], b1[P];
 		float xx0[P], xx1[P];
 		uint32_t unit = blockIdx.x;
-		if (unit < units) load_split_points<KB, P, LD, VEC>(b0, xx0, data, stride, (unit * MFMA_WAVES + wave) * P * TILE, col, h, dim, n);
+		if (unit < units) load_points(b0, xx0, (unit * MFMA_WAVES + wave) * P * TILE);
 		while (unit < units) {
 			uint32_t next = unit + gridDim.x;
-			if (next < units) load_split_points<KB, P, LD, VEC>(b1, xx1, data, stride, (next * MFMA_WAVES + wave) * P * TILE, col, h, dim, n);
+			if (next < units) load_points(b1, xx1, (next * MFMA_WAVES + wave) * P * TILE);
 			sweep(b0, xx0, (unit * MFMA_WAVES + wave) * P * TILE);
 			unit = next;
 			if (unit >= units) break;
 			next = unit + gridDim.x;
-			if (next < units) load_split_points<KB, P, LD, VEC>(b0, xx0, data, stride, (next * MFMA_WAVES + wave) * P * TILE, col, h, dim, n);
+			if (next < units) load_points(b0, xx0, (next * MFMA_WAVES + wave) * P * TILE);
 			sweep(b1, xx1, (unit * MFMA_WAVES + wave) * P * TILE);
 			unit = next;
 		}
@@ -488,7 +554,7 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 		SplitPoints<KB> b0[P];
 		float xx0[P];
 		for (uint32_t unit = blockIdx.x; unit < units; unit += gridDim.x) {
-			load_split_points<KB, P, LD, VEC>(b0, xx0, data, stride, (unit * MFMA_WAVES + wave) * P * TILE, col, h, dim, n);
+			load_points(b0, xx0, (unit * MFMA_WAVES + wave) * P * TILE);
 			sweep(b0, xx0, (unit * MFMA_WAVES + wave) * P * TILE);
 		}
 	}
@@ -698,11 +764,14 @@ template <int KB> struct SplitSweepShape {
 	static constexpr bool PREFETCH = KB <= 2;
 };
 
-template <int KB, int LD, bool VEC>
+/* rows of at most 4 dimensions: the four products of all dimensions in one block of MFMA slots (load_packed_points) */
+inline bool packed_rows(uint32_t dim) { return dim <= 4; }
+
+template <int KB, int LD, bool VEC, bool PACKED = false>
 static int launch_bf16_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev, uint32_t kp, float kd)
 {
 	constexpr uint32_t RS = KBLOCK * KB + ROW_PAD;
-	constexpr int P = SplitSweepShape<KB>::P;
+	constexpr int P = PACKED ? 4 : SplitSweepShape<KB>::P; /* one MFMA per tile: four point tiles share the centroid operand and the norms */
 	constexpr bool PF = SplitSweepShape<KB>::PREFETCH;
 	uint32_t budget = exec->shared_mem_bytes ? std::min(exec->shared_mem_bytes, dev.lds_bytes) : dev.lds_bytes;
 	const uint32_t static_bytes = (2 * FLAG_CAP * MFMA_WAVES + 64) * 4;
@@ -727,8 +796,8 @@ static int launch_bf16_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 	void (*kernel)(const float*, size_t, const float*, const float*, uint32_t*, uint32_t*, uint32_t*,
 	               uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, float, float) = nullptr;
 	if constexpr (KB <= 4) {
-		if (stream_mode) kernel = coarse ? assign_bf16_kernel<KB, P, LD, VEC, true, true, PF> : assign_bf16_kernel<KB, P, LD, VEC, true, false, PF>;
-		else kernel = coarse ? assign_bf16_kernel<KB, P, LD, VEC, false, true, PF> : assign_bf16_kernel<KB, P, LD, VEC, false, false, PF>;
+		if (stream_mode) kernel = coarse ? assign_bf16_kernel<KB, P, LD, VEC, true, true, PF, PACKED> : assign_bf16_kernel<KB, P, LD, VEC, true, false, PF, PACKED>;
+		else kernel = coarse ? assign_bf16_kernel<KB, P, LD, VEC, false, true, PF, PACKED> : assign_bf16_kernel<KB, P, LD, VEC, false, false, PF, PACKED>;
 	}
 	else {
 		kernel = assign_bf16_kernel<KB, P, LD, VEC, true, false, PF>;
@@ -751,8 +820,15 @@ static int launch_bf16_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 template <int KB>
 static int launch_bf16_kb(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev, uint32_t kp, float kd)
 {
-	if (a.layout == KMX_SOA) return launch_bf16_t<KB, KMX_SOA, false>(a, exec, ws, dev, kp, kd);
 	const bool aligned = a.dim % 4 == 0 && a.stride % 4 == 0 && ((uintptr_t)a.data % 16) == 0;
+	if constexpr (KB == 1) {
+		if (packed_rows(a.dim)) {
+			if (a.layout == KMX_SOA) return launch_bf16_t<KB, KMX_SOA, false, true>(a, exec, ws, dev, kp, kd);
+			if (aligned) return launch_bf16_t<KB, KMX_AOS, true, true>(a, exec, ws, dev, kp, kd);
+			return launch_bf16_t<KB, KMX_AOS, false, true>(a, exec, ws, dev, kp, kd);
+		}
+	}
+	if (a.layout == KMX_SOA) return launch_bf16_t<KB, KMX_SOA, false>(a, exec, ws, dev, kp, kd);
 	if (aligned) return launch_bf16_t<KB, KMX_AOS, true>(a, exec, ws, dev, kp, kd);
 	return launch_bf16_t<KB, KMX_AOS, false>(a, exec, ws, dev, kp, kd);
 }

@@ -164,10 +164,15 @@ int dispatch_assign(int variant, const AssignArgs& a, kmx_exec_params* exec, Wor
 		/* counterpart of BestCachedAssignmentKernel::run (reference kernels.cu:706-717): pick by shape.
 		 * Measured: the split-bf16 sweep is about twice as fast as the fp32 one wherever the sweep dominates; it hands
 		 * 2-3 times as many points to the exact pass, which costs more than it saves for very short rows and for
-		 * few centroids (HBM-bound shapes). The fp32 MFMA sweep beat the plain-VALU variant at every shape except
+		 * few centroids (HBM-bound shapes). Rows of 2 to 4 dimensions are the exception among the short ones: all their
+		 * products fit one MFMA per tile (the packed form), which beats the fp32 sweep from 128 centroids on (512 for
+		 * two dimensions; 1.14 against 1.53 ms per iteration at N = 4M, d = 4, k = 4096, exact pass included).
+		 * The fp32 MFMA sweep beat the plain-VALU variant at every shape except
 		 * a handful of centroids, where that variant reads them through the scalar cache. */
+		const bool packed_wins = !a.ranking_only /* the double path pays more per queued point: 2.35 against 1.91 ms there */ &&
+		                         ((a.dim >= 3 && a.dim <= 4 && a.k >= 128) || (a.dim == 2 && a.k >= 512));
 		if (a.k <= 32 && lds_fma_supports(a, dev) && lds_fma_reads_through_scalar_cache(a)) variant = KMX_ASSIGN_LDS_FMA;
-		else if (bf16_supports(a, dev) && a.dim >= 8 && a.k >= 64) variant = KMX_ASSIGN_MFMA_BF16X3;
+		else if (bf16_supports(a, dev) && ((a.dim >= 8 && a.k >= 64) || packed_wins)) variant = KMX_ASSIGN_MFMA_BF16X3;
 		else if (mfma_supports(a, dev)) variant = KMX_ASSIGN_MFMA;
 		else if (lds_fma_supports(a, dev)) variant = KMX_ASSIGN_LDS_FMA;
 		else variant = KMX_ASSIGN_BASE;
