@@ -61,22 +61,22 @@ pack_means_bf16_kernel(const float* __restrict__ means, size_t stride_means, flo
 	const uint32_t j = (blockIdx.x * blockDim.x + threadIdx.x) / WAVE;
 	if (blockIdx.x == 0 && threadIdx.x == 0) counters[0] = 0u; /* the recheck queue of this call starts empty */
 	if (j >= kp) return;
-	const uint32_t rs = dp + ROW_PAD;
+	const uint32_t rs = packed_slots ? row_floats<1, true>() : dp + ROW_PAD;
 	float* row = packed + packed_row(j, rs);
 	__bf16* parts = (__bf16*)row;
 	float c2 = 0.0f;
 	if (packed_slots) {
-		/* rows of at most 4 dimensions: slots 0..3 = hi, 4..7 = mid, 8..11 = hi, 12..15 = mid of -2c, the slots of a
-		 * half-wave in the row's "hi" unit (units 0 and 2); the "mid" units stay zero (load_packed_points has the
-		 * matching order of the point's parts) */
+		/* rows of at most 4 dimensions: slots 0..3 = hi, 4..7 = mid, 8..11 = hi, 12..15 = mid of -2c; inside the tile
+		 * the first halves of all rows, then the second halves (packed_half; load_packed_points has the matching order
+		 * of the point's parts) */
 		if (lane < KBLOCK) {
 			const uint32_t q = lane % 4;
 			const float v = (j < k && q < dim) ? means[elem<LM>(stride_means, j, q)] : 0.0f;
 			__bf16 hi, mid;
 			split_bf16(-2.0f * v, hi, mid);
-			const uint32_t unit = 2 * (lane / 8);
-			parts[8 * unit + lane % 8] = (lane / 4) % 2 == 1 ? mid : hi;
-			parts[8 * (unit + 1) + lane % 8] = (__bf16)0.0f;
+			float* tile = packed + (size_t)(j / TILE) * tile_floats(rs);
+			((__bf16*)(tile + packed_half(j % TILE, lane / 8)))[lane % 8] = (lane / 4) % 2 == 1 ? mid : hi;
+			if (j % TILE == TILE - 1 && lane < TILE_PAD) tile[TILE * rs + lane] = 0.0f;
 			if (lane < 4) {
 				c2 = v * v;
 				if (q < dim) means_t[(size_t)q * kp + j] = v; /* exact copy for the recheck pass */
@@ -96,7 +96,7 @@ pack_means_bf16_kernel(const float* __restrict__ means, size_t stride_means, flo
 		if (q < dim) means_t[(size_t)q * kp + j] = v; /* exact copy for the recheck pass */
 	}
 	const uint32_t pad_floats = ROW_PAD + (j % TILE == TILE - 1 ? TILE_PAD : 0);
-	if (lane < pad_floats) row[dp + lane] = 0.0f;
+	if (!packed_slots && lane < pad_floats) row[dp + lane] = 0.0f;
 	for (int off = WAVE / 2; off > 0; off >>= 1) c2 += __shfl_xor(c2, off);
 	if (lane == 0) norms[norm_at(j)] = j < k ? c2 : __builtin_inff();
 	if (lane < NORM_TILE - TILE && j % TILE == 0) norms[(j / TILE) * NORM_TILE + TILE + lane] = __builtin_inff();
@@ -142,7 +142,8 @@ int launch_assign_bf16(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws
 	const uint32_t kb = pick_kb(a.dim);
 	const uint32_t dp = KBLOCK * kb;
 	const uint32_t kp = round_up(a.k, TILE);
-	int rc = reserve_packed(ws, (size_t)(kp / TILE) * tile_floats(dp + ROW_PAD), (size_t)(kp / TILE) * NORM_TILE, (size_t)kp * a.dim);
+	const uint32_t rs = packed_rows(a.dim) ? row_floats<1, true>() : dp + ROW_PAD;
+	int rc = reserve_packed(ws, (size_t)(kp / TILE) * tile_floats(rs), (size_t)(kp / TILE) * NORM_TILE, (size_t)kp * a.dim);
 	if (rc) return rc;
 	rc = reserve_queue(ws, 2 * (size_t)a.n); /* (point, threshold) pairs */
 	if (rc) return rc;

@@ -19,6 +19,13 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 constexpr uint32_t KBLOCK = 16; /* dimensions per v_mfma_f32_32x32x16_bf16 */
 constexpr int STAGE_VECS = 9;   /* 16-byte pieces of a streamed chunk per lane: a chunk holds at most 9 * 512 * 16 bytes of tiles */
 
+/* Floats per packed centroid row. The PACKED form (rows of at most 4 dimensions) has 16 slots = 8 floats per row and no
+ * padding: inside a tile the slots 0..7 of the 32 rows come first, then their slots 8..15, so that the lanes of a
+ * half-wave read consecutive 16-byte pieces (no bank conflicts without padding, and 4096 centroids fit the LDS). */
+template <int KB, bool PACKED> constexpr uint32_t row_floats() { return PACKED ? 8 : KBLOCK * KB + ROW_PAD; }
+/* PACKED: where the 8 slots of half-wave h of row r (0..31) of a tile begin */
+__host__ __device__ constexpr uint32_t packed_half(uint32_t r, uint32_t h) { return h * (TILE * 4) + r * 4; }
+
 /* value = hi + mid + (at most 2^-18 |value|), both parts bf16 (round to nearest even) */
 __device__ __forceinline__ void split_bf16(float v, __bf16& hi, __bf16& mid)
 {
@@ -141,13 +148,13 @@ __device__ __forceinline__ void tile_step_bf16(const float* __restrict__ lds, co
                                                f32x16 (&acc_new)[P], const f32x16 (&acc_old)[P], uint32_t tile_old,
                                                Track (&st)[P], float neg_inf)
 {
-	constexpr uint32_t RS = KBLOCK * KB + ROW_PAD;
-	const float* arow = lds + (size_t)tile_new * tile_floats(RS) + (size_t)col * RS;
+	constexpr uint32_t RS = row_floats<KB, PACKED>();
+	const float* arow = lds + (size_t)tile_new * tile_floats(RS) + (PACKED ? packed_half(col, h) : col * RS);
 	bf16x8 chi[KB], cmid[KB];
 #pragma unroll
 	for (int kb = 0; kb < KB; ++kb) {
-		chi[kb] = row_unit(arow, 4 * kb + 2 * h);
-		cmid[kb] = row_unit(arow, 4 * kb + 2 * h + 1);
+		chi[kb] = PACKED ? *(const bf16x8*)arow : row_unit(arow, 4 * kb + 2 * h);
+		if (!PACKED) cmid[kb] = row_unit(arow, 4 * kb + 2 * h + 1);
 	}
 	/* C operand: |c|^2 of the 16 rows this lane receives: rows 8g + 4h + (0..3), g = 0..3 */
 	f32x16 cinit;
@@ -157,7 +164,7 @@ __device__ __forceinline__ void tile_step_bf16(const float* __restrict__ lds, co
 		cinit[4 * g] = v.x; cinit[4 * g + 1] = v.y; cinit[4 * g + 2] = v.z; cinit[4 * g + 3] = v.w;
 	}
 	if constexpr (PACKED) {
-		/* one MFMA per tile: the row's unit 2 h holds the half-wave's 8 slots, b.hi[0] the point's */
+		/* one MFMA per tile: chi[0] holds the half-wave's 8 slots of the row, b.hi[0] the point's */
 #pragma unroll
 		for (int p = 0; p < P; ++p) acc_new[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(chi[0], b[p].hi[0], cinit, 0, 0, 0);
 		if (TRACK) {
@@ -203,8 +210,8 @@ template <int KB, bool PACKED = false>
 __device__ __forceinline__ float row_dot_bf16(const float* row, uint32_t h, const SplitPoints<KB>& x)
 {
 	float part = 0.0f;
-	if constexpr (PACKED) { /* the half-wave's 8 slots of the packed row against the point's */
-		const bf16x8 ch = row_unit(row, 2 * h);
+	if constexpr (PACKED) { /* the half-wave's 8 slots of the packed row (row points at them) against the point's */
+		const bf16x8 ch = *(const bf16x8*)row;
 		const bf16x8 xh = x.hi[0];
 		part = KMX_DOT2_PAIR(part, ch, xh, 0); part = KMX_DOT2_PAIR(part, ch, xh, 1);
 		part = KMX_DOT2_PAIR(part, ch, xh, 2); part = KMX_DOT2_PAIR(part, ch, xh, 3);
@@ -230,7 +237,7 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
                    uint32_t* __restrict__ assignment, uint32_t* __restrict__ queue, uint32_t* __restrict__ counters,
                    uint32_t dim, uint32_t k, uint32_t kp, uint32_t n, uint32_t chunk_rows, float kd, float neg_inf)
 {
-	constexpr uint32_t RS = KBLOCK * KB + ROW_PAD;
+	constexpr uint32_t RS = row_floats<KB, PACKED>();
 	extern __shared__ float lds[];
 	__shared__ uint32_t wave_max[MFMA_WAVES];
 	__shared__ uint32_t flag_list[MFMA_WAVES][2 * FLAG_CAP]; /* (point, threshold) pairs */
@@ -480,7 +487,10 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 				float tot[ROWS];
 #pragma unroll
 				for (int r = 0; r < ROWS; ++r)
-					tot[r] = row_dot_bf16<KB, PACKED>(tile_base + (size_t)(8 * (sub + r / 4) + 4 * wh + (r % 4)) * RS, h, b[p]);
+				{
+					const uint32_t row = 8 * (sub + r / 4) + 4 * wh + (r % 4);
+					tot[r] = row_dot_bf16<KB, PACKED>(tile_base + (PACKED ? packed_half(row, h) : row * RS), h, b[p]);
+				}
 				float v1 = __builtin_inff(), v2 = __builtin_inff();
 				uint32_t rbest = 0;
 #pragma unroll
@@ -770,7 +780,7 @@ inline bool packed_rows(uint32_t dim) { return dim <= 4; }
 template <int KB, int LD, bool VEC, bool PACKED = false>
 static int launch_bf16_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev, uint32_t kp, float kd)
 {
-	constexpr uint32_t RS = KBLOCK * KB + ROW_PAD;
+	constexpr uint32_t RS = row_floats<KB, PACKED>();
 	constexpr int P = PACKED ? 4 : SplitSweepShape<KB>::P; /* one MFMA per tile: four point tiles share the centroid operand and the norms */
 	constexpr bool PF = SplitSweepShape<KB>::PREFETCH;
 	uint32_t budget = exec->shared_mem_bytes ? std::min(exec->shared_mem_bytes, dev.lds_bytes) : dev.lds_bytes;
