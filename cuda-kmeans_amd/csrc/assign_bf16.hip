@@ -171,8 +171,9 @@ int launch_assign_bf16(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws
 	if (rc) return rc;
 	if (a.ranking_only) return KMX_OK; /* the caller resolves the queued points */
 	/* wide rows and many centroids: a second sweep screens the queued points (narrow rows fit the registers of the
-	 * lane-per-centroid kernels, which then need fewer launches) */
-	return a.k >= 128 && a.dim > 32 ? launch_recheck_screened(a, ws, kp, dev) : launch_recheck(a, ws, kp);
+	 * lane-per-centroid kernels, which then need fewer launches); so do the packed rows, whose sweep queues four times
+	 * as many points as the fp32 one and screens a tile with a single MFMA */
+	return a.k >= 128 && (a.dim > 32 || packed_rows(a.dim)) ? launch_recheck_screened(a, ws, kp, dev) : launch_recheck(a, ws, kp);
 }
 
 } // namespace kmx

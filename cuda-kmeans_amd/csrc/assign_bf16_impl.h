@@ -26,6 +26,9 @@ template <int KB, bool PACKED> constexpr uint32_t row_floats() { return PACKED ?
 /* PACKED: where the 8 slots of half-wave h of row r (0..31) of a tile begin */
 __host__ __device__ constexpr uint32_t packed_half(uint32_t r, uint32_t h) { return h * (TILE * 4) + r * 4; }
 
+/* rows of at most 4 dimensions: the four products of all dimensions in one block of MFMA slots (load_packed_points) */
+inline bool packed_rows(uint32_t dim) { return dim <= 4; }
+
 /* value = hi + mid + (at most 2^-18 |value|), both parts bf16 (round to nearest even) */
 __device__ __forceinline__ void split_bf16(float v, __bf16& hi, __bf16& mid)
 {
@@ -591,14 +594,15 @@ static __device__ __attribute__((noinline)) void evaluate_pair_of_row(const floa
 	evaluate_pair<KMX_AOS>(rows, dim, means_t, dim, kp, row, j, &keys[row]);
 }
 
-template <int KB, int P>
+template <int KB, int P, bool PACKED = false>
 __global__ void __launch_bounds__(SCREEN_WAVES * WAVE)
 screen_bf16_kernel(const float* __restrict__ rows, const float* __restrict__ packed, const float* __restrict__ norms,
                    const float* __restrict__ means_t, const uint32_t* __restrict__ row_queue, const uint32_t* __restrict__ row_count,
                    uint32_t* __restrict__ pairs, uint32_t* __restrict__ item_pairs,
                    unsigned long long* __restrict__ keys, uint32_t dim, uint32_t k, uint32_t kp)
 {
-	constexpr uint32_t RS = KBLOCK * KB + ROW_PAD;
+	static_assert(!PACKED || KB == 1, "the packed form is one block of 16 slots");
+	constexpr uint32_t RS = row_floats<KB, PACKED>();
 	constexpr int G = KB < 4 ? KB : 4; /* blocks of 16 dimensions whose centroid operands travel together */
 	constexpr int GROUPS = KB / G;     /* 1, 2 or 4 */
 	static_assert(KB % G == 0 && (GROUPS == 1 || GROUPS % 2 == 0), "operand groups");
@@ -641,7 +645,8 @@ screen_bf16_kernel(const float* __restrict__ rows, const float* __restrict__ pac
 		written = 0;
 		SplitPoints<KB> b[P];
 		float xx[P];
-		load_split_points<KB, P, KMX_AOS, false>(b, xx, rows, dim, base, col, h, dim, count);
+		if constexpr (PACKED) load_packed_points<P, KMX_AOS, false>(b, xx, rows, dim, base, col, h, dim, count);
+		else load_split_points<KB, P, KMX_AOS, false>(b, xx, rows, dim, base, col, h, dim, count);
 		float thr[P];
 		bool valid[P];
 #pragma unroll
@@ -652,11 +657,11 @@ screen_bf16_kernel(const float* __restrict__ rows, const float* __restrict__ pac
 		}
 
 		auto fetch = [&](Operands& o, uint32_t tile, int group) {
-			const float* arow = packed + (size_t)tile * tile_floats(RS) + (size_t)col * RS;
+			const float* arow = packed + (size_t)tile * tile_floats(RS) + (PACKED ? packed_half(col, h) : col * RS);
 #pragma unroll
 			for (int i = 0; i < G; ++i) {
-				o.hi[i] = row_unit(arow, 4 * (group * G + i) + 2 * h);
-				o.mid[i] = row_unit(arow, 4 * (group * G + i) + 2 * h + 1);
+				o.hi[i] = PACKED ? *(const bf16x8*)arow : row_unit(arow, 4 * (group * G + i) + 2 * h);
+				if (!PACKED) o.mid[i] = row_unit(arow, 4 * (group * G + i) + 2 * h + 1);
 			}
 		};
 		auto fetch_norms = [&](f32x16& c, uint32_t tile) { /* |c|^2 of the 16 rows this lane receives */
@@ -700,6 +705,11 @@ screen_bf16_kernel(const float* __restrict__ rows, const float* __restrict__ pac
 				for (int p = 0; p < P; ++p) acc[p] = norms_next;
 				if (tile + 1 < tile_end) fetch_norms(norms_next, tile + 1);
 			}
+			if constexpr (PACKED) { /* one MFMA holds every product of the row (load_packed_points) */
+#pragma unroll
+				for (int p = 0; p < P; ++p) acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(o.hi[0], b[p].hi[0], acc[p], 0, 0, 0);
+			}
+			else
 #pragma unroll
 			for (int i = 0; i < G; ++i) {
 #pragma unroll
@@ -757,6 +767,9 @@ static int launch_screen_bf16_kb(const float* rows, const Workspace* ws, const u
                                  const DeviceInfo& dev, uint32_t* waves)
 {
 	auto kernel = screen_bf16_kernel<KB, ScreenShape<KB>::P>;
+	if constexpr (KB == 1) {
+		if (packed_rows(dim)) kernel = screen_bf16_kernel<KB, ScreenShape<KB>::P, true>;
+	}
 	/* as many wavefronts as the device holds at once: the partition of the work counts on all of them running together */
 	int per_cu = 1;
 	KMX_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)kernel, (int)(SCREEN_WAVES * WAVE), 0));
@@ -773,9 +786,6 @@ template <int KB> struct SplitSweepShape {
 	static constexpr int P = KB <= 4 ? 2 : 1;
 	static constexpr bool PREFETCH = KB <= 2;
 };
-
-/* rows of at most 4 dimensions: the four products of all dimensions in one block of MFMA slots (load_packed_points) */
-inline bool packed_rows(uint32_t dim) { return dim <= 4; }
 
 template <int KB, int LD, bool VEC, bool PACKED = false>
 static int launch_bf16_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev, uint32_t kp, float kd)
