@@ -113,6 +113,9 @@ SHAPES = [
     (48, 300, 3000),    # exact pass with one centroid row per lane, rows of 33..64 floats
     (37, 2100, 2500),   # the same with a padded row and three chunks of centroids
     (64, 1024, 6000),
+    (4, 9000, 3000),    # packed rows (at most 4 dimensions), more centroids than LDS holds: streamed
+    (3, 200, 4000),     # packed rows, padded to 4 dimensions, screened exact pass
+    (2, 600, 5000),
     (4, 1, 100),        # one centroid, one point
     (3, 5, 1),
     (40, 1, 1),
