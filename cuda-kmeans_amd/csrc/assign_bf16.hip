@@ -3,7 +3,7 @@
  * v_mfma_f32_32x32x16_bf16 tiles over SPLIT operands.
  *
  * Every fp32 value v is written as hi + mid + rest with hi = bf16(v), mid = bf16(v - hi) (round to nearest
- * even), |rest| <= 2^-18 |v|. The contraction keeps the three largest of the four hi/mid products,
+ * even), |mid| <= 2^-8 |v|, |rest| <= 2^-17 |v|. The contraction keeps the three largest of the four hi/mid products,
  *      c'.x  ~  sum_i  c'hi_i x_mid_i + c'mid_i x_hi_i + c'hi_i x_hi_i ,       c' = -2c,
  * each product exact in fp32 (8 x 8 significant bits), accumulated in fp32 by the matrix core. One block of
  * 16 dimensions costs 3 MFMAs of 8 passes where the fp32 kernel (v_mfma_f32_32x32x2_f32) spends 8 MFMAs of
@@ -12,23 +12,16 @@
  * Exactness. As in the fp32 kernel the result promised to the caller is the index the serial scan returns
  * (reference serial.hpp:21-35, metric_policies.hpp:23-28,40-44), established by the same certification:
  * a point whose two smallest a[j] are further apart than tau is decided, every other point goes to the
- * recheck queue and is re-evaluated with the serial arithmetic. Only tau differs. With u' = 2^-23 (one
- * unit allows for any rounding or truncation of the accumulator) and S = |x|^2 + max_j |c_j|^2:
- *   - dropped terms:   |c'_i x_i - (three products)| <= (2^-18 + 2^-18 + 2^-18)(1 + 2^-8) |c'_i||x_i|,
- *                      and sum_i |c'_i||x_i| <= 2|c||x| <= S            -> 3.02 * 2^-18 S  (= 96.6 u' S)
- *   - accumulation of 3d products and |c|^2 in fp32                      -> (3d + 2) u' * 2 S
- *   - the serial sum's own error and the sqrt collision margin           -> (2d + 12) u' S   (as for fp32)
- * tau must exceed twice the error of a[j] plus the serial margin: (12d + 8 + 193.3 + 2d + 12) u' S, so
- *      tau = (14 d + 224) 2^-23 (|x|^2 + max_j |c_j|^2).
+ * recheck queue and is re-evaluated with the serial arithmetic. Only tau differs: it has to cover the products
+ * the split drops. certificate.h derives it: tau = kd S + 2.06 * (bound of the dropped products), the bound
+ * evaluated from the norms of the parts actually dropped -- max_j |c'mid_j| and max_j |c'rest_j|, which the packing
+ * kernel below writes behind the norms, and |xmid| (or |xrest|) of the point -- not from their worst case.
  * The refinement (winning row inside the winning tile) re-evaluates rows with v_dot2c_f32_bf16 on the same
  * three products, so the same bound covers it.
  *
  * Rows of at most 4 dimensions (PACKED): a block of 16 MFMA slots holds ALL FOUR hi/mid products of every dimension
- * (4 d <= 16), so a tile costs one MFMA instead of three and nothing of (hi + mid)(hi + mid) is dropped:
- *   - operands cut to hi + mid:   |c'_i x_i - (four products)| <= (2^-18 + 2^-18 + 2^-36) |c'_i||x_i|  -> 2.0001 * 2^-18 S  (= 64.01 u' S)
- *   - accumulation of 4d products and |c|^2 in fp32                                              -> (4d + 2) u' * 2 S
- *   - serial margin as above                                                                          -> (2d + 12) u' S
- * tau > (128.02 + 16d + 8 + 2d + 12) u' S:   tau = (18 d + 149) 2^-23 (|x|^2 + max_j |c_j|^2).
+ * (4 d <= 16), so a tile costs one MFMA instead of three and nothing of (hi + mid)(hi + mid) is dropped; only the
+ * remainders of the split are (certificate.h, packed form).
  *
  * Data flow, tiling, tracking, flag buffering and the recheck hand-over are those of the fp32 kernel
  * (assign_mfma.hip); the packed centroid row holds hi and mid parts of -2c, 4 bytes per dimension as before.
@@ -64,7 +57,7 @@ pack_means_bf16_kernel(const float* __restrict__ means, size_t stride_means, flo
 	const uint32_t rs = packed_slots ? row_floats<1, true>() : dp + ROW_PAD;
 	float* row = packed + packed_row(j, rs);
 	__bf16* parts = (__bf16*)row;
-	float c2 = 0.0f;
+	float c2 = 0.0f, mid2 = 0.0f, rest2 = 0.0f; /* |c|^2 and, for the certificate, sum_i c'mid_i^2, sum_i c'rest_i^2 */
 	if (packed_slots) {
 		/* rows of at most 4 dimensions: slots 0..3 = hi, 4..7 = mid, 8..11 = hi, 12..15 = mid of -2c; inside the tile
 		 * the first halves of all rows, then the second halves (packed_half; load_packed_points has the matching order
@@ -73,12 +66,14 @@ pack_means_bf16_kernel(const float* __restrict__ means, size_t stride_means, flo
 			const uint32_t q = lane % 4;
 			const float v = (j < k && q < dim) ? means[elem<LM>(stride_means, j, q)] : 0.0f;
 			__bf16 hi, mid;
-			split_bf16(-2.0f * v, hi, mid);
+			const float rest = split_bf16(-2.0f * v, hi, mid);
 			float* tile = packed + (size_t)(j / TILE) * tile_floats(rs);
 			((__bf16*)(tile + packed_half(j % TILE, lane / 8)))[lane % 8] = (lane / 4) % 2 == 1 ? mid : hi;
 			if (j % TILE == TILE - 1 && lane < TILE_PAD) tile[TILE * rs + lane] = 0.0f;
 			if (lane < 4) {
 				c2 = v * v;
+				mid2 = (float)mid * (float)mid;
+				rest2 = rest * rest;
 				if (q < dim) means_t[(size_t)q * kp + j] = v; /* exact copy for the recheck pass */
 			}
 		}
@@ -88,7 +83,9 @@ pack_means_bf16_kernel(const float* __restrict__ means, size_t stride_means, flo
 		const float v = (j < k && q < dim) ? means[elem<LM>(stride_means, j, q)] : 0.0f;
 		c2 += v * v;
 		__bf16 hi, mid;
-		split_bf16(-2.0f * v, hi, mid);
+		const float rest = split_bf16(-2.0f * v, hi, mid);
+		mid2 += (float)mid * (float)mid;
+		rest2 += rest * rest;
 		/* block q / 16, half-wave (q % 16) / 8: 16-byte unit 4 kb + 2 h (hi), + 1 (mid) */
 		const uint32_t unit = 4 * (q / KBLOCK) + 2 * ((q % KBLOCK) / 8);
 		parts[8 * unit + q % 8] = hi;
@@ -97,8 +94,17 @@ pack_means_bf16_kernel(const float* __restrict__ means, size_t stride_means, flo
 	}
 	const uint32_t pad_floats = ROW_PAD + (j % TILE == TILE - 1 ? TILE_PAD : 0);
 	if (!packed_slots && lane < pad_floats) row[dp + lane] = 0.0f;
-	for (int off = WAVE / 2; off > 0; off >>= 1) c2 += __shfl_xor(c2, off);
-	if (lane == 0) norms[norm_at(j)] = j < k ? c2 : __builtin_inff();
+	for (int off = WAVE / 2; off > 0; off >>= 1) {
+		c2 += __shfl_xor(c2, off);
+		mid2 += __shfl_xor(mid2, off);
+		rest2 += __shfl_xor(rest2, off);
+	}
+	if (lane == 0) {
+		norms[norm_at(j)] = j < k ? c2 : __builtin_inff();
+		float* part_norms = norms + split_norms_offset(kp);
+		part_norms[j] = mid2;
+		part_norms[kp + j] = rest2;
+	}
 	if (lane < NORM_TILE - TILE && j % TILE == 0) norms[(j / TILE) * NORM_TILE + TILE + lane] = __builtin_inff();
 }
 
@@ -143,7 +149,7 @@ int launch_assign_bf16(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws
 	const uint32_t dp = KBLOCK * kb;
 	const uint32_t kp = round_up(a.k, TILE);
 	const uint32_t rs = packed_rows(a.dim) ? row_floats<1, true>() : dp + ROW_PAD;
-	int rc = reserve_packed(ws, (size_t)(kp / TILE) * tile_floats(rs), (size_t)(kp / TILE) * NORM_TILE, (size_t)kp * a.dim);
+	int rc = reserve_packed(ws, (size_t)(kp / TILE) * tile_floats(rs), split_norms_offset(kp) + 2 * (size_t)kp, (size_t)kp * a.dim);
 	if (rc) return rc;
 	rc = reserve_queue(ws, 2 * (size_t)a.n); /* (point, threshold) pairs */
 	if (rc) return rc;
@@ -156,9 +162,8 @@ int launch_assign_bf16(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws
 		                   a.means, a.stride_means, ws->packed_means, ws->norms, ws->means_t, a.dim, a.k, kp, dp, packed_rows(a.dim) ? 1u : 0u, ws->counters);
 	KMX_LAUNCH_CHECK("pack_means_bf16_kernel");
 
-	/* tau = kd (|x|^2 + max|c|^2), kd = (14 d + 224) 2^-23, or (18 d + 149) 2^-23 for the packed rows, which keep all
-	 * four products (see the bounds at the top of the file) */
-	const float kd = (packed_rows(a.dim) ? 18.0f * (float)a.dim + 149.0f : 14.0f * (float)a.dim + 224.0f) * 1.1920929e-07f + a.kd_extra;
+	/* tau = kd (|x|^2 + max|c|^2) + the bound of the dropped products (certificate.h) */
+	const float kd = (packed_rows(a.dim) ? cert_kd_packed(a.dim) : cert_kd_split(a.dim)) + a.kd_extra;
 	switch (kb) {
 	case 1: rc = launch_bf16_1(a, exec, ws, dev, kp, kd); break;
 	case 2: rc = launch_bf16_2(a, exec, ws, dev, kp, kd); break;

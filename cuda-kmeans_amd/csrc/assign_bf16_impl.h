@@ -7,6 +7,7 @@
 #define KMX_ASSIGN_BF16_IMPL_H
 
 #include "assign_mfma_impl.h"
+#include "certificate.h"
 
 #include <type_traits>
 
@@ -29,12 +30,19 @@ __host__ __device__ constexpr uint32_t packed_half(uint32_t r, uint32_t h) { ret
 /* rows of at most 4 dimensions: the four products of all dimensions in one block of MFMA slots (load_packed_points) */
 inline bool packed_rows(uint32_t dim) { return dim <= 4; }
 
-/* value = hi + mid + (at most 2^-18 |value|), both parts bf16 (round to nearest even) */
-__device__ __forceinline__ void split_bf16(float v, __bf16& hi, __bf16& mid)
+/* value = hi + mid + rest, both parts bf16 (round to nearest even), |mid| <= 2^-8 |value|, |rest| <= 2^-8 |mid|; returns
+ * rest (both subtractions are exact in fp32) */
+__device__ __forceinline__ float split_bf16(float v, __bf16& hi, __bf16& mid)
 {
 	hi = (__bf16)v;
-	mid = (__bf16)(v - (float)hi);
+	const float r = v - (float)hi;
+	mid = (__bf16)r;
+	return r - (float)mid;
 }
+
+/* The norms array of the split-bf16 kernels: the tiles of |c|^2 (NORM_TILE floats per tile), then per padded row
+ * sum_i c'mid_i^2 and, kp floats on, sum_i c'rest_i^2 (c' = -2c; what the certificate needs, see certificate.h). */
+__host__ __device__ __forceinline__ size_t split_norms_offset(uint32_t kp) { return (size_t)(kp / TILE) * NORM_TILE; }
 
 /* One tile of 32 points as B operands: per block of 16 dimensions the lane holds the 8 dimensions of its
  * half-wave (lanes 0-31: the first 8, lanes 32-63: the second 8) of ONE point, as hi and mid parts. */
@@ -69,18 +77,19 @@ __device__ __forceinline__ void load_packed_points(SplitPoints<1> (&b)[P], float
 #pragma unroll
 			for (int j = 0; j < 4; ++j) v[j] = (valid && (uint32_t)j < dim) ? data[elem<LD>(stride, pt, j)] : 0.0f;
 		}
-		float part = 0.0f;
+		float part = 0.0f, rest2 = 0.0f;
 #pragma unroll
 		for (int j = 0; j < 4; ++j) {
 			part += v[j] * v[j];
 			__bf16 hi, mid;
-			split_bf16(v[j], hi, mid);
+			const float rest = split_bf16(v[j], hi, mid);
+			rest2 += rest * rest;
 			b[p].hi[0][j] = h == 0 ? mid : hi;      /* slots 0..3: x_mid,  slots 8..11: x_hi   */
 			b[p].hi[0][4 + j] = h == 0 ? hi : mid;  /* slots 4..7: x_hi,   slots 12..15: x_mid */
 			b[p].mid[0][j] = (__bf16)0.0f;
 			b[p].mid[0][4 + j] = (__bf16)0.0f;
 		}
-		xx[p] = h == 0 ? part : 0.0f; /* the two half-waves hold the same point: |x|^2 once */
+		xx[p] = h == 0 ? part : rest2; /* the two half-waves hold the same point: |x|^2 in the first, sum_i xrest_i^2 in the second */
 	}
 }
 
@@ -242,7 +251,7 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 {
 	constexpr uint32_t RS = row_floats<KB, PACKED>();
 	extern __shared__ float lds[];
-	__shared__ uint32_t wave_max[MFMA_WAVES];
+	__shared__ uint32_t wave_max[3][MFMA_WAVES];
 	__shared__ uint32_t flag_list[MFMA_WAVES][2 * FLAG_CAP]; /* (point, threshold) pairs */
 
 	const uint32_t lane = threadIdx.x & (WAVE - 1);
@@ -250,15 +259,35 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 	const uint32_t col = lane & 31; /* point within a tile (B column) / centroid row fed to A */
 	const uint32_t h = lane >> 5;   /* half-wave: K split and the +4 row group of the result    */
 
-	/* max_j |c_j|^2 (bit pattern maximum: propagates NaN and +inf, which then flag every point) */
-	uint32_t cmax = 0;
-	for (uint32_t j = threadIdx.x; j < k; j += blockDim.x) cmax = max(cmax, __float_as_uint(norms[norm_at(j)]));
-	for (int off = WAVE / 2; off > 0; off >>= 1) cmax = max(cmax, (uint32_t)__shfl_xor((int)cmax, off));
-	if (lane == 0) wave_max[wave] = cmax;
-	__syncthreads();
-	cmax = 0;
-	for (uint32_t w = 0; w < MFMA_WAVES; ++w) cmax = max(cmax, wave_max[w]);
-	const float c2max = __uint_as_float(cmax);
+	/* max_j of |c_j|^2, sum_i c'mid_i^2 and sum_i c'rest_i^2 (bit pattern maxima: they propagate NaN and +inf, which then flag every point) */
+	CertCoeffs cert;
+	{
+		const float* part_norms = norms + split_norms_offset(kp);
+		uint32_t cmax[3] = { 0u, 0u, 0u };
+		for (uint32_t j = threadIdx.x; j < k; j += blockDim.x) {
+			cmax[0] = max(cmax[0], __float_as_uint(norms[norm_at(j)]));
+			cmax[1] = max(cmax[1], __float_as_uint(part_norms[j]));
+			cmax[2] = max(cmax[2], __float_as_uint(part_norms[kp + j]));
+		}
+#pragma unroll
+		for (int q = 0; q < 3; ++q) {
+			for (int off = WAVE / 2; off > 0; off >>= 1) cmax[q] = max(cmax[q], (uint32_t)__shfl_xor((int)cmax[q], off));
+			if (lane == 0) wave_max[q][wave] = cmax[q];
+		}
+		__syncthreads();
+#pragma unroll
+		for (int q = 0; q < 3; ++q) {
+			cmax[q] = 0;
+			for (uint32_t w = 0; w < MFMA_WAVES; ++w) cmax[q] = max(cmax[q], wave_max[q][w]);
+		}
+		const CentroidBounds cb{ __uint_as_float(cmax[0]), __uint_as_float(cmax[1]), __uint_as_float(cmax[2]) };
+		cert = PACKED ? cert_coeffs_packed(cb) : cert_coeffs_split(cb);
+		/* the same in every lane of the work-group: kept in scalar registers */
+		cert.c2max = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(cert.c2max)));
+		cert.a = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(cert.a)));
+		cert.b = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(cert.b)));
+	}
+	const float c2max = cert.c2max;
 
 	const uint32_t chunk_tiles = chunk_rows / TILE;
 	const uint32_t chunks = (kp + chunk_rows - 1) / chunk_rows;
@@ -419,7 +448,8 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 		Track st[P];
 #pragma unroll
 		for (int p = 0; p < P; ++p) {
-			x2[p] = xx[p] + __shfl_xor(xx[p], 32);
+			/* PACKED: the half-waves hold |x|^2 and sum_i xrest_i^2 of the same point; the pair is taken apart again below */
+			x2[p] = PACKED ? xx[p] : xx[p] + __shfl_xor(xx[p], 32);
 			st[p].m1 = __builtin_inff();
 			st[p].m2 = __builtin_inff();
 			st[p].tile = 0;
@@ -520,10 +550,28 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 				first = fminf(st[p].m1, o1);
 				second = fminf(fmaxf(st[p].m1, o1), fminf(st[p].m2, o2));
 			}
-			const float tau = kd * (x2[p] + c2max);
+			/* the certificate (certificate.h): the norms of the parts of the point that the products drop */
+			float xsq, tau;
+			if constexpr (PACKED) {
+				const float other = __shfl_xor(x2[p], 32);
+				xsq = h == 0 ? x2[p] : other;
+				tau = cert_tau(kd, xsq, h == 0 ? other : x2[p], cert);
+			}
+			else {
+				float xmid2 = 0.0f;
+#pragma unroll
+				for (int kb = 0; kb < KB; ++kb) {
+					const bf16x8 xm = b[p].mid[kb];
+					xmid2 = KMX_DOT2_PAIR(xmid2, xm, xm, 0); xmid2 = KMX_DOT2_PAIR(xmid2, xm, xm, 1);
+					xmid2 = KMX_DOT2_PAIR(xmid2, xm, xm, 2); xmid2 = KMX_DOT2_PAIR(xmid2, xm, xm, 3);
+				}
+				xmid2 += __shfl_xor(xmid2, 32);
+				xsq = x2[p];
+				tau = cert_tau(kd, xsq, xmid2, cert);
+			}
 			const uint32_t pt = base + p * TILE + col;
 			const bool mine = h == 0 && pt < n;
-			const bool decided = (second - first > tau) && (x2[p] + c2max > 1e-30f);
+			const bool decided = (second - first > tau) && (xsq + c2max > 1e-30f);
 			if (mine) assignment[pt] = idx < k ? idx : 0u;
 			const bool flag = mine && !decided;
 			const unsigned long long mask = __ballot(flag);

@@ -17,6 +17,7 @@
  * (KMX_ASSIGN_LDS_FMA, `hip_lds_fma`) so that the choice can be measured; KMX_ASSIGN_BEST picks it only for
  * k <= 32 with the scalar-cache path.
  */
+#include "certificate.h"
 #include "assign_mfma_impl.h"
 
 namespace kmx {
@@ -214,7 +215,7 @@ int launch_assign_lds_fma(const AssignArgs& a, kmx_exec_params* exec, Workspace*
 	const uint32_t kp = round_up(a.k, TILE);
 	int rc = launch_pack_means(a, ws, dp, kp);
 	if (rc) return rc;
-	const float kd = (8.0f * (float)a.dim + 24.0f) * 1.1920929e-07f + a.kd_extra;
+	const float kd = cert_kd_fp32(a.dim) + a.kd_extra;
 	switch (dp) {
 	case 4: rc = launch_fma_dp<4>(a, exec, ws, dev, kp, kd); break;
 	case 8: rc = launch_fma_dp<8>(a, exec, ws, dev, kp, kd); break;

@@ -36,6 +36,7 @@
  * is recomputed once per sweep; (2) sched_group_barrier groups the MFMAs of a tile and the tracking of
  * the previous tile into few large runs.
  */
+#include "certificate.h"
 #include "assign_mfma_impl.h"
 
 namespace kmx {
@@ -120,7 +121,7 @@ int launch_assign_mfma(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws
 	if (rc) return rc;
 
 	/* tau = kd (|x|^2 + max|c|^2), kd = (8 d + 24) 2^-23 (see the bound at the top of the file) */
-	const float kd = (8.0f * (float)a.dim + 24.0f) * 1.1920929e-07f + a.kd_extra;
+	const float kd = cert_kd_fp32(a.dim) + a.kd_extra;
 	switch (dph) {
 	case 2: rc = launch_mfma_2(a, exec, ws, dev, kp, kd); break;
 	case 4: rc = launch_mfma_4(a, exec, ws, dev, kp, kd); break;

@@ -1,0 +1,88 @@
+/*
+ * The certification bounds of the ranking sweeps, in one place, callable from device code and from the host
+ * (kmx_certificate_tau exposes them to the tests, which check them against an emulation of the split operands).
+ *
+ * A sweep ranks the centroids of a point by a[j] ~ A_j = |c_j|^2 - 2 c_j . x. It may decide the point without the
+ * serial arithmetic (reference serial.hpp:21-35, metric_policies.hpp:23-28,40-44) only if the two smallest a[j] are
+ * further apart than tau, where
+ *      tau  >=  2 max_j |a[j] - A_j|  +  (serial margin),
+ * the serial margin being the error of two serial sums plus what a correctly rounded sqrt can merge:
+ * (2 d + 12) u' S with u' = 2^-23 and S = |x|^2 + max_j |c_j|^2.
+ *
+ * fp32 sweeps: |a[j] - A_j| <= (d + 2) u' (|c_j|^2 + 2 |x||c_j|) <= (d + 2) u' 2 S  ->  tau = (8 d + 24) u' S
+ * (one u' per accumulation step allows for any rounding or truncation inside the matrix core).
+ *
+ * Split-bf16 sweeps. Every operand v is hi + mid + rest with hi = bf16(v), mid = bf16(v - hi), both rounded to nearest:
+ * a bf16 has 8 significant bits, so |mid| <= 2^-8 |v|, |rest| <= 2^-8 |mid| <= 2^-17 |v| (the worst case is
+ * attained: v = 1 + odd * 2^-17). The sweep adds the products it keeps exactly (8 x 8 bits fit an fp32) and accumulates
+ * them in fp32, so
+ *      |a[j] - A_j|  <=  (accumulation)  +  |sum_i of the dropped products|.
+ *   - three-product form (hi*hi + hi*mid + mid*hi per dimension, c' = -2 c, 3 d products and the norm):
+ *        accumulation <= (3 d + 2) u' 2 S
+ *        dropped = sum_i c'mid_i xmid_i + (c'hi_i + c'mid_i) xrest_i + c'rest_i x_i
+ *                <= |c'mid| |xmid| + (|c'| + |c'rest|) |xrest| + |c'rest| |x|               (Cauchy-Schwarz)
+ *        and elementwise |xrest_i| <= 2^-8 |xmid_i|, hence |xrest| <= 2^-8 |xmid|.
+ *     The bound is evaluated with the norms of the parts at hand instead of their worst case 2^-15 |c'||x| (= 256 u' S,
+ *     which would have to be doubled): |xmid| of the point from the operands the lane holds, max_j |c'mid_j| and
+ *     max_j |c'rest_j| from the packing kernel. With random mantissas it comes to about a third of the worst case.
+ *   - packed form (rows of at most 4 dimensions, all four hi/mid products kept, 4 d products and the norm):
+ *        accumulation <= (4 d + 2) u' 2 S
+ *        dropped = sum_i (c'hi_i + c'mid_i) xrest_i + c'rest_i x_i <= (|c'| + |c'rest|) |xrest| + |c'rest| |x|
+ *     with |xrest| of the point computed when it is split.
+ * tau = kd S + TRUNC_FACTOR * (bound of the dropped products); kd = (12 d + 8 + 2 d + 12 + slack) u' and
+ * (16 d + 8 + 2 d + 12 + slack) u'; TRUNC_FACTOR = 2 plus 1/16 for the fp32 roundings in the norms and square roots.
+ * Values the bound does not cover (NaN, infinities, sums that overflow) make tau NaN or infinite, and the
+ * comparison `second - first > tau` is then false: the point goes to the exact pass.
+ */
+#ifndef KMX_CERTIFICATE_H
+#define KMX_CERTIFICATE_H
+
+#if defined(__HIPCC__)
+#define KMX_HD __host__ __device__ inline __attribute__((always_inline))
+#else
+#define KMX_HD inline
+#endif
+
+namespace kmx {
+
+constexpr float CERT_UNIT = 1.1920929e-07f;   /* u' = 2^-23 */
+constexpr float CERT_TRUNC_FACTOR = 2.0625f;
+constexpr float CERT_BF16_UNIT = 0.00390625f; /* 2^-8: relative rounding error of a bf16 */
+
+/* what the packing kernel knows about the centroids of a call: max |c_j|^2, max sum_i c'mid_i^2, max sum_i c'rest_i^2 (c' = -2 c) */
+struct CentroidBounds {
+	float c2max, mid2max, rest2max;
+};
+
+KMX_HD float cert_kd_fp32(unsigned dim) { return (8.0f * (float)dim + 24.0f) * CERT_UNIT; }
+KMX_HD float cert_kd_split(unsigned dim) { return (14.0f * (float)dim + 28.0f) * CERT_UNIT; }
+KMX_HD float cert_kd_packed(unsigned dim) { return (18.0f * (float)dim + 28.0f) * CERT_UNIT; }
+
+/* The bound in the form the kernels evaluate per point: tau = kd (x2 + c2max) + a sqrt(xpart2) + b sqrt(x2), with
+ * xpart2 = sum_i xmid_i^2 (three-product form) or sum_i xrest_i^2 (packed form); a and b depend on the centroids only. */
+struct CertCoeffs {
+	float c2max, a, b;
+};
+
+KMX_HD CertCoeffs cert_coeffs_split(const CentroidBounds& c)
+{
+	const float cnorm = 2.0f * __builtin_sqrtf(c.c2max); /* |c'| */
+	const float cmid = __builtin_sqrtf(c.mid2max), crest = __builtin_sqrtf(c.rest2max);
+	return CertCoeffs{ c.c2max, CERT_TRUNC_FACTOR * (cmid + (cnorm + crest) * CERT_BF16_UNIT), CERT_TRUNC_FACTOR * crest };
+}
+
+KMX_HD CertCoeffs cert_coeffs_packed(const CentroidBounds& c)
+{
+	const float cnorm = 2.0f * __builtin_sqrtf(c.c2max);
+	const float crest = __builtin_sqrtf(c.rest2max);
+	return CertCoeffs{ c.c2max, CERT_TRUNC_FACTOR * (cnorm + crest), CERT_TRUNC_FACTOR * crest };
+}
+
+KMX_HD float cert_tau(float kd, float x2, float xpart2, const CertCoeffs& c)
+{
+	return kd * (x2 + c.c2max) + (c.a * __builtin_sqrtf(xpart2) + c.b * __builtin_sqrtf(x2));
+}
+
+} // namespace kmx
+
+#endif

@@ -24,6 +24,7 @@
  * Floating-point contraction is off for the whole file (the serial arithmetic must not fuse); the ranking uses
  * explicit fused multiply-adds.
  */
+#include "certificate.h"
 #include "assign_mfma_impl.h"
 
 #pragma clang fp contract(off)
@@ -300,7 +301,7 @@ static int launch_fused_layouts(const AssignArgs& a, float* means_out, uint32_t*
 	const uint32_t kp = round_up(a.k, TILE);
 	int rc = launch_pack_means(a, ws, dp, kp);
 	if (rc) return rc;
-	const float kd = (8.0f * (float)a.dim + 24.0f) * 1.1920929e-07f; /* the bound of the fp32 ranking, see assign_mfma.hip */
+	const float kd = cert_kd_fp32(a.dim); /* the bound of the fp32 ranking, see assign_mfma.hip */
 	switch (dp) {
 	case 4: rc = launch_fused_t<4, LD, LM>(a, means_out, sizes, exec, ws, dev, kd); break;
 	case 8: rc = launch_fused_t<8, LD, LM>(a, means_out, sizes, exec, ws, dev, kd); break;

@@ -3,6 +3,7 @@
  * validation and dispatch to the kernel launchers. Declared in include/kmx.h.
  */
 #include "kmx_internal.h"
+#include "certificate.h"
 
 #include <cstdarg>
 #include <cstring>
@@ -577,6 +578,19 @@ int kmx_set_queued_rows_limit(size_t bytes)
 	clear_error();
 	set_queued_rows_limit(bytes);
 	return KMX_OK;
+}
+
+int kmx_certificate_tau(int form, uint32_t dim, float x2, float xpart2, float c2max, float cmid2max, float crest2max, float* tau)
+{
+	clear_error();
+	if (!tau) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_certificate_tau: null pointer");
+	const CentroidBounds cb{ c2max, cmid2max, crest2max };
+	switch (form) {
+	case 0: *tau = cert_kd_fp32(dim) * (x2 + c2max); return KMX_OK;
+	case 1: *tau = cert_tau(cert_kd_split(dim), x2, xpart2, cert_coeffs_split(cb)); return KMX_OK;
+	case 2: *tau = cert_tau(cert_kd_packed(dim), x2, xpart2, cert_coeffs_packed(cb)); return KMX_OK;
+	default: return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_certificate_tau: unknown form %d", form);
+	}
 }
 
 int kmx_set_profiling(int enabled)

@@ -1,0 +1,227 @@
+"""The certification bound of the split-bf16 sweeps against an emulation of their arithmetic (CPU, no GPU).
+
+The sweeps rank centroids with a[j] = |c_j|^2 + sum_i (kept products of the split operands) and decide a point without
+the serial arithmetic when its two smallest a[j] differ by more than tau. The emulation here splits the operands
+exactly as the kernels do (bf16, round to nearest even), adds the kept products without error (float64 holds them
+exactly) and compares with the exact A_j = |c_j|^2 - 2 c_j . x: the difference is what the split drops. tau (from the
+library's own function, kmx_certificate_tau) must cover twice that plus the accumulation allowance plus the serial
+margin; and wherever the emulated ranking, disturbed by the full accumulation allowance, would certify a pair, the
+serial oracle must agree with the decision.
+
+The inputs are the worst cases of the split, which random data never reaches: coordinates 1 + odd * 2^-17 (both
+remainders at their maximum) against centroids c and about -c, plus near-ties at every scale.
+"""
+import numpy as np
+import pytest
+
+U = 2.0 ** -23
+
+
+def bf16_round(v):
+    """float32 -> nearest bf16 (ties to even), returned as float32."""
+    bits = np.asarray(v, np.float32).view(np.uint32).astype(np.uint64)
+    bits = (bits + 0x7FFF + ((bits >> 16) & 1)) & 0xFFFF0000
+    return bits.astype(np.uint32).view(np.float32)
+
+
+def split(v):
+    v = np.asarray(v, np.float32)
+    hi = bf16_round(v)
+    r = (v - hi).astype(np.float32)
+    mid = bf16_round(r)
+    rest = (r - mid).astype(np.float32)
+    assert np.array_equal(hi.astype(np.float64) + mid.astype(np.float64) + rest.astype(np.float64), v.astype(np.float64))
+    return hi, mid, rest
+
+
+def test_split_remainders_reach_their_stated_worst_case():
+    v = (1.0 + np.arange(1, 1 << 17, 2, dtype=np.float64) * 2.0 ** -17).astype(np.float32)
+    hi, mid, rest = split(v)
+    assert np.abs(mid / v).max() <= 2.0 ** -8 and np.abs(mid / v).max() > 0.99 * 2.0 ** -8
+    assert np.abs(rest / v).max() <= 2.0 ** -17 and np.abs(rest / v).max() > 0.99 * 2.0 ** -17
+    nz = mid != 0
+    assert np.all(np.abs(rest[nz]) <= 2.0 ** -8 * np.abs(mid[nz]))
+
+
+def adversarial(dim, n, k, rng):
+    """Coordinates 1 + m * 2^-17 with odd m up to 511 (|mid| / |v| and |rest| / |v| next to their maxima), random signs.
+    Centroids come in pairs (c, about -c) and half of the points are copies of a centroid: the products the split drops
+    then all have one sign for c and the other for -c, so the two ranking values move apart by the sum of the bounds."""
+    def worst(shape):
+        return (1.0 + (2 * rng.integers(128, 256, size=shape) + 1) * 2.0 ** -17).astype(np.float32)
+    c = worst((k, dim)) * rng.choice(np.float32([-1, 1]), size=(k, dim))
+    c[1::2] = -c[0::2][: c[1::2].shape[0]] * (1 + rng.integers(-3, 4, size=c[1::2].shape) * np.float32(2.0 ** -12))
+    x = worst((n, dim)) * rng.choice(np.float32([-1, 1]), size=(n, dim))
+    x[: n // 2] = c[rng.integers(0, k, size=n // 2)]
+    return x.astype(np.float32), c.astype(np.float32)
+
+
+def worst_parts(rng, shape, mid_sign, rest_sign):
+    """1 + m 2^-17 (m < 1024) whose split has a mid part of 0.8 to 1 times 2^-8 and a rest part of 2^-17, with the signs asked for.
+    m = 4j + 1 rounds down to 8 bits (rest +), 4j + 3 rounds up (rest -); 1024 - m gives hi = 1 + 2^-7 and a negative mid."""
+    j = rng.integers(100, 127, size=shape)
+    pos_mid, plus_rest = mid_sign > 0, rest_sign > 0
+    m = np.where(pos_mid, np.where(plus_rest, 4 * j + 1, 4 * j + 3), 1024 - np.where(plus_rest, 4 * j + 3, 4 * j + 1))
+    return 1.0 + m * 2.0 ** -17
+
+
+def worst_case_pairs(dim, pairs, per_pair, rng, shared_mid_signs):
+    """Near-ties on which every product the split drops has one sign for one centroid and the other sign for its rival.
+    All centroids of even index agree in sign with the points on half of the coordinates, those of odd index on the other
+    half, so a point is about equally far from both kinds; the signs of the mid and rest parts are chosen per coordinate
+    so that, for the even kind, c'mid xmid, c'hi xrest and c'rest xhi are all positive, and all negative for the odd kind.
+    The ranking values of the two kinds then move apart by twice the worst case of the dropped products (2 * 2^-15 S for
+    three products, 2 * 2^-16 S for the packed form) while the true gaps straddle zero."""
+    sx = rng.choice([-1.0, 1.0], size=(1, dim))
+    match = np.ones((1, dim))
+    match[0, rng.permutation(dim)[: dim // 2]] = -1           # +1: the point has the sign of the even kind there
+    mid_sign = rng.choice([-1.0, 1.0], size=(1, dim) if shared_mid_signs else (pairs, dim)) * np.ones((pairs, dim))
+    c = np.empty((2 * pairs, dim))
+    c[0::2] = sx * match * worst_parts(rng, (pairs, dim), match * mid_sign, match * np.ones((pairs, dim)))
+    c[1::2] = -sx * match * worst_parts(rng, (pairs, dim), match * mid_sign, match * np.ones((pairs, dim)))
+    pid = np.repeat(np.arange(pairs), per_pair)
+    x = sx * worst_parts(rng, (pairs * per_pair, dim), mid_sign[pid], match * np.ones((pairs * per_pair, dim)))
+    return x.astype(np.float32), c.astype(np.float32)
+
+
+# (dim, pairs, shared_mid_signs): shapes at which the inputs defeat a certificate derived for 9-bit parts
+WORST_CASE_SHAPES = [(2, 32, False), (3, 32, False), (4, 32, False), (8, 4, True), (16, 2, True), (32, 1, True), (64, 1, True)]
+
+
+def worst_case_inputs(dim, n=64000):
+    pairs, shared = next((p, s) for d, p, s in WORST_CASE_SHAPES if d == dim)
+    return worst_case_pairs(dim, pairs, n // pairs, np.random.default_rng(dim), shared)
+
+
+def near_ties(dim, n, k, rng, offset, centroids=None):
+    """Points close to the bisector of two centroids, true gap log-uniform over six decades, coordinates shifted by offset."""
+    c = centroids if centroids is not None else rng.normal(size=(k, dim)).astype(np.float32) * np.float32(3) + np.float32(offset)
+    a, b = rng.integers(0, k, size=n), rng.integers(0, k, size=n)
+    b = np.where(a == b, (b + 1) % k, b)
+    ca, cb = c[a].astype(np.float64), c[b].astype(np.float64)
+    gap = 10.0 ** rng.uniform(-9, -3, size=n) * rng.choice([-1.0, 1.0], size=n)
+    s = (ca ** 2).sum(1) + (cb ** 2).sum(1)
+    direction = cb - ca
+    length = np.maximum(np.sqrt((direction ** 2).sum(1)), 1e-30)
+    t = gap * s / (2 * length)
+    x = (ca + cb) / 2 + direction / length[:, None] * t[:, None]
+    return x.astype(np.float32), c
+
+
+def emulate(x, c, packed):
+    """The ranking values of the sweep without accumulation error, the exact ones, and the norms the certificate uses."""
+    xh, xm, xr = (p.astype(np.float64) for p in split(x))
+    cp = (np.float32(-2) * c).astype(np.float32)
+    ch, cm, cr = (p.astype(np.float64) for p in split(cp))
+    c2 = (c.astype(np.float32) ** 2).sum(1, dtype=np.float32).astype(np.float64)          # the packing kernel's fp32 norm
+    kept = ch @ xh.T + ch @ xm.T + cm @ xh.T
+    if packed:
+        kept = kept + cm @ xm.T
+    a = c2[:, None] + kept                                                                  # [k, n]
+    exact = (c.astype(np.float64) ** 2).sum(1)[:, None] + cp.astype(np.float64) @ x.astype(np.float64).T
+    norms = dict(x2=(x.astype(np.float32) ** 2).sum(1, dtype=np.float32), xmid2=(xm ** 2).sum(1), xrest2=(xr ** 2).sum(1),
+                 c2max=float(c2.max()), cmid2max=float((cm ** 2).sum(1).max()), crest2max=float((cr ** 2).sum(1).max()))
+    return a, exact, norms
+
+
+def serial_distances(x, c):
+    """sqrt(sum (x - c)^2) with every operation rounded to fp32 in ascending dimension (metric_policies.hpp:23-28,40-44)."""
+    n, dim = x.shape
+    out = np.zeros((c.shape[0], n), np.float32)
+    for j in range(c.shape[0]):
+        s = np.zeros(n, np.float32)
+        for q in range(dim):
+            diff = (x[:, q] - c[j, q]).astype(np.float32)
+            s = (s + (diff * diff).astype(np.float32)).astype(np.float32)
+        out[j] = np.sqrt(s, dtype=np.float32)
+    return out
+
+
+CASES = [(2, True), (3, True), (4, True), (2, False), (4, False), (8, False), (16, False), (32, False), (64, False), (256, False)]
+
+
+@pytest.mark.parametrize("dim,packed", CASES)
+@pytest.mark.parametrize("kind", ["adversarial", "pairs", "ties0", "ties100", "ties10000"])
+def test_tau_covers_the_split_and_the_serial_margin(km, dim, packed, kind):
+    rng = np.random.default_rng(dim * 31 + packed)
+    n, k = (4096, 16) if dim <= 64 else (1024, 8)
+    if kind == "adversarial":
+        x, c = adversarial(dim, n, k, rng)
+    elif kind == "pairs":
+        if dim > 64:
+            pytest.skip("the construction is used up to 64 dimensions")
+        x, c = worst_case_inputs(dim, 8192)
+        n = x.shape[0]
+    else:
+        x, c = near_ties(dim, n, k, rng, float(kind[4:]))
+    a, exact, nm = emulate(x, c, packed)
+    form = 2 if packed else 1
+    xpart = nm["xrest2"] if packed else nm["xmid2"]
+    tau = np.array([km.certificate_tau(form, dim, float(nm["x2"][i]), float(xpart[i]), nm["c2max"], nm["cmid2max"], nm["crest2max"])
+                    for i in range(n)], np.float64)
+    s_all = nm["x2"].astype(np.float64) + nm["c2max"]
+    products = 4 * dim if packed else 3 * dim
+    accumulation = (products + 2) * U * 2 * s_all          # allowance for the fp32 accumulation in the matrix core
+    margin = (2 * dim + 12) * U * s_all                    # two serial sums and the sqrt collision
+    dropped = np.abs(a - exact).max(0)
+    assert np.all(2 * dropped + 2 * accumulation + margin <= tau), \
+        "tau misses %d of %d points (worst ratio %.3f)" % (int((2 * dropped + 2 * accumulation + margin > tau).sum()), n,
+                                                          float(((2 * dropped + 2 * accumulation + margin) / tau).max()))
+    # decisions: a pair (winner j1, other j2) that could be certified under the full accumulation allowance must be a strict serial win
+    dist = serial_distances(x, c)
+    j1 = a.argmin(0)
+    certified = (a - a[j1, np.arange(n)][None, :]) + 2 * accumulation[None, :] > tau[None, :]
+    certified[j1, np.arange(n)] = False
+    wrong = certified & ~(dist[j1, np.arange(n)][None, :] < dist)
+    assert not wrong.any(), "%d certified pairs contradict the serial comparison" % int(wrong.sum())
+
+
+@pytest.mark.parametrize("dim,packed,old_units", [(2, True, 18 * 2 + 149), (8, False, 14 * 8 + 224), (16, False, 14 * 16 + 224)])
+def test_the_worst_case_inputs_defeat_a_bound_that_assumes_nine_bit_parts(dim, packed, old_units):
+    """The inputs have teeth: a bound derived from |mid| <= 2^-9 |v|, |rest| <= 2^-18 |v| (one bit too optimistic for a
+    bf16) does not cover what the split drops on them."""
+    rng = np.random.default_rng(5)
+    x, c = adversarial(dim, 8192, 16, rng)
+    a, exact, nm = emulate(x, c, packed)
+    s_all = nm["x2"].astype(np.float64) + nm["c2max"]
+    products = 4 * dim if packed else 3 * dim
+    needed = 2 * np.abs(a - exact).max(0) + 2 * (products + 2) * U * 2 * s_all + (2 * dim + 12) * U * s_all
+    assert (needed > old_units * U * s_all).any()
+
+
+def decisions(x, c, packed, tau):
+    """(points the ranking would decide, decided points whose serial result is another centroid)"""
+    a, _, _ = emulate(x, c, packed)
+    n = x.shape[0]
+    order = np.argsort(a, 0, kind="stable")
+    j1, j2 = order[0], order[1]
+    gap = a[j2, np.arange(n)] - a[j1, np.arange(n)]
+    serial = serial_distances(x, c).argmin(0)              # the first minimum: the serial scan's tie-break
+    decided = gap > tau
+    return int(decided.sum()), int((decided & (serial != j1)).sum())
+
+
+@pytest.mark.parametrize("dim,packed,old_units", [(2, True, 18 * 2 + 149), (4, True, 18 * 4 + 149), (8, False, 14 * 8 + 224),
+                                                  (16, False, 14 * 16 + 224)])
+def test_worst_case_pairs_are_decided_wrongly_by_the_nine_bit_bound_and_never_by_tau(km, dim, packed, old_units):
+    """The inputs of the GPU regression test (tests/test_gpu_certificate.py): even without any accumulation error a
+    certificate of (14 d + 224) u' S, or (18 d + 149) u' S for packed rows, decides some of them against the serial scan;
+    the library's tau decides none wrongly."""
+    x, c = worst_case_inputs(dim, 64000)
+    _, _, nm = emulate(x, c, packed)
+    s_all = nm["x2"].astype(np.float64) + nm["c2max"]
+    _, wrong_old = decisions(x, c, packed, old_units * U * s_all)
+    assert wrong_old > 0
+    xpart = nm["xrest2"] if packed else nm["xmid2"]
+    tau = np.array([km.certificate_tau(2 if packed else 1, dim, float(nm["x2"][i]), float(xpart[i]), nm["c2max"], nm["cmid2max"],
+                                       nm["crest2max"]) for i in range(x.shape[0])])
+    decided, wrong = decisions(x, c, packed, tau)
+    assert wrong == 0
+
+
+def test_fp32_form_and_argument_errors(km):
+    assert km.certificate_tau(0, 32, 3.0, 0.0, 5.0, 0.0, 0.0) == pytest.approx((8 * 32 + 24) * U * 8.0, rel=1e-6)
+    with pytest.raises(km.KmxError):
+        km.certificate_tau(7, 32, 1.0, 1.0, 1.0, 1.0, 1.0)
+    assert not np.isfinite(km.certificate_tau(1, 8, float("inf"), 1.0, 1.0, 1.0, 1.0))
+    assert np.isnan(km.certificate_tau(1, 8, float("nan"), 1.0, 1.0, 1.0, 1.0))
