@@ -34,6 +34,7 @@ ABI_SYMBOLS = [
     "kmx_assign_last_rechecked", "kmx_assign_last_variant", "kmx_update_f32", "kmx_bucket_sum_f32", "kmx_fused_f32", "kmx_assign_f64", "kmx_update_f64", "kmx_fused_f64", "kmx_bucket_sum_f64", "kmx_set_queued_rows_limit",
     "kmx_graph_begin", "kmx_graph_end", "kmx_graph_launch", "kmx_graph_destroy", "kmx_event_create", "kmx_event_destroy", "kmx_event_record",
     "kmx_event_elapsed_ms", "kmx_set_profiling", "kmx_last_kernel_ms", "kmx_last_error", "kmx_certificate_tau",
+    "kmx_update_f32_noalloc",
 ]
 
 
@@ -107,6 +108,7 @@ def hip_lib():
         lib.kmx_assign_last_variant.argtypes = [ctypes.POINTER(ctypes.c_int)]
         lib.kmx_update_f32.argtypes = [ctypes.c_int, vp, ctypes.c_int, sz, vp, vp, ctypes.c_int, sz, vp, u32, u32, u32,
                                        ctypes.POINTER(ExecParams)]
+        lib.kmx_update_f32_noalloc.argtypes = lib.kmx_update_f32.argtypes
         lib.kmx_bucket_sum_f32.argtypes = [ctypes.c_int, vp, ctypes.c_int, sz, vp, vp, ctypes.c_int, sz, u32, u32, u32,
                                            ctypes.POINTER(ExecParams)]
         lib.kmx_fused_f32.argtypes = [ctypes.c_int, vp, ctypes.c_int, sz, vp, vp, ctypes.c_int, sz, vp, u32, u32, u32,
@@ -307,6 +309,18 @@ def update(variant, data_buf, layout, stride, assignment_buf, means_buf, layout_
     fn = hip_lib().kmx_update_f64 if _is_double(dtype) else hip_lib().kmx_update_f32
     check(fn(variant, data_buf.ptr, layout, stride, assignment_buf.ptr, means_buf.ptr,
                                    layout_means, stride_means, sizes_buf.ptr, dim, k, n, ctypes.byref(ex)))
+    return ex
+
+
+NOALLOC_SCRATCH_BYTES = 64 << 20  # KMX_UPDATE_NOALLOC_SCRATCH_BYTES
+
+
+def update_noalloc(variant, data_buf, layout, stride, assignment_buf, means_buf, layout_means, stride_means, sizes_buf, dim, k,
+                   n, exec_params=None):
+    """kmx_update_f32_noalloc: kmx_update_f32 with its scratch memory in the library's static device array."""
+    ex = exec_params if exec_params is not None else ExecParams()
+    check(hip_lib().kmx_update_f32_noalloc(variant, data_buf.ptr, layout, stride, assignment_buf.ptr, means_buf.ptr,
+                                           layout_means, stride_means, sizes_buf.ptr, dim, k, n, ctypes.byref(ex)))
     return ex
 
 

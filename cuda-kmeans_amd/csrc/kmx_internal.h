@@ -28,6 +28,8 @@ hipStream_t stream();
 /* Brackets the dominant kernel of a call with events when kmx_set_profiling(1) is active (which: 0 assign, 1 update). */
 int profile_begin(int which);
 int profile_end(int which);
+/* while set, profile_begin / profile_end do nothing (they create events on first use: not for the entry point that allocates nothing) */
+void suspend_profiling(bool suspended);
 
 /* Properties of the current device, queried once. */
 struct DeviceInfo {
@@ -61,6 +63,7 @@ struct Workspace {
 	float* rows_copy = nullptr;           size_t rows_copy_cap = 0;     /* floats: AoS copy of SoA points for the tuned update */
 	float* queued_rows = nullptr;         size_t queued_rows_cap = 0;   /* floats */
 	uint32_t* queued_index = nullptr;     size_t queued_index_cap = 0;  /* words: per row 2 (queue) + 2 (assignment or 64-bit key), then the screen's pair counters and pairs */
+	bool fixed = false; /* the work space of the entry point that allocates nothing: its buffers never grow, a call that needs more is refused */
 };
 int workspace(Workspace** ws);
 int reserve_queue(Workspace* ws, size_t entries);
@@ -145,6 +148,8 @@ bool lds_fma_reads_through_scalar_cache(const AssignArgs& a); /* a handful of ce
 int launch_assign_lds_fma(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev);
 
 /* update.hip */
+/* the work space of kmx_update_f32_noalloc on the current device: `partials` is the library's static scratch array */
+int noalloc_workspace(Workspace** ws);
 int launch_update(int variant, const UpdateArgs& u, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev);
 int launch_divide_means(const UpdateArgs& u);
 

@@ -38,12 +38,14 @@ hipStream_t stream() { return g_capturing ? g_capture_stream : g_stream; }
 	} while (0)
 
 static bool g_profiling = false;
+static bool g_profiling_suspended = false;
+void suspend_profiling(bool suspended) { g_profiling_suspended = suspended; }
 static hipEvent_t g_prof[2][2] = { { nullptr, nullptr }, { nullptr, nullptr } };
 static bool g_prof_valid[2] = { false, false };
 
 int profile_begin(int which)
 {
-	if (!g_profiling || g_capturing) return KMX_OK;
+	if (!g_profiling || g_capturing || g_profiling_suspended) return KMX_OK;
 	for (int i = 0; i < 2; ++i)
 		if (!g_prof[which][i]) KMX_HIP(hipEventCreate(&g_prof[which][i]));
 	KMX_HIP(hipEventRecord(g_prof[which][0], g_stream));
@@ -52,7 +54,7 @@ int profile_begin(int which)
 
 int profile_end(int which)
 {
-	if (!g_profiling || g_capturing) return KMX_OK;
+	if (!g_profiling || g_capturing || g_profiling_suspended) return KMX_OK;
 	KMX_HIP(hipEventRecord(g_prof[which][1], g_stream));
 	g_prof_valid[which] = true;
 	return KMX_OK;
@@ -114,7 +116,15 @@ int reserve_packed(Workspace* ws, size_t packed_floats, size_t norm_floats, size
 	return grow(&ws->means_t, &ws->means_t_cap, transposed_floats);
 }
 
-int reserve_partials(Workspace* ws, size_t floats) { return grow(&ws->partials, &ws->partials_cap, floats); }
+int reserve_partials(Workspace* ws, size_t floats)
+{
+	if (ws->fixed) {
+		if (floats <= ws->partials_cap) return KMX_OK;
+		return fail(KMX_ERR_UNSUPPORTED, "the call needs %zu bytes of scratch memory for its partial sums; the entry point that allocates nothing holds %zu",
+		            floats * sizeof(float), ws->partials_cap * sizeof(float));
+	}
+	return grow(&ws->partials, &ws->partials_cap, floats);
+}
 int reserve_fused_assignment(Workspace* ws, size_t entries) { return grow(&ws->fused_assignment, &ws->fused_cap, entries); }
 int reserve_bucket_sizes(Workspace* ws, size_t entries) { return grow(&ws->bucket_sizes, &ws->bucket_cap, entries); }
 int reserve_f64(double** ptr, size_t* cap, size_t doubles) { return grow(ptr, cap, doubles); }
@@ -437,6 +447,40 @@ int kmx_update_f32(int variant,
 
 	UpdateArgs u{ data, layout, stride, assignment, means, layout_means, stride_means, cluster_sizes, dim, k, n };
 	return launch_update(variant, u, exec, ws, *dev);
+}
+
+int kmx_update_f32_noalloc(int variant,
+                           const float* data, int layout, size_t stride,
+                           const uint32_t* assignment,
+                           float* means, int layout_means, size_t stride_means,
+                           uint32_t* cluster_sizes,
+                           uint32_t dim, uint32_t k, uint32_t n, kmx_exec_params* exec)
+{
+	clear_error();
+	if (!exec) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_update_f32_noalloc: exec is null");
+	if (dim == 0 || k == 0) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_update_f32_noalloc: dim and k must be positive");
+	if (!means || !cluster_sizes) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_update_f32_noalloc: null device pointer");
+	if (n > 0 && (!data || !assignment)) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_update_f32_noalloc: null device pointer");
+	int rc = check_layout("kmx_update_f32_noalloc", "data", layout, stride, n, dim);
+	if (rc) return rc;
+	rc = check_layout("kmx_update_f32_noalloc", "means", layout_means, stride_means, k, dim);
+	if (rc) return rc;
+	rc = check_update_variant("kmx_update_f32_noalloc", variant);
+	if (rc) return rc;
+	if (exec->privatized_copies == 0) exec->privatized_copies = 1;
+
+	const DeviceInfo* dev = nullptr;
+	rc = device_info(&dev);
+	if (rc) return rc;
+	Workspace* ws = nullptr;
+	rc = noalloc_workspace(&ws); /* the static scratch array of this device; set up on the first call */
+	if (rc) return rc;
+
+	UpdateArgs u{ data, layout, stride, assignment, means, layout_means, stride_means, cluster_sizes, dim, k, n };
+	suspend_profiling(true);
+	rc = launch_update(variant, u, exec, ws, *dev);
+	suspend_profiling(false);
+	return rc;
 }
 
 int kmx_bucket_sum_f32(int variant,

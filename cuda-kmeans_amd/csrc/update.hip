@@ -866,9 +866,39 @@ rows_from_soa_kernel(const float* __restrict__ data, size_t stride, float* __res
 	}
 }
 
+/*
+ * Scratch memory of kmx_update_f32_noalloc: the per-chunk partial sums and counts of update_sorted_kernel, the only
+ * device memory beyond inputs and outputs the update uses with AoS points. One copy per GPU, held until the process
+ * ends. In host code the array's name is only a stand-in: its device address on the current device comes from
+ * hipGetSymbolAddress, once per device, and that pointer is what the kernels get.
+ */
+static __device__ __align__(256) float scratch[KMX_UPDATE_NOALLOC_SCRATCH_BYTES / sizeof(float)];
+
+constexpr int NOALLOC_MAX_DEVICES = 64;
+static Workspace g_noalloc_ws[NOALLOC_MAX_DEVICES];
+
+int noalloc_workspace(Workspace** ws)
+{
+	int device = 0;
+	KMX_HIP(hipGetDevice(&device));
+	if (device < 0 || device >= NOALLOC_MAX_DEVICES) return fail(KMX_ERR_UNSUPPORTED, "kmx_update_f32_noalloc: device %d is beyond the %d devices the library keeps scratch pointers for", device, NOALLOC_MAX_DEVICES);
+	Workspace& w = g_noalloc_ws[device];
+	if (!w.partials) {
+		float* ptr = nullptr;
+		KMX_HIP(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)));
+		if (!ptr) return fail(KMX_ERR_DEVICE, "kmx_update_f32_noalloc: the scratch array has no address on device %d", device);
+		w.partials = ptr;
+		w.partials_cap = KMX_UPDATE_NOALLOC_SCRATCH_BYTES / sizeof(float);
+		w.fixed = true;
+	}
+	*ws = &w;
+	return KMX_OK;
+}
+
 int launch_update(int variant, const UpdateArgs& u, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev)
 {
-	if (u.layout == KMX_SOA && (variant & ~KMX_UPDATE_EMULATED_ATOMICS) == KMX_UPDATE_ATOMIC_SHM && u.n > 0 && u.dim >= 8 &&
+	/* (the fixed work space has no room for a copy of the points: SoA points then stay with the element-wise kernels) */
+	if (!ws->fixed && u.layout == KMX_SOA && (variant & ~KMX_UPDATE_EMULATED_ATOMICS) == KMX_UPDATE_ATOMIC_SHM && u.n > 0 && u.dim >= 8 &&
 	    (size_t)u.n * u.dim * sizeof(float) <= ROWS_COPY_MAX_BYTES) {
 		int rc = reserve_rows_copy(ws, (size_t)u.n * u.dim);
 		if (rc) return rc;

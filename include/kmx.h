@@ -146,6 +146,26 @@ int kmx_update_f32(int variant,
                    uint32_t dim, uint32_t k, uint32_t n, kmx_exec_params* exec);
 
 /*
+ * kmx_update_f32 for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc). It has no counterpart in the reference, whose runners allocate nothing to begin
+ * with. Same arguments, variants and results as kmx_update_f32; the difference is where the scratch memory of the tuned
+ * variant (per-chunk partial sums and counts, chunks x k x (dim + 1) words) lives: in a static device array of
+ * KMX_UPDATE_NOALLOC_SCRATCH_BYTES that every GPU the library runs on holds until the process ends, instead of the
+ * work space that kmx_update_f32 grows with hipMalloc. The call allocates and frees nothing; a shape whose partial
+ * sums do not fit is refused with KMX_ERR_UNSUPPORTED (the message names both sizes). SoA points skip the AoS copy
+ * kmx_update_f32 makes of them and run the element-wise kernels (slower, same results). Per-kernel profiling
+ * (kmx_set_profiling) does not cover this call. All calls on one GPU share that GPU's array: calls that overlap in
+ * time on one GPU (different streams, different threads) race; calls on the library's one stream do not.
+ */
+#define KMX_UPDATE_NOALLOC_SCRATCH_BYTES (64u << 20)
+int kmx_update_f32_noalloc(int variant,
+                           const float* data, int layout, size_t stride,
+                           const uint32_t* assignment,
+                           float* means, int layout_means, size_t stride_means,
+                           uint32_t* cluster_sizes,
+                           uint32_t dim, uint32_t k, uint32_t n, kmx_exec_params* exec);
+
+/*
  * ---- KERNEL::run(ProblemInstance, CudaExecParameters&) of the update micro-benchmark
  *      (experimental/bucketing-cuda/bucketing-cuda/headers/kernels.cuh:7-22,44-63; called once per batch by
  *      CudaBucketingAlgorithm::run, bucketing-cuda/headers/cuda.hpp:56-63) ----
