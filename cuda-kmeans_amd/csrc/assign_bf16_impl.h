@@ -59,30 +59,44 @@ template <int KB> struct SplitPoints {
  * so a tile costs one MFMA instead of three and the mid * mid product is kept (bound at the top of assign_bf16.hip).
  * The lane holds the 8 slots of its half-wave in b.hi[0]; b.mid stays unused.
  */
+/* The coordinates a lane holds of P tiles of 32 points as they come from memory (rows beyond n read as zero): requested
+ * before a sweep and converted after it, so that the sweep hides the latency of the loads. */
+template <int KB, bool PACKED> struct RawPoints {
+	float v[PACKED ? 4 : KB * 8];
+};
+
 template <int P, int LD, bool VEC>
-__device__ __forceinline__ void load_packed_points(SplitPoints<1> (&b)[P], float (&xx)[P], const float* __restrict__ data, size_t stride,
-                                                   uint32_t base, uint32_t col, uint32_t h, uint32_t dim, uint32_t n)
+__device__ __forceinline__ void request_packed_points(RawPoints<1, true> (&raw)[P], const float* __restrict__ data, size_t stride,
+                                                      uint32_t base, uint32_t col, uint32_t dim, uint32_t n)
 {
 #pragma unroll
 	for (int p = 0; p < P; ++p) {
 		const uint32_t pt = base + p * TILE + col;
 		const bool valid = pt < n;
-		float v[4];
 		if (LD == KMX_AOS && VEC) { /* dim == 4, aligned rows */
 			f32x4 t = { 0.0f, 0.0f, 0.0f, 0.0f };
 			if (valid) t = *(const f32x4*)(data + (size_t)pt * stride);
-			v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+			raw[p].v[0] = t.x; raw[p].v[1] = t.y; raw[p].v[2] = t.z; raw[p].v[3] = t.w;
 		}
 		else {
 #pragma unroll
-			for (int j = 0; j < 4; ++j) v[j] = (valid && (uint32_t)j < dim) ? data[elem<LD>(stride, pt, j)] : 0.0f;
+			for (int j = 0; j < 4; ++j) raw[p].v[j] = (valid && (uint32_t)j < dim) ? data[elem<LD>(stride, pt, j)] : 0.0f;
 		}
+	}
+}
+
+template <int P>
+__device__ __forceinline__ void convert_packed_points(SplitPoints<1> (&b)[P], float (&xx)[P], const RawPoints<1, true> (&raw)[P], uint32_t h)
+{
+#pragma unroll
+	for (int p = 0; p < P; ++p) {
 		float part = 0.0f, rest2 = 0.0f;
 #pragma unroll
 		for (int j = 0; j < 4; ++j) {
-			part += v[j] * v[j];
+			const float v = raw[p].v[j];
+			part += v * v;
 			__bf16 hi, mid;
-			const float rest = split_bf16(v[j], hi, mid);
+			const float rest = split_bf16(v, hi, mid);
 			rest2 += rest * rest;
 			b[p].hi[0][j] = h == 0 ? mid : hi;      /* slots 0..3: x_mid,  slots 8..11: x_hi   */
 			b[p].hi[0][4 + j] = h == 0 ? hi : mid;  /* slots 4..7: x_hi,   slots 12..15: x_mid */
@@ -93,6 +107,77 @@ __device__ __forceinline__ void load_packed_points(SplitPoints<1> (&b)[P], float
 	}
 }
 
+template <int P, int LD, bool VEC>
+__device__ __forceinline__ void load_packed_points(SplitPoints<1> (&b)[P], float (&xx)[P], const float* __restrict__ data, size_t stride,
+                                                   uint32_t base, uint32_t col, uint32_t h, uint32_t dim, uint32_t n)
+{
+	RawPoints<1, true> raw[P];
+	request_packed_points<P, LD, VEC>(raw, data, stride, base, col, dim, n);
+	convert_packed_points<P>(b, xx, raw, h);
+}
+
+template <int KB, int P, int LD, bool VEC>
+__device__ __forceinline__ void request_split_points(RawPoints<KB, false> (&raw)[P], const float* __restrict__ data, size_t stride,
+                                                     uint32_t base, uint32_t col, uint32_t h, uint32_t dim, uint32_t n)
+{
+#pragma unroll
+	for (int p = 0; p < P; ++p) {
+		const uint32_t pt = base + p * TILE + col;
+		const bool valid = pt < n;
+#pragma unroll
+		for (int kb = 0; kb < KB; ++kb) {
+			const uint32_t d0 = kb * KBLOCK + h * 8;
+			float* v = raw[p].v + 8 * kb;
+			if (LD == KMX_AOS && VEC) {
+				const float* src = data + (size_t)pt * stride + d0;
+				f32x4 lo = { 0.0f, 0.0f, 0.0f, 0.0f }, up = { 0.0f, 0.0f, 0.0f, 0.0f };
+				if (valid && d0 < dim) lo = *(const f32x4*)src;
+				if (valid && d0 + 4 < dim) up = *(const f32x4*)(src + 4);
+				v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w;
+				v[4] = up.x; v[5] = up.y; v[6] = up.z; v[7] = up.w;
+			}
+			else if (LD == KMX_SOA) {
+				/* the address advances from load to load; long rows are loaded 16 coordinates at a time, so that only a few
+				 * of their 64-bit addresses are alive at once */
+				const float* src = data + (size_t)d0 * stride + pt;
+#pragma unroll
+				for (int j = 0; j < 8; ++j) {
+					v[j] = (valid && d0 + j < dim) ? *src : 0.0f;
+					src += stride;
+				}
+				if (KB > 4 && kb % 2 == 1) __builtin_amdgcn_sched_barrier(0);
+			}
+			else {
+#pragma unroll
+				for (int j = 0; j < 8; ++j) v[j] = (valid && d0 + j < dim) ? data[elem<LD>(stride, pt, d0 + j)] : 0.0f;
+			}
+		}
+	}
+}
+
+template <int KB, int P>
+__device__ __forceinline__ void convert_split_points(SplitPoints<KB> (&b)[P], float (&xx)[P], const RawPoints<KB, false> (&raw)[P])
+{
+#pragma unroll
+	for (int p = 0; p < P; ++p) {
+		float part = 0.0f;
+#pragma unroll
+		for (int kb = 0; kb < KB; ++kb) {
+#pragma unroll
+			for (int j = 0; j < 8; ++j) {
+				const float v = raw[p].v[8 * kb + j];
+				part += v * v;
+				__bf16 hi, mid;
+				split_bf16(v, hi, mid);
+				b[p].hi[kb][j] = hi;
+				b[p].mid[kb][j] = mid;
+			}
+		}
+		xx[p] = part;
+	}
+}
+
+/* request and conversion back to back, one block of 16 dimensions at a time (the rows of the widest kernels fill the registers) */
 template <int KB, int P, int LD, bool VEC>
 __device__ __forceinline__ void load_split_points(SplitPoints<KB> (&b)[P], float (&xx)[P], const float* __restrict__ data, size_t stride,
                                                   uint32_t base, uint32_t col, uint32_t h, uint32_t dim, uint32_t n)
@@ -115,8 +200,6 @@ __device__ __forceinline__ void load_split_points(SplitPoints<KB> (&b)[P], float
 				v[4] = up.x; v[5] = up.y; v[6] = up.z; v[7] = up.w;
 			}
 			else if (LD == KMX_SOA) {
-				/* the address advances from load to load; long rows are loaded 16 coordinates at a time, so that only a few
-				 * of their 64-bit addresses are alive at once */
 				const float* src = data + (size_t)d0 * stride + pt;
 #pragma unroll
 				for (int j = 0; j < 8; ++j) {
@@ -243,6 +326,124 @@ __device__ __forceinline__ float row_dot_bf16(const float* row, uint32_t h, cons
 	return part;
 }
 
+/* the same share of the dot product from the row's 16-byte pieces already in registers: piece 2 kb = hi parts, 2 kb + 1 = mid parts of block kb */
+template <int KB, bool PACKED = false>
+__device__ __forceinline__ float pieces_dot_bf16(const bf16x8 (&piece)[PACKED ? 1 : 2 * KB], const SplitPoints<KB>& x)
+{
+	float part = 0.0f;
+	if constexpr (PACKED) {
+		const bf16x8 ch = piece[0];
+		const bf16x8 xh = x.hi[0];
+		part = KMX_DOT2_PAIR(part, ch, xh, 0); part = KMX_DOT2_PAIR(part, ch, xh, 1);
+		part = KMX_DOT2_PAIR(part, ch, xh, 2); part = KMX_DOT2_PAIR(part, ch, xh, 3);
+		return part;
+	}
+	else {
+#pragma unroll
+		for (int kb = 0; kb < KB; ++kb) {
+			const bf16x8 ch = piece[2 * kb];
+			const bf16x8 cm = piece[2 * kb + 1];
+			const bf16x8 xh = x.hi[kb];
+			const bf16x8 xm = x.mid[kb];
+			part = KMX_DOT2_PAIR(part, ch, xm, 0); part = KMX_DOT2_PAIR(part, cm, xh, 0); part = KMX_DOT2_PAIR(part, ch, xh, 0);
+			part = KMX_DOT2_PAIR(part, ch, xm, 1); part = KMX_DOT2_PAIR(part, cm, xh, 1); part = KMX_DOT2_PAIR(part, ch, xh, 1);
+			part = KMX_DOT2_PAIR(part, ch, xm, 2); part = KMX_DOT2_PAIR(part, cm, xh, 2); part = KMX_DOT2_PAIR(part, ch, xh, 2);
+			part = KMX_DOT2_PAIR(part, ch, xm, 3); part = KMX_DOT2_PAIR(part, cm, xh, 3); part = KMX_DOT2_PAIR(part, ch, xh, 3);
+		}
+		return part;
+	}
+}
+
+/*
+ * The sweep with a SNAPSHOT of the leading group (rows of 17 to 64 dimensions, ten centroid tiles or more).
+ *
+ * What the counters and a few cut-down kernels showed at N = 2M, d = 32, k = 1024: VALU work next to
+ * v_mfma_f32_32x32x16_bf16 is free (a wavefront, or its partner on the SIMD, issues it while the matrix pipe works:
+ * 18 MFMAs + 48 VALU operations take the time of the 18 MFMAs); what is not free is the local data share. Recomputing the
+ * winning group of rows at the end of a sweep (the refinement of the other kernels) reads eight rows per point from
+ * per-lane addresses -- 32 conflicted 16-byte reads per point tile -- and cost 0.11 ms of a 0.36 ms sweep; and the
+ * operands of a tile, requested right before its MFMAs, cost another 0.08 ms of waiting. Hence
+ *   - tracking keeps, per lane and point tile, the 8 results of the group of rows that holds the smallest value so far
+ *     (8 conditional moves per group on top of the 8 operations of the minimum tracking): at the end of the sweep the
+ *     winner's row and the runner-up inside its group come from registers, nothing is read again;
+ *   - the centroid parts of tile t + 1 are requested before the MFMAs of tile t are issued (two register sets), and its
+ *     norms, which start the accumulators, as soon as the accumulators they go to have been tracked, a third of a step
+ *     before they are needed: no MFMA waits for the local data share;
+ *   - the tracking operations are spread between the MFMAs, a few after each.
+ */
+template <int KB> struct StepOperands {
+	bf16x8 chi[KB], cmid[KB];
+};
+
+template <int KB>
+__device__ __forceinline__ void fetch_operands(StepOperands<KB>& o, const float* __restrict__ lds_tiles, uint32_t tile, uint32_t col, uint32_t h)
+{
+	constexpr uint32_t RS = row_floats<KB, false>();
+	const float* arow = lds_tiles + (size_t)tile * tile_floats(RS) + col * RS;
+#pragma unroll
+	for (int kb = 0; kb < KB; ++kb) {
+		o.chi[kb] = row_unit(arow, 4 * kb + 2 * h);
+		o.cmid[kb] = row_unit(arow, 4 * kb + 2 * h + 1);
+	}
+}
+
+/* |c|^2 of the 16 rows of `tile` this lane receives (rows 8g + 4h + 0..3): the C operand of the tile's first MFMAs */
+__device__ __forceinline__ void fetch_norms(f32x16& c, const float* __restrict__ lds_norms, uint32_t tile, uint32_t h)
+{
+#pragma unroll
+	for (int g = 0; g < 4; ++g) {
+		const f32x4 v = *(const f32x4*)(lds_norms + tile * NORM_TILE + 8 * g + 4 * h);
+		c[4 * g] = v.x; c[4 * g + 1] = v.y; c[4 * g + 2] = v.z; c[4 * g + 3] = v.w;
+	}
+}
+
+/* The MFMAs of one centroid tile for P point tiles: per block of 16 dimensions hi*mid, mid*hi, hi*hi (small terms
+ * first). On entry acc[0] holds the tile's norms: they start every accumulator (acc[0] itself last). */
+template <int KB, int P>
+__device__ __forceinline__ void mfma_tile(f32x16 (&acc)[P], const StepOperands<KB>& o, const SplitPoints<KB> (&b)[P])
+{
+#pragma unroll
+	for (int p = P - 1; p >= 0; --p) acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(o.chi[0], b[p].mid[0], acc[0], 0, 0, 0);
+#pragma unroll
+	for (int kb = 0; kb < KB; ++kb) {
+		if (kb > 0) {
+#pragma unroll
+			for (int p = P - 1; p >= 0; --p) acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(o.chi[kb], b[p].mid[kb], acc[p], 0, 0, 0);
+		}
+#pragma unroll
+		for (int p = P - 1; p >= 0; --p) acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(o.cmid[kb], b[p].hi[kb], acc[p], 0, 0, 0);
+#pragma unroll
+		for (int p = P - 1; p >= 0; --p) acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(o.chi[kb], b[p].hi[kb], acc[p], 0, 0, 0);
+	}
+}
+
+/* Tracking with the snapshot: the minimum of the lane's 16 results of a tile (NaN-propagating tree, see track_tile), the two
+ * smallest tile minima so far (m1 <= m2), the tile that holds m1 and its 16 results. */
+constexpr int SNAP_ROWS = 16;
+__device__ __forceinline__ void track_snapshot(const f32x16& acc, Track& s, float (&snap)[SNAP_ROWS], uint32_t tile)
+{
+	auto lowest = [](float a, float b) { return __builtin_elementwise_minimum(a, b); };
+	float t = acc[0];
+#pragma unroll
+	for (int i = 1; i < 16; ++i) t = lowest(t, acc[i]);
+	s.m2 = __builtin_amdgcn_fmed3f(s.m1, s.m2, t); /* second smallest of {m1, m2, t} as m1 <= m2 */
+	const bool lt = t < s.m1;
+	s.tile = lt ? tile : s.tile;
+	s.m1 = lt ? t : s.m1;
+#pragma unroll
+	for (int i = 0; i < 16; ++i) snap[i] = lt ? acc[i] : snap[i];
+}
+
+/* which kernel instances sweep with the fenced, prefetching step (rows of 17 to 64 dimensions, ten centroid tiles or more) and
+ * which of those track with the snapshot (from 33 dimensions on: 9 MFMAs or more per point tile pay for its 32 operations, and
+ * the rows a refinement would recompute are long; at 6 MFMAs the snapshot saturates the instruction issue: 0.333 ms against
+ * the 0.30 ms of tracking group minima and refining at N = 2M, d = 32, k = 1024) */
+#ifndef KMX_SNAPSHOT_FROM_KB
+#define KMX_SNAPSHOT_FROM_KB 2
+#endif
+template <int KB, bool STREAM, bool COARSE, bool PACKED> constexpr bool pipelined_sweep() { return COARSE && !PACKED && !STREAM && KB >= 2 && KB <= 3; }
+template <int KB, bool STREAM, bool COARSE, bool PACKED> constexpr bool snapshot_sweep() { return pipelined_sweep<KB, STREAM, COARSE, PACKED>() && KB >= KMX_SNAPSHOT_FROM_KB; }
+
 template <int KB, int P, int LD, bool VEC, bool STREAM, bool COARSE, bool PREFETCH, bool PACKED = false>
 __global__ void __launch_bounds__(MFMA_WAVES * WAVE)
 assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* __restrict__ packed, const float* __restrict__ norms,
@@ -250,14 +451,16 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
                    uint32_t dim, uint32_t k, uint32_t kp, uint32_t n, uint32_t chunk_rows, float kd, float neg_inf)
 {
 	constexpr uint32_t RS = row_floats<KB, PACKED>();
-	extern __shared__ float lds[];
-	__shared__ uint32_t wave_max[3][MFMA_WAVES];
+	extern __shared__ __attribute__((aligned(16))) float lds[];
+	__shared__ uint32_t wave_max[4][MFMA_WAVES]; /* rows 0..2: maxima per wavefront; [3][0]: items of this work-group handed out so far */
 	__shared__ uint32_t flag_list[MFMA_WAVES][2 * FLAG_CAP]; /* (point, threshold) pairs */
+	uint32_t& claimed = wave_max[3][0]; /* (kept inside an array whose size is a multiple of 16 bytes: the tiles behind the static data must stay 16-byte aligned for their 128-bit reads) */
 
 	const uint32_t lane = threadIdx.x & (WAVE - 1);
 	const uint32_t wave = threadIdx.x / WAVE;
 	const uint32_t col = lane & 31; /* point within a tile (B column) / centroid row fed to A */
 	const uint32_t h = lane >> 5;   /* half-wave: K split and the +4 row group of the result    */
+	if (threadIdx.x == 0) claimed = 0u; /* (the barrier below publishes it) */
 
 	/* max_j of |c_j|^2, sum_i c'mid_i^2 and sum_i c'rest_i^2 (bit pattern maxima: they propagate NaN and +inf, which then flag every point) */
 	CertCoeffs cert;
@@ -456,8 +659,144 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 			st[p].loc = 0;
 		}
 		f32x16 acc0[P], acc1[P];
+		constexpr bool PIPE = pipelined_sweep<KB, STREAM, COARSE, PACKED>();
+		constexpr bool SNAP = snapshot_sweep<KB, STREAM, COARSE, PACKED>();
+		float snap[P][SNAP ? SNAP_ROWS : 1];
 		if constexpr (KB > 4) {
 			wide_sweep(b[0], st[0]);
+		}
+		else if constexpr (PIPE) {
+#pragma unroll
+			for (int p = 0; p < P; ++p) {
+#pragma unroll
+				for (int i = 0; i < (SNAP ? SNAP_ROWS : 1); ++i) snap[p][i] = __builtin_inff();
+			}
+			for (uint32_t chunk = 0; chunk < chunks; ++chunk) {
+				const uint32_t row0 = chunk * chunk_rows;
+				const uint32_t rows = min(chunk_rows, kp - row0);
+				const uint32_t next_row0 = chunk + 1 < chunks ? row0 + chunk_rows : 0;
+				const uint32_t next_rows = min(chunk_rows, kp - next_row0);
+				Staged incoming;
+				if (STREAM) request(incoming, next_row0, next_rows);
+				const float* lds_tiles = lds + (size_t)cur * buf_floats;
+				const float* lds_norms = lds_tiles + (size_t)chunk_tiles * tile_floats(RS);
+				const uint32_t tiles = rows / TILE;
+				const uint32_t tile0 = row0 / TILE;
+				constexpr int MFMAS = 3 * KB * P;
+				constexpr int CHUNKS = (SNAP ? 3 : 2) * P;    /* tracking comes in pieces of 8 to 12 operations: 2 per point tile, 3 with the snapshot */
+				static_assert(CHUNKS < MFMAS, "a step has more MFMAs than pieces of tracking");
+				/* One step: tile `t_new` is computed into acc_new (which holds its norms) with the centroid parts in `use`,
+				 * the centroid parts of the tile after it are requested into `fetch_into`, the tile in acc_old is tracked, and
+				 * then acc_old receives the norms of the tile that will be computed into it in the next step. The order of
+				 * the instructions is written out and fenced: the request first, then one piece of tracking behind each MFMA
+				 * (a wavefront issues them while the matrix pipe works on the MFMA), then the request for the norms, whose
+				 * answer the remaining MFMAs give time to arrive. */
+				auto step = [&](StepOperands<KB>& fetch_into, uint32_t t_new, f32x16 (&acc_new)[P], const StepOperands<KB>& use,
+				                f32x16 (&acc_old)[P], uint32_t tile_old) {
+					fetch_operands<KB>(fetch_into, lds_tiles, min(t_new + 1, tiles - 1), col, h);
+					__builtin_amdgcn_sched_barrier(0);
+					bool better[P][2];
+					int issued = 0;
+					auto after_mfma = [&](int i) {
+						__builtin_amdgcn_sched_barrier(0);
+						if (i < CHUNKS) {
+							auto lowest = [](float a, float b) { return __builtin_elementwise_minimum(a, b); };
+							if constexpr (SNAP) {
+								/* piece 0: minimum of the tile's 16 results, the two smallest tile minima so far, the tile of the smallest;
+								 * pieces 1 and 2: the 16 results replace the snapshot where the tile took the lead */
+								const int p = i / 3, part = i % 3;
+								const f32x16& a = acc_old[p];
+								if (part == 0) {
+									float t = a[0];
+#pragma unroll
+									for (int q = 1; q < 16; ++q) t = lowest(t, a[q]);
+									st[p].m2 = __builtin_amdgcn_fmed3f(st[p].m1, st[p].m2, t);
+									better[p][0] = t < st[p].m1;
+									st[p].tile = better[p][0] ? tile_old : st[p].tile;
+									st[p].m1 = better[p][0] ? t : st[p].m1;
+								}
+								else {
+#pragma unroll
+									for (int q = 8 * (part - 1); q < 8 * part; ++q) snap[p][q] = better[p][0] ? a[q] : snap[p][q];
+								}
+							}
+							else {
+								/* the minimum of a group of 8 results (NaN-propagating tree, see track_tile), the two smallest group
+								 * minima so far and the group of the smallest */
+								const int p = i / 2, g = i % 2, r = 8 * g;
+								const f32x16& a = acc_old[p];
+								const float t = lowest(lowest(lowest(lowest(lowest(lowest(lowest(a[r], a[r + 1]), a[r + 2]), a[r + 3]), a[r + 4]), a[r + 5]), a[r + 6]), a[r + 7]);
+								st[p].m2 = __builtin_amdgcn_fmed3f(st[p].m1, st[p].m2, t);
+								better[p][g] = t < st[p].m1;
+								st[p].tile = better[p][g] ? 2 * tile_old + g : st[p].tile;
+								st[p].m1 = better[p][g] ? t : st[p].m1;
+							}
+							__builtin_amdgcn_sched_barrier(0);
+						}
+						if (i == CHUNKS - 1) {
+							fetch_norms(acc_old[0], lds_norms, min(t_new + 1, tiles - 1), h);
+							__builtin_amdgcn_sched_barrier(0);
+						}
+					};
+#pragma unroll
+					for (int p = P - 1; p >= 0; --p) {
+						acc_new[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(use.chi[0], b[p].mid[0], acc_new[0], 0, 0, 0);
+						after_mfma(issued++);
+					}
+#pragma unroll
+					for (int kb = 0; kb < KB; ++kb) {
+						if (kb > 0) {
+#pragma unroll
+							for (int p = P - 1; p >= 0; --p) {
+								acc_new[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(use.chi[kb], b[p].mid[kb], acc_new[p], 0, 0, 0);
+								after_mfma(issued++);
+							}
+						}
+#pragma unroll
+						for (int p = P - 1; p >= 0; --p) {
+							acc_new[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(use.cmid[kb], b[p].hi[kb], acc_new[p], 0, 0, 0);
+							after_mfma(issued++);
+						}
+#pragma unroll
+						for (int p = P - 1; p >= 0; --p) {
+							acc_new[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(use.chi[kb], b[p].hi[kb], acc_new[p], 0, 0, 0);
+							after_mfma(issued++);
+						}
+					}
+				};
+				StepOperands<KB> o0, o1;
+				fetch_operands<KB>(o0, lds_tiles, 0, col, h);
+				fetch_norms(acc0[0], lds_norms, 0, h);
+				fetch_operands<KB>(o1, lds_tiles, min(1u, tiles - 1), col, h);
+				fetch_norms(acc1[0], lds_norms, min(1u, tiles - 1), h);
+				mfma_tile<KB, P>(acc0, o0, b);
+				uint32_t t = 0; /* acc0 holds tile t, not yet tracked; o1 and acc1[0] hold the centroid parts and norms of tile t + 1 */
+				while (t + 2 < tiles) {
+					step(o0, t + 1, acc1, o1, acc0, tile0 + t);
+					step(o1, t + 2, acc0, o0, acc1, tile0 + t + 1);
+					t += 2;
+				}
+				auto track = [&](const f32x16& acc, int p, uint32_t tile) {
+					if constexpr (SNAP) track_snapshot(acc, st[p], snap[p], tile);
+					else track_tile<true, true>(acc, st[p], tile, neg_inf);
+				};
+				if (t + 1 < tiles) {
+					mfma_tile<KB, P>(acc1, o1, b);
+#pragma unroll
+					for (int p = 0; p < P; ++p) track(acc0[p], p, tile0 + t);
+#pragma unroll
+					for (int p = 0; p < P; ++p) track(acc1[p], p, tile0 + t + 1);
+				}
+				else {
+#pragma unroll
+					for (int p = 0; p < P; ++p) track(acc0[p], p, tile0 + t);
+				}
+				if (STREAM) {
+					commit(incoming, cur ^ 1u, next_rows);
+					__syncthreads();
+					cur ^= 1u;
+				}
+			}
 		}
 		else
 		for (uint32_t chunk = 0; chunk < chunks; ++chunk) {
@@ -505,7 +844,28 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 			const bool win = st[p].m1 < o1 || (st[p].m1 == o1 && h == 0);
 			uint32_t idx;
 			float first, second;
-			if (COARSE) {
+			if constexpr (SNAP) {
+				/* the leading tile's 16 results are in registers: the winner's row and the runner-up among them; the half-wave
+				 * that holds the smaller minimum decides, everything outside its 16 rows is bounded below by W */
+				float v1 = __builtin_inff(), v2 = __builtin_inff();
+				uint32_t rbest = 0;
+#pragma unroll
+				for (int r = 0; r < SNAP_ROWS; ++r) {
+					const float v = snap[p][r];
+					v2 = __builtin_amdgcn_fmed3f(v1, v2, v);
+					const bool lt = v < v1;
+					rbest = lt ? (uint32_t)r : rbest;
+					v1 = lt ? v : v1;
+				}
+				const uint32_t mine_idx = st[p].tile * TILE + 8 * (rbest / 4) + 4 * h + (rbest % 4);
+				const uint32_t oi = (uint32_t)__shfl_xor((int)mine_idx, 32);
+				const float ov1 = __shfl_xor(v1, 32), ov2 = __shfl_xor(v2, 32);
+				const float W = win ? fminf(o1, st[p].m2) : fminf(st[p].m1, o2);
+				idx = win ? mine_idx : oi;
+				first = win ? v1 : ov1;
+				second = fminf(win ? v2 : ov2, W);
+			}
+			else if (COARSE) {
 				/* refinement of the winning group of 8 or 16 rows (see assign_mfma_impl.h); the rows are re-evaluated with
 				 * v_dot2c_f32_bf16 on the same three products, so the error bound of the MFMA results covers them */
 				constexpr bool FINE8 = fine8_bf16<KB>();
@@ -517,18 +877,35 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 				const float W = win ? fminf(o1, st[p].m2) : fminf(st[p].m1, o2);
 				const float* tile_base = STREAM ? packed + (size_t)ts * tile_floats(RS) : lds + (size_t)ts * tile_floats(RS);
 				const float* norm_base = STREAM ? norms + ts * NORM_TILE : lds + (size_t)chunk_tiles * tile_floats(RS) + ts * NORM_TILE;
+				/* all rows of the group are requested before the first one is used: one round trip to the local data share
+				 * (or to global memory) per point tile instead of one per row, which was most of the 15 000 cycles this phase
+				 * took per 96 points */
+				constexpr int UNITS = PACKED ? 1 : 2 * KB; /* 16-byte pieces of a row this half-wave multiplies */
+				constexpr int BATCH = UNITS >= 4 ? 4 : ROWS;  /* rows requested together (their pieces wait in registers) */
+				f32x4 group_norms[ROWS / 4];
+#pragma unroll
+				for (int g = 0; g < ROWS / 4; ++g) group_norms[g] = *(const f32x4*)(norm_base + 8 * (sub + g) + 4 * wh);
 				float tot[ROWS];
 #pragma unroll
-				for (int r = 0; r < ROWS; ++r)
-				{
-					const uint32_t row = 8 * (sub + r / 4) + 4 * wh + (r % 4);
-					tot[r] = row_dot_bf16<KB, PACKED>(tile_base + (PACKED ? packed_half(row, h) : row * RS), h, b[p]);
+				for (int r0 = 0; r0 < ROWS; r0 += BATCH) {
+					bf16x8 piece[BATCH][UNITS];
+#pragma unroll
+					for (int r = 0; r < BATCH; ++r) {
+						const uint32_t row = 8 * (sub + (r0 + r) / 4) + 4 * wh + ((r0 + r) % 4);
+						const float* at = tile_base + (PACKED ? packed_half(row, h) : row * RS);
+#pragma unroll
+						for (int u = 0; u < UNITS; ++u) piece[r][u] = PACKED ? *(const bf16x8*)at : row_unit(at, 4 * (u / 2) + 2 * h + (u % 2));
+					}
+					__builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+					for (int r = 0; r < BATCH; ++r) tot[r0 + r] = pieces_dot_bf16<KB, PACKED>(piece[r], b[p]);
+					__builtin_amdgcn_sched_barrier(0);
 				}
 				float v1 = __builtin_inff(), v2 = __builtin_inff();
 				uint32_t rbest = 0;
 #pragma unroll
 				for (int g = 0; g < ROWS / 4; ++g) {
-					const f32x4 c2 = *(const f32x4*)(norm_base + 8 * (sub + g) + 4 * wh);
+					const f32x4 c2 = group_norms[g];
 #pragma unroll
 					for (int q = 0; q < 4; ++q) {
 						const int r = 4 * g + q;
@@ -594,29 +971,69 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 		else load_split_points<KB, P, LD, VEC>(bb, xs, data, stride, first, col, h, dim, n);
 	};
 
+	/*
+	 * A work-group takes the units blockIdx.x, blockIdx.x + gridDim.x, ... (8 items of P tiles of 32 points each). With
+	 * resident centroids its wavefronts take those items one at a time from a counter in LDS instead of a fixed eighth
+	 * each: the matrix pipe of a SIMD serves its older wavefront first, so with equal shares the first four wavefronts of a
+	 * work-group were done after 70 % of the kernel's time and the other four swept the rest alone (measured with the
+	 * cycle counter: 440 k against 632 k cycles). (One global counter for all wavefronts was worse than either: 32768
+	 * returning atomics on one address take 14 ns each, longer than the whole sweep.) The next item is claimed, and its
+	 * points requested, before the current one is swept. Streamed centroids keep equal shares: every wavefront of the
+	 * work-group has to arrive at the barrier of every chunk, so all of them sweep the same number of times.
+	 */
+	const uint32_t my_units = blockIdx.x < units ? (units - blockIdx.x + gridDim.x - 1) / gridDim.x : 0u;
+	const uint32_t items = STREAM ? my_units : my_units * MFMA_WAVES;
+	uint32_t static_item = 0;
+	auto claim = [&]() -> uint32_t {
+		if (STREAM) return static_item++;
+		uint32_t item = 0;
+		if (lane == 0) item = atomicAdd(&claimed, 1u);
+		return item; /* lane 0's value; made uniform by the caller when it is needed */
+	};
+	auto uniform = [&](uint32_t v) -> uint32_t { return STREAM ? v : (uint32_t)__builtin_amdgcn_readfirstlane((int)v); };
+	/* first point of an item: unit blockIdx.x + (item / 8) gridDim.x, slice item % 8 (streamed: the wavefront's own slice of unit `item`) */
+	auto first_point = [&](uint32_t item) -> uint32_t {
+		const uint32_t unit = blockIdx.x + (STREAM ? item : item / MFMA_WAVES) * gridDim.x;
+		const uint32_t slice = STREAM ? wave : item % MFMA_WAVES;
+		return (unit * MFMA_WAVES + slice) * P * TILE;
+	};
 	if (PREFETCH) {
-		SplitPoints<KB> b0[P], b1[P];
-		float xx0[P], xx1[P];
-		uint32_t unit = blockIdx.x;
-		if (unit < units) load_points(b0, xx0, (unit * MFMA_WAVES + wave) * P * TILE);
-		while (unit < units) {
-			uint32_t next = unit + gridDim.x;
-			if (next < units) load_points(b1, xx1, (next * MFMA_WAVES + wave) * P * TILE);
-			sweep(b0, xx0, (unit * MFMA_WAVES + wave) * P * TILE);
-			unit = next;
-			if (unit >= units) break;
-			next = unit + gridDim.x;
-			if (next < units) load_points(b0, xx0, (next * MFMA_WAVES + wave) * P * TILE);
-			sweep(b1, xx1, (unit * MFMA_WAVES + wave) * P * TILE);
-			unit = next;
+		/* one set of split operands; the raw coordinates of the next item travel while the current one is swept */
+		RawPoints<KB, PACKED> raw[P];
+		SplitPoints<KB> b0[P];
+		float xx0[P];
+		auto request_points = [&](uint32_t first) {
+			if constexpr (PACKED) request_packed_points<P, LD, VEC>(raw, data, stride, first, col, dim, n);
+			else request_split_points<KB, P, LD, VEC>(raw, data, stride, first, col, h, dim, n);
+		};
+		auto convert_points = [&]() {
+			if constexpr (PACKED) convert_packed_points<P>(b0, xx0, raw, h);
+			else convert_split_points<KB, P>(b0, xx0, raw);
+		};
+		uint32_t item = uniform(claim());
+		uint32_t next = uniform(claim());
+		if (item < items) {
+			request_points(first_point(item));
+			convert_points();
+		}
+		while (item < items) {
+			const uint32_t after = claim();
+			if (next < items) request_points(first_point(next));
+			sweep(b0, xx0, first_point(item));
+			item = next;
+			next = uniform(after);
+			if (item < items) convert_points();
 		}
 	}
 	else {
 		SplitPoints<KB> b0[P];
 		float xx0[P];
-		for (uint32_t unit = blockIdx.x; unit < units; unit += gridDim.x) {
-			load_points(b0, xx0, (unit * MFMA_WAVES + wave) * P * TILE);
-			sweep(b0, xx0, (unit * MFMA_WAVES + wave) * P * TILE);
+		uint32_t item = uniform(claim());
+		while (item < items) {
+			const uint32_t after = claim();
+			load_points(b0, xx0, first_point(item));
+			sweep(b0, xx0, first_point(item));
+			item = uniform(after);
 		}
 	}
 	if (flagged) flush_flags();
@@ -843,7 +1260,7 @@ static int launch_bf16_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 	/* resident centroids and rows of 17 to 32 dimensions: a third point tile fits the registers (255, no spills; the
 	 * streamed kernel would spill) and the LDS reads of a step serve 18 MFMAs instead of 12: 0.348 against 0.356 ms at
 	 * N = 2M, d = 32, k = 1024 */
-	constexpr int PR = (!PACKED && KB == 2) ? 3 : P;
+	constexpr int PR = (!PACKED && KB == 2 && KMX_SNAPSHOT_FROM_KB > 2) ? 3 : P; /* a third point tile fits where the tracking keeps no snapshot */
 	constexpr bool PF = SplitSweepShape<KB>::PREFETCH;
 	uint32_t budget = exec->shared_mem_bytes ? std::min(exec->shared_mem_bytes, dev.lds_bytes) : dev.lds_bytes;
 	const uint32_t static_bytes = (2 * FLAG_CAP * MFMA_WAVES + 64) * 4;
