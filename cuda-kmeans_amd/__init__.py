@@ -23,6 +23,7 @@ AOS, SOA = 0, 1
 ASSIGN_BASE, ASSIGN_LDS_FMA, ASSIGN_MFMA, ASSIGN_BEST, ASSIGN_MFMA_BF16X3 = 0, 1, 2, 3, 4
 FUSED_TWO_PASS, FUSED_ONE_PASS, FUSED_BEST = 0, 1, 2
 UPDATE_ATOMIC_POINT, UPDATE_ATOMIC_FINE, UPDATE_ATOMIC_SHM, UPDATE_BASE, UPDATE_ATOMIC_WARP = 0, 1, 2, 3, 4
+UPDATE_ATOMIC_SHM2, UPDATE_FAKE, UPDATE_FAKE_SHM = 5, 6, 7  # the remaining kernels of the update micro-benchmark
 UPDATE_EMULATED_ATOMICS = 0x100  # flag for the point, fine and wavefront variants: compare-and-swap loops
 
 KMX_OK, KMX_ERR_INVALID_ARGUMENT, KMX_ERR_UNSUPPORTED, KMX_ERR_DEVICE, KMX_ERR_NO_DEVICE = 0, 1, 2, 3, 4

@@ -349,12 +349,15 @@ int kmx_fill_zero_u32(void* dptr, size_t count)
 }
 
 
-static int check_update_variant(const char* who, int variant)
+static int check_update_variant(const char* who, int variant, bool bucket_sum)
 {
 	const int base = variant & ~KMX_UPDATE_EMULATED_ATOMICS;
-	if (base < KMX_UPDATE_ATOMIC_POINT || base > KMX_UPDATE_ATOMIC_WARP) return fail(KMX_ERR_INVALID_ARGUMENT, "%s: unknown variant %d", who, variant);
-	if ((variant & KMX_UPDATE_EMULATED_ATOMICS) && (base == KMX_UPDATE_ATOMIC_SHM || base == KMX_UPDATE_BASE))
-		return fail(KMX_ERR_UNSUPPORTED, "%s: emulated atomics exist for the point, fine and wavefront variants only", who);
+	if (base < KMX_UPDATE_ATOMIC_POINT || base > KMX_UPDATE_FAKE_SHM) return fail(KMX_ERR_INVALID_ARGUMENT, "%s: unknown variant %d", who, variant);
+	if ((base == KMX_UPDATE_FAKE || base == KMX_UPDATE_FAKE_SHM) && !bucket_sum)
+		return fail(KMX_ERR_INVALID_ARGUMENT, "%s: variant %d ignores its inputs; it exists for kmx_bucket_sum_f32 only", who, variant);
+	if ((variant & KMX_UPDATE_EMULATED_ATOMICS) &&
+	    (base == KMX_UPDATE_ATOMIC_SHM || base == KMX_UPDATE_BASE || base == KMX_UPDATE_ATOMIC_SHM2 || base == KMX_UPDATE_FAKE_SHM))
+		return fail(KMX_ERR_UNSUPPORTED, "%s: emulated atomics exist for the point, fine, wavefront and fake variants only", who);
 	return KMX_OK;
 }
 
@@ -434,7 +437,7 @@ int kmx_update_f32(int variant,
 	if (rc) return rc;
 	rc = check_layout("kmx_update_f32", "means", layout_means, stride_means, k, dim);
 	if (rc) return rc;
-	rc = check_update_variant("kmx_update_f32", variant);
+	rc = check_update_variant("kmx_update_f32", variant, false);
 	if (rc) return rc;
 	if (exec->privatized_copies == 0) exec->privatized_copies = 1;
 
@@ -465,7 +468,7 @@ int kmx_update_f32_noalloc(int variant,
 	if (rc) return rc;
 	rc = check_layout("kmx_update_f32_noalloc", "means", layout_means, stride_means, k, dim);
 	if (rc) return rc;
-	rc = check_update_variant("kmx_update_f32_noalloc", variant);
+	rc = check_update_variant("kmx_update_f32_noalloc", variant, false);
 	if (rc) return rc;
 	if (exec->privatized_copies == 0) exec->privatized_copies = 1;
 
@@ -498,7 +501,7 @@ int kmx_bucket_sum_f32(int variant,
 	if (rc) return rc;
 	rc = check_layout("kmx_bucket_sum_f32", "result", layout_result, stride_result, k, dim);
 	if (rc) return rc;
-	rc = check_update_variant("kmx_bucket_sum_f32", variant);
+	rc = check_update_variant("kmx_bucket_sum_f32", variant, true);
 	if (rc) return rc;
 	if (exec->privatized_copies == 0) exec->privatized_copies = 1;
 

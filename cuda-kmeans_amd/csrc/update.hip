@@ -138,6 +138,88 @@ update_fine_kernel(const float* __restrict__ data, size_t stride, const uint32_t
 }
 
 /*
+ * atomicShm2Kernel of the update micro-benchmark (reference bucketing-cuda/kernels/kernels.cu:381-426): one lane per
+ * input element, the WHOLE k x dim block cached in LDS in `lds_copies` private copies (lane t adds to copy t % lds_copies),
+ * floating-point LDS atomics; at the end the copies of every element are summed and added to the result with one global
+ * atomic per element and work-group. (The reference sums resultCache[i + copy * dim] at :423-426, which is not where
+ * copy `copy` of element i was accumulated, (target * copies + copy) * dim + d, unless there is a single copy; here the
+ * copies of the element itself are summed.)
+ */
+template <int LD, int LM>
+__global__ void __launch_bounds__(1024)
+update_shm2_kernel(const float* __restrict__ data, size_t stride, const uint32_t* __restrict__ assignment,
+                   float* __restrict__ means, size_t stride_means, uint32_t* __restrict__ sizes,
+                   uint32_t dim, uint32_t k, uint32_t n, size_t copy_floats, uint32_t copies, uint32_t lds_copies)
+{
+	extern __shared__ float cache[];
+	const uint32_t cache_floats = k * dim * lds_copies;
+	for (uint32_t i = threadIdx.x; i < cache_floats; i += blockDim.x) cache[i] = 0.0f;
+	__syncthreads();
+	means = privatized<LM>(means, copy_floats, copies);
+	const size_t threads = (size_t)blockDim.x * gridDim.x;
+	const size_t size = (size_t)n * dim;
+	const uint32_t mine = threadIdx.x % lds_copies;
+	for (size_t i = threadIdx.x + (size_t)blockIdx.x * blockDim.x; i < size; i += threads) {
+		const uint32_t d = (uint32_t)(i % dim);
+		const uint32_t idx = (uint32_t)(i / dim);
+		const uint32_t target = assignment[idx];
+		atomic_add_f32(&cache[((size_t)target * lds_copies + mine) * dim + d], data[elem<LD>(stride, idx, d)]);
+		if (d == 0) atomicAdd(&sizes[target], 1u);
+	}
+	__syncthreads();
+	for (uint32_t i = threadIdx.x; i < k * dim; i += blockDim.x) {
+		const uint32_t c = i / dim, d = i % dim;
+		float sum = 0.0f;
+		for (uint32_t copy = 0; copy < lds_copies; ++copy) sum += cache[((size_t)c * lds_copies + copy) * dim + d];
+		atomic_add_f32(&means[elem<LM>(stride_means, c, d)], sum);
+	}
+}
+
+/*
+ * atomicFakeKernel / atomicShmFakeKernel of the update micro-benchmark (reference bucketing-cuda/kernels/kernels.cu:452-469,
+ * 495-531): probes of the raw cost of the atomic additions. One lane per input element, the inputs are ignored: element i
+ * adds the constant 0.1 to dimension i % dim of bucket (i / dim) % k with a real atomic, in global memory or, for the
+ * first `cached` buckets, in LDS (flushed with one global atomic per element and work-group). The result has a closed
+ * form: 0.1 * #{point numbers congruent to the bucket modulo k}.
+ */
+template <int LM, bool EMUL>
+__global__ void __launch_bounds__(1024)
+update_fake_kernel(float* __restrict__ means, size_t stride_means, uint32_t dim, uint32_t k, uint32_t n, size_t copy_floats, uint32_t copies)
+{
+	means = privatized<LM>(means, copy_floats, copies);
+	const size_t threads = (size_t)blockDim.x * gridDim.x;
+	const size_t size = (size_t)n * dim;
+	for (size_t i = threadIdx.x + (size_t)blockIdx.x * blockDim.x; i < size; i += threads) {
+		const uint32_t d = (uint32_t)(i % dim);
+		const uint32_t target = (uint32_t)((i / dim) % k);
+		atomic_add_global<EMUL>(&means[elem<LM>(stride_means, target, d)], 0.1f);
+	}
+}
+
+template <int LM>
+__global__ void __launch_bounds__(1024)
+update_fake_shm_kernel(float* __restrict__ means, size_t stride_means, uint32_t dim, uint32_t k, uint32_t n, size_t copy_floats, uint32_t copies,
+                       uint32_t cached)
+{
+	extern __shared__ float cache[];
+	const uint32_t cache_floats = cached * dim;
+	for (uint32_t i = threadIdx.x; i < cache_floats; i += blockDim.x) cache[i] = 0.0f;
+	__syncthreads();
+	means = privatized<LM>(means, copy_floats, copies);
+	const size_t threads = (size_t)blockDim.x * gridDim.x;
+	const size_t size = (size_t)n * dim;
+	for (size_t i = threadIdx.x + (size_t)blockIdx.x * blockDim.x; i < size; i += threads) {
+		const uint32_t d = (uint32_t)(i % dim);
+		const uint32_t target = (uint32_t)((i / dim) % k);
+		if (target < cached) atomic_add_f32(&cache[(size_t)target * dim + d], 0.1f);
+		else atomic_add_f32(&means[elem<LM>(stride_means, target, d)], 0.1f);
+	}
+	__syncthreads();
+	for (uint32_t i = threadIdx.x; i < cache_floats; i += blockDim.x)
+		atomic_add_f32(&means[elem<LM>(stride_means, i / dim, i % dim)], cache[i]);
+}
+
+/*
  * LDS-privatised update. Grid = (point chunks, dimension slices).
  * LDS: replicas x k x row floats of partial sums (row = slice width, +1 padding for SoA input so that
  * lanes holding different points of one dimension spread over the banks), then replicas x k counts.
@@ -795,6 +877,39 @@ static int launch_update_t(int variant, const UpdateArgs& u, kmx_exec_params* ex
 			size_t blocks = (threads + block - 1) / block;
 			exec->block_count = (uint32_t)std::min<size_t>(blocks, 1u << 20);
 			KMX_UPDATE_LAUNCH(update_fine_kernel, "update_fine_kernel");
+		}
+		else if (variant == KMX_UPDATE_ATOMIC_SHM2 || variant == KMX_UPDATE_FAKE || variant == KMX_UPDATE_FAKE_SHM) {
+			/* the micro-benchmark's launch shape: one lane per input element (or per items_per_thread elements) */
+			const size_t threads = ((size_t)u.n * u.dim + ipt - 1) / ipt;
+			exec->block_count = (uint32_t)std::min<size_t>((threads + block - 1) / block, 1u << 20);
+			const uint32_t budget = exec->shared_mem_bytes ? std::min(exec->shared_mem_bytes, dev.lds_bytes) : dev.lds_bytes;
+			if (variant == KMX_UPDATE_ATOMIC_SHM2) {
+				const size_t one_copy = (size_t)u.k * u.dim * sizeof(float);
+				const uint32_t lds_copies = (uint32_t)std::min<size_t>(budget / one_copy, block);
+				if (lds_copies < 1) return fail(KMX_ERR_UNSUPPORTED, "Insufficient shared memory size for given parameters.");
+				const uint32_t lds_bytes = (uint32_t)(lds_copies * one_copy);
+				auto kernel = update_shm2_kernel<LD, LM>;
+				KMX_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+				hipLaunchKernelGGL(kernel, dim3(exec->block_count), dim3(block), lds_bytes, stream(), u.data, u.stride, u.assignment,
+				                   u.means, u.stride_means, u.cluster_sizes, u.dim, u.k, u.n, copy_floats, copies, lds_copies);
+				KMX_LAUNCH_CHECK("update_shm2_kernel");
+			}
+			else if (variant == KMX_UPDATE_FAKE) {
+				if (emulated) hipLaunchKernelGGL((update_fake_kernel<LM, true>), dim3(exec->block_count), dim3(block), 0, stream(),
+				                                 u.means, u.stride_means, u.dim, u.k, u.n, copy_floats, copies);
+				else hipLaunchKernelGGL((update_fake_kernel<LM, false>), dim3(exec->block_count), dim3(block), 0, stream(),
+				                        u.means, u.stride_means, u.dim, u.k, u.n, copy_floats, copies);
+				KMX_LAUNCH_CHECK("update_fake_kernel");
+			}
+			else {
+				const uint32_t cached = (uint32_t)std::min<size_t>(budget / (u.dim * sizeof(float)), u.k);
+				const uint32_t lds_bytes = cached * u.dim * (uint32_t)sizeof(float);
+				auto kernel = update_fake_shm_kernel<LM>;
+				KMX_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+				hipLaunchKernelGGL(kernel, dim3(exec->block_count), dim3(block), lds_bytes, stream(),
+				                   u.means, u.stride_means, u.dim, u.k, u.n, copy_floats, copies, cached);
+				KMX_LAUNCH_CHECK("update_fake_shm_kernel");
+			}
 		}
 		else if (variant == KMX_UPDATE_BASE) {
 			exec->block_count = (u.k * u.dim + 255) / 256;

@@ -142,7 +142,10 @@ KMX_DEFINE_BUCKETING_KERNEL(BaseKernel, KMX_UPDATE_BASE, false)                /
 KMX_DEFINE_BUCKETING_KERNEL(AtomicPointKernel, KMX_UPDATE_ATOMIC_POINT, true)  /* :195-226 atomic_point */
 KMX_DEFINE_BUCKETING_KERNEL(AtomicWarpKernel, KMX_UPDATE_ATOMIC_WARP, true)    /* :234-266 atomic_warp, with 64-lane wavefronts */
 KMX_DEFINE_BUCKETING_KERNEL(AtomicFineKernel, KMX_UPDATE_ATOMIC_FINE, true)    /* :275-307 atomic_fine */
-KMX_DEFINE_BUCKETING_KERNEL(AtomicShmKernel, KMX_UPDATE_ATOMIC_SHM, false)     /* :317-372 atomic_shm (and the role of atomic_shm2, :381-447): here the tuned LDS kernels */
+KMX_DEFINE_BUCKETING_KERNEL(AtomicShmKernel, KMX_UPDATE_ATOMIC_SHM, false)     /* :317-372 atomic_shm: here the tuned LDS kernels */
+KMX_DEFINE_BUCKETING_KERNEL(AtomicShm2Kernel, KMX_UPDATE_ATOMIC_SHM2, false)   /* :381-447 atomic_shm2: the whole block in LDS, sharedMemorySize / (k dim sizeof F) private copies */
+KMX_DEFINE_BUCKETING_KERNEL(AtomicFakeKernel, KMX_UPDATE_FAKE, true)           /* :452-486 fake: constant 0.1 added atomically to bucket (i / dim) % k */
+KMX_DEFINE_BUCKETING_KERNEL(AtomicShmFakeKernel, KMX_UPDATE_FAKE_SHM, false)   /* :495-550 fake_shm: the same with the first buckets cached in LDS */
 
 /* = CudaBucketingAlgorithm (bucketing-cuda/headers/cuda.hpp:13-86): one buffer set per batch, one kernel call per batch */
 template<typename F = float, class LAYOUT = AoSLayoutPolicy<>, class KERNEL = AtomicShmKernel<F, LAYOUT>>

@@ -5,10 +5,11 @@
  * relative tolerance of 5e-5 :104-142). Inputs: data uniform in [0,1), indices uniform in [0,k), from mt19937(seed)
  * as in the reference (:177-178).
  *
- * Algorithms: serial, hip_base, hip_atomic_point, hip_atomic_warp, hip_atomic_fine, hip_atomic_shm (the reference's
- * cuda_* names are accepted; cuda_atomic_shm2 runs the same tuned LDS kernels as cuda_atomic_shm), --emul.
- * Not built: the two "fake" kernels (non-atomic additions that race on purpose: their results are wrong by design
- * and cannot be verified). --double: the serial algorithm and the atomic point, fine and shm kernels.
+ * Algorithms: serial, hip_base, hip_atomic_point, hip_atomic_warp, hip_atomic_fine, hip_atomic_shm, hip_atomic_shm2,
+ * hip_fake, hip_fake_shm (the reference's cuda_* names are accepted), --emul. The two "fake" algorithms are probes of the
+ * raw cost of atomic additions (bucketing-cuda/kernels/kernels.cu:452-531): they ignore the inputs and add the constant
+ * 0.1 to bucket (i / dim) % k, so --verify checks them against that closed form instead of the serial sums.
+ * --double: the serial algorithm and the atomic point, fine and shm kernels.
  */
 #include "bucketing.hpp"
 #include "cli_args.hpp"
@@ -47,8 +48,8 @@ std::string canonicalAlgorithm(const std::string& name)
 {
 	static const std::map<std::string, std::string> aliases = {
 		{ "cuda_base", "hip_base" }, { "cuda_atomic_point", "hip_atomic_point" }, { "cuda_atomic_warp", "hip_atomic_warp" },
-		{ "cuda_atomic_fine", "hip_atomic_fine" }, { "cuda_atomic_shm", "hip_atomic_shm" }, { "cuda_atomic_shm2", "hip_atomic_shm" },
-		{ "hip_atomic_shm2", "hip_atomic_shm" },
+		{ "cuda_atomic_fine", "hip_atomic_fine" }, { "cuda_atomic_shm", "hip_atomic_shm" }, { "cuda_atomic_shm2", "hip_atomic_shm2" },
+		{ "cuda_fake", "hip_fake" }, { "cuda_fake_shm", "hip_fake_shm" },
 	};
 	auto it = aliases.find(name);
 	return it == aliases.end() ? name : it->second;
@@ -111,8 +112,7 @@ void run(const ProgramArguments& args)
 	generate_random(indices, std::uniform_int_distribution<std::uint32_t>(0, (std::uint32_t)k - 1), seed);
 
 	const std::string algoName = canonicalAlgorithm(args.getString("algorithm"));
-	if (algoName == "cuda_fake" || algoName == "cuda_fake_shm" || algoName == "hip_fake" || algoName == "hip_fake_shm")
-		throw std::runtime_error("The 'fake' kernels (non-atomic additions that race on purpose) are not built.");
+	const bool fake = algoName == "hip_fake" || algoName == "hip_fake_shm";
 	HipExecParameters exec;
 	getHipExecParameters(args, exec);
 	std::map<std::string, std::unique_ptr<IBucketingAlgorithm<F>>> algorithms;
@@ -123,13 +123,17 @@ void run(const ProgramArguments& args)
 		algorithms["hip_atomic_warp"].reset(new HipBucketingAlgorithm<F, LAYOUT, AtomicWarpKernel<F, LAYOUT, true>>(exec));
 		algorithms["hip_atomic_fine"].reset(new HipBucketingAlgorithm<F, LAYOUT, AtomicFineKernel<F, LAYOUT, true>>(exec));
 		algorithms["hip_atomic_shm"].reset(new HipBucketingAlgorithm<F, LAYOUT, AtomicShmKernel<F, LAYOUT, true>>(exec));
+		algorithms["hip_fake"].reset(new HipBucketingAlgorithm<F, LAYOUT, AtomicFakeKernel<F, LAYOUT, true>>(exec));
 	}
 	else {
 		algorithms["hip_atomic_point"].reset(new HipBucketingAlgorithm<F, LAYOUT, AtomicPointKernel<F, LAYOUT>>(exec));
 		algorithms["hip_atomic_warp"].reset(new HipBucketingAlgorithm<F, LAYOUT, AtomicWarpKernel<F, LAYOUT>>(exec));
 		algorithms["hip_atomic_fine"].reset(new HipBucketingAlgorithm<F, LAYOUT, AtomicFineKernel<F, LAYOUT>>(exec));
 		algorithms["hip_atomic_shm"].reset(new HipBucketingAlgorithm<F, LAYOUT, AtomicShmKernel<F, LAYOUT>>(exec));
+		algorithms["hip_fake"].reset(new HipBucketingAlgorithm<F, LAYOUT, AtomicFakeKernel<F, LAYOUT>>(exec));
 	}
+	algorithms["hip_atomic_shm2"].reset(new HipBucketingAlgorithm<F, LAYOUT, AtomicShm2Kernel<F, LAYOUT>>(exec));
+	algorithms["hip_fake_shm"].reset(new HipBucketingAlgorithm<F, LAYOUT, AtomicShmFakeKernel<F, LAYOUT>>(exec));
 	auto it = algorithms.find(algoName);
 	if (it == algorithms.end()) throw std::runtime_error("Unkown algorithm '" + algoName + "'.");
 	std::cerr << "Selected algorithm: " << algoName << std::endl;
@@ -154,10 +158,21 @@ void run(const ProgramArguments& args)
 
 	if (args.getBool("verify")) {
 		std::cerr << "Verifying results ... "; std::cerr.flush();
-		SerialBucketingAlgorithm<F, LAYOUT> base;
-		base.initialize(dim, k, n, iter, data, indices);
-		base.run();
-		std::cerr << (verify(algorithm->getResult(), base.getResult(), dim, k) ? "OK" : "FAILED") << std::endl;
+		if (fake) {
+			/* what the probes add up to: 0.1 per point whose number is congruent to the bucket modulo k, in every dimension */
+			std::vector<F> expected(iter * k * dim); /* getResult() is iterations x k rows of dim sums, whatever the layout */
+			for (std::size_t i = 0; i < expected.size(); ++i) {
+				const std::size_t b = (i / dim) % k;
+				expected[i] = (F)(0.1 * (double)(n / k + (b < n % k ? 1 : 0)));
+			}
+			std::cerr << (verify(algorithm->getResult(), expected, dim, k) ? "OK" : "FAILED") << std::endl;
+		}
+		else {
+			SerialBucketingAlgorithm<F, LAYOUT> base;
+			base.initialize(dim, k, n, iter, data, indices);
+			base.run();
+			std::cerr << (verify(algorithm->getResult(), base.getResult(), dim, k) ? "OK" : "FAILED") << std::endl;
+		}
 	}
 	if (args.isPresent("out")) {
 		std::cerr << "Saving results to " << args.getString("out") << " ..." << std::endl;
@@ -189,8 +204,8 @@ int main(int argc, char* argv[])
 		args.registerInt("N", "Number of vectors in a batch.", 10240, 128);
 		args.registerInt("iterations", "Iterations to be performed (i.e., number of batches).", 1, 1);
 		args.registerInt("seed", "Random generator seed.", 42, 0);
-		args.registerString("algorithm", "Which algorithm is to be tested (serial, hip_base, hip_atomic_point, hip_atomic_warp, hip_atomic_fine, hip_atomic_shm).", "serial");
-		args.registerBool("emul", "Emulate atomic additions with atomic CAS operations (point, warp and fine algorithms).");
+		args.registerString("algorithm", "Which algorithm is to be tested (serial, hip_base, hip_atomic_point, hip_atomic_warp, hip_atomic_fine, hip_atomic_shm, hip_atomic_shm2, hip_fake, hip_fake_shm).", "serial");
+		args.registerBool("emul", "Emulate atomic additions with atomic CAS operations (point, warp, fine and fake algorithms).");
 		args.registerEnum("layout", "Type of data layout and alignment.", "aos", { "aos", "soa", "aos32", "soa32" });
 		args.registerBool("double", "Use doubles instead of floats (serial, hip_atomic_point, hip_atomic_fine, hip_atomic_shm).");
 		args.registerBool("verify", "Verify results against base (serial) algorithm.");

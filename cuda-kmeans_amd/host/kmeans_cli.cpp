@@ -56,6 +56,7 @@ std::string canonicalAlgorithm(const std::string& name)
 	static const std::map<std::string, std::string> aliases = {
 		{ "cuda_base", "hip_base" }, { "cuda_base_shm", "hip_base_shm" }, { "cuda_best", "hip_best" },
 		{ "cuda_cached_fixed", "hip_lds_fma" }, { "cuda_cached_regs", "hip_mfma" },
+		{ "cuda_cached_means", "hip_lds_fma" }, /* CachedAllMeansAssignmentKernel (k-means.cpp:72, kernels.cu:328-410): all centroids in LDS, which is what the LDS/FMA variant does */
 		{ "cuda_fused_fixed", "hip_fused" }, { "cuda_fused_regs", "hip_fused" },
 	};
 	auto it = aliases.find(name);

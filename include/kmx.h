@@ -73,7 +73,14 @@ typedef enum kmx_update_variant {
 	KMX_UPDATE_BASE = 3,         /* BaseKernel: no atomics, one lane per element of the result walks all points (sums in
 	                                point order, i.e. with the bits of the serial loop); O(n k dim), for small inputs */
 	KMX_UPDATE_ATOMIC_WARP = 4,  /* AtomicWarpKernel: one wavefront per point, lanes stride over the dimensions */
-	/* flag, or-ed to ATOMIC_POINT / ATOMIC_FINE / ATOMIC_WARP: additions as compare-and-swap loops instead of the hardware
+	KMX_UPDATE_ATOMIC_SHM2 = 5,  /* AtomicShm2Kernel (bucketing-cuda/kernels/kernels.cu:381-447): the whole k x dim block in LDS, in
+	                                shared_mem_bytes / (k dim 4) private copies (lane t uses copy t mod copies), LDS atomics;
+	                                KMX_ERR_UNSUPPORTED "Insufficient shared memory size ..." if not even one copy fits */
+	/* kmx_bucket_sum_f32 only: probes of the raw cost of atomic additions, inputs ignored (kernels.cu:452-541). Element i adds
+	 * 0.1 to dimension i mod dim of bucket (i / dim) mod k, so result[b][d] = 0.1 * #{points congruent to b modulo k} */
+	KMX_UPDATE_FAKE = 6,         /* AtomicFakeKernel: global atomics (may be or-ed with KMX_UPDATE_EMULATED_ATOMICS) */
+	KMX_UPDATE_FAKE_SHM = 7,     /* AtomicShmFakeKernel: the first shared_mem_bytes / (dim 4) buckets cached in LDS */
+	/* flag, or-ed to ATOMIC_POINT / ATOMIC_FINE / ATOMIC_WARP / FAKE: additions as compare-and-swap loops instead of the hardware
 	 * atomic (the micro-benchmark's --emul, AtomicEmulTrait, bucketing-cuda/kernels/kernels.cu:83-91) */
 	KMX_UPDATE_EMULATED_ATOMICS = 0x100
 } kmx_update_variant;

@@ -56,8 +56,8 @@ def test_errors(harness):
     assert rc == 2 and "Error: Unkown algorithm 'nope'." in out
     rc, out, err = run(harness, "--double", "--N", "1k", "--k", "8", "--dim", "3")   # the serial algorithm on doubles
     assert rc == 0 and len(out.split()) == 2
-    rc, out, err = run(harness, "--algorithm", "cuda_fake_shm")
-    assert rc == 2 and "not built" in out
+    rc, out, err = run(harness, "--help")
+    assert "hip_fake_shm" in out and "hip_atomic_shm2" in out
 
 
 @pytest.mark.gpu
@@ -85,18 +85,44 @@ def test_base_and_emulated_atomics(harness, gpu, tmp_path):
     for algo in ("hip_atomic_point", "hip_atomic_warp", "hip_atomic_fine", "hip_atomic_shm"):
         rc, out, err = run(harness, "--algorithm", algo, "--emul", "--verify", "--privatizedCopies", "2", *common)
         assert rc == 0 and "Verifying results ... OK" in err, algo + out + err
-    rc, out, err = run(harness, "--algorithm", "cuda_fake")
-    assert rc == 2 and "not built" in out
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("layout", ["aos", "soa", "aos32"])
+def test_fake_algorithms_add_up_to_their_closed_form(harness, gpu, layout):
+    """The atomic-throughput probes (kernels.cu:452-531): real atomic additions of the constant 0.1 to bucket
+    (i / dim) % k, checked by --verify against 0.1 * #{points congruent to the bucket modulo k} at the micro-benchmark's
+    tolerance (5e-5 relative)."""
+    for algo, extra in (("hip_fake", []), ("cuda_fake", ["--emul"]), ("hip_fake", ["--privatizedCopies", "3"]),
+                        ("cuda_fake_shm", []), ("hip_fake_shm", ["--cudaSharedMemorySize", "4096"]),
+                        ("hip_fake_shm", ["--k", "3000", "--dim", "24"])):
+        args = ["--algorithm", algo, "--layout", layout, "--N", "64k", "--k", "500", "--dim", "20", "--iterations", "2", "--verify"] + extra
+        rc, out, err = run(harness, *args)
+        assert rc == 0 and "Verifying results ... OK" in err, " ".join(args) + "\n" + out + err
+
+
+@pytest.mark.gpu
+def test_atomic_shm2_honours_its_lds_copies(harness, gpu):
+    """atomic_shm2 (kernels.cu:381-447): as many private copies of the whole k x dim block as the LDS budget holds; not
+    even one copy: the reference's error."""
+    for extra in ([], ["--cudaSharedMemorySize", "49152"], ["--cudaSharedMemorySize", "40960", "--privatizedCopies", "2"],
+                  ["--k", "16", "--dim", "16", "--layout", "soa"], ["--k", "1024", "--dim", "32", "--cudaBlockSize", "1024"]):
+        args = ["--algorithm", "cuda_atomic_shm2", "--N", "64k", "--k", "512", "--dim", "20", "--iterations", "2", "--verify"] + extra
+        rc, out, err = run(harness, *args)
+        assert rc == 0 and "Verifying results ... OK" in err, " ".join(args) + "\n" + out + err
+    rc, out, err = run(harness, "--algorithm", "hip_atomic_shm2", "--k", "512", "--dim", "20", "--cudaSharedMemorySize", "16384")
+    assert rc == 2 and "Insufficient shared memory size for given parameters." in out
 
 
 @pytest.mark.gpu
 def test_double_precision(harness, gpu):
-    for algo in ("hip_atomic_shm", "hip_atomic_fine", "hip_atomic_point", "cuda_atomic_shm2"):
+    for algo in ("hip_atomic_shm", "hip_atomic_fine", "hip_atomic_point"):
         for extra in (["--k", "512", "--dim", "20"], ["--k", "16", "--dim", "16", "--layout", "soa"], ["--k", "2048", "--dim", "32"]):
             rc, out, err = run(harness, "--double", "--algorithm", algo, "--N", "64k", "--iterations", "2", "--verify", *extra)
             assert rc == 0 and "Verifying results ... OK" in err, algo + " ".join(extra) + out + err
-    rc, out, err = run(harness, "--double", "--algorithm", "hip_base")   # the baselines of the micro-benchmark are float-only
-    assert rc == 2 and "doubles" in out
+    for algo in ("hip_base", "cuda_atomic_shm2", "hip_fake"):             # the baselines and probes of the micro-benchmark are float-only
+        rc, out, err = run(harness, "--double", "--algorithm", algo)
+        assert rc == 2 and "doubles" in out, algo + out
 
 
 @pytest.mark.gpu
@@ -120,7 +146,7 @@ def test_bucket_sum_entry_point_matches_numpy(km, gpu):
         np.add.at(want, idx, data.reshape(n, dim).astype(np.float64))
         d = km.DeviceBuffer(data.nbytes); d.write(data)
         i = km.DeviceBuffer(idx.nbytes); i.write(idx)
-        for variant in (km.UPDATE_ATOMIC_SHM, km.UPDATE_ATOMIC_FINE, km.UPDATE_ATOMIC_POINT, km.UPDATE_ATOMIC_WARP,
+        for variant in (km.UPDATE_ATOMIC_SHM, km.UPDATE_ATOMIC_FINE, km.UPDATE_ATOMIC_POINT, km.UPDATE_ATOMIC_WARP, km.UPDATE_ATOMIC_SHM2,
                         km.UPDATE_ATOMIC_FINE | km.UPDATE_EMULATED_ATOMICS, km.UPDATE_ATOMIC_WARP | km.UPDATE_EMULATED_ATOMICS):
             r = km.DeviceBuffer(4 * k * dim); r.zero()
             km.bucket_sum(variant, d, km.AOS, dim, i, r, km.AOS, dim, dim, k, n)
@@ -128,4 +154,19 @@ def test_bucket_sum_entry_point_matches_numpy(km, gpu):
             got = r.read(np.float32, k * dim).reshape(k, dim)
             r.free()
             assert np.allclose(got, want, rtol=5e-5, atol=1e-4), (dim, k, n, variant)
+        # the probes: result[b][d] = 0.1 * #{i < n : i % k == b}, whatever the inputs
+        closed = 0.1 * (n // k + (np.arange(k) < n % k))[:, None] * np.ones((1, dim))
+        for variant in (km.UPDATE_FAKE, km.UPDATE_FAKE | km.UPDATE_EMULATED_ATOMICS, km.UPDATE_FAKE_SHM):
+            r = km.DeviceBuffer(4 * k * dim); r.zero()
+            km.bucket_sum(variant, d, km.AOS, dim, i, r, km.AOS, dim, dim, k, n)
+            km.sync()
+            got = r.read(np.float32, k * dim).reshape(k, dim)
+            r.free()
+            # (thousands of fp32 additions of the same constant to one word round the same way every time: looser there)
+            assert np.allclose(got, closed, rtol=5e-5 if n // k <= 200 else 1e-3, atol=0), (dim, k, n, variant)
         d.free(); i.free()
+    # the probes are not an update: the k-means entry point refuses them
+    d = km.DeviceBuffer(64); s_ = km.DeviceBuffer(64)
+    with pytest.raises(km.KmxError, match="kmx_bucket_sum_f32 only"):
+        km.update(km.UPDATE_FAKE, d, km.AOS, 2, d, d, km.AOS, 2, s_, 2, 2, 4)
+    d.free(); s_.free()
