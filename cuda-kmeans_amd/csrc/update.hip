@@ -31,6 +31,7 @@
 
 #include <algorithm>
 
+
 namespace kmx {
 
 /* hardware fp32 atomic add without return value (global_atomic_add_f32 / ds_add_f32) */
@@ -396,7 +397,7 @@ update_private_kernel(const float* __restrict__ data, size_t stride, const uint3
  * partial layouts: [chunk][cluster][dim] and [chunk][cluster].
  */
 constexpr uint32_t SORT_SHIFT = 15; /* local point index bits: chunk_points <= 32768 */
-constexpr int SORT_UNROLL = 8;      /* row loads per batch and lane group in the segment-sum phase (two batches in flight) */
+constexpr int SORT_UNROLL = 8;      /* row loads per batch and lane group in the segment-sum phase (two batches in flight; 16 measured slower) */
 
 /* VEC consecutive floats of a row per lane: one 16-byte load when VEC = 4 (needs dim, stride % 4 == 0 and an aligned base). */
 template <int VEC> struct RowPart { float v[VEC]; };
@@ -428,7 +429,7 @@ __device__ __forceinline__ void store_part(float* p, const RowPart<VEC>& r)
 	}
 }
 
-template <int ITEMS, int GW, int VEC>
+template <int ITEMS, int GW, int VEC, bool WHOLE_ROWS = false>
 __global__ void __launch_bounds__(1024)
 update_sorted_kernel(const float* __restrict__ data, size_t stride, const uint32_t* __restrict__ assignment,
                      float* __restrict__ partial, uint32_t* __restrict__ partial_counts,
@@ -442,8 +443,11 @@ update_sorted_kernel(const float* __restrict__ data, size_t stride, const uint32
 	const uint32_t lane = tid & (WAVE - 1), wave = tid / WAVE;
 	const uint32_t p_begin = (uint32_t)min((uint64_t)blockIdx.x * chunk_points, (uint64_t)n);
 	const uint32_t count = min(chunk_points, n - p_begin);
-	const uint32_t d0 = blockIdx.y * 32;
-	const uint32_t width = min(32u, dim - d0);
+	/* The second grid dimension splits the work of a chunk: into slices of 32 dimensions, or (WHOLE_ROWS) into ranges of
+	 * clusters, every lane group then reading whole rows -- one contiguous kilobyte at 256 dimensions instead of eight
+	 * pieces of 128 bytes fetched by eight work-groups at unrelated times. */
+	const uint32_t d0 = WHOLE_ROWS ? 0u : blockIdx.y * 32;
+	const uint32_t width = WHOLE_ROWS ? dim : min(32u, dim - d0);
 
 	for (uint32_t i = tid; i <= k; i += 1024) offsets[i] = 0;
 	__syncthreads();
@@ -502,10 +506,11 @@ update_sorted_kernel(const float* __restrict__ data, size_t stride, const uint32
 	constexpr uint32_t GROUPS = 1024 / GW;
 	const uint32_t group = tid / GW, gl = tid % GW;
 	const uint32_t entries = offsets[k];
+	const uint32_t all_groups = WHOLE_ROWS ? GROUPS * gridDim.y : GROUPS; /* lane groups that share the chunk's sorted list */
 	auto first_cluster = [&](uint32_t g) -> uint32_t {
-		/* smallest c in [0, k] with offsets[c] >= g * entries / GROUPS */
-		if (g >= GROUPS) return k;
-		const uint32_t want = (uint32_t)((uint64_t)g * entries / GROUPS);
+		/* smallest c in [0, k] with offsets[c] >= g * entries / all_groups */
+		if (g >= all_groups) return k;
+		const uint32_t want = (uint32_t)((uint64_t)g * entries / all_groups);
 		uint32_t lo = 0, hi = k;
 		while (lo < hi) {
 			const uint32_t mid = (lo + hi) / 2;
@@ -513,7 +518,8 @@ update_sorted_kernel(const float* __restrict__ data, size_t stride, const uint32
 		}
 		return lo;
 	};
-	const uint32_t c_lo = first_cluster(group), c_hi = first_cluster(group + 1);
+	const uint32_t my_group = WHOLE_ROWS ? blockIdx.y * GROUPS + group : group;
+	const uint32_t c_lo = first_cluster(my_group), c_hi = first_cluster(my_group + 1);
 	const bool lane_on = gl * VEC < width;
 	const float* src = data + (size_t)p_begin * stride + d0 + (lane_on ? gl * VEC : 0);
 	float* out = partial + ((size_t)blockIdx.x * k) * dim + d0 + gl * VEC;
@@ -704,11 +710,18 @@ static uint32_t pow2_at_least(uint32_t v)
 }
 
 template <int ITEMS, int LM>
-static int launch_sorted(const UpdateArgs& u, Workspace* ws, uint32_t chunks, uint32_t slices, uint32_t chunk_points, uint32_t gw, uint32_t vec, uint32_t lds_bytes)
+static int launch_sorted(const UpdateArgs& u, Workspace* ws, uint32_t chunks, uint32_t slices, uint32_t chunk_points, uint32_t gw, uint32_t vec, uint32_t lds_bytes, bool whole_rows)
 {
 	void (*kernel)(const float*, size_t, const uint32_t*, float*, uint32_t*, uint32_t, uint32_t, uint32_t, uint32_t) = nullptr;
 	uint32_t* partial_counts = (uint32_t*)(ws->partials + (size_t)chunks * u.k * u.dim);
-	if (vec == 4) {
+	if (whole_rows) {
+		switch (gw) {
+		case 16: kernel = update_sorted_kernel<ITEMS, 16, 4, true>; break;
+		case 32: kernel = update_sorted_kernel<ITEMS, 32, 4, true>; break;
+		default: kernel = update_sorted_kernel<ITEMS, 64, 4, true>; break;
+		}
+	}
+	else if (vec == 4) {
 		switch (gw) {
 		case 1: kernel = update_sorted_kernel<ITEMS, 1, 4>; break;
 		case 2: kernel = update_sorted_kernel<ITEMS, 2, 4>; break;
@@ -771,8 +784,13 @@ static int launch_update_tuned(const UpdateArgs& u, kmx_exec_params* exec, Works
 	if (LD == KMX_AOS && u.k < (1u << (32 - SORT_SHIFT)) && (uint64_t)(u.k + 33) * 4 + 1024 * 4 <= budget) {
 		const uint32_t slices = (u.dim + 31) / 32;
 		/* 16-byte row parts where one slice covers the row and its alignment allows it (measured: no gain for sliced rows) */
-		const uint32_t vec = (u.dim <= 32 && u.dim % 4 == 0 && u.stride % 4 == 0 && ((uintptr_t)u.data & 15) == 0) ? 4 : 1;
-		const uint32_t gw = (u.dim > 16 ? 32 : pow2_at_least(std::max<uint32_t>(u.dim, 4))) / vec;
+		const bool aligned4 = u.dim % 4 == 0 && u.stride % 4 == 0 && ((uintptr_t)u.data & 15) == 0;
+		/* rows of 33 to 256 dimensions: the work-groups of a chunk take ranges of clusters and read whole rows (measured at
+		 * N = 1M, d = 256, k = 1024: 0.29 ms in slices of 32 dimensions) */
+		const bool whole_rows = u.dim > 32 && u.dim <= 256 && aligned4;
+		/* 16-byte row parts where one slice covers the row and its alignment allows it (measured: no gain for sliced rows) */
+		const uint32_t vec = ((u.dim <= 32 && aligned4) || whole_rows) ? 4 : 1;
+		const uint32_t gw = whole_rows ? std::max<uint32_t>(16, pow2_at_least(u.dim / 4)) : (u.dim > 16 ? 32 : pow2_at_least(std::max<uint32_t>(u.dim, 4))) / vec;
 		const uint32_t max_points = std::min<uint32_t>(1u << SORT_SHIFT, (budget - (u.k + 33) * 4) / 4 / 1024 * 1024);
 		uint32_t chunks = std::max<uint32_t>(1, dev.compute_units / slices);
 		uint32_t chunk_points = (u.n + chunks - 1) / chunks;
@@ -784,10 +802,10 @@ static int launch_update_tuned(const UpdateArgs& u, kmx_exec_params* exec, Works
 		exec->block_count = chunks * slices;
 		*state = 2;
 		const uint32_t items = chunk_points / 1024;
-		if (items <= 4) return launch_sorted<4, LM>(u, ws, chunks, slices, chunk_points, gw, vec, lds_bytes);
-		if (items <= 8) return launch_sorted<8, LM>(u, ws, chunks, slices, chunk_points, gw, vec, lds_bytes);
-		if (items <= 16) return launch_sorted<16, LM>(u, ws, chunks, slices, chunk_points, gw, vec, lds_bytes);
-		return launch_sorted<32, LM>(u, ws, chunks, slices, chunk_points, gw, vec, lds_bytes);
+		if (items <= 4) return launch_sorted<4, LM>(u, ws, chunks, slices, chunk_points, gw, vec, lds_bytes, whole_rows);
+		if (items <= 8) return launch_sorted<8, LM>(u, ws, chunks, slices, chunk_points, gw, vec, lds_bytes, whole_rows);
+		if (items <= 16) return launch_sorted<16, LM>(u, ws, chunks, slices, chunk_points, gw, vec, lds_bytes, whole_rows);
+		return launch_sorted<32, LM>(u, ws, chunks, slices, chunk_points, gw, vec, lds_bytes, whole_rows);
 	}
 
 	/* fallback: LDS-privatised floating-point atomics */
