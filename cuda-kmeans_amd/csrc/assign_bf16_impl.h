@@ -798,6 +798,52 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 				}
 			}
 		}
+		else if constexpr (PACKED && COARSE && !STREAM) {
+			/* Packed rows, all centroids resident: the fenced step of the wider rows with one MFMA per point tile. The tile's
+			 * 16-byte piece of centroid parts is requested a tile ahead; its norms go into the accumulator of the first
+			 * point tile as soon as that one has been tracked, three MFMAs before they are needed. */
+			const float* lds_norms = lds + (size_t)chunk_tiles * tile_floats(RS);
+			const uint32_t tiles = kp / TILE;
+			auto fetch_piece = [&](uint32_t tile) -> bf16x8 { return *(const bf16x8*)(lds + (size_t)tile * tile_floats(RS) + packed_half(col, h)); };
+			auto step = [&](bf16x8& fetch_into, uint32_t t_new, f32x16 (&acc_new)[P], const bf16x8& use, f32x16 (&acc_old)[P], uint32_t tile_old) {
+				fetch_into = fetch_piece(min(t_new + 1, tiles - 1));
+				__builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+				for (int i = 0; i < P; ++i) {
+					acc_new[P - 1 - i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(use, b[P - 1 - i].hi[0], acc_new[0], 0, 0, 0);
+					__builtin_amdgcn_sched_barrier(0);
+					track_tile<true, false>(acc_old[i], st[i], tile_old, neg_inf);
+					__builtin_amdgcn_sched_barrier(0);
+					if (i == 0) {
+						fetch_norms(acc_old[0], lds_norms, min(t_new + 1, tiles - 1), h);
+						__builtin_amdgcn_sched_barrier(0);
+					}
+				}
+			};
+			bf16x8 o0 = fetch_piece(0), o1 = fetch_piece(min(1u, tiles - 1));
+			fetch_norms(acc0[0], lds_norms, 0, h);
+			fetch_norms(acc1[0], lds_norms, min(1u, tiles - 1), h);
+#pragma unroll
+			for (int p = P - 1; p >= 0; --p) acc0[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(o0, b[p].hi[0], acc0[0], 0, 0, 0);
+			uint32_t t = 0; /* acc0 holds tile t, not yet tracked; o1 and acc1[0] hold the centroid parts and norms of tile t + 1 */
+			while (t + 2 < tiles) {
+				step(o0, t + 1, acc1, o1, acc0, t);
+				step(o1, t + 2, acc0, o0, acc1, t + 1);
+				t += 2;
+			}
+			if (t + 1 < tiles) {
+#pragma unroll
+				for (int p = P - 1; p >= 0; --p) acc1[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(o1, b[p].hi[0], acc1[0], 0, 0, 0);
+#pragma unroll
+				for (int p = 0; p < P; ++p) track_tile<true, false>(acc0[p], st[p], t, neg_inf);
+#pragma unroll
+				for (int p = 0; p < P; ++p) track_tile<true, false>(acc1[p], st[p], t + 1, neg_inf);
+			}
+			else {
+#pragma unroll
+				for (int p = 0; p < P; ++p) track_tile<true, false>(acc0[p], st[p], t, neg_inf);
+			}
+		}
 		else
 		for (uint32_t chunk = 0; chunk < chunks; ++chunk) {
 			const uint32_t row0 = chunk * chunk_rows;

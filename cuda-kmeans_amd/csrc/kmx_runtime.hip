@@ -236,6 +236,10 @@ int kmx_set_device(int device)
 		(void)hipGetLastError();
 		return fail(KMX_ERR_NO_DEVICE, "No HIP devices found!");
 	}
+	/* the work space, the cached device properties and the stream belong to the device they were made on */
+	if (g_ws.counters && g_dev.device >= 0 && g_dev.device != device)
+		return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_set_device: the library holds a work space on device %d; call kmx_shutdown() before moving to device %d",
+		            g_dev.device, device);
 	KMX_HIP(hipSetDevice(device));
 	return KMX_OK;
 }

@@ -18,7 +18,9 @@
  *     called) and the calls return without waiting, except kmx_sync, kmx_d2h and
  *     kmx_event_elapsed_ms. Stream order is the only dependency mechanism, as in the reference
  *     (cuda.hpp:70-88: one cudaDeviceSynchronize after the iteration loop).
- *   - Not thread-safe: one host thread drives one device, as in the reference.
+ *   - Not thread-safe: one host thread drives one device, as in the reference. The library keeps one work space, one
+ *     stream and the properties of one device per process; kmx_set_device to another device is refused until
+ *     kmx_shutdown() has released the work space.
  *   - layout: KMX_AOS element (idx, dim) = base[idx*stride + dim]; KMX_SOA = base[dim*stride + idx]
  *     (layout_policies.hpp:22-25,46-49); stride = LAYOUT::precomputeConstants(count, dim).
  */
@@ -44,7 +46,14 @@ typedef enum kmx_layout { KMX_AOS = 0, KMX_SOA = 1 } kmx_layout;
 
 /* = CudaExecParameters (kernels.cuh:55-70). In/out: runners overwrite block_count like the reference
  * (kernels.cu:203,311,750). Unlike the reference (kernels.cu:384,676,713) they never write the
- * other fields back, so one struct can serve the assignment and the update of every iteration. */
+ * other fields back, so one struct can serve the assignment and the update of every iteration.
+ * Who reads what: block_size and items_per_thread shape the launches of KMX_ASSIGN_BASE and of the update variants
+ * ATOMIC_POINT / _FINE / _WARP / _SHM2 / FAKE / FAKE_SHM (one lane per point or element, as in the reference);
+ * shared_mem_bytes bounds the LDS of every variant that stages data there (0 = all of it); privatized_copies is read by
+ * the update variants with global replicas. The tuned variants (KMX_ASSIGN_LDS_FMA / _MFMA / _MFMA_BF16X3 / _BEST,
+ * KMX_UPDATE_ATOMIC_SHM, the fused kernels) fix their own work-group shape -- 8 wavefronts around the LDS-resident
+ * centroids, 16 around a sorted chunk -- and ignore block_size, items_per_thread and regs_cache: the register tile the
+ * reference exposes as regs_cache is the MFMA tile here. */
 typedef struct kmx_exec_params {
 	uint32_t block_size;        /* work-group size for the variants that honour it (default 256)   */
 	uint32_t block_count;       /* out: number of work-groups of the main kernel last launched      */
