@@ -35,7 +35,7 @@ ABI_SYMBOLS = [
     "kmx_assign_last_rechecked", "kmx_assign_last_variant", "kmx_update_f32", "kmx_bucket_sum_f32", "kmx_fused_f32", "kmx_assign_f64", "kmx_update_f64", "kmx_fused_f64", "kmx_bucket_sum_f64", "kmx_set_queued_rows_limit",
     "kmx_graph_begin", "kmx_graph_end", "kmx_graph_launch", "kmx_graph_destroy", "kmx_event_create", "kmx_event_destroy", "kmx_event_record",
     "kmx_event_elapsed_ms", "kmx_set_profiling", "kmx_last_kernel_ms", "kmx_last_error", "kmx_certificate_tau",
-    "kmx_update_f32_noalloc",
+    "kmx_update_f32_noalloc", "kmx_reserve_f32",
 ]
 
 
@@ -110,6 +110,7 @@ def hip_lib():
         lib.kmx_update_f32.argtypes = [ctypes.c_int, vp, ctypes.c_int, sz, vp, vp, ctypes.c_int, sz, vp, u32, u32, u32,
                                        ctypes.POINTER(ExecParams)]
         lib.kmx_update_f32_noalloc.argtypes = lib.kmx_update_f32.argtypes
+        lib.kmx_reserve_f32.argtypes = [ctypes.c_int] * 4 + [u32] * 3
         lib.kmx_bucket_sum_f32.argtypes = [ctypes.c_int, vp, ctypes.c_int, sz, vp, vp, ctypes.c_int, sz, u32, u32, u32,
                                            ctypes.POINTER(ExecParams)]
         lib.kmx_fused_f32.argtypes = [ctypes.c_int, vp, ctypes.c_int, sz, vp, vp, ctypes.c_int, sz, vp, u32, u32, u32,
@@ -377,6 +378,11 @@ def certificate_tau(form, dim, x2, xpart2, c2max, cmid2max, crest2max):
     out = ctypes.c_float()
     check(hip_lib().kmx_certificate_tau(form, dim, x2, xpart2, c2max, cmid2max, crest2max, ctypes.byref(out)))
     return out.value
+
+
+def reserve(assign_variant, update_variant, layout, layout_means, dim, k, n):
+    """kmx_reserve_f32: sizes the work space so that assignment / update calls of this shape allocate nothing."""
+    check(hip_lib().kmx_reserve_f32(assign_variant, update_variant, layout, layout_means, dim, k, n))
 
 
 def set_queued_rows_limit(nbytes):

@@ -155,10 +155,10 @@ int launch_assign_bf16(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws
 	if (rc) return rc;
 	const uint32_t pack_blocks = (kp * WAVE + 255) / 256;
 	if (a.layout_means == KMX_AOS)
-		hipLaunchKernelGGL((pack_means_bf16_kernel<KMX_AOS>), dim3(pack_blocks), dim3(256), 0, stream(),
+		KMX_LAUNCH_KERNEL((pack_means_bf16_kernel<KMX_AOS>), dim3(pack_blocks), dim3(256), 0, stream(),
 		                   a.means, a.stride_means, ws->packed_means, ws->norms, ws->means_t, a.dim, a.k, kp, dp, packed_rows(a.dim) ? 1u : 0u, ws->counters);
 	else
-		hipLaunchKernelGGL((pack_means_bf16_kernel<KMX_SOA>), dim3(pack_blocks), dim3(256), 0, stream(),
+		KMX_LAUNCH_KERNEL((pack_means_bf16_kernel<KMX_SOA>), dim3(pack_blocks), dim3(256), 0, stream(),
 		                   a.means, a.stride_means, ws->packed_means, ws->norms, ws->means_t, a.dim, a.k, kp, dp, packed_rows(a.dim) ? 1u : 0u, ws->counters);
 	KMX_LAUNCH_CHECK("pack_means_bf16_kernel");
 

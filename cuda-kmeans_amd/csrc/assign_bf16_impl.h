@@ -1286,7 +1286,7 @@ static int launch_screen_bf16_kb(const float* rows, const Workspace* ws, const u
 	KMX_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)kernel, (int)(SCREEN_WAVES * WAVE), 0));
 	const uint32_t grid = std::min<uint32_t>(dev.compute_units * (uint32_t)std::max(1, per_cu), SCREEN_MAX_WAVES / SCREEN_WAVES);
 	*waves = grid * SCREEN_WAVES;
-	hipLaunchKernelGGL(kernel, dim3(grid), dim3(SCREEN_WAVES * WAVE), 0, stream(),
+	KMX_LAUNCH_KERNEL(kernel, dim3(grid), dim3(SCREEN_WAVES * WAVE), 0, stream(),
 	                   rows, ws->packed_means, ws->norms, ws->means_t, row_queue, row_count, pairs, item_pairs, keys, dim, k, kp);
 	KMX_LAUNCH_CHECK("screen_bf16_kernel");
 	return KMX_OK;
@@ -1345,7 +1345,7 @@ static int launch_bf16_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 	exec->block_count = grid;
 	int rc = profile_begin(0);
 	if (rc) return rc;
-	hipLaunchKernelGGL(kernel, dim3(grid), dim3(MFMA_WAVES * WAVE), lds_bytes, stream(),
+	KMX_LAUNCH_KERNEL(kernel, dim3(grid), dim3(MFMA_WAVES * WAVE), lds_bytes, stream(),
 	                   a.data, a.stride, ws->packed_means, ws->norms, a.assignment, ws->queue, ws->counters,
 	                   a.dim, a.k, kp, a.n, chunk_rows, kd, -__builtin_inff());
 	KMX_LAUNCH_CHECK("assign_bf16_kernel");

@@ -525,7 +525,7 @@ static int launch_base_t(const AssignArgs& a, kmx_exec_params* exec, uint32_t* c
 	exec->block_count = (a.n + block - 1) / block;
 	int rc = profile_begin(0);
 	if (rc) return rc;
-	hipLaunchKernelGGL((assign_base_kernel<LD, LM>), dim3(exec->block_count), dim3(block), 0, stream(),
+	KMX_LAUNCH_KERNEL((assign_base_kernel<LD, LM>), dim3(exec->block_count), dim3(block), 0, stream(),
 	                   a.data, a.stride, a.means, a.stride_means, a.assignment, a.dim, a.k, a.n, counters);
 	KMX_LAUNCH_CHECK("assign_base_kernel");
 	return profile_end(0);
@@ -549,7 +549,7 @@ static int launch_recheck_t(const AssignArgs& a, Workspace* ws, uint32_t kp)
 	const size_t lds = (size_t)PB * ((a.dim + 3) / 4 * 4) * sizeof(float);
 	auto kernel = recheck_kernel<LD, PB>;
 	if (lds > 48 * 1024) KMX_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-	hipLaunchKernelGGL(kernel, dim3(blocks), dim3(block), lds, stream(),
+	KMX_LAUNCH_KERNEL(kernel, dim3(blocks), dim3(block), lds, stream(),
 	                   a.data, a.stride, ws->means_t, kp, a.assignment, a.dim, a.k, ws->queue, ws->counters);
 	KMX_LAUNCH_CHECK("recheck_kernel");
 	return KMX_OK;
@@ -558,7 +558,7 @@ static int launch_recheck_t(const AssignArgs& a, Workspace* ws, uint32_t kp)
 template <int LD, int L, int PB, int DPAD>
 static int launch_recheck_reg(const AssignArgs& a, Workspace* ws, uint32_t kp)
 {
-	hipLaunchKernelGGL((recheck_reg_kernel<LD, L, PB, DPAD>), dim3(2048), dim3(256), 0, stream(),
+	KMX_LAUNCH_KERNEL((recheck_reg_kernel<LD, L, PB, DPAD>), dim3(2048), dim3(256), 0, stream(),
 	                   a.data, a.stride, ws->means_t, kp, a.assignment, a.dim, a.k, ws->queue, ws->counters);
 	KMX_LAUNCH_CHECK("recheck_reg_kernel");
 	return KMX_OK;
@@ -582,7 +582,7 @@ static int launch_recheck_points(const AssignArgs& a, Workspace* ws, uint32_t kp
 	const uint32_t threads = std::min<uint32_t>(1024, round_up(two ? (a.k + 1) / 2 : a.k, WAVE));
 	const dim3 grid(DPAD <= 32 ? 512 : 256); /* two work-groups fit a compute unit while the rows of a lane take at most 64 registers */
 #define KMX_RECHECK_POINTS(FULL, C) \
-	hipLaunchKernelGGL((recheck_points_kernel<LD, DPAD, FULL, C>), grid, dim3(threads), 0, stream(), \
+	KMX_LAUNCH_KERNEL((recheck_points_kernel<LD, DPAD, FULL, C>), grid, dim3(threads), 0, stream(), \
 	                   a.data, a.stride, ws->means_t, ws->norms, a.assignment, a.dim, a.k, kp, ws->queue, ws->counters)
 	if (a.dim == DPAD) { if (two) KMX_RECHECK_POINTS(true, CPL); else KMX_RECHECK_POINTS(true, 1); }
 	else { if (two) KMX_RECHECK_POINTS(false, CPL); else KMX_RECHECK_POINTS(false, 1); }
@@ -597,10 +597,10 @@ static int launch_recheck_sliced(const AssignArgs& a, Workspace* ws, uint32_t kp
 	const uint32_t threads = std::min<uint32_t>(1024, round_up(a.k, WAVE));
 	const dim3 grid(256);
 	if (a.dim % SLICE == 0)
-		hipLaunchKernelGGL((recheck_sliced_kernel<LD, true>), grid, dim3(threads), 0, stream(),
+		KMX_LAUNCH_KERNEL((recheck_sliced_kernel<LD, true>), grid, dim3(threads), 0, stream(),
 		                   a.data, a.stride, ws->means_t, ws->norms, a.assignment, a.dim, a.k, kp, ws->queue, ws->counters);
 	else
-		hipLaunchKernelGGL((recheck_sliced_kernel<LD, false>), grid, dim3(threads), 0, stream(),
+		KMX_LAUNCH_KERNEL((recheck_sliced_kernel<LD, false>), grid, dim3(threads), 0, stream(),
 		                   a.data, a.stride, ws->means_t, ws->norms, a.assignment, a.dim, a.k, kp, ws->queue, ws->counters);
 	KMX_LAUNCH_CHECK("recheck_sliced_kernel");
 	return KMX_OK;
@@ -744,19 +744,19 @@ int launch_recheck_screened(const AssignArgs& a, Workspace* ws, uint32_t kp, con
 	uint32_t* item_pairs = ws->queued_index + 4 * (size_t)cap;
 	uint32_t* pairs = item_pairs + items_max;
 	if (a.layout == KMX_AOS)
-		hipLaunchKernelGGL((gather_queued_rows_kernel<KMX_AOS>), dim3(1024), dim3(256), 0, stream(),
+		KMX_LAUNCH_KERNEL((gather_queued_rows_kernel<KMX_AOS>), dim3(1024), dim3(256), 0, stream(),
 		                   a.data, a.stride, a.dim, ws->queue, ws->counters, ws->queued_rows, row_queue, keys, cap, group_shift);
 	else
-		hipLaunchKernelGGL((gather_queued_rows_kernel<KMX_SOA>), dim3(1024), dim3(256), 0, stream(),
+		KMX_LAUNCH_KERNEL((gather_queued_rows_kernel<KMX_SOA>), dim3(1024), dim3(256), 0, stream(),
 		                   a.data, a.stride, a.dim, ws->queue, ws->counters, ws->queued_rows, row_queue, keys, cap, group_shift);
 	KMX_LAUNCH_CHECK("gather_queued_rows_kernel");
 	uint32_t screen_waves = 0;
 	rc = launch_screen_bf16(ws->queued_rows, ws, row_queue, ws->counters + 1, pairs, item_pairs, keys, a.dim, a.k, kp, dev, &screen_waves);
 	if (rc) return rc;
-	hipLaunchKernelGGL(evaluate_pairs_kernel, dim3(1024), dim3(256), 0, stream(),
+	KMX_LAUNCH_KERNEL(evaluate_pairs_kernel, dim3(1024), dim3(256), 0, stream(),
 	                   ws->queued_rows, a.dim, ws->means_t, kp, pairs, item_pairs, ws->counters + 1, unit_rows, screen_waves, keys);
 	KMX_LAUNCH_CHECK("evaluate_pairs_kernel");
-	hipLaunchKernelGGL(scatter_row_keys_kernel, dim3(512), dim3(256), 0, stream(), ws->queue, ws->counters, keys, a.assignment);
+	KMX_LAUNCH_KERNEL(scatter_row_keys_kernel, dim3(512), dim3(256), 0, stream(), ws->queue, ws->counters, keys, a.assignment);
 	KMX_LAUNCH_CHECK("scatter_row_keys_kernel");
 	if (cap == a.n) return KMX_OK; /* every point has a row: nothing can be left over */
 	Workspace rest = *ws; /* the launchers only read the pointers */
@@ -777,7 +777,7 @@ int launch_recheck(const AssignArgs& a, Workspace* ws, uint32_t kp)
 	const uint32_t group_shift = row_group_shift(a.dim);
 	uint32_t* row_queue = ws->queued_index;
 	uint32_t* row_assignment = ws->queued_index + 2 * (size_t)cap;
-	hipLaunchKernelGGL((gather_queued_rows_kernel<KMX_SOA>), dim3(2048), dim3(256), 0, stream(),
+	KMX_LAUNCH_KERNEL((gather_queued_rows_kernel<KMX_SOA>), dim3(2048), dim3(256), 0, stream(),
 	                   a.data, a.stride, a.dim, ws->queue, ws->counters, ws->queued_rows, row_queue, (unsigned long long*)nullptr, cap, group_shift);
 	KMX_LAUNCH_CHECK("gather_queued_rows_kernel");
 	AssignArgs rows = a;
@@ -786,7 +786,7 @@ int launch_recheck(const AssignArgs& a, Workspace* ws, uint32_t kp)
 	view.queue = row_queue; view.counters = ws->counters + 1;
 	rc = launch_recheck_l<KMX_AOS>(rows, &view, kp);
 	if (rc) return rc;
-	hipLaunchKernelGGL(scatter_row_results_kernel, dim3(512), dim3(256), 0, stream(), ws->queue, ws->counters, row_assignment, a.assignment);
+	KMX_LAUNCH_KERNEL(scatter_row_results_kernel, dim3(512), dim3(256), 0, stream(), ws->queue, ws->counters, row_assignment, a.assignment);
 	KMX_LAUNCH_CHECK("scatter_row_results_kernel");
 	if (cap == a.n) return KMX_OK; /* every point has a row: nothing can be left over */
 	view.queue = ws->queue + 2 * (size_t)cap; view.counters = ws->counters + 2;

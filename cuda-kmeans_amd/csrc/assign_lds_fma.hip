@@ -203,7 +203,7 @@ static int launch_fma_dp(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 	else kernel = scalar ? assign_lds_fma_kernel<DP, KMX_SOA, true> : assign_lds_fma_kernel<DP, KMX_SOA, false>;
 	int rc = profile_begin(0);
 	if (rc) return rc;
-	hipLaunchKernelGGL(kernel, dim3(grid), dim3(FMA_WAVES * WAVE), lds_bytes, stream(),
+	KMX_LAUNCH_KERNEL(kernel, dim3(grid), dim3(FMA_WAVES * WAVE), lds_bytes, stream(),
 	                   a.data, a.stride, ws->packed_means, ws->norms, a.assignment, ws->queue, ws->counters, a.dim, a.k, kp, a.n, chunk_rows, kd, vec4);
 	KMX_LAUNCH_CHECK("assign_lds_fma_kernel");
 	return profile_end(0);

@@ -103,10 +103,10 @@ int launch_pack_means(const AssignArgs& a, Workspace* ws, uint32_t dp, uint32_t 
 	if (rc) return rc;
 	const uint32_t pack_blocks = (kp * WAVE + 255) / 256;
 	if (a.layout_means == KMX_AOS)
-		hipLaunchKernelGGL((pack_means_kernel<KMX_AOS>), dim3(pack_blocks), dim3(256), 0, stream(),
+		KMX_LAUNCH_KERNEL((pack_means_kernel<KMX_AOS>), dim3(pack_blocks), dim3(256), 0, stream(),
 		                   a.means, a.stride_means, ws->packed_means, ws->norms, ws->means_t, a.dim, a.k, kp, dp, ws->counters);
 	else
-		hipLaunchKernelGGL((pack_means_kernel<KMX_SOA>), dim3(pack_blocks), dim3(256), 0, stream(),
+		KMX_LAUNCH_KERNEL((pack_means_kernel<KMX_SOA>), dim3(pack_blocks), dim3(256), 0, stream(),
 		                   a.means, a.stride_means, ws->packed_means, ws->norms, ws->means_t, a.dim, a.k, kp, dp, ws->counters);
 	KMX_LAUNCH_CHECK("pack_means_kernel");
 	return KMX_OK;

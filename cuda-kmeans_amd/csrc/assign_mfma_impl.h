@@ -547,7 +547,7 @@ static int launch_mfma_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 	exec->block_count = grid;
 	int rc = profile_begin(0);
 	if (rc) return rc;
-	hipLaunchKernelGGL(kernel, dim3(grid), dim3(MFMA_WAVES * WAVE), lds_bytes, stream(),
+	KMX_LAUNCH_KERNEL(kernel, dim3(grid), dim3(MFMA_WAVES * WAVE), lds_bytes, stream(),
 	                   a.data, a.stride, ws->packed_means, ws->norms, a.assignment, ws->queue, ws->counters,
 	                   a.dim, a.k, kp, a.n, chunk_rows, kd, -__builtin_inff());
 	KMX_LAUNCH_CHECK("assign_mfma_kernel");

@@ -628,7 +628,7 @@ int launch_assign_f64_ld(int variant, const double* data, size_t stride, uint32_
 	const uint32_t* exact_length = (const uint32_t*)g_misc;
 	if (float_queue) { exact_queue = float_queue; exact_stride = 2; exact_length = float_queue_length; } /* ... or the float sweep's (pairs) */
 #define KMX_F64_EXACT(DPAD, G) \
-	hipLaunchKernelGGL((assign_f64_kernel<LD, DPAD, G>), grid, block, 0, stream(), data, stride, g_means_t, assignment, dim, k, kp, n)
+	KMX_LAUNCH_KERNEL((assign_f64_kernel<LD, DPAD, G>), grid, block, 0, stream(), data, stride, g_means_t, assignment, dim, k, kp, n)
 	/* queued points: many centroids and rows long enough to pay for the work-group-wide minimum -> batches of points
 	 * against one lane per centroid; else 16 lanes (2 for few centroids) share a point */
 	const bool batched = k >= 256 && dim >= 16 && (size_t)BATCH * dim * sizeof(double) <= 48 * 1024; /* dynamic + static LDS stay below 64 KB */
@@ -638,18 +638,18 @@ int launch_assign_f64_ld(int variant, const double* data, size_t stride, uint32_
 	const dim3 qgrid((uint32_t)std::min<size_t>(((size_t)n * (many ? 16 : 2) + 255) / 256, (size_t)dev.compute_units * 8));
 #define KMX_F64_REQUEUED(DPAD) \
 	do { \
-		if (many) hipLaunchKernelGGL((requeued_f64_kernel<LD, DPAD, 16>), qgrid, block, 0, stream(), data, stride, g_means_t, assignment, \
+		if (many) KMX_LAUNCH_KERNEL((requeued_f64_kernel<LD, DPAD, 16>), qgrid, block, 0, stream(), data, stride, g_means_t, assignment, \
 		                             dim, k, kp, exact_queue, exact_stride, exact_length); \
-		else hipLaunchKernelGGL((requeued_f64_kernel<LD, DPAD, 2>), qgrid, block, 0, stream(), data, stride, g_means_t, assignment, \
+		else KMX_LAUNCH_KERNEL((requeued_f64_kernel<LD, DPAD, 2>), qgrid, block, 0, stream(), data, stride, g_means_t, assignment, \
 		                        dim, k, kp, exact_queue, exact_stride, exact_length); \
 	} while (0)
 #define KMX_F64_REQUEUED_BY_DIM() \
 	do { \
 		if (batched && float_queue) \
-			hipLaunchKernelGGL((requeued_batch_f64_kernel<LD, true>), bgrid, dim3(batch_threads), (size_t)BATCH * dim * sizeof(double), stream(), \
+			KMX_LAUNCH_KERNEL((requeued_batch_f64_kernel<LD, true>), bgrid, dim3(batch_threads), (size_t)BATCH * dim * sizeof(double), stream(), \
 			                   data, stride, g_means_t, g_norms, assignment, dim, k, kp, exact_queue, exact_stride, exact_length); \
 		else if (batched) \
-			hipLaunchKernelGGL((requeued_batch_f64_kernel<LD, false>), bgrid, dim3(batch_threads), (size_t)BATCH * dim * sizeof(double), stream(), \
+			KMX_LAUNCH_KERNEL((requeued_batch_f64_kernel<LD, false>), bgrid, dim3(batch_threads), (size_t)BATCH * dim * sizeof(double), stream(), \
 			                   data, stride, g_means_t, g_norms, assignment, dim, k, kp, exact_queue, exact_stride, exact_length); \
 		else if (dim > 32) KMX_F64_REQUEUED(0); \
 		else if (dim <= 8) KMX_F64_REQUEUED(8); \
@@ -673,7 +673,7 @@ int launch_assign_f64_ld(int variant, const double* data, size_t stride, uint32_
 	constexpr int P = 1; /* points per lane of the ranking sweep (2 measured no faster: fewer wavefronts hide less scalar-load latency) */
 	const dim3 rgrid((n + 256 * P - 1) / (256 * P));
 #define KMX_F64_RANK(DPAD, G) \
-	hipLaunchKernelGGL((rank_f64_kernel<LD, DPAD, G, P>), rgrid, block, 0, stream(), data, stride, g_means_t, g_norms, misc, queue, assignment, dim, k, kp, n, kd)
+	KMX_LAUNCH_KERNEL((rank_f64_kernel<LD, DPAD, G, P>), rgrid, block, 0, stream(), data, stride, g_means_t, g_norms, misc, queue, assignment, dim, k, kp, n, kd)
 	if (dim > 32) KMX_F64_RANK(0, 16);
 	else if (dim <= 8) KMX_F64_RANK(8, GROUP);
 	else if (dim <= 16) KMX_F64_RANK(16, GROUP);
@@ -713,21 +713,21 @@ int launch_update_f64_t(int variant, const double* data, size_t stride, const ui
 		const size_t per_slice = std::max<size_t>(1024, 16 * (size_t)range_size * dim);
 		const uint32_t slices = (uint32_t)std::max<size_t>(1, std::min<size_t>((total + per_slice - 1) / per_slice, std::max<size_t>(1, (size_t)dev.compute_units * 2 / ranges)));
 		exec->block_count = slices * ranges;
-		hipLaunchKernelGGL((update_ranges_f64_kernel<LD, LM>), dim3(slices * ranges), wide, range_bytes, stream(),
+		KMX_LAUNCH_KERNEL((update_ranges_f64_kernel<LD, LM>), dim3(slices * ranges), wide, range_bytes, stream(),
 		                   data, stride, assignment, means, stride_means, sizes, dim, k, n, range_size, slices);
 		KMX_LAUNCH_CHECK("update_ranges_f64_kernel");
 	}
 	else if (n > 0) {
 		if (use_private)
-			hipLaunchKernelGGL((update_f64_kernel<LD, LM, true>), grid, block, private_bytes, stream(),
+			KMX_LAUNCH_KERNEL((update_f64_kernel<LD, LM, true>), grid, block, private_bytes, stream(),
 			                   data, stride, assignment, means, stride_means, sizes, dim, k, n);
 		else
-			hipLaunchKernelGGL((update_f64_kernel<LD, LM, false>), grid, block, 0, stream(),
+			KMX_LAUNCH_KERNEL((update_f64_kernel<LD, LM, false>), grid, block, 0, stream(),
 			                   data, stride, assignment, means, stride_means, sizes, dim, k, n);
 		KMX_LAUNCH_CHECK("update_f64_kernel");
 	}
 	if (!divide) return KMX_OK; /* the update micro-benchmark wants the sums */
-	hipLaunchKernelGGL((divide_means_f64_kernel<LM>), dim3((k * dim + 255) / 256), dim3(256), 0, stream(), means, stride_means, sizes, dim, k);
+	KMX_LAUNCH_KERNEL((divide_means_f64_kernel<LM>), dim3((k * dim + 255) / 256), dim3(256), 0, stream(), means, stride_means, sizes, dim, k);
 	KMX_LAUNCH_CHECK("divide_means_f64_kernel");
 	return KMX_OK;
 }
@@ -783,13 +783,13 @@ extern "C" int kmx_assign_f64(int variant,
 	rc = reserve_f64(&g_misc, &g_misc_cap, 4);
 	if (rc) return rc;
 	unsigned long long* misc = (unsigned long long*)g_misc;
-	hipLaunchKernelGGL(reset_f64_kernel, dim3(1), dim3(64), 0, stream(), misc);
+	KMX_LAUNCH_KERNEL(reset_f64_kernel, dim3(1), dim3(64), 0, stream(), misc);
 	KMX_LAUNCH_CHECK("reset_f64_kernel");
 	const dim3 pgrid((kp + 255) / 256);
 	if (layout_means == KMX_AOS)
-		hipLaunchKernelGGL((prepare_means_f64_kernel<KMX_AOS>), pgrid, dim3(256), 0, stream(), means, stride_means, g_means_t, g_norms, misc, dim, k, kp);
+		KMX_LAUNCH_KERNEL((prepare_means_f64_kernel<KMX_AOS>), pgrid, dim3(256), 0, stream(), means, stride_means, g_means_t, g_norms, misc, dim, k, kp);
 	else
-		hipLaunchKernelGGL((prepare_means_f64_kernel<KMX_SOA>), pgrid, dim3(256), 0, stream(), means, stride_means, g_means_t, g_norms, misc, dim, k, kp);
+		KMX_LAUNCH_KERNEL((prepare_means_f64_kernel<KMX_SOA>), pgrid, dim3(256), 0, stream(), means, stride_means, g_means_t, g_norms, misc, dim, k, kp);
 	KMX_LAUNCH_CHECK("prepare_means_f64_kernel");
 
 	const uint32_t* float_queue = nullptr;
@@ -802,9 +802,9 @@ extern "C" int kmx_assign_f64(int variant,
 		if (rc) return rc;
 		rc = reserve_f64(&g_means32, &g_means32_cap, means_extent / 2 + 1);
 		if (rc) return rc;
-		hipLaunchKernelGGL(round_to_float_kernel, dim3((uint32_t)std::min<size_t>((data_extent + 1023) / 1024, (size_t)dev->compute_units * 32)), dim3(256), 0,
+		KMX_LAUNCH_KERNEL(round_to_float_kernel, dim3((uint32_t)std::min<size_t>((data_extent + 1023) / 1024, (size_t)dev->compute_units * 32)), dim3(256), 0,
 		                   stream(), data, (float*)g_data32, data_extent);
-		hipLaunchKernelGGL(round_to_float_kernel, dim3((uint32_t)std::min<size_t>((means_extent + 1023) / 1024, (size_t)dev->compute_units * 32)), dim3(256), 0,
+		KMX_LAUNCH_KERNEL(round_to_float_kernel, dim3((uint32_t)std::min<size_t>((means_extent + 1023) / 1024, (size_t)dev->compute_units * 32)), dim3(256), 0,
 		                   stream(), means, (float*)g_means32, means_extent);
 		KMX_LAUNCH_CHECK("round_to_float_kernel");
 		Workspace* ws = nullptr;
@@ -837,7 +837,7 @@ extern "C" int kmx_assign_f64(int variant,
 	Workspace* ws = nullptr;
 	rc = workspace(&ws);
 	if (rc) return rc;
-	hipLaunchKernelGGL(publish_queue_length_kernel, dim3(1), dim3(64), 0, stream(), misc, ws->counters, variant == KMX_ASSIGN_LDS_FMA);
+	KMX_LAUNCH_KERNEL(publish_queue_length_kernel, dim3(1), dim3(64), 0, stream(), misc, ws->counters, variant == KMX_ASSIGN_LDS_FMA);
 	KMX_LAUNCH_CHECK("publish_queue_length_kernel");
 	return KMX_OK;
 }

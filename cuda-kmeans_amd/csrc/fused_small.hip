@@ -287,7 +287,7 @@ static int launch_fused_t(const AssignArgs& a, float* means_out, uint32_t* sizes
 	const uint32_t vec4 = (a.layout == KMX_AOS && a.dim % 4 == 0 && a.stride % 4 == 0 && ((uintptr_t)a.data % 16) == 0) ? 1u : 0u;
 	int rc = profile_begin(0);
 	if (rc) return rc;
-	hipLaunchKernelGGL(kernel, dim3(grid), dim3(FUSED_WAVES * WAVE), lds_bytes, stream(),
+	KMX_LAUNCH_KERNEL(kernel, dim3(grid), dim3(FUSED_WAVES * WAVE), lds_bytes, stream(),
 	                   a.data, a.stride, ws->packed_means, ws->norms, a.means, a.stride_means, means_out, sizes,
 	                   ws->queue, ws->counters, a.dim, a.k, a.n, kd, vec4);
 	KMX_LAUNCH_CHECK("fused_small_kernel");
@@ -314,7 +314,7 @@ static int launch_fused_layouts(const AssignArgs& a, float* means_out, uint32_t*
 	/* the unresolved points: exact pass into the work-space assignment vector, then their share of the sums */
 	rc = launch_recheck(a, ws, kp);
 	if (rc) return rc;
-	hipLaunchKernelGGL((fused_fixup_kernel<LD, LM>), dim3(64), dim3(256), 0, stream(),
+	KMX_LAUNCH_KERNEL((fused_fixup_kernel<LD, LM>), dim3(64), dim3(256), 0, stream(),
 	                   a.data, a.stride, a.assignment, means_out, a.stride_means, sizes, ws->queue, ws->counters, a.dim, a.k);
 	KMX_LAUNCH_CHECK("fused_fixup_kernel");
 	return KMX_OK;

@@ -81,6 +81,14 @@ int reserve_queued_rows(Workspace* ws, size_t rows, size_t dim, size_t extra_wor
 			return ::kmx::fail(KMX_ERR_DEVICE, "%s failed: %s", #call, hipGetErrorString(kmx_e_));           \
 	} while (0)
 
+/* Every kernel of the library is launched through this: while kmx_reserve_f32 walks the launchers to size the work space
+ * (sizing_only()), the reservations happen and the kernels do not run. */
+bool sizing_only();
+#define KMX_LAUNCH_KERNEL(...)                                                                                \
+	do {                                                                                                      \
+		if (!::kmx::sizing_only()) hipLaunchKernelGGL(__VA_ARGS__);                                           \
+	} while (0)
+
 #define KMX_LAUNCH_CHECK(name)                                                                                \
 	do {                                                                                                      \
 		hipError_t kmx_e_ = hipGetLastError();                                                                \

@@ -37,6 +37,9 @@ hipStream_t stream() { return g_capturing ? g_capture_stream : g_stream; }
 		if (g_capturing) return fail(KMX_ERR_INVALID_ARGUMENT, name ": not allowed between kmx_graph_begin and kmx_graph_end"); \
 	} while (0)
 
+static bool g_sizing = false;
+bool sizing_only() { return g_sizing; }
+
 static bool g_profiling = false;
 static bool g_profiling_suspended = false;
 void suspend_profiling(bool suspended) { g_profiling_suspended = suspended; }
@@ -45,7 +48,7 @@ static bool g_prof_valid[2] = { false, false };
 
 int profile_begin(int which)
 {
-	if (!g_profiling || g_capturing || g_profiling_suspended) return KMX_OK;
+	if (!g_profiling || g_capturing || g_profiling_suspended || g_sizing) return KMX_OK;
 	for (int i = 0; i < 2; ++i)
 		if (!g_prof[which][i]) KMX_HIP(hipEventCreate(&g_prof[which][i]));
 	KMX_HIP(hipEventRecord(g_prof[which][0], g_stream));
@@ -54,7 +57,7 @@ int profile_begin(int which)
 
 int profile_end(int which)
 {
-	if (!g_profiling || g_capturing || g_profiling_suspended) return KMX_OK;
+	if (!g_profiling || g_capturing || g_profiling_suspended || g_sizing) return KMX_OK;
 	KMX_HIP(hipEventRecord(g_prof[which][1], g_stream));
 	g_prof_valid[which] = true;
 	return KMX_OK;
@@ -347,7 +350,7 @@ int kmx_fill_zero_u32(void* dptr, size_t count)
 	const unsigned block = 256;
 	size_t blocks = (count + block - 1) / block;
 	if (blocks > 4096) blocks = 4096;
-	hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)blocks), dim3(block), 0, stream(), (uint32_t*)dptr, count);
+	KMX_LAUNCH_KERNEL(fill_zero_kernel, dim3((unsigned)blocks), dim3(block), 0, stream(), (uint32_t*)dptr, count);
 	KMX_LAUNCH_CHECK("fill_zero_kernel");
 	return KMX_OK;
 }
@@ -399,6 +402,32 @@ int kmx_assign_f32(int variant,
 
 	AssignArgs a{ data, layout, stride, means, layout_means, stride_means, assignment, dim, k, n };
 	return dispatch_assign(variant, a, exec, ws, *dev, nullptr);
+}
+
+int kmx_reserve_f32(int assign_variant, int update_variant, int layout, int layout_means, uint32_t dim, uint32_t k, uint32_t n)
+{
+	clear_error();
+	KMX_NOT_WHILE_CAPTURING("kmx_reserve_f32");
+	if (dim == 0 || k == 0) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_reserve_f32: dim and k must be positive");
+	if (n == 0) return KMX_OK;
+	/* the launchers themselves say what they need: they are walked with the launches switched off, on pointers that are
+	 * never followed (16-byte aligned, like buffers from kmx_malloc) */
+	float* const points = (float*)(uintptr_t)4096;
+	uint32_t* const words = (uint32_t*)(uintptr_t)4096;
+	const size_t stride = layout == KMX_AOS ? dim : n, stride_means = layout_means == KMX_AOS ? dim : k;
+	kmx_exec_params exec = { 256, 0, 0, 1, 1, 1 };
+	const int last_variant = g_last_assign_variant;
+	g_sizing = true;
+	int rc = kmx_assign_f32(assign_variant, points, layout, stride, points, layout_means, stride_means, nullptr, words, dim, k, n, &exec);
+	if (rc == KMX_OK) rc = kmx_update_f32(update_variant, points, layout, stride, words, points, layout_means, stride_means, words, dim, k, n, &exec);
+	if (rc == KMX_OK) {
+		Workspace* ws = nullptr;
+		rc = workspace(&ws);
+		if (rc == KMX_OK) rc = reserve_fused_assignment(ws, n); /* kmx_fused_f32 keeps its assignment vector in the work space */
+	}
+	g_sizing = false;
+	g_last_assign_variant = last_variant;
+	return rc;
 }
 
 int kmx_assign_last_variant(int* variant)

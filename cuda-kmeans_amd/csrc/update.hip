@@ -697,7 +697,7 @@ static int clear_outputs(const UpdateArgs& u)
 {
 	const size_t words = copy_floats_of(u);
 	const uint32_t blocks = (uint32_t)std::min<size_t>((words + u.k + 255) / 256, 1024);
-	hipLaunchKernelGGL(clear_outputs_kernel, dim3(std::max(blocks, 1u)), dim3(256), 0, stream(), (uint32_t*)u.means, words, u.cluster_sizes, u.k);
+	KMX_LAUNCH_KERNEL(clear_outputs_kernel, dim3(std::max(blocks, 1u)), dim3(256), 0, stream(), (uint32_t*)u.means, words, u.cluster_sizes, u.k);
 	KMX_LAUNCH_CHECK("clear_outputs_kernel");
 	return KMX_OK;
 }
@@ -737,12 +737,12 @@ static int launch_sorted(const UpdateArgs& u, Workspace* ws, uint32_t chunks, ui
 		}
 	}
 	KMX_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-	hipLaunchKernelGGL(kernel, dim3(chunks, slices), dim3(1024), lds_bytes, stream(),
+	KMX_LAUNCH_KERNEL(kernel, dim3(chunks, slices), dim3(1024), lds_bytes, stream(),
 	                   u.data, u.stride, u.assignment, ws->partials, partial_counts, u.dim, u.k, u.n, chunk_points);
 	KMX_LAUNCH_CHECK("update_sorted_kernel");
 	const uint32_t total = u.k * u.dim;
 	const uint32_t shares = std::max<uint32_t>(1, std::min<uint32_t>(REDUCE_SHARES, chunks / 8));
-	hipLaunchKernelGGL((reduce_partials_kernel<LM>), dim3((total + 63) / 64), dim3(64 * shares), 0, stream(),
+	KMX_LAUNCH_KERNEL((reduce_partials_kernel<LM>), dim3((total + 63) / 64), dim3(64 * shares), 0, stream(),
 	                   ws->partials, partial_counts, u.means, u.stride_means, u.cluster_sizes, u.dim, u.k, chunks, u.divide ? 1u : 0u);
 	KMX_LAUNCH_CHECK("reduce_partials_kernel");
 	return KMX_OK;
@@ -773,7 +773,7 @@ static int launch_update_tuned(const UpdateArgs& u, kmx_exec_params* exec, Works
 			exec->block_count = chunks;
 			int rc = clear_outputs(u);
 			if (rc) return rc;
-			hipLaunchKernelGGL((update_private_kernel<LM>), dim3(chunks), dim3(256), (uint32_t)lds_bytes, stream(),
+			KMX_LAUNCH_KERNEL((update_private_kernel<LM>), dim3(chunks), dim3(256), (uint32_t)lds_bytes, stream(),
 			                   u.data, u.stride, u.assignment, u.means, u.stride_means, u.cluster_sizes,
 			                   u.dim, u.k, u.n, gw, (uint32_t)copy_stride, chunk_points);
 			KMX_LAUNCH_CHECK("update_private_kernel");
@@ -840,7 +840,7 @@ static int launch_update_tuned(const UpdateArgs& u, kmx_exec_params* exec, Works
 	auto kernel = update_lds_kernel<LD, LM>;
 	KMX_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
 	exec->block_count = chunks * slices;
-	hipLaunchKernelGGL(kernel, dim3(chunks, slices), dim3(wg), lds_bytes, stream(),
+	KMX_LAUNCH_KERNEL(kernel, dim3(chunks, slices), dim3(wg), lds_bytes, stream(),
 	                   u.data, u.stride, u.assignment, u.means, u.stride_means, u.cluster_sizes,
 	                   u.dim, u.k, u.n, slice, chunk_points, replicas);
 	KMX_LAUNCH_CHECK("update_lds_kernel");
@@ -874,9 +874,9 @@ static int launch_update_t(int variant, const UpdateArgs& u, kmx_exec_params* ex
 		}
 #define KMX_UPDATE_LAUNCH(KERNEL, NAME) \
 	do { \
-		if (emulated) hipLaunchKernelGGL((KERNEL<LD, LM, true>), dim3(exec->block_count), dim3(block), 0, stream(), u.data, u.stride, u.assignment, \
+		if (emulated) KMX_LAUNCH_KERNEL((KERNEL<LD, LM, true>), dim3(exec->block_count), dim3(block), 0, stream(), u.data, u.stride, u.assignment, \
 		                                 u.means, u.stride_means, u.cluster_sizes, u.dim, u.k, u.n, copy_floats, copies); \
-		else hipLaunchKernelGGL((KERNEL<LD, LM, false>), dim3(exec->block_count), dim3(block), 0, stream(), u.data, u.stride, u.assignment, \
+		else KMX_LAUNCH_KERNEL((KERNEL<LD, LM, false>), dim3(exec->block_count), dim3(block), 0, stream(), u.data, u.stride, u.assignment, \
 		                        u.means, u.stride_means, u.cluster_sizes, u.dim, u.k, u.n, copy_floats, copies); \
 		KMX_LAUNCH_CHECK(NAME); \
 	} while (0)
@@ -908,14 +908,14 @@ static int launch_update_t(int variant, const UpdateArgs& u, kmx_exec_params* ex
 				const uint32_t lds_bytes = (uint32_t)(lds_copies * one_copy);
 				auto kernel = update_shm2_kernel<LD, LM>;
 				KMX_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-				hipLaunchKernelGGL(kernel, dim3(exec->block_count), dim3(block), lds_bytes, stream(), u.data, u.stride, u.assignment,
+				KMX_LAUNCH_KERNEL(kernel, dim3(exec->block_count), dim3(block), lds_bytes, stream(), u.data, u.stride, u.assignment,
 				                   u.means, u.stride_means, u.cluster_sizes, u.dim, u.k, u.n, copy_floats, copies, lds_copies);
 				KMX_LAUNCH_CHECK("update_shm2_kernel");
 			}
 			else if (variant == KMX_UPDATE_FAKE) {
-				if (emulated) hipLaunchKernelGGL((update_fake_kernel<LM, true>), dim3(exec->block_count), dim3(block), 0, stream(),
+				if (emulated) KMX_LAUNCH_KERNEL((update_fake_kernel<LM, true>), dim3(exec->block_count), dim3(block), 0, stream(),
 				                                 u.means, u.stride_means, u.dim, u.k, u.n, copy_floats, copies);
-				else hipLaunchKernelGGL((update_fake_kernel<LM, false>), dim3(exec->block_count), dim3(block), 0, stream(),
+				else KMX_LAUNCH_KERNEL((update_fake_kernel<LM, false>), dim3(exec->block_count), dim3(block), 0, stream(),
 				                        u.means, u.stride_means, u.dim, u.k, u.n, copy_floats, copies);
 				KMX_LAUNCH_CHECK("update_fake_kernel");
 			}
@@ -924,7 +924,7 @@ static int launch_update_t(int variant, const UpdateArgs& u, kmx_exec_params* ex
 				const uint32_t lds_bytes = cached * u.dim * (uint32_t)sizeof(float);
 				auto kernel = update_fake_shm_kernel<LM>;
 				KMX_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-				hipLaunchKernelGGL(kernel, dim3(exec->block_count), dim3(block), lds_bytes, stream(),
+				KMX_LAUNCH_KERNEL(kernel, dim3(exec->block_count), dim3(block), lds_bytes, stream(),
 				                   u.means, u.stride_means, u.dim, u.k, u.n, copy_floats, copies, cached);
 				KMX_LAUNCH_CHECK("update_fake_shm_kernel");
 			}
@@ -932,7 +932,7 @@ static int launch_update_t(int variant, const UpdateArgs& u, kmx_exec_params* ex
 		else if (variant == KMX_UPDATE_BASE) {
 			exec->block_count = (u.k * u.dim + 255) / 256;
 			copies = 1; /* no replicas: every element of the result has one owner */
-			hipLaunchKernelGGL((update_base_kernel<LD, LM>), dim3(exec->block_count), dim3(256), 0, stream(),
+			KMX_LAUNCH_KERNEL((update_base_kernel<LD, LM>), dim3(exec->block_count), dim3(256), 0, stream(),
 			                   u.data, u.stride, u.assignment, u.means, u.stride_means, u.cluster_sizes, u.dim, u.k, u.n);
 			KMX_LAUNCH_CHECK("update_base_kernel");
 		}
@@ -946,11 +946,11 @@ static int launch_update_t(int variant, const UpdateArgs& u, kmx_exec_params* ex
 	const uint32_t total = u.k * u.dim;
 	const uint32_t blocks = std::min<uint32_t>((total + 255) / 256, 1024);
 	if (copies > 1) {
-		hipLaunchKernelGGL((reduce_copies_kernel<LM>), dim3(blocks), dim3(256), 0, stream(), u.means, u.stride_means, copy_floats, u.dim, u.k, copies);
+		KMX_LAUNCH_KERNEL((reduce_copies_kernel<LM>), dim3(blocks), dim3(256), 0, stream(), u.means, u.stride_means, copy_floats, u.dim, u.k, copies);
 		KMX_LAUNCH_CHECK("reduce_copies_kernel");
 	}
 	if (u.divide) {
-		hipLaunchKernelGGL((divide_means_kernel<LM>), dim3(blocks), dim3(256), 0, stream(), u.means, u.stride_means, u.cluster_sizes, u.dim, u.k);
+		KMX_LAUNCH_KERNEL((divide_means_kernel<LM>), dim3(blocks), dim3(256), 0, stream(), u.means, u.stride_means, u.cluster_sizes, u.dim, u.k);
 		KMX_LAUNCH_CHECK("divide_means_kernel");
 	}
 	return KMX_OK;
@@ -962,9 +962,9 @@ int launch_divide_means(const UpdateArgs& u)
 	const uint32_t total = u.k * u.dim;
 	const uint32_t blocks = std::min<uint32_t>((total + 255) / 256, 1024);
 	if (u.layout_means == KMX_AOS)
-		hipLaunchKernelGGL((divide_means_kernel<KMX_AOS>), dim3(blocks), dim3(256), 0, stream(), u.means, u.stride_means, u.cluster_sizes, u.dim, u.k);
+		KMX_LAUNCH_KERNEL((divide_means_kernel<KMX_AOS>), dim3(blocks), dim3(256), 0, stream(), u.means, u.stride_means, u.cluster_sizes, u.dim, u.k);
 	else
-		hipLaunchKernelGGL((divide_means_kernel<KMX_SOA>), dim3(blocks), dim3(256), 0, stream(), u.means, u.stride_means, u.cluster_sizes, u.dim, u.k);
+		KMX_LAUNCH_KERNEL((divide_means_kernel<KMX_SOA>), dim3(blocks), dim3(256), 0, stream(), u.means, u.stride_means, u.cluster_sizes, u.dim, u.k);
 	KMX_LAUNCH_CHECK("divide_means_kernel");
 	return KMX_OK;
 }
@@ -1036,7 +1036,7 @@ int launch_update(int variant, const UpdateArgs& u, kmx_exec_params* exec, Works
 		int rc = reserve_rows_copy(ws, (size_t)u.n * u.dim);
 		if (rc) return rc;
 		const size_t tiles = (size_t)((u.n + 63) / 64) * ((u.dim + 31) / 32);
-		hipLaunchKernelGGL(rows_from_soa_kernel, dim3((uint32_t)std::min<size_t>(tiles, (size_t)dev.compute_units * 32)), dim3(256), 0, stream(),
+		KMX_LAUNCH_KERNEL(rows_from_soa_kernel, dim3((uint32_t)std::min<size_t>(tiles, (size_t)dev.compute_units * 32)), dim3(256), 0, stream(),
 		                   u.data, u.stride, ws->rows_copy, u.dim, u.n);
 		KMX_LAUNCH_CHECK("rows_from_soa_kernel");
 		UpdateArgs rows = u;

@@ -137,6 +137,15 @@ int kmx_assign_f32(int variant,
                    const uint32_t* last_assignment, uint32_t* assignment,
                    uint32_t dim, uint32_t k, uint32_t n, kmx_exec_params* exec);
 
+/*
+ * Sizes the library's work space (packed centroids, recheck queue, copied rows, partial sums) for kmx_assign_f32 /
+ * kmx_update_f32 / kmx_fused_f32 calls of this shape and these variants, so that those calls allocate nothing afterwards
+ * (no counterpart in the reference, whose runners allocate nothing: cuda.hpp:54-64 allocates everything in initialize()).
+ * Without it the first call of a shape grows the work space itself, which waits for the stream and calls hipMalloc; a
+ * call with a different LDS budget (shared_mem_bytes) than the default may still grow it. Not while a graph is recorded.
+ */
+int kmx_reserve_f32(int assign_variant, int update_variant, int layout, int layout_means, uint32_t dim, uint32_t k, uint32_t n);
+
 /* Number of points the last kmx_assign_f32 call re-evaluated with the serial arithmetic (waits for the stream). */
 int kmx_assign_last_rechecked(uint64_t* count);
 

@@ -645,3 +645,35 @@ def test_recording_refuses_what_cannot_be_recorded(km, gpu):
     g.destroy()
     for b in (buf, d, m, a):
         b.free()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dim,k,n,layout", [(4, 1024, 1 << 16, AOS), (32, 256, 1 << 15, SOA), (64, 128, 1 << 14, AOS), (2, 16, 1 << 14, AOS)])
+def test_reserved_work_space_is_enough(km, orc, gpu, dim, k, n, layout):
+    """kmx_reserve_f32 on a released work space: the assignment and the update of that shape can then be recorded, which
+    refuses every call that would have to allocate; the recorded pair gives the oracle's assignment and counts."""
+    rng = np.random.default_rng(dim * 7 + k)
+    rows = rng.normal(size=(n, dim)).astype(np.float32)
+    cents = rows[rng.choice(n, k, replace=False)].copy()
+    host = rows.ravel() if layout == AOS else rows.T.copy().ravel()
+    stride = dim if layout == AOS else n
+    d = km.DeviceBuffer(4 * n * dim); d.write(host)
+    m = km.DeviceBuffer(4 * k * dim); m.write(cents.ravel())
+    a = km.DeviceBuffer(4 * n); out = km.DeviceBuffer(4 * k * dim); sizes = km.DeviceBuffer(4 * k)
+    km.sync()
+    km.check(km.hip_lib().kmx_shutdown())
+    km.reserve(km.ASSIGN_BEST, km.UPDATE_ATOMIC_SHM, layout, AOS, dim, k, n)
+    with km.Graph() as g:
+        km.assign(km.ASSIGN_BEST, d, layout, stride, m, AOS, dim, a, dim, k, n)
+        km.update(km.UPDATE_ATOMIC_SHM, d, layout, stride, a, out, AOS, dim, sizes, dim, k, n)
+    g.launch()
+    km.sync()
+    g.destroy()
+    ga = a.read(np.uint32, n)
+    oa = orc.assign(rows.ravel(), cents.ravel(), dim, k, n, threads=0, fast=True)
+    assert np.array_equal(ga, oa)
+    om, osz = orc.update(rows.ravel(), ga, dim, k, n, threads=0)
+    assert np.array_equal(sizes.read(np.uint32, k), osz)
+    assert rel_err(out.read(np.float32, k * dim), om) < CENTROID_RTOL
+    for b in (d, m, a, out, sizes):
+        b.free()
