@@ -417,6 +417,18 @@ __device__ __forceinline__ void mfma_tile(f32x16 (&acc)[P], const StepOperands<K
 	}
 }
 
+/* `if_set` in the lanes of `mask`, `otherwise` in the others, as one v_cndmask on a mask held in scalar registers. */
+__device__ __forceinline__ float select_lanes(uint64_t mask, float if_set, float otherwise)
+{
+	asm("v_cndmask_b32_e64 %0, %0, %1, %2" : "+v"(otherwise) : "v"(if_set), "s"(mask));
+	return otherwise;
+}
+__device__ __forceinline__ uint32_t select_lanes(uint64_t mask, uint32_t if_set, uint32_t otherwise)
+{
+	asm("v_cndmask_b32_e64 %0, %0, %1, %2" : "+v"(otherwise) : "v"(if_set), "s"(mask));
+	return otherwise;
+}
+
 /* Tracking with the snapshot: the minimum of the lane's 16 results of a tile (NaN-propagating tree, see track_tile), the two
  * smallest tile minima so far (m1 <= m2), the tile that holds m1 and its 16 results. */
 constexpr int SNAP_ROWS = 16;
@@ -683,42 +695,52 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 				const uint32_t tiles = rows / TILE;
 				const uint32_t tile0 = row0 / TILE;
 				constexpr int MFMAS = 3 * KB * P;
-				constexpr int CHUNKS = (SNAP ? 3 : 2) * P;    /* tracking comes in pieces of 8 to 12 operations: 2 per point tile, 3 with the snapshot */
-				static_assert(CHUNKS < MFMAS, "a step has more MFMAs than pieces of tracking");
+				/* Tracking comes in pieces that are issued one behind each MFMA, so that a wavefront is back with its next MFMA before
+				 * the matrix pipe has finished the last one. With the snapshot a point tile costs 28 operations (SNAP_OPS), spread
+				 * evenly over its share of the step's MFMAs; without it, two pieces of 11 operations. */
+				constexpr int SLOTS = MFMAS / P;                             /* MFMAs per point tile and step */
+				constexpr int SNAP_OPS = 12 + SNAP_ROWS;
+				constexpr int OPS_PER_SLOT = (SNAP_OPS + SLOTS - 1) / SLOTS;
+				constexpr int CHUNKS = SNAP ? MFMAS : 2 * P;
+				constexpr int NORMS_AFTER = SNAP ? SLOTS - 1 : CHUNKS - 1;   /* acc_old[0] is free once point tile 0 has been tracked */
+				static_assert(CHUNKS <= MFMAS, "a step has at least as many MFMAs as pieces of tracking");
 				/* One step: tile `t_new` is computed into acc_new (which holds its norms) with the centroid parts in `use`,
 				 * the centroid parts of the tile after it are requested into `fetch_into`, the tile in acc_old is tracked, and
 				 * then acc_old receives the norms of the tile that will be computed into it in the next step. The order of
 				 * the instructions is written out and fenced: the request first, then one piece of tracking behind each MFMA
-				 * (a wavefront issues them while the matrix pipe works on the MFMA), then the request for the norms, whose
-				 * answer the remaining MFMAs give time to arrive. */
+				 * (a wavefront issues them while the matrix pipe works on the MFMA), the request for the norms as soon as
+				 * acc_old[0] has been tracked: the remaining MFMAs give its answer time to arrive. */
 				auto step = [&](StepOperands<KB>& fetch_into, uint32_t t_new, f32x16 (&acc_new)[P], const StepOperands<KB>& use,
 				                f32x16 (&acc_old)[P], uint32_t tile_old) {
 					fetch_operands<KB>(fetch_into, lds_tiles, min(t_new + 1, tiles - 1), col, h);
 					__builtin_amdgcn_sched_barrier(0);
 					bool better[P][2];
+					float lowest_of_tile[P];
+					uint64_t leads[P]; /* lanes whose tile took the lead, as a mask in scalar registers */
 					int issued = 0;
+					auto lowest = [](float a, float b) { return __builtin_elementwise_minimum(a, b); };
+					/* operation u of the snapshot tracking of point tile p: 0..7 the minimum of the lane's 16 results (NaN-propagating
+					 * tree, see track_tile), 8 the second smallest tile minimum so far, 9..11 the smallest and its tile, 12.. the 16
+					 * results replace the snapshot where the tile took the lead. The selections are written as v_cndmask on the mask:
+					 * from a condition the compiler makes one branch around all of them, which undoes the spreading. */
+					auto snapshot_op = [&](int p, int u) {
+						const f32x16& a = acc_old[p];
+						if (u == 0) lowest_of_tile[p] = lowest(a[0], a[1]);
+						else if (u < 8) lowest_of_tile[p] = lowest(lowest(lowest_of_tile[p], a[2 * u]), a[2 * u + 1]);
+						else if (u == 8) st[p].m2 = __builtin_amdgcn_fmed3f(st[p].m1, st[p].m2, lowest_of_tile[p]);
+						else if (u == 9) leads[p] = __builtin_amdgcn_ballot_w64(lowest_of_tile[p] < st[p].m1);
+						else if (u == 10) st[p].tile = select_lanes(leads[p], tile_old, st[p].tile);
+						else if (u == 11) st[p].m1 = select_lanes(leads[p], lowest_of_tile[p], st[p].m1);
+						else snap[p][u - 12] = select_lanes(leads[p], a[u - 12], snap[p][u - 12]);
+					};
 					auto after_mfma = [&](int i) {
 						__builtin_amdgcn_sched_barrier(0);
 						if (i < CHUNKS) {
-							auto lowest = [](float a, float b) { return __builtin_elementwise_minimum(a, b); };
 							if constexpr (SNAP) {
-								/* piece 0: minimum of the tile's 16 results, the two smallest tile minima so far, the tile of the smallest;
-								 * pieces 1 and 2: the 16 results replace the snapshot where the tile took the lead */
-								const int p = i / 3, part = i % 3;
-								const f32x16& a = acc_old[p];
-								if (part == 0) {
-									float t = a[0];
+								const int p = i / SLOTS, first_op = (i % SLOTS) * OPS_PER_SLOT;
 #pragma unroll
-									for (int q = 1; q < 16; ++q) t = lowest(t, a[q]);
-									st[p].m2 = __builtin_amdgcn_fmed3f(st[p].m1, st[p].m2, t);
-									better[p][0] = t < st[p].m1;
-									st[p].tile = better[p][0] ? tile_old : st[p].tile;
-									st[p].m1 = better[p][0] ? t : st[p].m1;
-								}
-								else {
-#pragma unroll
-									for (int q = 8 * (part - 1); q < 8 * part; ++q) snap[p][q] = better[p][0] ? a[q] : snap[p][q];
-								}
+								for (int u = first_op; u < first_op + OPS_PER_SLOT; ++u)
+									if (u < SNAP_OPS) snapshot_op(p, u);
 							}
 							else {
 								/* the minimum of a group of 8 results (NaN-propagating tree, see track_tile), the two smallest group
@@ -733,7 +755,7 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 							}
 							__builtin_amdgcn_sched_barrier(0);
 						}
-						if (i == CHUNKS - 1) {
+						if (i == NORMS_AFTER) {
 							fetch_norms(acc_old[0], lds_norms, min(t_new + 1, tiles - 1), h);
 							__builtin_amdgcn_sched_barrier(0);
 						}
