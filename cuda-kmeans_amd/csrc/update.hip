@@ -389,10 +389,12 @@ update_private_kernel(const float* __restrict__ data, size_t stride, const uint3
  * Larger k. Grid = (point chunks, 32-wide dimension slices); work-group = 1024 lanes.
  *   1. histogram of the chunk's assignments with ds_add_rtn_u32 (the returned value is the point's rank
  *      inside its cluster); 2. exclusive scan -> cluster offsets; 3. scatter (cluster << 15 | local index)
- *      into the sorted list; 4. the sorted list is cut into one range of whole clusters per lane group
- *      (groups of GW lanes, lane = dimension), balanced by entry count; a group walks its range in batches
- *      of 8 entries (8 row loads in flight), adds in a register and stores a cluster's row of sums when the
- *      cluster changes -- zero rows for clusters without members, so the partial buffer needs no clearing.
+ *      into the sorted list; 4. the sorted list is cut into one range per lane group (groups of GW lanes,
+ *      lane = dimension), every range the same number of entries; a group walks its range in batches of 8
+ *      entries (8 row loads in flight), adds in a register and stores a cluster's row of sums when the cluster
+ *      changes -- zero rows for clusters without members, so the partial buffer needs no clearing. The pieces
+ *      of a cluster that spans ranges meet in LDS (measured at N = 2M, d = 32, k = 1024: 58 us with ranges of
+ *      whole clusters, whose sizes differed by a cluster; 50 us with equal ranges).
  * Per-chunk counts go to a second partial array (dimension slice 0 only), so that nothing has to be zero beforehand.
  * partial layouts: [chunk][cluster][dim] and [chunk][cluster].
  */
@@ -435,10 +437,10 @@ update_sorted_kernel(const float* __restrict__ data, size_t stride, const uint32
                      float* __restrict__ partial, uint32_t* __restrict__ partial_counts,
                      uint32_t dim, uint32_t k, uint32_t n, uint32_t chunk_points)
 {
-	extern __shared__ uint32_t sm[];
+	extern __shared__ __attribute__((aligned(16))) uint32_t sm[];
 	uint32_t* offsets = sm;                   /* k + 1 words: histogram, then exclusive offsets */
 	uint32_t* scratch = sm + k + 1;           /* 32 words */
-	uint32_t* sorted = scratch + 32;          /* chunk_points words */
+	uint32_t* sorted = sm + ((k + 36) & ~3u); /* chunk_points words (a multiple of 1024), then the 16-byte rows of `heads` */
 	const uint32_t tid = threadIdx.x;
 	const uint32_t lane = tid & (WAVE - 1), wave = tid / WAVE;
 	const uint32_t p_begin = (uint32_t)min((uint64_t)blockIdx.x * chunk_points, (uint64_t)n);
@@ -506,39 +508,73 @@ update_sorted_kernel(const float* __restrict__ data, size_t stride, const uint32
 	constexpr uint32_t GROUPS = 1024 / GW;
 	const uint32_t group = tid / GW, gl = tid % GW;
 	const uint32_t entries = offsets[k];
-	const uint32_t all_groups = WHOLE_ROWS ? GROUPS * gridDim.y : GROUPS; /* lane groups that share the chunk's sorted list */
-	auto first_cluster = [&](uint32_t g) -> uint32_t {
-		/* smallest c in [0, k] with offsets[c] >= g * entries / all_groups */
-		if (g >= all_groups) return k;
-		const uint32_t want = (uint32_t)((uint64_t)g * entries / all_groups);
-		uint32_t lo = 0, hi = k;
-		while (lo < hi) {
-			const uint32_t mid = (lo + hi) / 2;
-			if (offsets[mid] >= want) hi = mid; else lo = mid + 1;
-		}
-		return lo;
-	};
-	const uint32_t my_group = WHOLE_ROWS ? blockIdx.y * GROUPS + group : group;
-	const uint32_t c_lo = first_cluster(my_group), c_hi = first_cluster(my_group + 1);
 	const bool lane_on = gl * VEC < width;
 	const float* src = data + (size_t)p_begin * stride + d0 + (lane_on ? gl * VEC : 0);
 	float* out = partial + ((size_t)blockIdx.x * k) * dim + d0 + gl * VEC;
-	uint32_t cur = c_lo;
+	constexpr uint32_t LOCAL_MASK = (1u << SORT_SHIFT) - 1u;
+
+	/* the clusters [c_begin, c_stop) and their entries [e_begin, e_stop) that this work-group sums: all of them, or (WHOLE_ROWS)
+	 * one of gridDim.y ranges of whole clusters, balanced by entry count */
+	uint32_t c_begin = 0, c_stop = k;
+	if constexpr (WHOLE_ROWS) {
+		auto first_cluster = [&](uint32_t y) -> uint32_t {
+			/* smallest c in [0, k] with offsets[c] >= y * entries / gridDim.y */
+			if (y >= gridDim.y) return k;
+			const uint32_t want = (uint32_t)((uint64_t)y * entries / gridDim.y);
+			uint32_t lo = 0, hi = k;
+			while (lo < hi) {
+				const uint32_t mid = (lo + hi) / 2;
+				if (offsets[mid] >= want) hi = mid; else lo = mid + 1;
+			}
+			return lo;
+		};
+		c_begin = first_cluster(blockIdx.y);
+		c_stop = first_cluster(blockIdx.y + 1);
+	}
+	const uint32_t e_begin = offsets[c_begin], e_stop = offsets[c_stop];
+	auto cluster_at = [&](uint32_t e) -> uint32_t { return e < e_stop ? sorted[e] >> SORT_SHIFT : c_stop; };
+	auto range_begin = [&](uint32_t g) -> uint32_t { return e_begin + (uint32_t)((uint64_t)g * (e_stop - e_begin) / GROUPS); };
+
+	/* Lane group g takes the entries [range_begin(g), range_begin(g + 1)): every group the same number of rows, whatever
+	 * the cluster sizes (cut at cluster boundaries the ranges differed by a cluster's size, and the last group to finish set
+	 * the time of the work-group). A cluster that spans ranges is summed in pieces: the range it starts in keeps its piece in
+	 * registers, the ranges it continues in leave theirs in LDS, and after a barrier the first adds them up. */
+	uint32_t e = range_begin(group), e_end = range_begin(group + 1);
+	uint32_t cur, c_end;       /* cluster whose sum `acc` holds; cluster the range's last flush runs up to */
+	bool head_pending = false; /* the first cluster of the range began in an earlier range: its sum goes to `heads` */
+	bool tail_open = false;    /* the last cluster of the range goes on in later ranges: its sum waits in `acc` */
+	float* heads = (float*)(sorted + chunk_points);     /* GROUPS rows of GW * VEC floats */
+	uint32_t* whole = (uint32_t*)(heads + 1024 * VEC); /* GROUPS flags: the range lies inside one cluster that goes on behind it */
+	if (gl == 0) whole[group] = 0u;
+	if (e < e_end) {
+		const uint32_t c_first = cluster_at(e), c_last = cluster_at(e_end - 1);
+		head_pending = offsets[c_first] < e;
+		tail_open = offsets[c_last + 1] > e_end;
+		cur = e == e_begin ? c_begin : c_first; /* the group of the first entry also writes the rows of the empty clusters before it */
+		c_end = cluster_at(e_end);              /* ... and every group those behind its last cluster */
+	}
+	else {
+		/* no entry for this group; clusters without any entry still owe a row of zeros each */
+		const bool none = e_begin == e_stop;
+		cur = none ? c_begin + (uint32_t)((uint64_t)group * (c_stop - c_begin) / GROUPS) : 0u;
+		c_end = none ? c_begin + (uint32_t)((uint64_t)(group + 1) * (c_stop - c_begin) / GROUPS) : 0u;
+	}
 	RowPart<VEC> acc;
 #pragma unroll
 	for (int i = 0; i < VEC; ++i) acc.v[i] = 0.0f;
 	auto flush_to = [&](uint32_t t) {
 		while (cur < t) {
-			if (lane_on) store_part<VEC>(out + (size_t)cur * dim, acc);
+			if (head_pending) {
+				store_part<VEC>(heads + (size_t)group * (GW * VEC) + gl * VEC, acc);
+				head_pending = false;
+			}
+			else if (lane_on) store_part<VEC>(out + (size_t)cur * dim, acc);
 #pragma unroll
 			for (int i = 0; i < VEC; ++i) acc.v[i] = 0.0f;
 			++cur;
 		}
 	};
-	uint32_t e = offsets[c_lo];
-	const uint32_t e_end = offsets[c_hi];
 	/* software pipeline: the row loads of the next batch are issued before the current batch is summed */
-	constexpr uint32_t LOCAL_MASK = (1u << SORT_SHIFT) - 1u;
 	uint32_t ent[SORT_UNROLL];
 	RowPart<VEC> v[SORT_UNROLL];
 	bool have = e + SORT_UNROLL <= e_end;
@@ -574,14 +610,42 @@ update_sorted_kernel(const float* __restrict__ data, size_t stride, const uint32
 		}
 		have = more;
 	}
-	for (; e < e_end; ++e) {
-		const uint32_t one = sorted[e];
-		const RowPart<VEC> row = load_part<VEC>(src + (size_t)(one & LOCAL_MASK) * stride);
-		flush_to(one >> SORT_SHIFT);
+	if (e < e_end) {
+		/* the last entries of the range, fewer than a batch: requested together like a batch */
 #pragma unroll
-		for (int i = 0; i < VEC; ++i) acc.v[i] += row.v[i];
+		for (int u = 0; u < SORT_UNROLL; ++u) ent[u] = e + u < e_end ? sorted[e + u] : 0xFFFFFFFFu;
+#pragma unroll
+		for (int u = 0; u < SORT_UNROLL; ++u)
+			if (ent[u] != 0xFFFFFFFFu) v[u] = load_part<VEC>(src + (size_t)(ent[u] & LOCAL_MASK) * stride);
+#pragma unroll
+		for (int u = 0; u < SORT_UNROLL; ++u)
+			if (ent[u] != 0xFFFFFFFFu) {
+				flush_to(ent[u] >> SORT_SHIFT);
+#pragma unroll
+				for (int i = 0; i < VEC; ++i) acc.v[i] += v[u].v[i];
+			}
 	}
-	flush_to(c_hi);
+	bool collect = false;
+	if (tail_open) {
+		if (head_pending) {
+			/* the whole range lies inside one cluster that began before it and goes on behind it */
+			store_part<VEC>(heads + (size_t)group * (GW * VEC) + gl * VEC, acc);
+			if (gl == 0) whole[group] = 1u;
+		}
+		else collect = true;
+	}
+	else flush_to(c_end);
+	__syncthreads();
+	if (collect) {
+		for (uint32_t g = group + 1; g < GROUPS; ++g) {
+			if (range_begin(g) == range_begin(g + 1)) continue;
+			const RowPart<VEC> piece = load_part<VEC>(heads + (size_t)g * (GW * VEC) + gl * VEC);
+#pragma unroll
+			for (int i = 0; i < VEC; ++i) acc.v[i] += piece.v[i];
+			if (!whole[g]) break;
+		}
+		if (lane_on) store_part<VEC>(out + (size_t)cur * dim, acc);
+	}
 }
 
 /*
@@ -781,7 +845,7 @@ static int launch_update_tuned(const UpdateArgs& u, kmx_exec_params* exec, Works
 		}
 	}
 
-	if (LD == KMX_AOS && u.k < (1u << (32 - SORT_SHIFT)) && (uint64_t)(u.k + 33) * 4 + 1024 * 4 <= budget) {
+	if (LD == KMX_AOS && u.k < (1u << (32 - SORT_SHIFT)) && (uint64_t)(u.k + 36) * 4 + 1024 * 4 + 1024 * 5 * 4 <= budget) {
 		const uint32_t slices = (u.dim + 31) / 32;
 		/* 16-byte row parts where one slice covers the row and its alignment allows it (measured: no gain for sliced rows) */
 		const bool aligned4 = u.dim % 4 == 0 && u.stride % 4 == 0 && ((uintptr_t)u.data & 15) == 0;
@@ -791,12 +855,13 @@ static int launch_update_tuned(const UpdateArgs& u, kmx_exec_params* exec, Works
 		/* 16-byte row parts where one slice covers the row and its alignment allows it (measured: no gain for sliced rows) */
 		const uint32_t vec = ((u.dim <= 32 && aligned4) || whole_rows) ? 4 : 1;
 		const uint32_t gw = whole_rows ? std::max<uint32_t>(16, pow2_at_least(u.dim / 4)) : (u.dim > 16 ? 32 : pow2_at_least(std::max<uint32_t>(u.dim, 4))) / vec;
-		const uint32_t max_points = std::min<uint32_t>(1u << SORT_SHIFT, (budget - (u.k + 33) * 4) / 4 / 1024 * 1024);
+		const uint32_t pieces_bytes = 1024u * (vec + 1) * 4; /* sums of clusters cut by a range boundary, and a flag per lane group */
+		const uint32_t max_points = std::min<uint32_t>(1u << SORT_SHIFT, (budget - (u.k + 36) * 4 - pieces_bytes) / 4 / 1024 * 1024);
 		uint32_t chunks = std::max<uint32_t>(1, dev.compute_units / slices);
 		uint32_t chunk_points = (u.n + chunks - 1) / chunks;
 		chunk_points = std::min(max_points, (chunk_points + 1023) / 1024 * 1024);
 		chunks = (u.n + chunk_points - 1) / chunk_points;
-		const uint32_t lds_bytes = (u.k + 33 + chunk_points) * 4;
+		const uint32_t lds_bytes = (u.k + 36 + chunk_points) * 4 + pieces_bytes;
 		int rc = reserve_partials(ws, (size_t)chunks * u.k * u.dim + (size_t)chunks * u.k); /* sums, then counts */
 		if (rc) return rc;
 		exec->block_count = chunks * slices;

@@ -270,6 +270,35 @@ def test_update_matches_oracle(km, orc, gpu, dim, k, n, layout, layout_means):
             assert np.all(lm[1] == 0), "empty cluster must stay at the origin"
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("dim,k,n", [(32, 1024, 300000), (4, 4096, 200000), (256, 1024, 70000), (24, 700, 100000), (7, 300, 50000),
+                                     (64, 2048, 1 << 20), (32, 1024, 700)])
+def test_update_with_clusters_that_span_the_ranges_of_many_lane_groups(km, gpu, dim, k, n):
+    """The sorted update cuts a chunk's sorted points into equal ranges per lane group; a cluster larger than a range is
+    summed in pieces. Assignments that make such clusters (everything in one cluster, nine points in ten, sorted points,
+    two clusters) against float64 sums of the same assignment; counts exact, empty clusters at the origin."""
+    rng = np.random.default_rng(dim + k)
+    rows = (rng.normal(size=(n, dim)) * 3 + 1).astype(np.float32)
+    patterns = {
+        "all in the last": np.full(n, k - 1, np.uint32),
+        "all in the first": np.zeros(n, np.uint32),
+        "nine in ten in one": np.where(rng.random(n) < 0.9, k // 3, rng.integers(0, k, n)).astype(np.uint32),
+        "sorted": np.sort(rng.integers(0, k, n)).astype(np.uint32),
+        "two clusters": np.where(rng.random(n) < 0.5, 5, k - 2).astype(np.uint32),
+        "runs": (np.arange(n) // 1500 % k).astype(np.uint32),
+    }
+    for name, asg in patterns.items():
+        means, sizes = gpu_update(km, km.UPDATE_ATOMIC_SHM, rows.ravel(), asg, dim, k, n, AOS, AOS, km.ExecParams(), dirty=True)
+        counts = np.bincount(asg, minlength=k)
+        assert np.array_equal(sizes, counts), name
+        sums = np.zeros((k, dim)); np.add.at(sums, asg, rows.astype(np.float64))
+        want = np.where(counts[:, None] > 0, sums / np.maximum(counts, 1)[:, None], 0.0)
+        got = means.reshape(k, dim)
+        assert np.all(got[counts == 0] == 0), name
+        scale = float(np.sqrt(np.mean(want[counts > 0] ** 2)))
+        assert float(np.abs(got - want).max()) / scale < 1e-5, name
+
+
 @pytest.mark.parametrize("dim,k,n", UPDATE_SHAPES + [(8, 64, 0), (32, 1024, 0), (8, 1024, 9000000)])   # the last: more than 256 chunks of sorted points
 @pytest.mark.parametrize("layout,layout_means", [(AOS, AOS), (SOA, SOA), (AOS, SOA), (SOA, AOS)])
 def test_tuned_update_needs_no_zeroed_outputs(km, orc, gpu, dim, k, n, layout, layout_means):
