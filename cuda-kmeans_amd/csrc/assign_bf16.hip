@@ -53,6 +53,32 @@ pack_means_bf16_kernel(const float* __restrict__ means, size_t stride_means, flo
 	const uint32_t lane = threadIdx.x & (WAVE - 1);
 	const uint32_t j = (blockIdx.x * blockDim.x + threadIdx.x) / WAVE;
 	if (blockIdx.x == 0 && threadIdx.x == 0) counters[0] = 0u; /* the recheck queue of this call starts empty */
+	/* packed rows: the frame of the sweep, the mean of the first centroids (up to 1024 of them, the finite coordinates; any
+	 * vector would do, this one is near the middle of the data). Every work-group computes it, in the same order. */
+	__shared__ float frame_parts[4][4];
+	float frame[4] = { 0.0f, 0.0f, 0.0f, 0.0f };
+	if (packed_slots & 2u) {
+		const uint32_t sample = min(k, 1024u);
+		float sum[4] = { 0.0f, 0.0f, 0.0f, 0.0f };
+		for (uint32_t r = threadIdx.x; r < sample; r += 256) {
+#pragma unroll
+			for (int q = 0; q < 4; ++q) {
+				const float v = (uint32_t)q < dim ? means[elem<LM>(stride_means, r, q)] : 0.0f;
+				sum[q] += __builtin_fabsf(v) < __builtin_inff() ? v : 0.0f;
+			}
+		}
+		for (int off = WAVE / 2; off > 0; off >>= 1)
+			for (int q = 0; q < 4; ++q) sum[q] += __shfl_xor(sum[q], off);
+		if (lane == 0)
+			for (int q = 0; q < 4; ++q) frame_parts[threadIdx.x / WAVE][q] = sum[q];
+		__syncthreads();
+		for (int q = 0; q < 4; ++q) frame[q] = (frame_parts[0][q] + frame_parts[1][q] + frame_parts[2][q] + frame_parts[3][q]) / (float)sample;
+	}
+	if ((packed_slots & 1u) && blockIdx.x == 0) {
+#pragma unroll
+		for (int q = 0; q < 4; ++q)
+			if (threadIdx.x == (uint32_t)q) norms[frame_offset(kp) + q] = frame[q];
+	}
 	if (j >= kp) return;
 	const uint32_t rs = packed_slots ? row_floats<1, true>() : dp + ROW_PAD;
 	float* row = packed + packed_row(j, rs);
@@ -64,7 +90,8 @@ pack_means_bf16_kernel(const float* __restrict__ means, size_t stride_means, flo
 		 * of the point's parts) */
 		if (lane < KBLOCK) {
 			const uint32_t q = lane % 4;
-			const float v = (j < k && q < dim) ? means[elem<LM>(stride_means, j, q)] : 0.0f;
+			const float exact = (j < k && q < dim) ? means[elem<LM>(stride_means, j, q)] : 0.0f;
+			const float v = (j < k && q < dim) ? exact - (q == 0 ? frame[0] : q == 1 ? frame[1] : q == 2 ? frame[2] : frame[3]) : 0.0f;
 			__bf16 hi, mid;
 			const float rest = split_bf16(-2.0f * v, hi, mid);
 			float* tile = packed + (size_t)(j / TILE) * tile_floats(rs);
@@ -74,7 +101,7 @@ pack_means_bf16_kernel(const float* __restrict__ means, size_t stride_means, flo
 				c2 = v * v;
 				mid2 = (float)mid * (float)mid;
 				rest2 = rest * rest;
-				if (q < dim) means_t[(size_t)q * kp + j] = v; /* exact copy for the recheck pass */
+				if (q < dim) means_t[(size_t)q * kp + j] = exact; /* exact copy for the recheck pass */
 			}
 		}
 	}
@@ -143,23 +170,30 @@ int launch_screen_bf16(const float* rows, const Workspace* ws, const uint32_t* r
 #undef KMX_SCREEN_CASE
 }
 
-int launch_assign_bf16(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev)
+int launch_assign_bf16(const AssignArgs& args, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev)
 {
+	AssignArgs a = args;
+	/* wide rows and many centroids: a second sweep screens the queued points (narrow rows fit the registers of the
+	 * lane-per-centroid kernels, which then need fewer launches); so do the packed rows, whose sweep queues more points
+	 * than the fp32 one and screens a tile with a single MFMA */
+	const bool screened = !a.ranking_only && a.k >= 128 && (a.dim > 32 || packed_rows(a.dim));
+	a.shift_rows = screened && packed_rows(a.dim);
+	a.shifted_cap = a.shift_rows ? screened_rows_cap(a) : 0xFFFFFFFFu;
 	const uint32_t kb = pick_kb(a.dim);
 	const uint32_t dp = KBLOCK * kb;
 	const uint32_t kp = round_up(a.k, TILE);
 	const uint32_t rs = packed_rows(a.dim) ? row_floats<1, true>() : dp + ROW_PAD;
-	int rc = reserve_packed(ws, (size_t)(kp / TILE) * tile_floats(rs), split_norms_offset(kp) + 2 * (size_t)kp, (size_t)kp * a.dim);
+	int rc = reserve_packed(ws, (size_t)(kp / TILE) * tile_floats(rs), frame_offset(kp) + 4, (size_t)kp * a.dim);
 	if (rc) return rc;
 	rc = reserve_queue(ws, 2 * (size_t)a.n); /* (point, threshold) pairs */
 	if (rc) return rc;
 	const uint32_t pack_blocks = (kp * WAVE + 255) / 256;
 	if (a.layout_means == KMX_AOS)
 		KMX_LAUNCH_KERNEL((pack_means_bf16_kernel<KMX_AOS>), dim3(pack_blocks), dim3(256), 0, stream(),
-		                   a.means, a.stride_means, ws->packed_means, ws->norms, ws->means_t, a.dim, a.k, kp, dp, packed_rows(a.dim) ? 1u : 0u, ws->counters);
+		                   a.means, a.stride_means, ws->packed_means, ws->norms, ws->means_t, a.dim, a.k, kp, dp, (packed_rows(a.dim) ? 1u : 0u) | (a.shift_rows ? 2u : 0u), ws->counters);
 	else
 		KMX_LAUNCH_KERNEL((pack_means_bf16_kernel<KMX_SOA>), dim3(pack_blocks), dim3(256), 0, stream(),
-		                   a.means, a.stride_means, ws->packed_means, ws->norms, ws->means_t, a.dim, a.k, kp, dp, packed_rows(a.dim) ? 1u : 0u, ws->counters);
+		                   a.means, a.stride_means, ws->packed_means, ws->norms, ws->means_t, a.dim, a.k, kp, dp, (packed_rows(a.dim) ? 1u : 0u) | (a.shift_rows ? 2u : 0u), ws->counters);
 	KMX_LAUNCH_CHECK("pack_means_bf16_kernel");
 
 	/* tau = kd (|x|^2 + max|c|^2) + the bound of the dropped products (certificate.h) */
@@ -175,10 +209,7 @@ int launch_assign_bf16(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws
 	}
 	if (rc) return rc;
 	if (a.ranking_only) return KMX_OK; /* the caller resolves the queued points */
-	/* wide rows and many centroids: a second sweep screens the queued points (narrow rows fit the registers of the
-	 * lane-per-centroid kernels, which then need fewer launches); so do the packed rows, whose sweep queues four times
-	 * as many points as the fp32 one and screens a tile with a single MFMA */
-	return a.k >= 128 && (a.dim > 32 || packed_rows(a.dim)) ? launch_recheck_screened(a, ws, kp, dev) : launch_recheck(a, ws, kp);
+	return screened ? launch_recheck_screened(a, ws, kp, dev) : launch_recheck(a, ws, kp);
 }
 
 } // namespace kmx

@@ -43,6 +43,9 @@ __device__ __forceinline__ float split_bf16(float v, __bf16& hi, __bf16& mid)
 /* The norms array of the split-bf16 kernels: the tiles of |c|^2 (NORM_TILE floats per tile), then per padded row
  * sum_i c'mid_i^2 and, kp floats on, sum_i c'rest_i^2 (c' = -2c; what the certificate needs, see certificate.h). */
 __host__ __device__ __forceinline__ size_t split_norms_offset(uint32_t kp) { return (size_t)(kp / TILE) * NORM_TILE; }
+/* ... and behind those the 4 coordinates of the frame the packed rows are swept in (zeros: the frame of the data) */
+__host__ __device__ __forceinline__ size_t frame_offset(uint32_t kp) { return split_norms_offset(kp) + 2 * (size_t)kp; }
+struct Frame { float m[4]; };
 
 /* One tile of 32 points as B operands: per block of 16 dimensions the lane holds the 8 dimensions of its
  * half-wave (lanes 0-31: the first 8, lanes 32-63: the second 8) of ONE point, as hi and mid parts. */
@@ -86,14 +89,14 @@ __device__ __forceinline__ void request_packed_points(RawPoints<1, true> (&raw)[
 }
 
 template <int P>
-__device__ __forceinline__ void convert_packed_points(SplitPoints<1> (&b)[P], float (&xx)[P], const RawPoints<1, true> (&raw)[P], uint32_t h)
+__device__ __forceinline__ void convert_packed_points(SplitPoints<1> (&b)[P], float (&xx)[P], const RawPoints<1, true> (&raw)[P], uint32_t h, const Frame& frame)
 {
 #pragma unroll
 	for (int p = 0; p < P; ++p) {
 		float part = 0.0f, rest2 = 0.0f;
 #pragma unroll
 		for (int j = 0; j < 4; ++j) {
-			const float v = raw[p].v[j];
+			const float v = raw[p].v[j] - frame.m[j];
 			part += v * v;
 			__bf16 hi, mid;
 			const float rest = split_bf16(v, hi, mid);
@@ -109,11 +112,11 @@ __device__ __forceinline__ void convert_packed_points(SplitPoints<1> (&b)[P], fl
 
 template <int P, int LD, bool VEC>
 __device__ __forceinline__ void load_packed_points(SplitPoints<1> (&b)[P], float (&xx)[P], const float* __restrict__ data, size_t stride,
-                                                   uint32_t base, uint32_t col, uint32_t h, uint32_t dim, uint32_t n)
+                                                   uint32_t base, uint32_t col, uint32_t h, uint32_t dim, uint32_t n, const Frame& frame)
 {
 	RawPoints<1, true> raw[P];
 	request_packed_points<P, LD, VEC>(raw, data, stride, base, col, dim, n);
-	convert_packed_points<P>(b, xx, raw, h);
+	convert_packed_points<P>(b, xx, raw, h, frame);
 }
 
 template <int KB, int P, int LD, bool VEC>
@@ -460,10 +463,15 @@ template <int KB, int P, int LD, bool VEC, bool STREAM, bool COARSE, bool PREFET
 __global__ void __launch_bounds__(MFMA_WAVES * WAVE)
 assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* __restrict__ packed, const float* __restrict__ norms,
                    uint32_t* __restrict__ assignment, uint32_t* __restrict__ queue, uint32_t* __restrict__ counters,
-                   uint32_t dim, uint32_t k, uint32_t kp, uint32_t n, uint32_t chunk_rows, float kd, float neg_inf)
+                   uint32_t dim, uint32_t k, uint32_t kp, uint32_t n, uint32_t chunk_rows, float kd, float neg_inf, uint32_t shifted_cap)
 {
 	constexpr uint32_t RS = row_floats<KB, PACKED>();
 	extern __shared__ __attribute__((aligned(16))) float lds[];
+	Frame frame = { { 0.0f, 0.0f, 0.0f, 0.0f } }; /* PACKED: the rows are swept as x - frame (pack_means_bf16_kernel moved the centroids alike) */
+	if constexpr (PACKED) {
+#pragma unroll
+		for (int j = 0; j < 4; ++j) frame.m[j] = norms[frame_offset(kp) + j];
+	}
 	__shared__ uint32_t wave_max[4][MFMA_WAVES]; /* rows 0..2: maxima per wavefront; [3][0]: items of this work-group handed out so far */
 	__shared__ uint32_t flag_list[MFMA_WAVES][2 * FLAG_CAP]; /* (point, threshold) pairs */
 	uint32_t& claimed = wave_max[3][0]; /* (kept inside an array whose size is a multiple of 16 bytes: the tiles behind the static data must stay 16-byte aligned for their 128-bit reads) */
@@ -565,7 +573,9 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 		uint32_t slot = 0;
 		if (lane == 0) slot = atomicAdd(&counters[0], flagged);
 		slot = (uint32_t)__shfl((int)slot, 0);
-		for (uint32_t i = lane; i < 2 * flagged; i += WAVE) queue[2 * (size_t)slot + i] = flag_list[wave][i];
+		/* (entries from shifted_cap on: thresholds of a moved frame mean nothing to the kernels that will read them) */
+		for (uint32_t i = lane; i < 2 * flagged; i += WAVE)
+			queue[2 * (size_t)slot + i] = (PACKED && (i & 1u) && slot + i / 2 >= shifted_cap) ? __float_as_uint(__builtin_inff()) : flag_list[wave][i];
 		__builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
 		__builtin_amdgcn_wave_barrier();
 		flagged = 0;
@@ -1035,7 +1045,7 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 
 	static_assert(!PACKED || KB == 1, "the packed form is one block of 16 slots");
 	auto load_points = [&](SplitPoints<KB> (&bb)[P], float (&xs)[P], uint32_t first) {
-		if constexpr (PACKED) load_packed_points<P, LD, VEC>(bb, xs, data, stride, first, col, h, dim, n);
+		if constexpr (PACKED) load_packed_points<P, LD, VEC>(bb, xs, data, stride, first, col, h, dim, n, frame);
 		else load_split_points<KB, P, LD, VEC>(bb, xs, data, stride, first, col, h, dim, n);
 	};
 
@@ -1075,7 +1085,7 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 			else request_split_points<KB, P, LD, VEC>(raw, data, stride, first, col, h, dim, n);
 		};
 		auto convert_points = [&]() {
-			if constexpr (PACKED) convert_packed_points<P>(b0, xx0, raw, h);
+			if constexpr (PACKED) convert_packed_points<P>(b0, xx0, raw, h, frame);
 			else convert_split_points<KB, P>(b0, xx0, raw);
 		};
 		uint32_t item = uniform(claim());
@@ -1147,6 +1157,11 @@ screen_bf16_kernel(const float* __restrict__ rows, const float* __restrict__ pac
 	const uint32_t tiles = kp / TILE;
 	const uint32_t waves = gridDim.x * SCREEN_WAVES;
 	const ScreenItems work = screen_items(count, unit_rows, tiles, waves);
+	Frame frame = { { 0.0f, 0.0f, 0.0f, 0.0f } }; /* PACKED: the frame of the first sweep */
+	if constexpr (PACKED) {
+#pragma unroll
+		for (int j = 0; j < 4; ++j) frame.m[j] = norms[frame_offset(kp) + j];
+	}
 
 	struct Operands { bf16x8 hi[G], mid[G]; };
 
@@ -1178,7 +1193,7 @@ screen_bf16_kernel(const float* __restrict__ rows, const float* __restrict__ pac
 		written = 0;
 		SplitPoints<KB> b[P];
 		float xx[P];
-		if constexpr (PACKED) load_packed_points<P, KMX_AOS, false>(b, xx, rows, dim, base, col, h, dim, count);
+		if constexpr (PACKED) load_packed_points<P, KMX_AOS, false>(b, xx, rows, dim, base, col, h, dim, count, frame);
 		else load_split_points<KB, P, KMX_AOS, false>(b, xx, rows, dim, base, col, h, dim, count);
 		float thr[P];
 		bool valid[P];
@@ -1351,7 +1366,7 @@ static int launch_bf16_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 	const uint32_t unit_points = MFMA_WAVES * (stream_mode ? P : PR) * TILE;
 	const uint32_t units = (a.n + unit_points - 1) / unit_points;
 	void (*kernel)(const float*, size_t, const float*, const float*, uint32_t*, uint32_t*, uint32_t*,
-	               uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, float, float) = nullptr;
+	               uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, float, float, uint32_t) = nullptr;
 	if constexpr (KB <= 4) {
 		if (stream_mode) kernel = coarse ? assign_bf16_kernel<KB, P, LD, VEC, true, true, PF, PACKED> : assign_bf16_kernel<KB, P, LD, VEC, true, false, PF, PACKED>;
 		else kernel = coarse ? assign_bf16_kernel<KB, PR, LD, VEC, false, true, PF, PACKED> : assign_bf16_kernel<KB, PR, LD, VEC, false, false, PF, PACKED>;
@@ -1369,7 +1384,7 @@ static int launch_bf16_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 	if (rc) return rc;
 	KMX_LAUNCH_KERNEL(kernel, dim3(grid), dim3(MFMA_WAVES * WAVE), lds_bytes, stream(),
 	                   a.data, a.stride, ws->packed_means, ws->norms, a.assignment, ws->queue, ws->counters,
-	                   a.dim, a.k, kp, a.n, chunk_rows, kd, -__builtin_inff());
+	                   a.dim, a.k, kp, a.n, chunk_rows, kd, -__builtin_inff(), a.shifted_cap);
 	KMX_LAUNCH_CHECK("assign_bf16_kernel");
 	return profile_end(0);
 }

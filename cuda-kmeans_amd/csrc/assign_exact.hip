@@ -730,9 +730,14 @@ static uint32_t queued_rows_cap(const AssignArgs& a)
 	return (uint32_t)std::min<size_t>(a.n, std::max<size_t>(1024, g_queued_rows_bytes / ((size_t)a.dim * sizeof(float))));
 }
 
+uint32_t screened_rows_cap(const AssignArgs& a)
+{
+	return std::min<uint32_t>(queued_rows_cap(a), 4u << 20); /* the pair list takes 32 bytes per row */
+}
+
 int launch_recheck_screened(const AssignArgs& a, Workspace* ws, uint32_t kp, const DeviceInfo& dev)
 {
-	const uint32_t cap = std::min<uint32_t>(queued_rows_cap(a), 4u << 20); /* the pair list takes 32 bytes per row */
+	const uint32_t cap = screened_rows_cap(a);
 	const uint32_t unit_rows = screen_unit_rows(a.dim);
 	const uint32_t items_max = screen_items_max(cap, unit_rows);
 	const size_t slice_words = 2 * (size_t)SCREEN_SLICE_PER_ROW * unit_rows;

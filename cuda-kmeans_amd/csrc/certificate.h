@@ -29,8 +29,12 @@
  *        accumulation <= (4 d + 2) u' 2 S
  *        dropped = sum_i (c'hi_i + c'mid_i) xrest_i + c'rest_i x_i <= (|c'| + |c'rest|) |xrest| + |c'rest| |x|
  *     with |xrest| of the point computed when it is split.
+ *     The packed sweep may work in a frame moved by a vector m (the middle of the centroids), on x' = fl(x - m) and
+ *     c' = fl(c - m): distances do not depend on the frame, S becomes |x'|^2 + max_j |c'_j|^2, which is what makes tau
+ *     small for data far from the origin, and the two roundings move a distance by at most 2 u (|x'| + |c'|)^2 <= 2 u' S,
+ *     a difference of two distances by 4 u' S: 8 u' more in kd.
  * tau = kd S + TRUNC_FACTOR * (bound of the dropped products); kd = (12 d + 8 + 2 d + 12 + slack) u' and
- * (16 d + 8 + 2 d + 12 + slack) u'; TRUNC_FACTOR = 2 plus 1/16 for the fp32 roundings in the norms and square roots.
+ * (16 d + 8 + 2 d + 12 + 8 + slack) u'; TRUNC_FACTOR = 2 plus 1/16 for the fp32 roundings in the norms and square roots.
  * Values the bound does not cover (NaN, infinities, sums that overflow) make tau NaN or infinite, and the
  * comparison `second - first > tau` is then false: the point goes to the exact pass.
  */
@@ -56,7 +60,7 @@ struct CentroidBounds {
 
 KMX_HD float cert_kd_fp32(unsigned dim) { return (8.0f * (float)dim + 24.0f) * CERT_UNIT; }
 KMX_HD float cert_kd_split(unsigned dim) { return (14.0f * (float)dim + 28.0f) * CERT_UNIT; }
-KMX_HD float cert_kd_packed(unsigned dim) { return (18.0f * (float)dim + 28.0f) * CERT_UNIT; }
+KMX_HD float cert_kd_packed(unsigned dim) { return (18.0f * (float)dim + 36.0f) * CERT_UNIT; }
 
 /* The bound in the form the kernels evaluate per point: tau = kd (x2 + c2max) + a sqrt(xpart2) + b sqrt(x2), with
  * xpart2 = sum_i xmid_i^2 (three-product form) or sum_i xrest_i^2 (packed form); a and b depend on the centroids only. */

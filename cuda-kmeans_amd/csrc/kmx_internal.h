@@ -114,6 +114,11 @@ struct AssignArgs {
 	 * uncertified points (pairs of point number and threshold, length in counters[0]) to the caller. */
 	float kd_extra = 0.0f;
 	bool ranking_only = false;
+	/* Packed rows (at most 4 dimensions) whose exact pass is the screened one are swept in a frame moved to the middle of the
+	 * centroids (shift_rows): the thresholds of the queue are then values of that frame, which only the screen shares, so
+	 * entries from position shifted_cap on -- those the screen has no rows for -- get an infinite threshold. */
+	bool shift_rows = false;
+	uint32_t shifted_cap = 0xFFFFFFFFu;
 };
 
 struct UpdateArgs {
@@ -138,6 +143,7 @@ void set_queued_rows_limit(size_t bytes); /* bound of the block of copied rows *
  * split-bf16 sweep over them notes the (row, centroid) pairs within the threshold (assign_bf16.hip), and one lane
  * per pair evaluates the serial arithmetic. */
 int launch_recheck_screened(const AssignArgs& a, Workspace* ws, uint32_t kp, const DeviceInfo& dev);
+uint32_t screened_rows_cap(const AssignArgs& a); /* queue entries the screened exact pass has rows for */
 int launch_screen_bf16(const float* rows, const Workspace* ws, const uint32_t* row_queue, const uint32_t* row_count,
                        uint32_t* pairs, uint32_t* item_pairs, unsigned long long* keys, uint32_t dim, uint32_t k, uint32_t kp,
                        const DeviceInfo& dev, uint32_t* waves);

@@ -65,7 +65,7 @@ def worst_parts(rng, shape, mid_sign, rest_sign):
     return 1.0 + m * 2.0 ** -17
 
 
-def worst_case_pairs(dim, pairs, per_pair, rng, shared_mid_signs):
+def worst_case_pairs(dim, pairs, per_pair, rng, shared_mid_signs, mirrored=False):
     """Near-ties on which every product the split drops has one sign for one centroid and the other sign for its rival.
     All centroids of even index agree in sign with the points on half of the coordinates, those of odd index on the other
     half, so a point is about equally far from both kinds; the signs of the mid and rest parts are chosen per coordinate
@@ -79,6 +79,8 @@ def worst_case_pairs(dim, pairs, per_pair, rng, shared_mid_signs):
     c = np.empty((2 * pairs, dim))
     c[0::2] = sx * match * worst_parts(rng, (pairs, dim), match * mid_sign, match * np.ones((pairs, dim)))
     c[1::2] = -sx * match * worst_parts(rng, (pairs, dim), match * mid_sign, match * np.ones((pairs, dim)))
+    if mirrored:   # the odd kind the exact negatives of the even kind: every product changes sign, and the centroids' mean is 0
+        c[1::2] = -c[0::2]
     pid = np.repeat(np.arange(pairs), per_pair)
     x = sx * worst_parts(rng, (pairs * per_pair, dim), mid_sign[pid], match * np.ones((pairs * per_pair, dim)))
     return x.astype(np.float32), c.astype(np.float32)
@@ -88,9 +90,10 @@ def worst_case_pairs(dim, pairs, per_pair, rng, shared_mid_signs):
 WORST_CASE_SHAPES = [(2, 32, False), (3, 32, False), (4, 32, False), (8, 4, True), (16, 2, True), (32, 1, True), (64, 1, True)]
 
 
-def worst_case_inputs(dim, n=64000):
-    pairs, shared = next((p, s) for d, p, s in WORST_CASE_SHAPES if d == dim)
-    return worst_case_pairs(dim, pairs, n // pairs, np.random.default_rng(dim), shared)
+def worst_case_inputs(dim, n=64000, mirrored=False, pairs=None):
+    default_pairs, shared = next((p, s) for d, p, s in WORST_CASE_SHAPES if d == dim)
+    pairs = pairs or default_pairs
+    return worst_case_pairs(dim, pairs, n // pairs, np.random.default_rng(dim), shared, mirrored)
 
 
 def near_ties(dim, n, k, rng, offset, centroids=None):
@@ -174,6 +177,49 @@ def test_tau_covers_the_split_and_the_serial_margin(km, dim, packed, kind):
     certified[j1, np.arange(n)] = False
     wrong = certified & ~(dist[j1, np.arange(n)][None, :] < dist)
     assert not wrong.any(), "%d certified pairs contradict the serial comparison" % int(wrong.sum())
+
+
+@pytest.mark.parametrize("dim", [2, 3, 4])
+@pytest.mark.parametrize("kind", ["ties0", "ties100", "ties10000", "uniform", "mirrored pairs"])
+def test_tau_in_a_moved_frame_covers_the_distances_of_the_data(km, dim, kind):
+    """Packed rows are swept as fl(x - m), fl(c - m) with m near the middle of the centroids. The ranking values of that
+    frame, against the exact ones of the unrounded differences (distances do not depend on the frame): the frame's tau,
+    from the frame's norms, covers what the split drops and the two roundings; what it certifies is a strict serial win on
+    the data as given."""
+    rng = np.random.default_rng(dim * 17 + len(kind))
+    n, k = 4096, 160
+    if kind == "uniform":
+        x, c = rng.random((n, dim)).astype(np.float32), rng.random((k, dim)).astype(np.float32)
+    elif kind == "mirrored pairs":
+        x, c = worst_case_inputs(dim, 8192, mirrored=True, pairs=80)
+        n = x.shape[0]
+    else:
+        x, c = near_ties(dim, n, k, rng, float(kind[4:]))
+    m = (c.sum(0, dtype=np.float32) / np.float32(c.shape[0])).astype(np.float32)
+    if kind == "mirrored pairs":
+        assert not m.any()
+    xs, cs = (x - m).astype(np.float32), (c - m).astype(np.float32)
+    a, _, nm = emulate(xs, cs, True)
+    xd, cd = x.astype(np.float64) - m.astype(np.float64), c.astype(np.float64) - m.astype(np.float64)
+    exact = (cd ** 2).sum(1)[:, None] - 2 * cd @ xd.T
+    tau = np.array([km.certificate_tau(2, dim, float(nm["x2"][i]), float(nm["xrest2"][i]), nm["c2max"], nm["cmid2max"], nm["crest2max"])
+                    for i in range(n)], np.float64)
+    s_all = nm["x2"].astype(np.float64) + nm["c2max"]
+    accumulation = (4 * dim + 2) * U * 2 * s_all
+    margin = (2 * dim + 12) * U * s_all
+    off = np.abs(a - exact).max(0)
+    assert np.all(2 * off + 2 * accumulation + margin <= tau), "worst ratio %.3f" % float(((2 * off + 2 * accumulation + margin) / tau).max())
+    dist = serial_distances(x, c)
+    j1 = a.argmin(0)
+    certified = (a - a[j1, np.arange(n)][None, :]) + 2 * accumulation[None, :] > tau[None, :]
+    certified[j1, np.arange(n)] = False
+    wrong = certified & ~(dist[j1, np.arange(n)][None, :] < dist)
+    assert not wrong.any(), "%d certified pairs contradict the serial comparison" % int(wrong.sum())
+    if kind in ("ties100", "ties10000"):   # the point of the frame: tau follows the spread of the data, not its distance from the origin
+        _, _, nm0 = emulate(x, c, True)
+        tau0 = np.array([km.certificate_tau(2, dim, float(nm0["x2"][i]), float(nm0["xrest2"][i]), nm0["c2max"], nm0["cmid2max"],
+                                            nm0["crest2max"]) for i in range(n)])
+        assert np.median(tau) < np.median(tau0) / 50   # (the points with the largest gaps lie far from the centroids in any frame)
 
 
 @pytest.mark.parametrize("dim,packed,old_units", [(2, True, 18 * 2 + 149), (8, False, 14 * 8 + 224), (16, False, 14 * 16 + 224)])

@@ -48,6 +48,24 @@ def test_worst_case_pairs_match_the_serial_scan(km, orc, gpu, dim):
     d.free()
 
 
+@pytest.mark.parametrize("dim", [2, 3, 4])
+def test_worst_case_pairs_in_the_moved_frame_of_the_packed_sweep(km, orc, gpu, dim):
+    """From 128 centroids on the packed sweep works in a frame moved to the centroids' mean. 128 centroids in mirrored pairs
+    have the mean 0 exactly, so the frame is the data's own and the worst-case signs of the dropped products survive."""
+    x, c = worst_case_inputs(dim, 64000, mirrored=True, pairs=64)
+    n, k = x.shape[0], c.shape[0]
+    assert k == 128
+    data, means = np.ascontiguousarray(x).ravel(), np.ascontiguousarray(c).ravel()
+    want = orc.assign(data, means, dim, k, n, threads=0, fast=True)
+    d = km.DeviceBuffer(data.nbytes); d.write(data)
+    for v in (km.ASSIGN_BEST, km.ASSIGN_MFMA_BF16X3):
+        got, rechecked = assign_all(km, d, means, dim, k, n, v)
+        bad = np.nonzero(got != want)[0]
+        assert bad.size == 0, "variant %d: %d of %d points differ from the serial scan (first %s), %d went to the exact pass" % (
+            v, bad.size, n, bad[:5], rechecked)
+    d.free()
+
+
 def test_quoted_packed_example_of_a_wrong_decision(km, orc, gpu):
     """Two dimensions, x between c1 and c2 with a true gap below what the split drops: the ranking values differ by more
     than (18 d + 149) u' S in favour of c2 while the serial scan returns c1."""
