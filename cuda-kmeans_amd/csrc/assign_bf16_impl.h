@@ -442,7 +442,7 @@ __device__ __forceinline__ void track_snapshot(const f32x16& acc, Track& s, floa
 #pragma unroll
 	for (int i = 1; i < 16; ++i) t = lowest(t, acc[i]);
 	s.m2 = __builtin_amdgcn_fmed3f(s.m1, s.m2, t); /* second smallest of {m1, m2, t} as m1 <= m2 */
-	const bool lt = t < s.m1;
+	const bool lt = t < s.m1 || tile == 0; /* tile 0 fills the snapshot, whatever its values */
 	s.tile = lt ? tile : s.tile;
 	s.m1 = lt ? t : s.m1;
 #pragma unroll
@@ -691,7 +691,7 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 #pragma unroll
 			for (int p = 0; p < P; ++p) {
 #pragma unroll
-				for (int i = 0; i < (SNAP ? SNAP_ROWS : 1); ++i) snap[p][i] = __builtin_inff();
+				for (int i = 0; i < (SNAP ? SNAP_ROWS : 1); ++i) asm volatile("" : "=v"(snap[p][i])); /* no value yet: tile 0 always takes the lead */
 			}
 			for (uint32_t chunk = 0; chunk < chunks; ++chunk) {
 				const uint32_t row0 = chunk * chunk_rows;
@@ -738,7 +738,7 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 						if (u == 0) lowest_of_tile[p] = lowest(a[0], a[1]);
 						else if (u < 8) lowest_of_tile[p] = lowest(lowest(lowest_of_tile[p], a[2 * u]), a[2 * u + 1]);
 						else if (u == 8) st[p].m2 = __builtin_amdgcn_fmed3f(st[p].m1, st[p].m2, lowest_of_tile[p]);
-						else if (u == 9) leads[p] = __builtin_amdgcn_ballot_w64(lowest_of_tile[p] < st[p].m1);
+						else if (u == 9) leads[p] = tile_old == 0 ? ~0ull : __builtin_amdgcn_ballot_w64(lowest_of_tile[p] < st[p].m1); /* (tile 0 fills the snapshot, whatever its values) */
 						else if (u == 10) st[p].tile = select_lanes(leads[p], tile_old, st[p].tile);
 						else if (u == 11) st[p].m1 = select_lanes(leads[p], lowest_of_tile[p], st[p].m1);
 						else snap[p][u - 12] = select_lanes(leads[p], a[u - 12], snap[p][u - 12]);

@@ -82,9 +82,21 @@ KMX_HD CertCoeffs cert_coeffs_packed(const CentroidBounds& c)
 	return CertCoeffs{ c.c2max, CERT_TRUNC_FACTOR * (cnorm + crest), CERT_TRUNC_FACTOR * crest };
 }
 
+/* a square root that is never below the true one: on the device the hardware's approximation (1 ulp) of an argument kept out
+ * of the subnormal range, a millionth added, instead of the correctly rounded sequence of 18 instructions the kernels are
+ * compiled with; NaN stays NaN */
+KMX_HD float cert_sqrt_upper(float v)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+	return __builtin_amdgcn_sqrtf(v < 1e-30f ? 1e-30f : v) * 1.000001f;
+#else
+	return __builtin_sqrtf(v);
+#endif
+}
+
 KMX_HD float cert_tau(float kd, float x2, float xpart2, const CertCoeffs& c)
 {
-	return kd * (x2 + c.c2max) + (c.a * __builtin_sqrtf(xpart2) + c.b * __builtin_sqrtf(x2));
+	return kd * (x2 + c.c2max) + (c.a * cert_sqrt_upper(xpart2) + c.b * cert_sqrt_upper(x2));
 }
 
 } // namespace kmx
