@@ -2,7 +2,7 @@
  * Assignment on the vector ALUs: one lane per point, the point's coordinates in registers, the packed centroids
  * (-2c rows and |c|^2, the same block pack_means_kernel writes for the MFMA variant) in LDS, read as broadcasts;
  * a[j] = |c_j|^2 - 2 c_j . x by plain v_fma_f32, exact (min, second min, argmin) tracking per lane, and the same
- * certification / recheck queue as the MFMA variant (see assign_mfma.hip for the error bound).
+ * certification / recheck queue as the MFMA variant (the bound of a chain of fused multiply-adds: certificate.h).
  *
  * With a handful of centroids (the packed block within 8 KB: k = 16 at d = 16, k = 64 at d = 8) the rows are not staged
  * in LDS at all: they are read with wave-uniform addresses, i.e. as scalar loads through the scalar cache, and feed
@@ -215,7 +215,7 @@ int launch_assign_lds_fma(const AssignArgs& a, kmx_exec_params* exec, Workspace*
 	const uint32_t kp = round_up(a.k, TILE);
 	int rc = launch_pack_means(a, ws, dp, kp);
 	if (rc) return rc;
-	const float kd = cert_kd_fp32(a.dim) + a.kd_extra;
+	const float kd = cert_kd_fma(a.dim) + a.kd_extra;
 	switch (dp) {
 	case 4: rc = launch_fma_dp<4>(a, exec, ws, dev, kp, kd); break;
 	case 8: rc = launch_fma_dp<8>(a, exec, ws, dev, kp, kd); break;

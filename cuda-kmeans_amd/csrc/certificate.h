@@ -9,8 +9,13 @@
  * the serial margin being the error of two serial sums plus what a correctly rounded sqrt can merge:
  * (2 d + 12) u' S with u' = 2^-23 and S = |x|^2 + max_j |c_j|^2.
  *
- * fp32 sweeps: |a[j] - A_j| <= (d + 2) u' (|c_j|^2 + 2 |x||c_j|) <= (d + 2) u' 2 S  ->  tau = (8 d + 24) u' S
+ * fp32 MFMA sweeps: |a[j] - A_j| <= (d + 2) u' (|c_j|^2 + 2 |x||c_j|) <= (d + 2) u' 2 S  ->  tau = (8 d + 24) u' S
  * (one u' per accumulation step allows for any rounding or truncation inside the matrix core).
+ *
+ * Sweeps on the vector ALU (a chain of d v_fma_f32 that starts from the fp32 norm; round to nearest, unit roundoff
+ * u = u'/2): the norm carries at most 7 u |c_j|^2 (one product per lane, six levels of the wavefront sum), every fused
+ * multiply-add rounds a running value of at most |c_j|^2 + 2 |c_j||x| <= 2 S once, so |a[j] - A_j| <= (2 d + 7) u S and
+ * twice that plus the serial margin is (4 d + 19) u' S  ->  tau = (4 d + 24) u' S, about half the MFMA bound.
  *
  * Split-bf16 sweeps. Every operand v is hi + mid + rest with hi = bf16(v), mid = bf16(v - hi), both rounded to nearest:
  * a bf16 has 8 significant bits, so |mid| <= 2^-8 |v|, |rest| <= 2^-8 |mid| <= 2^-17 |v| (the worst case is
@@ -59,6 +64,7 @@ struct CentroidBounds {
 };
 
 KMX_HD float cert_kd_fp32(unsigned dim) { return (8.0f * (float)dim + 24.0f) * CERT_UNIT; }
+KMX_HD float cert_kd_fma(unsigned dim) { return (4.0f * (float)dim + 24.0f) * CERT_UNIT; }
 KMX_HD float cert_kd_split(unsigned dim) { return (14.0f * (float)dim + 28.0f) * CERT_UNIT; }
 KMX_HD float cert_kd_packed(unsigned dim) { return (18.0f * (float)dim + 36.0f) * CERT_UNIT; }
 

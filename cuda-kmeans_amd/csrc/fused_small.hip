@@ -301,7 +301,7 @@ static int launch_fused_layouts(const AssignArgs& a, float* means_out, uint32_t*
 	const uint32_t kp = round_up(a.k, TILE);
 	int rc = launch_pack_means(a, ws, dp, kp);
 	if (rc) return rc;
-	const float kd = cert_kd_fp32(a.dim); /* the bound of the fp32 ranking, see assign_mfma.hip */
+	const float kd = cert_kd_fma(a.dim); /* the bound of a ranking by chains of fused multiply-adds, see certificate.h */
 	switch (dp) {
 	case 4: rc = launch_fused_t<4, LD, LM>(a, means_out, sizes, exec, ws, dev, kd); break;
 	case 8: rc = launch_fused_t<8, LD, LM>(a, means_out, sizes, exec, ws, dev, kd); break;

@@ -667,6 +667,7 @@ int kmx_certificate_tau(int form, uint32_t dim, float x2, float xpart2, float c2
 	const CentroidBounds cb{ c2max, cmid2max, crest2max };
 	switch (form) {
 	case 0: *tau = cert_kd_fp32(dim) * (x2 + c2max); return KMX_OK;
+	case 3: *tau = cert_kd_fma(dim) * (x2 + c2max); return KMX_OK;
 	case 1: *tau = cert_tau(cert_kd_split(dim), x2, xpart2, cert_coeffs_split(cb)); return KMX_OK;
 	case 2: *tau = cert_tau(cert_kd_packed(dim), x2, xpart2, cert_coeffs_packed(cb)); return KMX_OK;
 	default: return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_certificate_tau: unknown form %d", form);

@@ -309,7 +309,8 @@ int kmx_set_queued_rows_limit(size_t bytes);
  * counterpart in the reference, whose kernels evaluate every pair directly; no device needed). A sweep decides a point
  * without the serial arithmetic only if its two smallest ranking values differ by more than tau; the tests check tau
  * against an emulation of the split operands on adversarial inputs.
- *   form 0: fp32 sweeps (KMX_ASSIGN_MFMA, _LDS_FMA)               tau = kd (x2 + c2max); xpart2, cmid2max, crest2max ignored
+ *   form 0: fp32 MFMA sweep (KMX_ASSIGN_MFMA)                      tau = kd (x2 + c2max); xpart2, cmid2max, crest2max ignored
+ *   form 3: sweeps on the vector ALU (KMX_ASSIGN_LDS_FMA, the single-pass fused kernel): the same with a smaller kd
  *   form 1: split-bf16 sweep, three products per dimension         xpart2 = sum_i xmid_i^2
  *   form 2: split-bf16 sweep, packed rows (dim <= 4, four products) xpart2 = sum_i xrest_i^2
  * x2 = |x|^2, c2max = max_j |c_j|^2, cmid2max / crest2max = max_j of the squared norms of the mid / rest parts of -2 c_j;

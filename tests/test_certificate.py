@@ -179,6 +179,41 @@ def test_tau_covers_the_split_and_the_serial_margin(km, dim, packed, kind):
     assert not wrong.any(), "%d certified pairs contradict the serial comparison" % int(wrong.sum())
 
 
+@pytest.mark.parametrize("dim", [2, 4, 8, 16, 32, 64])
+@pytest.mark.parametrize("kind", ["adversarial", "ties0", "ties100", "ties10000"])
+def test_tau_of_the_vector_alu_sweeps_covers_a_chain_of_fused_multiply_adds(km, dim, kind):
+    """KMX_ASSIGN_LDS_FMA and the single-pass fused kernel rank by a[j] = fma(c'_d, x_d, ... fma(c'_1, x_1, |c_j|^2)) in fp32,
+    round to nearest (form 3 of kmx_certificate_tau: (4 d + 24) u' S). The chain is emulated with exact products and one
+    rounding per step; twice its distance from the exact value plus the serial margin stays below tau, and what tau
+    certifies is a strict serial win."""
+    rng = np.random.default_rng(dim * 13 + len(kind))
+    n, k = 4096, 16
+    x, c = adversarial(dim, n, k, rng) if kind == "adversarial" else near_ties(dim, n, k, rng, float(kind[4:]))
+    cp = (np.float32(-2) * c).astype(np.float32)
+    c2 = np.zeros(k, np.float32)
+    for q in range(dim):
+        c2 = (c2 + (c[:, q] * c[:, q]).astype(np.float32)).astype(np.float32)      # any fp32 sum of the squares: at most d roundings
+    a = np.repeat(c2[:, None], n, 1)
+    for q in range(dim):
+        a = (cp[:, q].astype(np.float64)[:, None] * x[:, q].astype(np.float64)[None, :] + a.astype(np.float64)).astype(np.float32)
+    exact = (c.astype(np.float64) ** 2).sum(1)[:, None] + cp.astype(np.float64) @ x.astype(np.float64).T
+    x2 = (x.astype(np.float32) ** 2).sum(1, dtype=np.float32)
+    c2max = float(c2.max())
+    tau = np.array([km.certificate_tau(3, dim, float(x2[i]), 0.0, c2max, 0.0, 0.0) for i in range(n)], np.float64)
+    assert tau[0] == pytest.approx((4 * dim + 24) * U * (float(x2[0]) + c2max), rel=1e-6)
+    s_all = x2.astype(np.float64) + c2max
+    margin = (2 * dim + 12) * U * s_all
+    off = np.abs(a.astype(np.float64) - exact).max(0)
+    assert np.all(off <= (2 * dim + 7) * (U / 2) * s_all)          # the bound of the chain itself
+    assert np.all(2 * off + margin <= tau)
+    dist = serial_distances(x, c)
+    j1 = a.argmin(0)
+    certified = (a.astype(np.float64) - a[j1, np.arange(n)].astype(np.float64)[None, :]) > tau[None, :]
+    certified[j1, np.arange(n)] = False
+    wrong = certified & ~(dist[j1, np.arange(n)][None, :] < dist)
+    assert not wrong.any(), "%d certified pairs contradict the serial comparison" % int(wrong.sum())
+
+
 @pytest.mark.parametrize("dim", [2, 3, 4])
 @pytest.mark.parametrize("kind", ["ties0", "ties100", "ties10000", "uniform", "mirrored pairs"])
 def test_tau_in_a_moved_frame_covers_the_distances_of_the_data(km, dim, kind):
