@@ -53,12 +53,12 @@ pack_means_bf16_kernel(const float* __restrict__ means, size_t stride_means, flo
 	const uint32_t lane = threadIdx.x & (WAVE - 1);
 	const uint32_t j = (blockIdx.x * blockDim.x + threadIdx.x) / WAVE;
 	if (blockIdx.x == 0 && threadIdx.x == 0) counters[0] = 0u; /* the recheck queue of this call starts empty */
-	/* packed rows: the frame of the sweep, the mean of the first centroids (up to 1024 of them, the finite coordinates; any
-	 * vector would do, this one is near the middle of the data). Every work-group computes it, in the same order. */
+	/* packed rows: the frame of the sweep, the mean of the first centroids (up to 256 of them, one per lane; the finite
+	 * coordinates; any vector would do, this one is near the middle of the data). Every work-group computes it, in the same order. */
 	__shared__ float frame_parts[4][4];
 	float frame[4] = { 0.0f, 0.0f, 0.0f, 0.0f };
 	if (packed_slots & 2u) {
-		const uint32_t sample = min(k, 1024u);
+		const uint32_t sample = min(k, 256u);
 		float sum[4] = { 0.0f, 0.0f, 0.0f, 0.0f };
 		for (uint32_t r = threadIdx.x; r < sample; r += 256) {
 #pragma unroll

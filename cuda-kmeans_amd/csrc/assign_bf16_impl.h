@@ -420,7 +420,18 @@ __device__ __forceinline__ void mfma_tile(f32x16 (&acc)[P], const StepOperands<K
 	}
 }
 
-/* `if_set` in the lanes of `mask`, `otherwise` in the others, as one v_cndmask on a mask held in scalar registers. */
+/* A lane mask that a vector compare has just written to scalar registers, for use by select_lanes: on gfx940 and later a
+ * vector instruction may read a scalar register that a vector instruction wrote only two wait states later. The compiler
+ * keeps that distance for its own instructions but does not look inside inline assembly, so the wait is written out here;
+ * the selections take the mask from this function's result and are thereby ordered behind it. */
+__device__ __forceinline__ uint64_t settled_mask(uint64_t mask)
+{
+	asm volatile("s_nop 1" : "+s"(mask));
+	return mask;
+}
+
+/* `if_set` in the lanes of `mask`, `otherwise` in the others, as one v_cndmask on a mask held in scalar registers
+ * (a mask from settled_mask, see there). */
 __device__ __forceinline__ float select_lanes(uint64_t mask, float if_set, float otherwise)
 {
 	asm("v_cndmask_b32_e64 %0, %0, %1, %2" : "+v"(otherwise) : "v"(if_set), "s"(mask));
@@ -738,7 +749,7 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 						if (u == 0) lowest_of_tile[p] = lowest(a[0], a[1]);
 						else if (u < 8) lowest_of_tile[p] = lowest(lowest(lowest_of_tile[p], a[2 * u]), a[2 * u + 1]);
 						else if (u == 8) st[p].m2 = __builtin_amdgcn_fmed3f(st[p].m1, st[p].m2, lowest_of_tile[p]);
-						else if (u == 9) leads[p] = tile_old == 0 ? ~0ull : __builtin_amdgcn_ballot_w64(lowest_of_tile[p] < st[p].m1); /* (tile 0 fills the snapshot, whatever its values) */
+						else if (u == 9) leads[p] = settled_mask(tile_old == 0 ? ~0ull : __builtin_amdgcn_ballot_w64(lowest_of_tile[p] < st[p].m1)); /* (tile 0 fills the snapshot, whatever its values) */
 						else if (u == 10) st[p].tile = select_lanes(leads[p], tile_old, st[p].tile);
 						else if (u == 11) st[p].m1 = select_lanes(leads[p], lowest_of_tile[p], st[p].m1);
 						else snap[p][u - 12] = select_lanes(leads[p], a[u - 12], snap[p][u - 12]);

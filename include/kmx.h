@@ -315,7 +315,7 @@ int kmx_set_queued_rows_limit(size_t bytes);
  *   form 2: split-bf16 sweep, packed rows (dim <= 4, four products) xpart2 = sum_i xrest_i^2
  * x2 = |x|^2, c2max = max_j |c_j|^2, cmid2max / crest2max = max_j of the squared norms of the mid / rest parts of -2 c_j;
  * for form 2 all of them in the frame the packed sweep works in: with 128 centroids or more it subtracts the mean of the
- * (first 1024) centroids from points and centroids, so the norms are those of the moved data.
+ * (first 256) centroids from points and centroids, so the norms are those of the moved data.
  */
 int kmx_certificate_tau(int form, uint32_t dim, float x2, float xpart2, float c2max, float cmid2max, float crest2max, float* tau);
 
