@@ -460,10 +460,10 @@ __device__ __forceinline__ void track_snapshot(const f32x16& acc, Track& s, floa
 	for (int i = 0; i < 16; ++i) snap[i] = lt ? acc[i] : snap[i];
 }
 
-/* which kernel instances sweep with the fenced, prefetching step (rows of 17 to 64 dimensions, ten centroid tiles or more) and
- * which of those track with the snapshot (from 33 dimensions on: 9 MFMAs or more per point tile pay for its 32 operations, and
- * the rows a refinement would recompute are long; at 6 MFMAs the snapshot saturates the instruction issue: 0.333 ms against
- * the 0.30 ms of tracking group minima and refining at N = 2M, d = 32, k = 1024) */
+/* which kernel instances sweep with the fenced, prefetching step (rows of 17 to 48 dimensions, ten centroid tiles or more, all
+ * centroids resident) and which of those track with the snapshot: all of them. (Measured on one box at N = 2M, d = 32, k = 1024:
+ * 0.325 ms with the snapshot and two point tiles against 0.344 ms with group minima, a refinement and three point tiles, which
+ * spills 9 registers; KMX_SNAPSHOT_FROM_KB = 3 builds the latter for rows of 17 to 32 dimensions.) */
 #ifndef KMX_SNAPSHOT_FROM_KB
 #define KMX_SNAPSHOT_FROM_KB 2
 #endif
