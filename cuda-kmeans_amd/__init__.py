@@ -35,7 +35,7 @@ ABI_SYMBOLS = [
     "kmx_assign_last_rechecked", "kmx_assign_last_variant", "kmx_update_f32", "kmx_bucket_sum_f32", "kmx_fused_f32", "kmx_assign_f64", "kmx_update_f64", "kmx_fused_f64", "kmx_bucket_sum_f64", "kmx_set_queued_rows_limit",
     "kmx_graph_begin", "kmx_graph_end", "kmx_graph_launch", "kmx_graph_destroy", "kmx_event_create", "kmx_event_destroy", "kmx_event_record",
     "kmx_event_elapsed_ms", "kmx_set_profiling", "kmx_last_kernel_ms", "kmx_last_error", "kmx_certificate_tau",
-    "kmx_update_f32_noalloc", "kmx_reserve_f32",
+    "kmx_update_f32_noalloc", "kmx_reserve_f32", "kmx_prepare_points_f64", "kmx_forget_points_f64",
 ]
 
 
@@ -111,6 +111,8 @@ def hip_lib():
                                        ctypes.POINTER(ExecParams)]
         lib.kmx_update_f32_noalloc.argtypes = lib.kmx_update_f32.argtypes
         lib.kmx_reserve_f32.argtypes = [ctypes.c_int] * 4 + [u32] * 3
+        lib.kmx_prepare_points_f64.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t, u32, u32]
+        lib.kmx_forget_points_f64.argtypes = []
         lib.kmx_bucket_sum_f32.argtypes = [ctypes.c_int, vp, ctypes.c_int, sz, vp, vp, ctypes.c_int, sz, u32, u32, u32,
                                            ctypes.POINTER(ExecParams)]
         lib.kmx_fused_f32.argtypes = [ctypes.c_int, vp, ctypes.c_int, sz, vp, vp, ctypes.c_int, sz, vp, u32, u32, u32,
@@ -446,6 +448,8 @@ class HipKMeansAlgorithm:
         self.cu_assignment = [DeviceBuffer(4 * self.n) for _ in range(2)]
         self._bufs = [self.cu_data, self.cu_sizes] + self.cu_means + self.cu_assignment
         self.cu_data.write(data)
+        if _is_double(self.dtype):   # the points never change after the upload (cuda.hpp:54-64): their float copy is made once
+            check(hip_lib().kmx_prepare_points_f64(self.cu_data.ptr, self.layout, self.stride, self.dim, self.n))
         self.reset(means)
 
     def reset(self, means):
@@ -506,6 +510,8 @@ class HipKMeansAlgorithm:
         return self.cu_sizes.read(np.uint32, self.k)
 
     def cleanup(self):
+        if _is_double(self.dtype):
+            check(hip_lib().kmx_forget_points_f64())
         for b in self._bufs:
             b.free()
         self._bufs = []
@@ -537,6 +543,8 @@ class HipFusedKMeansAlgorithm:
         self.cu_means = [DeviceBuffer(self.item * self.means_size) for _ in range(2)]
         self._bufs = [self.cu_data, self.cu_sizes] + self.cu_means
         self.cu_data.write(data)
+        if _is_double(self.dtype):   # see HipKMeansAlgorithm.initialize
+            check(hip_lib().kmx_prepare_points_f64(self.cu_data.ptr, self.layout, self.stride, self.dim, self.n))
         self.last = 0
         self.cu_means[0].write(means)
         self.cu_sizes.zero()
@@ -579,6 +587,8 @@ class HipFusedKMeansAlgorithm:
             out.free()
 
     def cleanup(self):
+        if _is_double(self.dtype):
+            check(hip_lib().kmx_forget_points_f64())
         for b in self._bufs:
             b.free()
         self._bufs = []

@@ -17,11 +17,15 @@
  * evaluated from the norms of the parts actually dropped -- max_j |c'mid_j| and max_j |c'rest_j|, which the packing
  * kernel below writes behind the norms, and |xmid| (or |xrest|) of the point -- not from their worst case.
  * The refinement (winning row inside the winning tile) re-evaluates rows with v_dot2c_f32_bf16 on the same
- * three products, so the same bound covers it.
+ * three products, so the same bound covers it; the sweep of rows of 17 to 48 dimensions with resident centroids keeps the
+ * 16 results of the leading tile in registers instead (the snapshot, assign_bf16_impl.h) and has nothing to re-evaluate.
  *
  * Rows of at most 4 dimensions (PACKED): a block of 16 MFMA slots holds ALL FOUR hi/mid products of every dimension
  * (4 d <= 16), so a tile costs one MFMA instead of three and nothing of (hi + mid)(hi + mid) is dropped; only the
- * remainders of the split are (certificate.h, packed form).
+ * remainders of the split are (certificate.h, packed form). With 128 centroids or more these rows are swept in a frame moved
+ * to the mean of the centroids (pack_means_bf16_kernel below subtracts it from the centroids, the sweep and the screen of the
+ * exact pass from the points): tau scales with |x|^2 + max |c|^2, which the frame makes the spread of the data instead of its
+ * distance from the origin.
  *
  * Data flow, tiling, tracking, flag buffering and the recheck hand-over are those of the fp32 kernel
  * (assign_mfma.hip); the packed centroid row holds hi and mid parts of -2c, 4 bytes per dimension as before.

@@ -64,6 +64,16 @@ static double* g_misc = nullptr;                   /* 64-bit words: [0] queue le
 static size_t g_misc_cap = 0;
 static double* g_data32 = nullptr;                 /* float copy of the points (same layout and stride) */
 static size_t g_data32_cap = 0;
+/* the points whose float copy g_data32 currently holds because the caller announced them with kmx_prepare_points_f64 and has
+ * promised to leave them alone: kmx_assign_f64 then skips the conversion (null: nobody's) */
+struct PreparedPoints {
+	const double* data = nullptr;
+	int layout = 0;
+	size_t stride = 0;
+	uint32_t dim = 0, n = 0;
+	bool holds(const double* d, int l, size_t s, uint32_t dm, uint32_t nn) const { return data && data == d && layout == l && stride == s && dim == dm && n == nn; }
+};
+static PreparedPoints g_prepared;
 static double* g_means32 = nullptr;                /* float copy of the centroids */
 static size_t g_means32_cap = 0;
 
@@ -736,6 +746,7 @@ int launch_update_f64_t(int variant, const double* data, size_t stride, const ui
 
 int release_f64_workspace()
 {
+	g_prepared = PreparedPoints();
 	double** buffers[] = { &g_means_t, &g_norms, &g_queue, &g_misc, &g_data32, &g_means32 };
 	size_t* caps[] = { &g_means_t_cap, &g_norms_cap, &g_queue_cap, &g_misc_cap, &g_data32_cap, &g_means32_cap };
 	for (int b = 0; b < 6; ++b) {
@@ -749,6 +760,35 @@ int release_f64_workspace()
 } // namespace kmx
 
 using namespace kmx;
+
+extern "C" int kmx_prepare_points_f64(const double* data, int layout, size_t stride, uint32_t dim, uint32_t n)
+{
+	clear_error();
+	if (dim == 0) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_prepare_points_f64: dim must be positive");
+	g_prepared = PreparedPoints();
+	if (n == 0) return KMX_OK;
+	if (!data) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_prepare_points_f64: null device pointer");
+	int rc = check_layout_f64("kmx_prepare_points_f64", "data", layout, stride, n, dim);
+	if (rc) return rc;
+	const DeviceInfo* dev = nullptr;
+	rc = device_info(&dev);
+	if (rc) return rc;
+	const size_t data_extent = layout == KMX_AOS ? (size_t)(n - 1) * stride + dim : (size_t)(dim - 1) * stride + n;
+	rc = reserve_f64(&g_data32, &g_data32_cap, data_extent / 2 + 1);
+	if (rc) return rc;
+	KMX_LAUNCH_KERNEL(round_to_float_kernel, dim3((uint32_t)std::min<size_t>((data_extent + 1023) / 1024, (size_t)dev->compute_units * 32)), dim3(256), 0,
+	                   stream(), data, (float*)g_data32, data_extent);
+	KMX_LAUNCH_CHECK("round_to_float_kernel");
+	g_prepared.data = data; g_prepared.layout = layout; g_prepared.stride = stride; g_prepared.dim = dim; g_prepared.n = n;
+	return KMX_OK;
+}
+
+extern "C" int kmx_forget_points_f64(void)
+{
+	clear_error();
+	g_prepared = PreparedPoints();
+	return KMX_OK;
+}
 
 extern "C" int kmx_assign_f64(int variant,
                               const double* data, int layout, size_t stride,
@@ -798,12 +838,15 @@ extern "C" int kmx_assign_f64(int variant,
 		/* float copies with the layouts and strides of the originals */
 		const size_t data_extent = layout == KMX_AOS ? (size_t)(n - 1) * stride + dim : (size_t)(dim - 1) * stride + n;
 		const size_t means_extent = layout_means == KMX_AOS ? (size_t)(k - 1) * stride_means + dim : (size_t)(dim - 1) * stride_means + k;
-		rc = reserve_f64(&g_data32, &g_data32_cap, data_extent / 2 + 1);
-		if (rc) return rc;
 		rc = reserve_f64(&g_means32, &g_means32_cap, means_extent / 2 + 1);
 		if (rc) return rc;
-		KMX_LAUNCH_KERNEL(round_to_float_kernel, dim3((uint32_t)std::min<size_t>((data_extent + 1023) / 1024, (size_t)dev->compute_units * 32)), dim3(256), 0,
-		                   stream(), data, (float*)g_data32, data_extent);
+		if (!g_prepared.holds(data, layout, stride, dim, n)) {
+			g_prepared = PreparedPoints(); /* the copy is about to hold other points */
+			rc = reserve_f64(&g_data32, &g_data32_cap, data_extent / 2 + 1);
+			if (rc) return rc;
+			KMX_LAUNCH_KERNEL(round_to_float_kernel, dim3((uint32_t)std::min<size_t>((data_extent + 1023) / 1024, (size_t)dev->compute_units * 32)), dim3(256), 0,
+			                   stream(), data, (float*)g_data32, data_extent);
+		}
 		KMX_LAUNCH_KERNEL(round_to_float_kernel, dim3((uint32_t)std::min<size_t>((means_extent + 1023) / 1024, (size_t)dev->compute_units * 32)), dim3(256), 0,
 		                   stream(), means, (float*)g_means32, means_extent);
 		KMX_LAUNCH_CHECK("round_to_float_kernel");

@@ -121,6 +121,26 @@ inline int fused_call(int variant, const double* data, int ld, std::size_t strid
 	std::size_t strideMeans, std::uint32_t* sizes, std::uint32_t dim, std::uint32_t k, std::uint32_t n, kmx_exec_params* exec)
 { return kmx_fused_f64(variant, data, ld, stride, meansIn, meansOut, lm, strideMeans, sizes, dim, k, n, exec); }
 
+/* The points of a run are uploaded once and never change (cuda.hpp:54-64): the double-precision entry points are told so and
+ * keep the float copy their ranking sweeps work on, instead of converting the points in every call. Floats need nothing. */
+inline int prepare_points_call(const float*, int, std::size_t, std::uint32_t, std::uint32_t) { return KMX_OK; }
+inline int prepare_points_call(const double* data, int ld, std::size_t stride, std::uint32_t dim, std::uint32_t n)
+{ return kmx_prepare_points_f64(data, ld, stride, dim, n); }
+inline int forget_points_call(const float*) { return KMX_OK; }
+inline int forget_points_call(const double*) { return kmx_forget_points_f64(); }
+
+template<typename F, class LAYOUT>
+void preparePoints(const F* data, std::size_t n, std::size_t dim)
+{
+	KMX_CHECK(prepare_points_call(data, LAYOUT::ID, LAYOUT::precomputeConstants(n, dim), (std::uint32_t)dim, (std::uint32_t)n));
+}
+
+template<typename F>
+void forgetPoints(const F* data)
+{
+	KMX_CHECK(forget_points_call(data));
+}
+
 template<typename F, typename IDX_T, class LAYOUT, class LAYOUT_MEANS>
 void assign(int variant, const AssignmentProblemInstance<F, IDX_T>& in, HipExecParameters& exec)
 {

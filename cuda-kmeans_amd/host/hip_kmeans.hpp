@@ -119,6 +119,7 @@ public:
 		for (auto& b : mDevMeans) b.realloc(meansSize() * copies);
 		for (auto& b : mDevAssignment) b.realloc(n);
 		mDevData.write(data);
+		hip_detail::preparePoints<F, LAYOUT>(*mDevData, n, dim);
 		mLast = 0;
 		mDevMeans[mLast].write(means);
 		runFillZeros<IDX_T>(*mDevAssignment[mLast], n);
@@ -218,6 +219,7 @@ public:
 	void cleanup() override
 	{
 		IKMeansAlgorithm<F, IDX_T>::cleanup();
+		hip_detail::forgetPoints<F>(*mDevData);
 		mDevData.free();
 		for (auto& b : mDevMeans) b.free();
 		for (auto& b : mDevAssignment) b.free();
@@ -258,6 +260,7 @@ public:
 		mDevClusterSizes.realloc(k);
 		for (auto& b : mDevMeans) b.realloc(meansSize());
 		mDevData.write(data);
+		hip_detail::preparePoints<F, LAYOUT>(*mDevData, n, dim);
 		mLast = 0;
 		mDevMeans[mLast].write(means);
 		runFillZeros<IDX_T>(*mDevClusterSizes, k);
@@ -304,6 +307,7 @@ public:
 	void cleanup() override
 	{
 		IKMeansAlgorithm<F, IDX_T>::cleanup();
+		hip_detail::forgetPoints<F>(*mDevData);
 		mDevData.free();
 		for (auto& b : mDevMeans) b.free();
 		mDevClusterSizes.free();

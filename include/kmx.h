@@ -240,7 +240,15 @@ int kmx_fused_f32(int variant,
  *   Precondition as for kmx_update_f32: means and cluster_sizes are zero (kmx_fill_zero_u32 with twice the count).
  * kmx_fused_f64: KMX_FUSED_TWO_PASS / KMX_FUSED_BEST (assignment into the work space, then the update);
  *   KMX_FUSED_ONE_PASS is float-only: KMX_ERR_UNSUPPORTED.
+ * kmx_prepare_points_f64: the float copy of the points that the ranking sweeps of kmx_assign_f64 work on is made once, now,
+ *   and kmx_assign_f64 / kmx_fused_f64 calls with the same pointer, layout, stride, dim and n reuse it instead of converting
+ *   n * dim doubles per call -- the counterpart of the reference's upload in initialize() (cuda.hpp:54-64), after which the
+ *   points never change. The caller promises exactly that: not to modify the points until kmx_forget_points_f64(), the next
+ *   kmx_prepare_points_f64() or kmx_shutdown(). A call with other points makes the library forget by itself. Without
+ *   this call every kmx_assign_f64 converts its points (correct for points that change between calls).
  */
+int kmx_prepare_points_f64(const double* data, int layout, size_t stride, uint32_t dim, uint32_t n);
+int kmx_forget_points_f64(void);
 int kmx_assign_f64(int variant,
                    const double* data, int layout, size_t stride,
                    const double* means, int layout_means, size_t stride_means,

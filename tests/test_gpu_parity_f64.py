@@ -207,3 +207,40 @@ def test_fused_call_and_argument_errors(km, orc, gpu):
     assert e.value.code == km.KMX_ERR_UNSUPPORTED
     # empty input: nothing to do
     assert gpu_assign(km, km.ASSIGN_BEST, np.zeros(0), means0, spec.dim, spec.k, 0).size == 0
+
+
+def test_prepared_points_are_converted_once_and_forgotten_on_request(km, orc, gpu):
+    """kmx_prepare_points_f64: assignment calls on the announced points reuse their float copy; the result is the one without the
+    announcement; other points in between, and new values after kmx_forget_points_f64, are converted afresh."""
+    dim, k, n = 32, 256, 20000
+    rng = np.random.default_rng(11)
+    first = rng.normal(size=n * dim) * 3
+    other = rng.normal(size=n * dim) * 3 + 1
+    means = first.reshape(n, dim)[:k].copy().ravel()
+    lib = km.hip_lib()
+    d1 = km.DeviceBuffer(8 * n * dim); d1.write(first)
+    d2 = km.DeviceBuffer(8 * n * dim); d2.write(other)
+    m = km.DeviceBuffer(8 * k * dim); m.write(means)
+    a = km.DeviceBuffer(4 * n)
+
+    def run(buf):
+        km.assign(km.ASSIGN_BEST, buf, km.AOS, dim, m, km.AOS, dim, a, dim, k, n, dtype=np.float64)
+        km.sync()
+        return a.read(np.uint32, n)
+
+    want_first = orc.assign_f64(first, means, dim, k, n, threads=0)
+    want_other = orc.assign_f64(other, means, dim, k, n, threads=0)
+    assert np.array_equal(run(d1), want_first)
+    km.check(lib.kmx_prepare_points_f64(d1.ptr, km.AOS, dim, dim, n))
+    assert np.array_equal(run(d1), want_first)
+    assert np.array_equal(run(d1), want_first)
+    assert np.array_equal(run(d2), want_other)          # other points: the library forgets by itself
+    assert np.array_equal(run(d1), want_first)
+    km.check(lib.kmx_prepare_points_f64(d1.ptr, km.AOS, dim, dim, n))
+    km.check(lib.kmx_forget_points_f64())
+    d1.write(other)                                      # allowed again: nothing is kept
+    assert np.array_equal(run(d1), want_other)
+    with pytest.raises(km.KmxError):
+        km.check(lib.kmx_prepare_points_f64(d1.ptr, km.AOS, dim - 1, dim, n))   # stride < dim
+    for b in (d1, d2, m, a):
+        b.free()
