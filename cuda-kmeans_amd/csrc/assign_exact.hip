@@ -193,8 +193,9 @@ template <int LD, int L, int PB, int DPAD>
 __global__ void __launch_bounds__(256)
 recheck_reg_kernel(const float* __restrict__ data, size_t stride, const float* __restrict__ means_t, uint32_t kp,
                    uint32_t* __restrict__ assignment, uint32_t dim, uint32_t k,
-                   const uint32_t* __restrict__ queue, const uint32_t* __restrict__ counters)
+                   const uint32_t* __restrict__ queue, const uint32_t* __restrict__ counters, uint32_t vec4)
 {
+	typedef float f4 __attribute__((ext_vector_type(4)));
 	constexpr uint32_t GROUPS = 256 / L;
 	const uint32_t group = threadIdx.x / L;
 	const uint32_t gl = threadIdx.x % L;
@@ -210,8 +211,18 @@ recheck_reg_kernel(const float* __restrict__ data, size_t stride, const float* _
 			const size_t entry = 2 * (size_t)min(batch * PB + p, count - 1);
 			idx[p] = queue[entry];
 			thr[p] = __uint_as_float(queue[entry + 1]);
+			if (LD == KMX_AOS && vec4) { /* rows of whole, aligned 16-byte pieces: a quarter of the load instructions */
 #pragma unroll
-			for (int d = 0; d < DPAD; ++d) x[p][d] = (uint32_t)d < dim ? data[elem<LD>(stride, idx[p], d)] : 0.0f;
+				for (int d = 0; d < DPAD; d += 4) {
+					f4 v = { 0.0f, 0.0f, 0.0f, 0.0f };
+					if ((uint32_t)d < dim) v = *(const f4*)(data + (size_t)idx[p] * stride + d);
+					x[p][d] = v.x; x[p][d + 1] = v.y; x[p][d + 2] = v.z; x[p][d + 3] = v.w;
+				}
+			}
+			else {
+#pragma unroll
+				for (int d = 0; d < DPAD; ++d) x[p][d] = (uint32_t)d < dim ? data[elem<LD>(stride, idx[p], d)] : 0.0f;
+			}
 		}
 		float best[PB];
 		uint32_t bestIdx[PB];
@@ -558,8 +569,9 @@ static int launch_recheck_t(const AssignArgs& a, Workspace* ws, uint32_t kp)
 template <int LD, int L, int PB, int DPAD>
 static int launch_recheck_reg(const AssignArgs& a, Workspace* ws, uint32_t kp)
 {
+	const uint32_t vec4 = LD == KMX_AOS && a.dim % 4 == 0 && a.stride % 4 == 0 && ((uintptr_t)a.data & 15) == 0;
 	KMX_LAUNCH_KERNEL((recheck_reg_kernel<LD, L, PB, DPAD>), dim3(2048), dim3(256), 0, stream(),
-	                   a.data, a.stride, ws->means_t, kp, a.assignment, a.dim, a.k, ws->queue, ws->counters);
+	                   a.data, a.stride, ws->means_t, kp, a.assignment, a.dim, a.k, ws->queue, ws->counters, vec4);
 	KMX_LAUNCH_CHECK("recheck_reg_kernel");
 	return KMX_OK;
 }
