@@ -596,8 +596,8 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 	const uint32_t units = (n + unit_points - 1) / unit_points;
 
 	/*
-	 * Rows of more than 64 dimensions (always streamed, one point tile per wavefront, whose split operands take half of the
-	 * register file). Per centroid tile: one chain of 3 KB MFMAs into a single accumulator that starts from the norms;
+	 * Rows of more than 64 dimensions (always streamed; two point tiles per wavefront up to 128 dimensions, one above, where
+	 * the split operands of a tile take half of the register file). Per centroid tile and point tile: one chain of 3 KB MFMAs into a single accumulator that starts from the norms;
 	 * the centroid operands of block kb + 2 are requested from LDS before the MFMAs of block kb are issued
 	 * (sched_group_barrier pins that order: left to itself the scheduler reads each block right before its MFMAs and the
 	 * matrix pipe waits out an LDS round trip per block). The next chunk travels in pieces, one per tile step: requested
@@ -606,7 +606,7 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 	 */
 	constexpr int AHEAD = 2; /* blocks of centroid operands requested before the first MFMA of a step (one in flight behind the one in use; a deeper pipeline measured no faster) */
 	constexpr uint32_t PIECE_VECS = (tile_floats(RS) / 4 + MFMA_WAVES * WAVE - 1) / (MFMA_WAVES * WAVE); /* 16-byte pieces per lane that cover one tile */
-	auto wide_sweep = [&](const SplitPoints<KB>& x, Track& st) {
+	auto wide_sweep = [&](const SplitPoints<KB> (&x)[P], Track (&st)[P]) {
 		for (uint32_t chunk = 0; chunk < chunks; ++chunk) {
 			const uint32_t row0 = chunk * chunk_rows;
 			const uint32_t rows = min(chunk_rows, kp - row0);
@@ -629,12 +629,14 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 				for (uint32_t i = 0; i < PIECE_VECS; ++i) pv[i] = src[min(piece + i * (MFMA_WAVES * WAVE), last_vec)];
 				const f32x4 nv = nsrc[norm_vec];
 				const float* arow = lds_tiles + (size_t)t * tile_floats(RS) + (size_t)col * RS;
-				f32x16 acc;
+				f32x16 acc[P];
 #pragma unroll
 				for (int g = 0; g < 4; ++g) {
 					f32x4 v = *(const f32x4*)(lds_norms + t * NORM_TILE + 8 * g + 4 * h);
-					acc[4 * g] = v.x; acc[4 * g + 1] = v.y; acc[4 * g + 2] = v.z; acc[4 * g + 3] = v.w;
+					acc[0][4 * g] = v.x; acc[0][4 * g + 1] = v.y; acc[0][4 * g + 2] = v.z; acc[0][4 * g + 3] = v.w;
 				}
+#pragma unroll
+				for (int p = 1; p < P; ++p) acc[p] = acc[0];
 				bf16x8 chi[KB], cmid[KB];
 #pragma unroll
 				for (int kb = 0; kb < AHEAD; ++kb) {
@@ -647,11 +649,15 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 						chi[kb + AHEAD] = row_unit(arow, 4 * (kb + AHEAD) + 2 * h);
 						cmid[kb + AHEAD] = row_unit(arow, 4 * (kb + AHEAD) + 2 * h + 1);
 					}
-					acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(chi[kb], x.mid[kb], acc, 0, 0, 0);
-					acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cmid[kb], x.hi[kb], acc, 0, 0, 0);
-					acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(chi[kb], x.hi[kb], acc, 0, 0, 0);
+#pragma unroll
+					for (int p = 0; p < P; ++p) acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(chi[kb], x[p].mid[kb], acc[p], 0, 0, 0);
+#pragma unroll
+					for (int p = 0; p < P; ++p) acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cmid[kb], x[p].hi[kb], acc[p], 0, 0, 0);
+#pragma unroll
+					for (int p = 0; p < P; ++p) acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(chi[kb], x[p].hi[kb], acc[p], 0, 0, 0);
 				}
-				track_tile<false, false>(acc, st, tile0 + t, neg_inf);
+#pragma unroll
+				for (int p = 0; p < P; ++p) track_tile<false, false>(acc[p], st[p], tile0 + t, neg_inf);
 #pragma unroll
 				for (uint32_t i = 0; i < PIECE_VECS; ++i) dst[min(piece + i * (MFMA_WAVES * WAVE), last_vec)] = pv[i];
 				ndst[norm_vec] = nv;
@@ -662,7 +668,7 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 				__builtin_amdgcn_sched_group_barrier(0x100, 4 + 2 * AHEAD, 0);
 #pragma unroll
 				for (int kb = 0; kb < KB; ++kb) {
-					__builtin_amdgcn_sched_group_barrier(0x008, 3, 0);
+					__builtin_amdgcn_sched_group_barrier(0x008, 3 * P, 0);
 					if (kb + AHEAD < KB) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
 				}
 			}
@@ -696,7 +702,7 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 		constexpr bool SNAP = snapshot_sweep<KB, STREAM, COARSE, PACKED>();
 		float snap[P][SNAP ? SNAP_ROWS : 1];
 		if constexpr (KB > 4) {
-			wide_sweep(b[0], st[0]);
+			wide_sweep(b, st);
 		}
 		else if constexpr (PIPE) {
 #pragma unroll
@@ -1342,7 +1348,7 @@ static int launch_screen_bf16_kb(const float* rows, const Workspace* ws, const u
 
 /* point tiles per wavefront and sweep, and whether the next sweep's points are prefetched: bounded by the register file */
 template <int KB> struct SplitSweepShape {
-	static constexpr int P = KB <= 4 ? 2 : 1;
+	static constexpr int P = KB <= 8 ? 2 : 1; /* (rows of 65 to 128 dimensions: 128 registers of split operands; measured 6 % faster than one tile, whose centroid operands serve half the MFMAs) */
 	static constexpr bool PREFETCH = KB <= 2;
 };
 
