@@ -18,6 +18,8 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr uint32_t KBLOCK = 16; /* dimensions per v_mfma_f32_32x32x16_bf16 */
+constexpr uint32_t SLICED_MIN_POINTS = 1u << 16; /* fewer points: the streamed kernel, one launch */
+constexpr uint32_t SLICED_MAX_SLICES = 8;
 constexpr int STAGE_VECS = 9;   /* 16-byte pieces of a streamed chunk per lane: a chunk holds at most 9 * 512 * 16 bytes of tiles */
 
 /* Floats per packed centroid row. The PACKED form (rows of at most 4 dimensions) has 16 slots = 8 floats per row and no
@@ -470,18 +472,43 @@ __device__ __forceinline__ void track_snapshot(const f32x16& acc, Track& s, floa
 template <int KB, bool STREAM, bool COARSE, bool PACKED> constexpr bool pipelined_sweep() { return COARSE && !PACKED && !STREAM && KB >= 2 && KB <= 3; }
 template <int KB, bool STREAM, bool COARSE, bool PACKED> constexpr bool snapshot_sweep() { return pipelined_sweep<KB, STREAM, COARSE, PACKED>() && KB >= KMX_SNAPSHOT_FROM_KB; }
 
-template <int KB, int P, int LD, bool VEC, bool STREAM, bool COARSE, bool PREFETCH, bool PACKED = false>
+/*
+ * A sweep may cover a slice of the centroids only (rows slice.row_base .. slice.row_base + kp of the packed block; `packed`
+ * and `norms` then point at the slice). The launcher cuts the centroids into slices that fit the LDS when streaming them
+ * through it would be slower than sweeping the points once per slice. Between the launches a point's leader and its two
+ * smallest ranking values travel in `carried` (three arrays of n words); the last slice decides. tau is the same in every
+ * slice: its coefficients are maxima over all centroids.
+ */
+struct CentroidSlice {
+	const float* all_norms; /* the norms block of all centroids (the maxima of the certificate, the frame) */
+	uint32_t* carried;      /* [3][n]: leader, smallest and second smallest ranking value over the earlier slices */
+	uint32_t all_k, all_kp;
+	uint32_t row_base;      /* first centroid of the slice */
+	uint32_t mode;          /* CARRY_IN: earlier slices have been swept; CARRY_OUT: later ones follow, nothing is decided yet */
+};
+constexpr uint32_t CARRY_IN = 1u, CARRY_OUT = 2u;
+__device__ __forceinline__ CentroidSlice slice_of() { return CentroidSlice{ nullptr, nullptr, 0u, 0u, 0u, 0u }; }
+__device__ __forceinline__ CentroidSlice slice_of(const CentroidSlice& s) { return s; }
+
+/* (Slice: nothing, or CentroidSlice for the instances that sweep slices; the others are compiled without any of it) */
+template <int KB, int P, int LD, bool VEC, bool STREAM, bool COARSE, bool PREFETCH, bool PACKED = false, class... Slice>
 __global__ void __launch_bounds__(MFMA_WAVES * WAVE)
 assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* __restrict__ packed, const float* __restrict__ norms,
                    uint32_t* __restrict__ assignment, uint32_t* __restrict__ queue, uint32_t* __restrict__ counters,
-                   uint32_t dim, uint32_t k, uint32_t kp, uint32_t n, uint32_t chunk_rows, float kd, float neg_inf, uint32_t shifted_cap)
+                   uint32_t dim, uint32_t k, uint32_t kp, uint32_t n, uint32_t chunk_rows, float kd, float neg_inf, uint32_t shifted_cap,
+                   Slice... slice_argument)
 {
+	static_assert(sizeof...(Slice) <= 1, "at most one slice");
+	constexpr bool SLICED = sizeof...(Slice) == 1;
+	[[maybe_unused]] const CentroidSlice slice = slice_of(slice_argument...);
+	const float* __restrict__ all_norms = SLICED ? slice.all_norms : norms;
+	const uint32_t all_k = SLICED ? slice.all_k : k, all_kp = SLICED ? slice.all_kp : kp;
 	constexpr uint32_t RS = row_floats<KB, PACKED>();
 	extern __shared__ __attribute__((aligned(16))) float lds[];
 	Frame frame = { { 0.0f, 0.0f, 0.0f, 0.0f } }; /* PACKED: the rows are swept as x - frame (pack_means_bf16_kernel moved the centroids alike) */
 	if constexpr (PACKED) {
 #pragma unroll
-		for (int j = 0; j < 4; ++j) frame.m[j] = norms[frame_offset(kp) + j];
+		for (int j = 0; j < 4; ++j) frame.m[j] = all_norms[frame_offset(all_kp) + j];
 	}
 	__shared__ uint32_t wave_max[4][MFMA_WAVES]; /* rows 0..2: maxima per wavefront; [3][0]: items of this work-group handed out so far */
 	__shared__ uint32_t flag_list[MFMA_WAVES][2 * FLAG_CAP]; /* (point, threshold) pairs */
@@ -496,12 +523,12 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 	/* max_j of |c_j|^2, sum_i c'mid_i^2 and sum_i c'rest_i^2 (bit pattern maxima: they propagate NaN and +inf, which then flag every point) */
 	CertCoeffs cert;
 	{
-		const float* part_norms = norms + split_norms_offset(kp);
+		const float* part_norms = all_norms + split_norms_offset(all_kp);
 		uint32_t cmax[3] = { 0u, 0u, 0u };
-		for (uint32_t j = threadIdx.x; j < k; j += blockDim.x) {
-			cmax[0] = max(cmax[0], __float_as_uint(norms[norm_at(j)]));
+		for (uint32_t j = threadIdx.x; j < all_k; j += blockDim.x) {
+			cmax[0] = max(cmax[0], __float_as_uint(all_norms[norm_at(j)]));
 			cmax[1] = max(cmax[1], __float_as_uint(part_norms[j]));
-			cmax[2] = max(cmax[2], __float_as_uint(part_norms[kp + j]));
+			cmax[2] = max(cmax[2], __float_as_uint(part_norms[all_kp + j]));
 		}
 #pragma unroll
 		for (int q = 0; q < 3; ++q) {
@@ -1043,8 +1070,29 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 			}
 			const uint32_t pt = base + p * TILE + col;
 			const bool mine = h == 0 && pt < n;
+			if constexpr (SLICED) {
+			idx += slice.row_base;
+			if (slice.mode & CARRY_IN) {
+				/* the smallest two of both pairs; on equal values either leader will do: such a point is not decided here */
+				const uint32_t ci = mine ? slice.carried[pt] : 0u;
+				const float cf = mine ? __uint_as_float(slice.carried[(size_t)n + pt]) : 0.0f;
+				const float cs = mine ? __uint_as_float(slice.carried[2 * (size_t)n + pt]) : 0.0f;
+				const bool theirs = cf <= first;
+				second = fminf(fminf(cs, second), theirs ? first : cf);
+				idx = theirs ? ci : idx;
+				first = theirs ? cf : first;
+			}
+			if (slice.mode & CARRY_OUT) {
+				if (mine) {
+					slice.carried[pt] = idx;
+					slice.carried[(size_t)n + pt] = __float_as_uint(first);
+					slice.carried[2 * (size_t)n + pt] = __float_as_uint(second);
+				}
+				continue;
+			}
+			}
 			const bool decided = (second - first > tau) && (xsq + c2max > 1e-30f);
-			if (mine) assignment[pt] = idx < k ? idx : 0u;
+			if (mine) assignment[pt] = idx < all_k ? idx : 0u;
 			const bool flag = mine && !decided;
 			const unsigned long long mask = __ballot(flag);
 			if (mask) {
@@ -1369,7 +1417,24 @@ static int launch_bf16_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 	/* everything resident if it fits (rows up to 64 dimensions only: the wider kernels always stream); otherwise two
 	 * buffers of as many tiles as fit, bounded by what a work-group carries in registers (STAGE_VECS) */
 	uint32_t chunk_rows = std::min<uint32_t>(kp, (budget - static_bytes) / tile_bytes * TILE);
-	const bool stream_mode = KB > 4 || chunk_rows < kp;
+	bool stream_mode = KB > 4 || chunk_rows < kp;
+	/* Rows of 17 to 64 dimensions whose centroids do not fit: slices of centroids that do, one launch of the resident kernel
+	 * each (see CentroidSlice), when the points are many enough to pay for the launches. The resident kernels hand out their
+	 * items dynamically and keep the pipelined step; the streamed one has a barrier per chunk and item. (N = 1M, k = 1024:
+	 * d = 48 0.373 -> 0.284 ms, d = 64 0.50 -> 0.43 ms; d = 32, k = 2048: 0.429 -> 0.367 ms, k = 4096: no difference. Rows of
+	 * up to 16 dimensions stream as fast as they sweep resident centroids.) */
+	uint32_t slices = 1;
+	if (stream_mode && KB >= 2 && KB <= 4 && !PACKED && a.n >= SLICED_MIN_POINTS) {
+		const uint32_t tiles = kp / TILE, fit = chunk_rows / TILE;
+		const uint32_t wanted = (tiles + fit - 1) / fit;
+		if (wanted <= SLICED_MAX_SLICES) {
+			slices = wanted;
+			chunk_rows = (tiles + slices - 1) / slices * TILE; /* equal slices; the last one may be shorter */
+			stream_mode = false;
+			int rc = reserve_carried(ws, 3 * (size_t)a.n);
+			if (rc) return rc;
+		}
+	}
 	if (stream_mode) {
 		const uint32_t by_lds = (budget - static_bytes) / (2 * tile_bytes);
 		const uint32_t by_regs = (uint32_t)STAGE_VECS * MFMA_WAVES * WAVE * 16 / (tile_floats(RS) * 4);
@@ -1378,12 +1443,17 @@ static int launch_bf16_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 		if (chunk_tiles == 0) return fail(KMX_ERR_UNSUPPORTED, "assign (split-bf16 MFMA): two tiles of %u-dimension rows do not fit the LDS budget of %u bytes", KBLOCK * KB, budget);
 		chunk_rows = chunk_tiles * TILE;
 	}
-	const bool coarse = kp / TILE >= COARSE_MIN_TILES && KB <= 4;
+	const bool coarse = (slices > 1 ? chunk_rows : kp) / TILE >= COARSE_MIN_TILES && KB <= 4;
 	const uint32_t lds_bytes = (stream_mode ? 2u : 1u) * (chunk_rows / TILE) * tile_bytes;
 	const uint32_t unit_points = MFMA_WAVES * (stream_mode ? P : PR) * TILE;
 	const uint32_t units = (a.n + unit_points - 1) / unit_points;
 	void (*kernel)(const float*, size_t, const float*, const float*, uint32_t*, uint32_t*, uint32_t*,
 	               uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, float, float, uint32_t) = nullptr;
+	void (*sliced_kernel)(const float*, size_t, const float*, const float*, uint32_t*, uint32_t*, uint32_t*,
+	                      uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, float, float, uint32_t, CentroidSlice) = nullptr;
+	if constexpr (KB >= 2 && KB <= 4 && !PACKED) {
+		if (slices > 1) sliced_kernel = coarse ? assign_bf16_kernel<KB, PR, LD, VEC, false, true, PF, PACKED, CentroidSlice> : assign_bf16_kernel<KB, PR, LD, VEC, false, false, PF, PACKED, CentroidSlice>;
+	}
 	if constexpr (KB <= 4) {
 		if (stream_mode) kernel = coarse ? assign_bf16_kernel<KB, P, LD, VEC, true, true, PF, PACKED> : assign_bf16_kernel<KB, P, LD, VEC, true, false, PF, PACKED>;
 		else kernel = coarse ? assign_bf16_kernel<KB, PR, LD, VEC, false, true, PF, PACKED> : assign_bf16_kernel<KB, PR, LD, VEC, false, false, PF, PACKED>;
@@ -1391,18 +1461,34 @@ static int launch_bf16_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 	else {
 		kernel = assign_bf16_kernel<KB, P, LD, VEC, true, false, PF>;
 	}
-	KMX_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+	const void* launched = slices > 1 ? (const void*)sliced_kernel : (const void*)kernel;
+	KMX_HIP(hipFuncSetAttribute(launched, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
 	int per_cu = 1;
-	KMX_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)kernel, (int)(MFMA_WAVES * WAVE), lds_bytes));
+	KMX_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, launched, (int)(MFMA_WAVES * WAVE), lds_bytes));
 	per_cu = std::max(1, std::min(per_cu, 4));
 	const uint32_t grid = std::min(units, dev.compute_units * (uint32_t)per_cu);
 	exec->block_count = grid;
 	int rc = profile_begin(0);
 	if (rc) return rc;
-	KMX_LAUNCH_KERNEL(kernel, dim3(grid), dim3(MFMA_WAVES * WAVE), lds_bytes, stream(),
-	                   a.data, a.stride, ws->packed_means, ws->norms, a.assignment, ws->queue, ws->counters,
-	                   a.dim, a.k, kp, a.n, chunk_rows, kd, -__builtin_inff(), a.shifted_cap);
-	KMX_LAUNCH_CHECK("assign_bf16_kernel");
+	if (slices == 1) {
+		KMX_LAUNCH_KERNEL(kernel, dim3(grid), dim3(MFMA_WAVES * WAVE), lds_bytes, stream(),
+		                   a.data, a.stride, ws->packed_means, ws->norms, a.assignment, ws->queue, ws->counters,
+		                   a.dim, a.k, kp, a.n, chunk_rows, kd, -__builtin_inff(), a.shifted_cap);
+		KMX_LAUNCH_CHECK("assign_bf16_kernel");
+	}
+	else {
+		for (uint32_t s = 0; s < slices; ++s) {
+			const uint32_t row0 = s * chunk_rows;
+			const uint32_t rows = std::min(chunk_rows, kp - row0);
+			const CentroidSlice slice = { ws->norms, ws->carried, a.k, kp, row0, (s > 0 ? CARRY_IN : 0u) | (s + 1 < slices ? CARRY_OUT : 0u) };
+			/* (the kernel's view: `rows` resident centroids, all of them one chunk) */
+			KMX_LAUNCH_KERNEL(sliced_kernel, dim3(grid), dim3(MFMA_WAVES * WAVE), lds_bytes, stream(),
+			                   a.data, a.stride, ws->packed_means + packed_row(row0, RS), ws->norms + (size_t)(row0 / TILE) * NORM_TILE,
+			                   a.assignment, ws->queue, ws->counters,
+			                   a.dim, std::min(a.k - std::min(a.k, row0), rows), rows, a.n, rows, kd, -__builtin_inff(), a.shifted_cap, slice);
+			KMX_LAUNCH_CHECK("assign_bf16_kernel (a slice of the centroids)");
+		}
+	}
 	return profile_end(0);
 }
 

@@ -63,6 +63,7 @@ struct Workspace {
 	float* rows_copy = nullptr;           size_t rows_copy_cap = 0;     /* floats: AoS copy of SoA points for the tuned update */
 	float* queued_rows = nullptr;         size_t queued_rows_cap = 0;   /* floats */
 	uint32_t* queued_index = nullptr;     size_t queued_index_cap = 0;  /* words: per row 2 (queue) + 2 (assignment or 64-bit key), then the screen's pair counters and pairs */
+	uint32_t* carried = nullptr;          size_t carried_cap = 0;       /* words: per point the leader and the two smallest ranking values over the slices of centroids swept so far */
 	bool fixed = false; /* the work space of the entry point that allocates nothing: its buffers never grow, a call that needs more is refused */
 };
 int workspace(Workspace** ws);
@@ -73,6 +74,7 @@ int reserve_fused_assignment(Workspace* ws, size_t entries);
 int reserve_bucket_sizes(Workspace* ws, size_t entries);
 int reserve_rows_copy(Workspace* ws, size_t floats);
 int reserve_queued_rows(Workspace* ws, size_t rows, size_t dim, size_t extra_words);
+int reserve_carried(Workspace* ws, size_t words);
 
 #define KMX_HIP(call)                                                                                         \
 	do {                                                                                                      \

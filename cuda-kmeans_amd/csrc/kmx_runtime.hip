@@ -139,6 +139,8 @@ int reserve_queued_rows(Workspace* ws, size_t rows, size_t dim, size_t extra_wor
 	return grow(&ws->queued_index, &ws->queued_index_cap, 4 * rows + extra_words);
 }
 
+int reserve_carried(Workspace* ws, size_t words) { return grow(&ws->carried, &ws->carried_cap, words); }
+
 static int release_workspace()
 {
 	if (g_ws.queue) KMX_HIP(hipFree(g_ws.queue));
@@ -152,6 +154,7 @@ static int release_workspace()
 	if (g_ws.rows_copy) KMX_HIP(hipFree(g_ws.rows_copy));
 	if (g_ws.queued_rows) KMX_HIP(hipFree(g_ws.queued_rows));
 	if (g_ws.queued_index) KMX_HIP(hipFree(g_ws.queued_index));
+	if (g_ws.carried) KMX_HIP(hipFree(g_ws.carried));
 	g_ws = Workspace();
 	return release_f64_workspace();
 }

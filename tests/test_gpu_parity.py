@@ -172,6 +172,53 @@ def test_hard_inputs(km, orc, gpu, dim, k, n):
                 name, v, bad.size, bad[:5], got[bad[:5]], want[bad[:5]])
 
 
+@pytest.mark.parametrize("dim,k,n,lds_budget", [
+    (32, 2048, 66000, 0),       # two slices of 32 tiles
+    (48, 1024, 65536, 0),       # two slices of the pipelined kernel for rows of 33..48 dimensions
+    (64, 1100, 65537, 0),       # k not a multiple of the tile: the last slice is shorter and padded
+    (33, 300, 65600, 40000),    # a small LDS budget: many short slices
+    (17, 250, 70000, 24000),
+    (20, 3000, 70001, 0),
+])
+def test_centroids_swept_in_slices(km, orc, gpu, dim, k, n, lds_budget):
+    """From 65536 points on, rows of 17 to 64 dimensions whose centroids do not fit the LDS are swept once per slice of
+    centroids; the leader and the two smallest values of a point travel between the launches. Plain data in all layouts;
+    then duplicates of a centroid in the first and the last slice (a tie across slices), a NaN and an infinite centroid in
+    the last slice, ties on a grid."""
+    rng = np.random.default_rng(dim * 31 + k)
+    centres = rng.uniform(-10, 10, (40, dim)).astype(np.float32)
+    base = centres[rng.integers(0, 40, n)] + rng.normal(size=(n, dim)).astype(np.float32)
+    means = base[rng.permutation(n)[:k]].copy()
+    ex = lambda: km.ExecParams(shared_mem_bytes=lds_budget) if lds_budget else None
+    v = km.ASSIGN_MFMA_BF16X3
+    want = orc.assign(base.ravel(), means.ravel(), dim, k, n, threads=0, fast=True)
+    for layout, layout_means in [(AOS, AOS), (SOA, SOA), (AOS, SOA)]:
+        d = base if layout == AOS else np.ascontiguousarray(base.T)
+        m = means if layout_means == AOS else np.ascontiguousarray(means.T)
+        got, rechecked = gpu_assign(km, v, d.ravel(), m.ravel(), dim, k, n, layout, layout_means, ex())
+        bad = np.nonzero(got != want)[0]
+        assert bad.size == 0, "layouts %s/%s: %d mismatches, first at %s" % (layout, layout_means, bad.size, bad[:5])
+        assert rechecked < n // 4    # the certificate decides most points: the slices were merged, not each one flagged
+    cases = {}
+    m = means.copy(); m[k - 1] = m[3]; m[k // 2] = m[3]
+    d = base.copy(); d[:k] = m
+    cases["duplicates_across_slices"] = (d, m)
+    m = means.copy(); m[k - 2, 1] = np.nan
+    cases["nan_centroid_in_the_last_slice"] = (base, m)
+    m = means.copy(); m[k - 3, 0] = np.inf
+    cases["inf_centroid_in_the_last_slice"] = (base, m)
+    d = base.copy(); d[5, 0] = np.nan; d[9, dim - 1] = np.inf
+    cases["nan_inf_points"] = (d, means)
+    cases["grid_ties"] = (np.round(base), np.round(means))
+    for name, (d, m) in cases.items():
+        d = np.ascontiguousarray(d, dtype=np.float32).ravel()
+        m = np.ascontiguousarray(m, dtype=np.float32).ravel()
+        want = orc.assign(d, m, dim, k, n, threads=0, fast=True)
+        got, _ = gpu_assign(km, v, d, m, dim, k, n, AOS, AOS, ex())
+        bad = np.nonzero(got != want)[0]
+        assert bad.size == 0, "%s: %d mismatches, first at %s (gpu %s, oracle %s)" % (name, bad.size, bad[:5], got[bad[:5]], want[bad[:5]])
+
+
 @pytest.mark.parametrize("dim,k,n", [(32, 256, 3000), (21, 1500, 4000), (96, 200, 1500), (4, 512, 5000)])
 def test_soa_points_in_the_exact_pass(km, orc, gpu, dim, k, n):
     """SoA points: the exact pass copies the rows of the queued points into a compact block. Inputs that queue every point
@@ -677,7 +724,8 @@ def test_recording_refuses_what_cannot_be_recorded(km, gpu):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("dim,k,n,layout", [(4, 1024, 1 << 16, AOS), (32, 256, 1 << 15, SOA), (64, 128, 1 << 14, AOS), (2, 16, 1 << 14, AOS)])
+@pytest.mark.parametrize("dim,k,n,layout", [(4, 1024, 1 << 16, AOS), (32, 256, 1 << 15, SOA), (64, 128, 1 << 14, AOS), (2, 16, 1 << 14, AOS),
+                                                 (32, 2048, 1 << 16, AOS)])   # (the last one: centroids swept in two slices)
 def test_reserved_work_space_is_enough(km, orc, gpu, dim, k, n, layout):
     """kmx_reserve_f32 on a released work space: the assignment and the update of that shape can then be recorded, which
     refuses every call that would have to allocate; the recorded pair gives the oracle's assignment and counts."""
