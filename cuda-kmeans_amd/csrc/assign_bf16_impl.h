@@ -469,6 +469,8 @@ __device__ __forceinline__ void track_snapshot(const f32x16& acc, Track& s, floa
 #ifndef KMX_SNAPSHOT_FROM_KB
 #define KMX_SNAPSHOT_FROM_KB 2
 #endif
+/* the wide-row step (wide_sweep): rows of more than 64 dimensions, and streamed centroids from 49 dimensions on */
+template <int KB, bool STREAM> constexpr bool wide_rows_sweep() { return KB > 4 || (KB == 4 && STREAM); }
 template <int KB, bool STREAM, bool COARSE, bool PACKED> constexpr bool pipelined_sweep() { return COARSE && !PACKED && !STREAM && KB >= 2 && KB <= 3; }
 template <int KB, bool STREAM, bool COARSE, bool PACKED> constexpr bool snapshot_sweep() { return pipelined_sweep<KB, STREAM, COARSE, PACKED>() && KB >= KMX_SNAPSHOT_FROM_KB; }
 
@@ -728,7 +730,7 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 		constexpr bool PIPE = pipelined_sweep<KB, STREAM, COARSE, PACKED>();
 		constexpr bool SNAP = snapshot_sweep<KB, STREAM, COARSE, PACKED>();
 		float snap[P][SNAP ? SNAP_ROWS : 1];
-		if constexpr (KB > 4) {
+		if constexpr (wide_rows_sweep<KB, STREAM>()) {
 			wide_sweep(b, st);
 		}
 		else if constexpr (PIPE) {
@@ -1418,13 +1420,15 @@ static int launch_bf16_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 	 * buffers of as many tiles as fit, bounded by what a work-group carries in registers (STAGE_VECS) */
 	uint32_t chunk_rows = std::min<uint32_t>(kp, (budget - static_bytes) / tile_bytes * TILE);
 	bool stream_mode = KB > 4 || chunk_rows < kp;
-	/* Rows of 17 to 64 dimensions whose centroids do not fit: slices of centroids that do, one launch of the resident kernel
+	/* Rows of 17 to 48 dimensions whose centroids do not fit: slices of centroids that do, one launch of the resident kernel
 	 * each (see CentroidSlice), when the points are many enough to pay for the launches. The resident kernels hand out their
-	 * items dynamically and keep the pipelined step; the streamed one has a barrier per chunk and item. (N = 1M, k = 1024:
-	 * d = 48 0.373 -> 0.284 ms, d = 64 0.50 -> 0.43 ms; d = 32, k = 2048: 0.429 -> 0.367 ms, k = 4096: no difference. Rows of
-	 * up to 16 dimensions stream as fast as they sweep resident centroids.) */
+	 * items dynamically and keep the pipelined step; the streamed one has a barrier per chunk and item. (N = 1M: d = 48,
+	 * k = 1024 0.373 -> 0.270 ms; d = 32, k = 2048 0.429 -> 0.350 ms, k = 4096 no difference. Rows of up to 16 dimensions
+	 * stream as fast as they sweep resident centroids. Rows of 49 to 64 dimensions, whose resident kernel has the earlier
+	 * step, stream through the wide-row step instead: N = 1M, d = 64: k = 1024 0.50 -> 0.40 ms (slices: 0.42), k = 4096
+	 * 1.69 (slices) -> 1.45 ms.) */
 	uint32_t slices = 1;
-	if (stream_mode && KB >= 2 && KB <= 4 && !PACKED && a.n >= SLICED_MIN_POINTS) {
+	if (stream_mode && KB >= 2 && KB <= 3 && !PACKED && a.n >= SLICED_MIN_POINTS) {
 		const uint32_t tiles = kp / TILE, fit = chunk_rows / TILE;
 		const uint32_t wanted = (tiles + fit - 1) / fit;
 		if (wanted <= SLICED_MAX_SLICES) {
@@ -1443,7 +1447,8 @@ static int launch_bf16_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 		if (chunk_tiles == 0) return fail(KMX_ERR_UNSUPPORTED, "assign (split-bf16 MFMA): two tiles of %u-dimension rows do not fit the LDS budget of %u bytes", KBLOCK * KB, budget);
 		chunk_rows = chunk_tiles * TILE;
 	}
-	const bool coarse = (slices > 1 ? chunk_rows : kp) / TILE >= COARSE_MIN_TILES && KB <= 4;
+	const uint32_t swept_tiles = (slices > 1 ? chunk_rows : kp) / TILE;
+	const bool coarse = swept_tiles >= COARSE_MIN_TILES && KB <= 4 && !(KB == 4 && stream_mode); /* (the wide-row step tracks single rows) */
 	const uint32_t lds_bytes = (stream_mode ? 2u : 1u) * (chunk_rows / TILE) * tile_bytes;
 	const uint32_t unit_points = MFMA_WAVES * (stream_mode ? P : PR) * TILE;
 	const uint32_t units = (a.n + unit_points - 1) / unit_points;
@@ -1451,10 +1456,14 @@ static int launch_bf16_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 	               uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, float, float, uint32_t) = nullptr;
 	void (*sliced_kernel)(const float*, size_t, const float*, const float*, uint32_t*, uint32_t*, uint32_t*,
 	                      uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, float, float, uint32_t, CentroidSlice) = nullptr;
-	if constexpr (KB >= 2 && KB <= 4 && !PACKED) {
+	if constexpr (KB >= 2 && KB <= 3 && !PACKED) {
 		if (slices > 1) sliced_kernel = coarse ? assign_bf16_kernel<KB, PR, LD, VEC, false, true, PF, PACKED, CentroidSlice> : assign_bf16_kernel<KB, PR, LD, VEC, false, false, PF, PACKED, CentroidSlice>;
 	}
-	if constexpr (KB <= 4) {
+	if constexpr (KB == 4) {
+		if (stream_mode) kernel = assign_bf16_kernel<KB, P, LD, VEC, true, false, PF, PACKED>;
+		else kernel = coarse ? assign_bf16_kernel<KB, PR, LD, VEC, false, true, PF, PACKED> : assign_bf16_kernel<KB, PR, LD, VEC, false, false, PF, PACKED>;
+	}
+	else if constexpr (KB <= 4) {
 		if (stream_mode) kernel = coarse ? assign_bf16_kernel<KB, P, LD, VEC, true, true, PF, PACKED> : assign_bf16_kernel<KB, P, LD, VEC, true, false, PF, PACKED>;
 		else kernel = coarse ? assign_bf16_kernel<KB, PR, LD, VEC, false, true, PF, PACKED> : assign_bf16_kernel<KB, PR, LD, VEC, false, false, PF, PACKED>;
 	}
