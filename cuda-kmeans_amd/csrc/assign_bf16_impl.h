@@ -20,6 +20,10 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 constexpr uint32_t KBLOCK = 16; /* dimensions per v_mfma_f32_32x32x16_bf16 */
 constexpr uint32_t SLICED_MIN_POINTS = 1u << 16; /* fewer points: the streamed kernel, one launch */
 constexpr uint32_t SLICED_MAX_SLICES = 8;
+/* rows of 49 to 64 dimensions: their streamed step catches up with more centroids (N = 1M, d = 64, k = 1024: 0.398 ms in
+ * two slices, 0.422 ms streamed; k = 2048: the same; k = 4096: 1.50 against 1.45 ms), and SoA points cost more to read
+ * twice than the slices save (d = 56, k = 1024: 0.434 against 0.380 ms) */
+constexpr uint32_t SLICED_MAX_SLICES_WIDE = 2;
 constexpr int STAGE_VECS = 9;   /* 16-byte pieces of a streamed chunk per lane: a chunk holds at most 9 * 512 * 16 bytes of tiles */
 
 /* Floats per packed centroid row. The PACKED form (rows of at most 4 dimensions) has 16 slots = 8 floats per row and no
@@ -469,8 +473,8 @@ __device__ __forceinline__ void track_snapshot(const f32x16& acc, Track& s, floa
 #ifndef KMX_SNAPSHOT_FROM_KB
 #define KMX_SNAPSHOT_FROM_KB 2
 #endif
-/* the wide-row step (wide_sweep): rows of more than 64 dimensions, and streamed centroids from 49 dimensions on */
-template <int KB, bool STREAM> constexpr bool wide_rows_sweep() { return KB > 4 || (KB == 4 && STREAM); }
+/* the wide-row step (wide_sweep): rows of 49 dimensions and more */
+template <int KB> constexpr bool wide_rows_sweep() { return KB >= 4; }
 template <int KB, bool STREAM, bool COARSE, bool PACKED> constexpr bool pipelined_sweep() { return COARSE && !PACKED && !STREAM && KB >= 2 && KB <= 3; }
 template <int KB, bool STREAM, bool COARSE, bool PACKED> constexpr bool snapshot_sweep() { return pipelined_sweep<KB, STREAM, COARSE, PACKED>() && KB >= KMX_SNAPSHOT_FROM_KB; }
 
@@ -625,13 +629,17 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 	const uint32_t units = (n + unit_points - 1) / unit_points;
 
 	/*
-	 * Rows of more than 64 dimensions (always streamed; two point tiles per wavefront up to 128 dimensions, one above, where
-	 * the split operands of a tile take half of the register file). Per centroid tile and point tile: one chain of 3 KB MFMAs into a single accumulator that starts from the norms;
+	 * Rows of 49 dimensions and more (two point tiles per wavefront up to 128 dimensions, one above, where the split operands
+	 * of a tile take half of the register file; rows of more than 64 dimensions are always streamed, the narrower ones when
+	 * their centroids do not fit the LDS). Per centroid tile and point tile: one chain of 3 KB MFMAs into a single accumulator that starts from the norms;
 	 * the centroid operands of block kb + 2 are requested from LDS before the MFMAs of block kb are issued
 	 * (sched_group_barrier pins that order: left to itself the scheduler reads each block right before its MFMAs and the
 	 * matrix pipe waits out an LDS round trip per block). The next chunk travels in pieces, one per tile step: requested
 	 * from global memory before the step's MFMAs, written to the other LDS buffer after them (a few registers instead of a
 	 * whole chunk's share). Lanes beyond the end of the chunk repeat its last piece, so the step has no branches.
+	 * (Rows of 49 to 64 dimensions had the step of the narrower rows before, tracking groups of 8 rows behind the MFMAs of
+	 * the next tile with a refinement at the end: 255 registers resident, spills when streamed. This step measured faster
+	 * at every k: N = 1M, d = 64: k = 512 0.202 -> 0.187 ms, k = 1024 0.50 -> 0.40 ms, k = 2048 1.0 -> 0.745 ms.)
 	 */
 	constexpr int AHEAD = 2; /* blocks of centroid operands requested before the first MFMA of a step (one in flight behind the one in use; a deeper pipeline measured no faster) */
 	constexpr uint32_t PIECE_VECS = (tile_floats(RS) / 4 + MFMA_WAVES * WAVE - 1) / (MFMA_WAVES * WAVE); /* 16-byte pieces per lane that cover one tile */
@@ -653,10 +661,12 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 			const uint32_t norm_vec = min((uint32_t)threadIdx.x, (next_rows / TILE) * NORM_TILE / 4 - 1);
 			uint32_t piece = threadIdx.x; /* first 16-byte piece of this lane in the current step */
 			for (uint32_t t = 0; t < tiles; ++t) {
-				f32x4 pv[PIECE_VECS];
+				f32x4 pv[PIECE_VECS], nv;
+				if constexpr (STREAM) {
 #pragma unroll
-				for (uint32_t i = 0; i < PIECE_VECS; ++i) pv[i] = src[min(piece + i * (MFMA_WAVES * WAVE), last_vec)];
-				const f32x4 nv = nsrc[norm_vec];
+					for (uint32_t i = 0; i < PIECE_VECS; ++i) pv[i] = src[min(piece + i * (MFMA_WAVES * WAVE), last_vec)];
+					nv = nsrc[norm_vec];
+				}
 				const float* arow = lds_tiles + (size_t)t * tile_floats(RS) + (size_t)col * RS;
 				f32x16 acc[P];
 #pragma unroll
@@ -687,13 +697,15 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 				}
 #pragma unroll
 				for (int p = 0; p < P; ++p) track_tile<false, false>(acc[p], st[p], tile0 + t, neg_inf);
+				if constexpr (STREAM) {
 #pragma unroll
-				for (uint32_t i = 0; i < PIECE_VECS; ++i) dst[min(piece + i * (MFMA_WAVES * WAVE), last_vec)] = pv[i];
-				ndst[norm_vec] = nv;
-				piece += PIECE_VECS * (MFMA_WAVES * WAVE);
+					for (uint32_t i = 0; i < PIECE_VECS; ++i) dst[min(piece + i * (MFMA_WAVES * WAVE), last_vec)] = pv[i];
+					ndst[norm_vec] = nv;
+					piece += PIECE_VECS * (MFMA_WAVES * WAVE);
+				}
 				/* the order of the step: global requests; norms and AHEAD blocks of operands; then per block its MFMAs
 				 * and the request for the block AHEAD blocks on; tracking and the LDS writes come last by their dependences */
-				__builtin_amdgcn_sched_group_barrier(0x020, PIECE_VECS + 1, 0);
+				if constexpr (STREAM) __builtin_amdgcn_sched_group_barrier(0x020, PIECE_VECS + 1, 0);
 				__builtin_amdgcn_sched_group_barrier(0x100, 4 + 2 * AHEAD, 0);
 #pragma unroll
 				for (int kb = 0; kb < KB; ++kb) {
@@ -701,16 +713,18 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 					if (kb + AHEAD < KB) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
 				}
 			}
-			/* a short chunk (the last one) has fewer steps than the next chunk has tiles: the remaining pieces */
-			for (; piece - threadIdx.x <= last_vec; piece += PIECE_VECS * (MFMA_WAVES * WAVE)) {
+			if constexpr (STREAM) {
+				/* a short chunk (the last one) has fewer steps than the next chunk has tiles: the remaining pieces */
+				for (; piece - threadIdx.x <= last_vec; piece += PIECE_VECS * (MFMA_WAVES * WAVE)) {
 #pragma unroll
-				for (uint32_t i = 0; i < PIECE_VECS; ++i) {
-					const uint32_t at = min(piece + i * (MFMA_WAVES * WAVE), last_vec);
-					dst[at] = src[at];
+					for (uint32_t i = 0; i < PIECE_VECS; ++i) {
+						const uint32_t at = min(piece + i * (MFMA_WAVES * WAVE), last_vec);
+						dst[at] = src[at];
+					}
 				}
+				__syncthreads();
+				cur ^= 1u;
 			}
-			__syncthreads();
-			cur ^= 1u;
 		}
 	};
 
@@ -730,7 +744,7 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 		constexpr bool PIPE = pipelined_sweep<KB, STREAM, COARSE, PACKED>();
 		constexpr bool SNAP = snapshot_sweep<KB, STREAM, COARSE, PACKED>();
 		float snap[P][SNAP ? SNAP_ROWS : 1];
-		if constexpr (wide_rows_sweep<KB, STREAM>()) {
+		if constexpr (wide_rows_sweep<KB>()) {
 			wide_sweep(b, st);
 		}
 		else if constexpr (PIPE) {
@@ -1420,18 +1434,16 @@ static int launch_bf16_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 	 * buffers of as many tiles as fit, bounded by what a work-group carries in registers (STAGE_VECS) */
 	uint32_t chunk_rows = std::min<uint32_t>(kp, (budget - static_bytes) / tile_bytes * TILE);
 	bool stream_mode = KB > 4 || chunk_rows < kp;
-	/* Rows of 17 to 48 dimensions whose centroids do not fit: slices of centroids that do, one launch of the resident kernel
+	/* Rows of 17 to 64 dimensions whose centroids do not fit: slices of centroids that do, one launch of the resident kernel
 	 * each (see CentroidSlice), when the points are many enough to pay for the launches. The resident kernels hand out their
 	 * items dynamically and keep the pipelined step; the streamed one has a barrier per chunk and item. (N = 1M: d = 48,
-	 * k = 1024 0.373 -> 0.270 ms; d = 32, k = 2048 0.429 -> 0.350 ms, k = 4096 no difference. Rows of up to 16 dimensions
-	 * stream as fast as they sweep resident centroids. Rows of 49 to 64 dimensions, whose resident kernel has the earlier
-	 * step, stream through the wide-row step instead: N = 1M, d = 64: k = 1024 0.50 -> 0.40 ms (slices: 0.42), k = 4096
-	 * 1.69 (slices) -> 1.45 ms.) */
+	 * k = 1024 0.373 -> 0.270 ms; d = 32, k = 2048 0.429 -> 0.350 ms, k = 4096 no difference; SoA points gain as much. Rows
+	 * of up to 16 dimensions stream as fast as they sweep resident centroids.) */
 	uint32_t slices = 1;
-	if (stream_mode && KB >= 2 && KB <= 3 && !PACKED && a.n >= SLICED_MIN_POINTS) {
+	if (stream_mode && KB >= 2 && KB <= 4 && !PACKED && a.n >= SLICED_MIN_POINTS) {
 		const uint32_t tiles = kp / TILE, fit = chunk_rows / TILE;
 		const uint32_t wanted = (tiles + fit - 1) / fit;
-		if (wanted <= SLICED_MAX_SLICES) {
+		if (wanted <= (KB < 4 ? SLICED_MAX_SLICES : LD == KMX_AOS ? SLICED_MAX_SLICES_WIDE : 1u)) {
 			slices = wanted;
 			chunk_rows = (tiles + slices - 1) / slices * TILE; /* equal slices; the last one may be shorter */
 			stream_mode = false;
@@ -1448,7 +1460,7 @@ static int launch_bf16_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 		chunk_rows = chunk_tiles * TILE;
 	}
 	const uint32_t swept_tiles = (slices > 1 ? chunk_rows : kp) / TILE;
-	const bool coarse = swept_tiles >= COARSE_MIN_TILES && KB <= 4 && !(KB == 4 && stream_mode); /* (the wide-row step tracks single rows) */
+	const bool coarse = swept_tiles >= COARSE_MIN_TILES && !wide_rows_sweep<KB>(); /* (the wide-row step tracks single rows) */
 	const uint32_t lds_bytes = (stream_mode ? 2u : 1u) * (chunk_rows / TILE) * tile_bytes;
 	const uint32_t unit_points = MFMA_WAVES * (stream_mode ? P : PR) * TILE;
 	const uint32_t units = (a.n + unit_points - 1) / unit_points;
@@ -1456,12 +1468,14 @@ static int launch_bf16_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 	               uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, float, float, uint32_t) = nullptr;
 	void (*sliced_kernel)(const float*, size_t, const float*, const float*, uint32_t*, uint32_t*, uint32_t*,
 	                      uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, float, float, uint32_t, CentroidSlice) = nullptr;
-	if constexpr (KB >= 2 && KB <= 3 && !PACKED) {
+	if constexpr (KB == 4) {
+		if (slices > 1) sliced_kernel = assign_bf16_kernel<KB, PR, LD, VEC, false, false, PF, PACKED, CentroidSlice>;
+	}
+	else if constexpr (KB >= 2 && KB <= 3 && !PACKED) {
 		if (slices > 1) sliced_kernel = coarse ? assign_bf16_kernel<KB, PR, LD, VEC, false, true, PF, PACKED, CentroidSlice> : assign_bf16_kernel<KB, PR, LD, VEC, false, false, PF, PACKED, CentroidSlice>;
 	}
 	if constexpr (KB == 4) {
-		if (stream_mode) kernel = assign_bf16_kernel<KB, P, LD, VEC, true, false, PF, PACKED>;
-		else kernel = coarse ? assign_bf16_kernel<KB, PR, LD, VEC, false, true, PF, PACKED> : assign_bf16_kernel<KB, PR, LD, VEC, false, false, PF, PACKED>;
+		kernel = stream_mode ? assign_bf16_kernel<KB, P, LD, VEC, true, false, PF, PACKED> : assign_bf16_kernel<KB, PR, LD, VEC, false, false, PF, PACKED>;
 	}
 	else if constexpr (KB <= 4) {
 		if (stream_mode) kernel = coarse ? assign_bf16_kernel<KB, P, LD, VEC, true, true, PF, PACKED> : assign_bf16_kernel<KB, P, LD, VEC, true, false, PF, PACKED>;

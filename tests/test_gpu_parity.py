@@ -175,14 +175,17 @@ def test_hard_inputs(km, orc, gpu, dim, k, n):
 @pytest.mark.parametrize("dim,k,n,lds_budget", [
     (32, 2048, 66000, 0),       # two slices of 32 tiles
     (48, 1024, 65536, 0),       # two slices of the pipelined kernel for rows of 33..48 dimensions
-    (64, 1100, 65537, 0),       # k not a multiple of the tile: the last slice is shorter and padded
+    (64, 1100, 65537, 0),       # three slices would be needed: rows of 49..64 dimensions then stream (wide-row step)
+    (60, 1000, 66000, 0),       # two slices of the wide-row kernel (AoS points; SoA points stream)
+    (40, 1100, 65537, 0),       # k not a multiple of the tile: the last slice is shorter and padded
     (33, 300, 65600, 40000),    # a small LDS budget: many short slices
     (17, 250, 70000, 24000),
     (20, 3000, 70001, 0),
 ])
 def test_centroids_swept_in_slices(km, orc, gpu, dim, k, n, lds_budget):
     """From 65536 points on, rows of 17 to 64 dimensions whose centroids do not fit the LDS are swept once per slice of
-    centroids; the leader and the two smallest values of a point travel between the launches. Plain data in all layouts;
+    centroids (49 to 64 dimensions: two slices at most, AoS points only); the leader and the two smallest values of a point
+    travel between the launches. Plain data in all layouts;
     then duplicates of a centroid in the first and the last slice (a tie across slices), a NaN and an infinite centroid in
     the last slice, ties on a grid."""
     rng = np.random.default_rng(dim * 31 + k)
