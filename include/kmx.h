@@ -138,7 +138,8 @@ int kmx_assign_f32(int variant,
                    uint32_t dim, uint32_t k, uint32_t n, kmx_exec_params* exec);
 
 /*
- * Sizes the library's work space (packed centroids, recheck queue, copied rows, partial sums) for kmx_assign_f32 /
+ * Sizes the library's work space (packed centroids, recheck queue, copied rows, partial sums, the values carried between
+ * the sweeps of slices of centroids) for kmx_assign_f32 /
  * kmx_update_f32 / kmx_fused_f32 calls of this shape and these variants, so that those calls allocate nothing afterwards
  * (no counterpart in the reference, whose runners allocate nothing: cuda.hpp:54-64 allocates everything in initialize()).
  * Without it the first call of a shape grows the work space itself, which waits for the stream and calls hipMalloc; a
