@@ -475,6 +475,12 @@ __device__ __forceinline__ void track_snapshot(const f32x16& acc, Track& s, floa
 #endif
 /* the wide-row step (wide_sweep): rows of 49 dimensions and more */
 template <int KB> constexpr bool wide_rows_sweep() { return KB >= 4; }
+/* ... which of them track with the snapshot (track_snapshot: 29 operations per tile instead of the 66 of the row-by-row
+ * tracking, 16 registers per point tile): rows of 49 to 64 dimensions, whose 12 MFMAs per tile are short of hiding 66 */
+#ifndef KMX_WIDE_SNAPSHOT_UP_TO_KB
+#define KMX_WIDE_SNAPSHOT_UP_TO_KB 4
+#endif
+template <int KB> constexpr bool wide_rows_snapshot() { return wide_rows_sweep<KB>() && KB <= KMX_WIDE_SNAPSHOT_UP_TO_KB; }
 template <int KB, bool STREAM, bool COARSE, bool PACKED> constexpr bool pipelined_sweep() { return COARSE && !PACKED && !STREAM && KB >= 2 && KB <= 3; }
 template <int KB, bool STREAM, bool COARSE, bool PACKED> constexpr bool snapshot_sweep() { return pipelined_sweep<KB, STREAM, COARSE, PACKED>() && KB >= KMX_SNAPSHOT_FROM_KB; }
 
@@ -643,7 +649,8 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 	 */
 	constexpr int AHEAD = 2; /* blocks of centroid operands requested before the first MFMA of a step (one in flight behind the one in use; a deeper pipeline measured no faster) */
 	constexpr uint32_t PIECE_VECS = (tile_floats(RS) / 4 + MFMA_WAVES * WAVE - 1) / (MFMA_WAVES * WAVE); /* 16-byte pieces per lane that cover one tile */
-	auto wide_sweep = [&](const SplitPoints<KB> (&x)[P], Track (&st)[P]) {
+	constexpr bool WSNAP = wide_rows_snapshot<KB>();
+	auto wide_sweep = [&](const SplitPoints<KB> (&x)[P], Track (&st)[P], float (&snap)[P][WSNAP ? SNAP_ROWS : 1]) {
 		for (uint32_t chunk = 0; chunk < chunks; ++chunk) {
 			const uint32_t row0 = chunk * chunk_rows;
 			const uint32_t rows = min(chunk_rows, kp - row0);
@@ -696,7 +703,10 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 					for (int p = 0; p < P; ++p) acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(chi[kb], x[p].hi[kb], acc[p], 0, 0, 0);
 				}
 #pragma unroll
-				for (int p = 0; p < P; ++p) track_tile<false, false>(acc[p], st[p], tile0 + t, neg_inf);
+				for (int p = 0; p < P; ++p) {
+					if constexpr (WSNAP) track_snapshot(acc[p], st[p], snap[p], tile0 + t);
+					else track_tile<false, false>(acc[p], st[p], tile0 + t, neg_inf);
+				}
 				if constexpr (STREAM) {
 #pragma unroll
 					for (uint32_t i = 0; i < PIECE_VECS; ++i) dst[min(piece + i * (MFMA_WAVES * WAVE), last_vec)] = pv[i];
@@ -742,10 +752,17 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 		}
 		f32x16 acc0[P], acc1[P];
 		constexpr bool PIPE = pipelined_sweep<KB, STREAM, COARSE, PACKED>();
-		constexpr bool SNAP = snapshot_sweep<KB, STREAM, COARSE, PACKED>();
+		constexpr bool SNAP = snapshot_sweep<KB, STREAM, COARSE, PACKED>() || WSNAP;
 		float snap[P][SNAP ? SNAP_ROWS : 1];
 		if constexpr (wide_rows_sweep<KB>()) {
-			wide_sweep(b, st);
+			if constexpr (WSNAP) {
+#pragma unroll
+				for (int p = 0; p < P; ++p) {
+#pragma unroll
+					for (int i = 0; i < SNAP_ROWS; ++i) asm volatile("" : "=v"(snap[p][i])); /* no value yet: tile 0 always takes the lead */
+				}
+			}
+			wide_sweep(b, st, snap);
 		}
 		else if constexpr (PIPE) {
 #pragma unroll
