@@ -466,12 +466,14 @@ __device__ __forceinline__ void track_snapshot(const f32x16& acc, Track& s, floa
 	for (int i = 0; i < 16; ++i) snap[i] = lt ? acc[i] : snap[i];
 }
 
-/* which kernel instances sweep with the fenced, prefetching step (rows of 17 to 48 dimensions, ten centroid tiles or more, all
- * centroids resident) and which of those track with the snapshot: all of them. (Measured on one box at N = 2M, d = 32, k = 1024:
- * 0.325 ms with the snapshot and two point tiles against 0.344 ms with group minima, a refinement and three point tiles, which
- * spills 9 registers; KMX_SNAPSHOT_FROM_KB = 3 builds the latter for rows of 17 to 32 dimensions.) */
+/* which kernel instances sweep with the fenced, prefetching step (unpacked rows of up to 48 dimensions, ten centroid tiles or
+ * more, all centroids resident) and which of those track with the snapshot: all of them. (Measured on one box at N = 2M, d = 32,
+ * k = 1024: 0.325 ms with the snapshot and two point tiles against 0.344 ms with group minima, a refinement and three point
+ * tiles, which spills 9 registers; KMX_SNAPSHOT_FROM_KB = 3 builds the latter for rows of 17 to 32 dimensions. Rows of 5 to 16
+ * dimensions, three MFMAs per tile: N = 2M, d = 16: k = 320 0.136 -> 0.110 ms, k = 1024 0.238 -> 0.235 ms; d = 12, k = 512:
+ * 0.160 -> 0.144 ms; no shape slower.) */
 #ifndef KMX_SNAPSHOT_FROM_KB
-#define KMX_SNAPSHOT_FROM_KB 2
+#define KMX_SNAPSHOT_FROM_KB 1
 #endif
 /* the wide-row step (wide_sweep): rows of 49 dimensions and more */
 template <int KB> constexpr bool wide_rows_sweep() { return KB >= 4; }
@@ -481,7 +483,7 @@ template <int KB> constexpr bool wide_rows_sweep() { return KB >= 4; }
 #define KMX_WIDE_SNAPSHOT_UP_TO_KB 4
 #endif
 template <int KB> constexpr bool wide_rows_snapshot() { return wide_rows_sweep<KB>() && KB <= KMX_WIDE_SNAPSHOT_UP_TO_KB; }
-template <int KB, bool STREAM, bool COARSE, bool PACKED> constexpr bool pipelined_sweep() { return COARSE && !PACKED && !STREAM && KB >= 2 && KB <= 3; }
+template <int KB, bool STREAM, bool COARSE, bool PACKED> constexpr bool pipelined_sweep() { return COARSE && !PACKED && !STREAM && KB <= 3; }
 template <int KB, bool STREAM, bool COARSE, bool PACKED> constexpr bool snapshot_sweep() { return pipelined_sweep<KB, STREAM, COARSE, PACKED>() && KB >= KMX_SNAPSHOT_FROM_KB; }
 
 /*

@@ -45,7 +45,7 @@ def close_reads(code):
     return found
 
 
-@pytest.mark.parametrize("blocks", [2, 3])
+@pytest.mark.parametrize("blocks", [1, 2, 3])
 def test_selections_on_a_fresh_mask_keep_two_wait_states(tmp_path, blocks):
     hipcc = "/opt/rocm/bin/hipcc"
     if not os.path.exists(hipcc):
