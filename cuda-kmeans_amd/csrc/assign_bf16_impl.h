@@ -1479,7 +1479,12 @@ static int launch_bf16_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 		chunk_rows = chunk_tiles * TILE;
 	}
 	const uint32_t swept_tiles = (slices > 1 ? chunk_rows : kp) / TILE;
-	const bool coarse = swept_tiles >= COARSE_MIN_TILES && !wide_rows_sweep<KB>(); /* (the wide-row step tracks single rows) */
+	/* per-tile tracking pays from COARSE_MIN_TILES tiles on where a refinement follows the sweep; the snapshot needs none
+	 * (N = 2-4M: d = 16, k = 256 0.219 -> 0.174 ms; d = 32, k = 256 0.150 -> 0.127 ms, k = 128 0.105 -> 0.096 ms; two tiles,
+	 * k = 64: 0.108 -> 0.110 ms, left with the row-by-row tracking) */
+	constexpr uint32_t SNAPSHOT_MIN_TILES = 3;
+	const uint32_t coarse_from = (snapshot_sweep<KB, false, true, PACKED>() && !stream_mode) ? SNAPSHOT_MIN_TILES : COARSE_MIN_TILES;
+	const bool coarse = swept_tiles >= coarse_from && !wide_rows_sweep<KB>(); /* (the wide-row step tracks single rows) */
 	const uint32_t lds_bytes = (stream_mode ? 2u : 1u) * (chunk_rows / TILE) * tile_bytes;
 	const uint32_t unit_points = MFMA_WAVES * (stream_mode ? P : PR) * TILE;
 	const uint32_t units = (a.n + unit_points - 1) / unit_points;
