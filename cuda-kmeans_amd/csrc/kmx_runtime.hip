@@ -179,17 +179,24 @@ int dispatch_assign(int variant, const AssignArgs& a, kmx_exec_params* exec, Wor
 {
 	if (variant == KMX_ASSIGN_BEST) {
 		/* counterpart of BestCachedAssignmentKernel::run (reference kernels.cu:706-717): pick by shape.
-		 * Measured: the split-bf16 sweep is about twice as fast as the fp32 one wherever the sweep dominates; it hands
-		 * 2-3 times as many points to the exact pass, which costs more than it saves for very short rows and for
-		 * few centroids (HBM-bound shapes). Rows of 2 to 4 dimensions are the exception among the short ones: all their
-		 * products fit one MFMA per tile (the packed form), which beats the fp32 sweep from 128 centroids on (512 for
-		 * two dimensions; 1.14 against 1.53 ms per iteration at N = 4M, d = 4, k = 4096, exact pass included).
-		 * The fp32 MFMA sweep beat the plain-VALU variant at every shape except
-		 * a handful of centroids, where that variant reads them through the scalar cache. */
-		const bool packed_wins = !a.ranking_only /* the double path pays more per queued point: 2.35 against 1.91 ms there */ &&
-		                         ((a.dim >= 3 && a.dim <= 4 && a.k >= 128) || (a.dim == 2 && a.k >= 512));
-		if (a.k <= 32 && lds_fma_supports(a, dev) && lds_fma_reads_through_scalar_cache(a)) variant = KMX_ASSIGN_LDS_FMA;
-		else if (bf16_supports(a, dev) && ((a.dim >= 8 && a.k >= 64) || packed_wins)) variant = KMX_ASSIGN_MFMA_BF16X3;
+		 * Measured (one call, exact pass included, N = 2-4M): the split-bf16 sweep is about twice as fast as the fp32 one
+		 * wherever the sweep dominates; it hands 2-3 times as many points to the exact pass. Rows of 16 dimensions and more:
+		 * ahead or level at every k (d = 64, k = 16: 0.25 against 0.32 ms; d = 32, k = 33: 0.108 against 0.137 ms; d = 16,
+		 * k = 32: level). Rows of 5 to 15 dimensions: ahead from three centroid tiles on (d = 5, k = 100: 0.153 against
+		 * 0.181 ms; k = 1024: 0.279 against 0.385 ms), behind with one or two (d = 8, k = 64: 0.120 against 0.116 ms).
+		 * Rows of 2 to 4 dimensions: all their products fit one MFMA per tile (the packed form), which beats the fp32 sweep
+		 * from 128 centroids on (512 for two dimensions; 1.14 against 1.53 ms per iteration at N = 4M, d = 4, k = 4096).
+		 * The plain-VALU variant, which reads a small centroid block through the scalar cache, wins with at most 16
+		 * centroids of at most 16 dimensions (d = 16, k = 16: 0.086 against 0.105 ms; d = 8, k = 8: 0.049 against 0.080 ms)
+		 * and loses from there on (d = 16, k = 32: 0.128 against 0.110 ms; d = 32, k = 16: 0.183 against 0.161 ms).
+		 * The double path keeps the earlier bounds: it pays more per queued point (2.35 against 1.91 ms with the packed
+		 * form there), and the new ones were not measured for it. */
+		const bool packed_wins = !a.ranking_only && ((a.dim >= 3 && a.dim <= 4 && a.k >= 128) || (a.dim == 2 && a.k >= 512));
+		const bool split_wins = a.ranking_only ? (a.dim >= 8 && a.k >= 64)
+		                                       : (a.dim >= 16 || (a.dim >= 5 && a.k > 64));
+		const bool few = a.ranking_only ? a.k <= 32 : (a.k <= 16 && a.dim <= 16);
+		if (few && lds_fma_supports(a, dev) && lds_fma_reads_through_scalar_cache(a)) variant = KMX_ASSIGN_LDS_FMA;
+		else if (bf16_supports(a, dev) && (split_wins || packed_wins)) variant = KMX_ASSIGN_MFMA_BF16X3;
 		else if (mfma_supports(a, dev)) variant = KMX_ASSIGN_MFMA;
 		else if (lds_fma_supports(a, dev)) variant = KMX_ASSIGN_LDS_FMA;
 		else variant = KMX_ASSIGN_BASE;
