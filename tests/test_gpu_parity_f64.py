@@ -96,6 +96,24 @@ def test_assignment_is_bit_exact(km, orc, gpu, dim, k, n, layout, layout_means):
         assert bad.size == 0, "variant %d: %d mismatches, first at %s" % (v, bad.size, bad[:5])
 
 
+@pytest.mark.parametrize("dim,k,n", [(32, 2048, 66000), (48, 1100, 65536), (64, 1000, 65600)])
+@pytest.mark.parametrize("layout,layout_means", [(AOS, AOS), (SOA, SOA)])
+def test_centroids_swept_in_slices(km, orc, gpu, dim, k, n, layout, layout_means):
+    """Doubles, ranked by the float sweeps: from 65536 points on, rows of 17 to 64 dimensions whose centroids do not fit the
+    LDS are swept once per slice of centroids (the float copy of the points is read once per slice)."""
+    rng = np.random.default_rng(dim * 13 + k)
+    centres = rng.uniform(-10, 10, (40, dim))
+    base = centres[rng.integers(0, 40, n)] + rng.normal(size=(n, dim))
+    means = base[rng.permutation(n)[:k]].copy()
+    d = base if layout == AOS else np.ascontiguousarray(base.T)
+    m = means if layout_means == AOS else np.ascontiguousarray(means.T)
+    want = orc.assign_f64(d.ravel(), m.ravel(), dim, k, n, layout, layout_means, threads=0)
+    for v in (km.ASSIGN_MFMA_BF16X3, km.ASSIGN_BEST):
+        got = gpu_assign(km, v, d.ravel(), m.ravel(), dim, k, n, layout, layout_means)
+        bad = np.nonzero(got != want)[0]
+        assert bad.size == 0, "variant %d: %d mismatches, first at %s" % (v, bad.size, bad[:5])
+
+
 @pytest.mark.parametrize("dim,k,n", [(8, 64, 4096), (32, 256, 3000), (40, 70, 1000)])
 def test_hard_inputs(km, orc, gpu, dim, k, n):
     """Exact ties, duplicated centroids, coincident points, NaN / inf / huge / tiny values, float-invisible gaps."""
