@@ -1238,7 +1238,7 @@ static __device__ __attribute__((noinline)) void evaluate_pair_of_row(const floa
 }
 
 template <int KB, int P, bool PACKED = false>
-__global__ void __launch_bounds__(SCREEN_WAVES * WAVE)
+__global__ void __launch_bounds__(SCREEN_WAVES * WAVE) __attribute__((amdgpu_waves_per_eu(KB <= 3 ? 2 : 1)))
 screen_bf16_kernel(const float* __restrict__ rows, const float* __restrict__ packed, const float* __restrict__ norms,
                    const float* __restrict__ means_t, const uint32_t* __restrict__ row_queue, const uint32_t* __restrict__ row_count,
                    uint32_t* __restrict__ pairs, uint32_t* __restrict__ item_pairs,

@@ -82,6 +82,18 @@ __host__ __device__ __forceinline__ ScreenItems screen_items(uint32_t rows, uint
 	ScreenItems w;
 	w.units = (rows + unit_rows - 1) / unit_rows;
 	uint32_t want = w.units ? waves / w.units : 1u;
+	if (want < 2u && w.units) {
+		/* about as many units as wavefronts, or more: the wavefronts go round ceil(items / waves) times, and the last round
+		 * may be nearly empty (1225 units on 1024 wavefronts: two rounds for 1.2 rounds of work). Shares of the tiles make
+		 * the rounds shorter: the split with the least rounds of whole sweeps, while the items stay within the bound of
+		 * screen_items_max. */
+		uint32_t best_rounds = (w.units + waves - 1) / waves * 8u; /* in eighths of a whole sweep */
+		want = 1u;
+		for (uint32_t p = 2; p <= 8u && p <= tiles && w.units * p <= SCREEN_MAX_WAVES; p *= 2) {
+			const uint32_t rounds = (w.units * p + waves - 1) / waves * (8u / p);
+			if (rounds < best_rounds) { best_rounds = rounds; want = p; }
+		}
+	}
 	want = want < 1u ? 1u : (want > tiles ? tiles : want);
 	w.part_tiles = (tiles + want - 1) / want;
 	w.parts = (tiles + w.part_tiles - 1) / w.part_tiles;
