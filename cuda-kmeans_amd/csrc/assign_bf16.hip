@@ -61,7 +61,7 @@ pack_means_bf16_kernel(const float* __restrict__ means, size_t stride_means, flo
 	 * coordinates; any vector would do, this one is near the middle of the data). Every work-group computes it, in the same order. */
 	__shared__ float frame_parts[4][4];
 	float frame[4] = { 0.0f, 0.0f, 0.0f, 0.0f };
-	if (packed_slots & 2u) {
+	if ((packed_slots & 3u) == 3u) {
 		const uint32_t sample = min(k, 256u);
 		float sum[4] = { 0.0f, 0.0f, 0.0f, 0.0f };
 		for (uint32_t r = threadIdx.x; r < sample; r += 256) {
@@ -83,12 +83,48 @@ pack_means_bf16_kernel(const float* __restrict__ means, size_t stride_means, flo
 		for (int q = 0; q < 4; ++q)
 			if (threadIdx.x == (uint32_t)q) norms[frame_offset(kp) + q] = frame[q];
 	}
+	/* unpacked rows: the same for rows of up to FRAME_DIMS dimensions, from the first 16 centroids (a thread per dimension,
+	 * its 16 loads in flight together: every work-group repeats this; zeros when the sweep keeps the frame of the data);
+	 * the first work-group stores it with |m|^2 and an upper bound of |m| */
+	__shared__ float wide_frame[FRAME_DIMS];
+	if (!(packed_slots & 1u)) {
+		constexpr uint32_t SAMPLE = 16;
+		const uint32_t sample = min(k, SAMPLE);
+		for (uint32_t q = threadIdx.x; q < dp; q += blockDim.x) {
+			float sum = 0.0f;
+			if ((packed_slots & 2u) && q < dim) {
+				float v[SAMPLE];
+#pragma unroll
+				for (uint32_t r = 0; r < SAMPLE; ++r) v[r] = r < sample ? means[elem<LM>(stride_means, r, q)] : 0.0f;
+#pragma unroll
+				for (uint32_t r = 0; r < SAMPLE; ++r) sum += __builtin_fabsf(v[r]) < __builtin_inff() ? v[r] : 0.0f;
+				sum = sum / (float)sample;
+				sum = __builtin_fabsf(sum) < __builtin_inff() ? sum : 0.0f; /* (the sum of finite values may overflow) */
+			}
+			wide_frame[q] = sum;
+		}
+		__syncthreads();
+		if (blockIdx.x == 0) {
+			for (uint32_t q = threadIdx.x; q < dp; q += blockDim.x) norms[frame_offset(kp) + q] = wide_frame[q];
+			if (threadIdx.x < WAVE) {
+				float m2 = 0.0f;
+				for (uint32_t q = lane; q < dp; q += WAVE) m2 += wide_frame[q] * wide_frame[q];
+				for (int off = WAVE / 2; off > 0; off >>= 1) m2 += __shfl_xor(m2, off);
+				if (lane == 0) {
+					norms[frame_offset(kp) + FRAME_DIMS] = m2; /* (as computed: it enters the shift of the thresholds) */
+					norms[frame_offset(kp) + FRAME_DIMS + 1] = __builtin_sqrtf(m2) * 1.0001f;
+				}
+			}
+		}
+	}
 	if (j >= kp) return;
-	const uint32_t rs = packed_slots ? row_floats<1, true>() : dp + ROW_PAD;
+	const bool packed_form = (packed_slots & 1u) != 0;
+	const uint32_t rs = packed_form ? row_floats<1, true>() : dp + ROW_PAD;
 	float* row = packed + packed_row(j, rs);
 	__bf16* parts = (__bf16*)row;
-	float c2 = 0.0f, mid2 = 0.0f, rest2 = 0.0f; /* |c|^2 and, for the certificate, sum_i c'mid_i^2, sum_i c'rest_i^2 */
-	if (packed_slots) {
+	float c2 = 0.0f, mid2 = 0.0f, rest2 = 0.0f; /* |c|^2 (of the moved centroid) and, for the certificate, sum_i c'mid_i^2, sum_i c'rest_i^2 */
+	float exact2 = 0.0f; /* unpacked rows: |c|^2 of the centroid as given */
+	if (packed_form) {
 		/* rows of at most 4 dimensions: slots 0..3 = hi, 4..7 = mid, 8..11 = hi, 12..15 = mid of -2c; inside the tile
 		 * the first halves of all rows, then the second halves (packed_half; load_packed_points has the matching order
 		 * of the point's parts) */
@@ -103,6 +139,7 @@ pack_means_bf16_kernel(const float* __restrict__ means, size_t stride_means, flo
 			if (j % TILE == TILE - 1 && lane < TILE_PAD) tile[TILE * rs + lane] = 0.0f;
 			if (lane < 4) {
 				c2 = v * v;
+				exact2 = exact * exact;
 				mid2 = (float)mid * (float)mid;
 				rest2 = rest * rest;
 				if (q < dim) means_t[(size_t)q * kp + j] = exact; /* exact copy for the recheck pass */
@@ -111,7 +148,9 @@ pack_means_bf16_kernel(const float* __restrict__ means, size_t stride_means, flo
 	}
 	else
 	for (uint32_t q = lane; q < dp; q += WAVE) {
-		const float v = (j < k && q < dim) ? means[elem<LM>(stride_means, j, q)] : 0.0f;
+		const float exact = (j < k && q < dim) ? means[elem<LM>(stride_means, j, q)] : 0.0f;
+		const float v = (j < k && q < dim) ? exact - wide_frame[q] : 0.0f;
+		exact2 += exact * exact;
 		c2 += v * v;
 		__bf16 hi, mid;
 		const float rest = split_bf16(-2.0f * v, hi, mid);
@@ -121,22 +160,27 @@ pack_means_bf16_kernel(const float* __restrict__ means, size_t stride_means, flo
 		const uint32_t unit = 4 * (q / KBLOCK) + 2 * ((q % KBLOCK) / 8);
 		parts[8 * unit + q % 8] = hi;
 		parts[8 * (unit + 1) + q % 8] = mid;
-		if (q < dim) means_t[(size_t)q * kp + j] = v; /* exact copy for the recheck pass */
+		if (q < dim) means_t[(size_t)q * kp + j] = exact; /* exact copy for the recheck pass */
 	}
 	const uint32_t pad_floats = ROW_PAD + (j % TILE == TILE - 1 ? TILE_PAD : 0);
-	if (!packed_slots && lane < pad_floats) row[dp + lane] = 0.0f;
+	if (!packed_form && lane < pad_floats) row[dp + lane] = 0.0f;
 	for (int off = WAVE / 2; off > 0; off >>= 1) {
 		c2 += __shfl_xor(c2, off);
 		mid2 += __shfl_xor(mid2, off);
 		rest2 += __shfl_xor(rest2, off);
+		exact2 += __shfl_xor(exact2, off);
 	}
 	if (lane == 0) {
 		norms[norm_at(j)] = j < k ? c2 : __builtin_inff();
+		norms[exact_norms_offset(kp) + norm_at(j)] = j < k ? exact2 : __builtin_inff();
 		float* part_norms = norms + split_norms_offset(kp);
 		part_norms[j] = mid2;
 		part_norms[kp + j] = rest2;
 	}
-	if (lane < NORM_TILE - TILE && j % TILE == 0) norms[(j / TILE) * NORM_TILE + TILE + lane] = __builtin_inff();
+	if (lane < NORM_TILE - TILE && j % TILE == 0) {
+		norms[(j / TILE) * NORM_TILE + TILE + lane] = __builtin_inff();
+		norms[exact_norms_offset(kp) + (j / TILE) * NORM_TILE + TILE + lane] = __builtin_inff();
+	}
 }
 
 bool bf16_supports(const AssignArgs& a, const DeviceInfo& dev)
@@ -181,13 +225,19 @@ int launch_assign_bf16(const AssignArgs& args, kmx_exec_params* exec, Workspace*
 	 * lane-per-centroid kernels, which then need fewer launches); so do the packed rows, whose sweep queues more points
 	 * than the fp32 one and screens a tile with a single MFMA */
 	const bool screened = !a.ranking_only && a.k >= 128 && (a.dim > 32 || packed_rows(a.dim));
-	a.shift_rows = screened && packed_rows(a.dim);
-	a.shifted_cap = a.shift_rows ? screened_rows_cap(a) : 0xFFFFFFFFu;
+	/* The sweep works in a frame moved to the middle of the centroids (certificate.h): tau then scales with the spread of
+	 * the data instead of its distance from the origin. The screen shares the frame and takes the thresholds as they are
+	 * (queue entries beyond its block of copied rows, which other kernels read, get infinite ones); for the other kernels
+	 * of the exact pass the sweep takes the thresholds back to the frame of the data. The packed rows move only where the
+	 * screen follows; the double path ranks float copies of its points, whose rounding is relative to the origin anyway. */
+	a.shift_rows = packed_rows(a.dim) ? screened : !a.ranking_only;
+	a.shifted_cap = (a.shift_rows && screened) ? screened_rows_cap(a) : 0xFFFFFFFFu;
+	a.unmoved_thresholds = a.shift_rows && !screened;
 	const uint32_t kb = pick_kb(a.dim);
 	const uint32_t dp = KBLOCK * kb;
 	const uint32_t kp = round_up(a.k, TILE);
 	const uint32_t rs = packed_rows(a.dim) ? row_floats<1, true>() : dp + ROW_PAD;
-	int rc = reserve_packed(ws, (size_t)(kp / TILE) * tile_floats(rs), frame_offset(kp) + 4, (size_t)kp * a.dim);
+	int rc = reserve_packed(ws, (size_t)(kp / TILE) * tile_floats(rs), split_norms_floats(kp), (size_t)kp * a.dim);
 	if (rc) return rc;
 	rc = reserve_queue(ws, 2 * (size_t)a.n); /* (point, threshold) pairs */
 	if (rc) return rc;
@@ -201,7 +251,7 @@ int launch_assign_bf16(const AssignArgs& args, kmx_exec_params* exec, Workspace*
 	KMX_LAUNCH_CHECK("pack_means_bf16_kernel");
 
 	/* tau = kd (|x|^2 + max|c|^2) + the bound of the dropped products (certificate.h) */
-	const float kd = (packed_rows(a.dim) ? cert_kd_packed(a.dim) : cert_kd_split(a.dim)) + a.kd_extra;
+	const float kd = (packed_rows(a.dim) ? cert_kd_packed(a.dim) : cert_kd_split(a.dim) + (a.shift_rows ? 8.0f * CERT_UNIT : 0.0f)) + a.kd_extra;
 	switch (kb) {
 	case 1: rc = launch_bf16_1(a, exec, ws, dev, kp, kd); break;
 	case 2: rc = launch_bf16_2(a, exec, ws, dev, kp, kd); break;
@@ -213,7 +263,10 @@ int launch_assign_bf16(const AssignArgs& args, kmx_exec_params* exec, Workspace*
 	}
 	if (rc) return rc;
 	if (a.ranking_only) return KMX_OK; /* the caller resolves the queued points */
-	return screened ? launch_recheck_screened(a, ws, kp, dev) : launch_recheck(a, ws, kp);
+	ws->exact_norms = ws->norms + exact_norms_offset(kp);
+	rc = screened ? launch_recheck_screened(a, ws, kp, dev) : launch_recheck(a, ws, kp);
+	ws->exact_norms = nullptr;
+	return rc;
 }
 
 } // namespace kmx

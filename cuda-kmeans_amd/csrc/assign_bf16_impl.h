@@ -49,8 +49,14 @@ __device__ __forceinline__ float split_bf16(float v, __bf16& hi, __bf16& mid)
 /* The norms array of the split-bf16 kernels: the tiles of |c|^2 (NORM_TILE floats per tile), then per padded row
  * sum_i c'mid_i^2 and, kp floats on, sum_i c'rest_i^2 (c' = -2c; what the certificate needs, see certificate.h). */
 __host__ __device__ __forceinline__ size_t split_norms_offset(uint32_t kp) { return (size_t)(kp / TILE) * NORM_TILE; }
-/* ... and behind those the 4 coordinates of the frame the packed rows are swept in (zeros: the frame of the data) */
+/* ... and behind those the frame the rows are swept in: FRAME_DIMS coordinates of the vector m that is subtracted from
+ * every point and centroid before they are split (zeros: the frame of the data), then |m|^2 and an upper bound of |m| */
+constexpr uint32_t FRAME_DIMS = 256;
+constexpr uint32_t FRAME_FLOATS = FRAME_DIMS + 4;
 __host__ __device__ __forceinline__ size_t frame_offset(uint32_t kp) { return split_norms_offset(kp) + 2 * (size_t)kp; }
+/* ... and behind the frame |c|^2 of the centroids as given, in the layout of the first block (for the exact pass) */
+__host__ __device__ __forceinline__ size_t exact_norms_offset(uint32_t kp) { return frame_offset(kp) + FRAME_FLOATS; }
+__host__ __device__ __forceinline__ size_t split_norms_floats(uint32_t kp) { return exact_norms_offset(kp) + split_norms_offset(kp); }
 struct Frame { float m[4]; };
 
 /* One tile of 32 points as B operands: per block of 16 dimensions the lane holds the 8 dimensions of its
@@ -164,18 +170,25 @@ __device__ __forceinline__ void request_split_points(RawPoints<KB, false> (&raw)
 	}
 }
 
+/* The rows are swept as x - m (`frame`: the FRAME_DIMS coordinates of m, zero beyond the row; the packing kernel moved the
+ * centroids alike). xx = the lane's share of |x - m|^2, xm = its share of (x - m) . m (which takes a threshold back to the
+ * frame of the data, see unmoved_threshold). */
 template <int KB, int P>
-__device__ __forceinline__ void convert_split_points(SplitPoints<KB> (&b)[P], float (&xx)[P], const RawPoints<KB, false> (&raw)[P])
+__device__ __forceinline__ void convert_split_points(SplitPoints<KB> (&b)[P], float (&xx)[P], float (&xm)[P], const RawPoints<KB, false> (&raw)[P],
+                                                     const float* frame, uint32_t h)
 {
 #pragma unroll
 	for (int p = 0; p < P; ++p) {
-		float part = 0.0f;
+		float part = 0.0f, along = 0.0f;
 #pragma unroll
 		for (int kb = 0; kb < KB; ++kb) {
+			const f32x4 m0 = *(const f32x4*)(frame + kb * KBLOCK + h * 8), m1 = *(const f32x4*)(frame + kb * KBLOCK + h * 8 + 4);
+			const float m[8] = { m0.x, m0.y, m0.z, m0.w, m1.x, m1.y, m1.z, m1.w };
 #pragma unroll
 			for (int j = 0; j < 8; ++j) {
-				const float v = raw[p].v[8 * kb + j];
+				const float v = raw[p].v[8 * kb + j] - m[j];
 				part += v * v;
+				along += v * m[j];
 				__bf16 hi, mid;
 				split_bf16(v, hi, mid);
 				b[p].hi[kb][j] = hi;
@@ -183,54 +196,83 @@ __device__ __forceinline__ void convert_split_points(SplitPoints<KB> (&b)[P], fl
 			}
 		}
 		xx[p] = part;
+		xm[p] = along;
 	}
 }
 
-/* request and conversion back to back, one block of 16 dimensions at a time (the rows of the widest kernels fill the registers) */
-template <int KB, int P, int LD, bool VEC>
-__device__ __forceinline__ void load_split_points(SplitPoints<KB> (&b)[P], float (&xx)[P], const float* __restrict__ data, size_t stride,
-                                                  uint32_t base, uint32_t col, uint32_t h, uint32_t dim, uint32_t n)
+/* Request and conversion of the rows of P tiles. FENCED (the sweeps of rows of more than 64 dimensions, which fill the
+ * registers): all coordinates of a point are requested first, then the blocks of 16 dimensions are converted one at a time
+ * behind a fence each, so that the coordinates of the frame are not requested ahead and held as well. Otherwise the
+ * scheduler is left to interleave the blocks. */
+template <int KB, int P, int LD, bool VEC, bool FENCED = false>
+__device__ __forceinline__ void load_split_points(SplitPoints<KB> (&b)[P], float (&xx)[P], float (&xm)[P], const float* __restrict__ data, size_t stride,
+                                                  uint32_t base, uint32_t col, uint32_t h, uint32_t dim, uint32_t n, const float* frame)
 {
 #pragma unroll
 	for (int p = 0; p < P; ++p) {
 		const uint32_t pt = base + p * TILE + col;
 		const bool valid = pt < n;
-		float part = 0.0f;
-#pragma unroll
-		for (int kb = 0; kb < KB; ++kb) {
+		float v[KB][8];
+		auto request = [&](int kb) {
 			const uint32_t d0 = kb * KBLOCK + h * 8;
-			float v[8];
 			if (LD == KMX_AOS && VEC) {
 				const float* src = data + (size_t)pt * stride + d0;
 				f32x4 lo = { 0.0f, 0.0f, 0.0f, 0.0f }, up = { 0.0f, 0.0f, 0.0f, 0.0f };
 				if (valid && d0 < dim) lo = *(const f32x4*)src;
 				if (valid && d0 + 4 < dim) up = *(const f32x4*)(src + 4);
-				v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w;
-				v[4] = up.x; v[5] = up.y; v[6] = up.z; v[7] = up.w;
+				v[kb][0] = lo.x; v[kb][1] = lo.y; v[kb][2] = lo.z; v[kb][3] = lo.w;
+				v[kb][4] = up.x; v[kb][5] = up.y; v[kb][6] = up.z; v[kb][7] = up.w;
 			}
 			else if (LD == KMX_SOA) {
+				/* the address advances from load to load; long rows are loaded 16 coordinates at a time, so that only a few
+				 * of their 64-bit addresses are alive at once */
 				const float* src = data + (size_t)d0 * stride + pt;
 #pragma unroll
 				for (int j = 0; j < 8; ++j) {
-					v[j] = (valid && d0 + j < dim) ? *src : 0.0f;
+					v[kb][j] = (valid && d0 + j < dim) ? *src : 0.0f;
 					src += stride;
 				}
 				if (KB > 4 && kb % 2 == 1) __builtin_amdgcn_sched_barrier(0);
 			}
 			else {
 #pragma unroll
-				for (int j = 0; j < 8; ++j) v[j] = (valid && d0 + j < dim) ? data[elem<LD>(stride, pt, d0 + j)] : 0.0f;
+				for (int j = 0; j < 8; ++j) v[kb][j] = (valid && d0 + j < dim) ? data[elem<LD>(stride, pt, d0 + j)] : 0.0f;
 			}
+		};
+		float part = 0.0f, along = 0.0f;
+		auto convert = [&](int kb) {
+			const uint32_t d0 = kb * KBLOCK + h * 8;
+			const f32x4 m0 = *(const f32x4*)(frame + d0), m1 = *(const f32x4*)(frame + d0 + 4);
+			const float m[8] = { m0.x, m0.y, m0.z, m0.w, m1.x, m1.y, m1.z, m1.w };
 #pragma unroll
 			for (int j = 0; j < 8; ++j) {
-				part += v[j] * v[j];
+				const float w = v[kb][j] - m[j];
+				part += w * w;
+				along += w * m[j];
 				__bf16 hi, mid;
-				split_bf16(v[j], hi, mid);
+				split_bf16(w, hi, mid);
 				b[p].hi[kb][j] = hi;
 				b[p].mid[kb][j] = mid;
 			}
+		};
+		if (FENCED) {
+#pragma unroll
+			for (int kb = 0; kb < KB; ++kb) request(kb);
+#pragma unroll
+			for (int kb = 0; kb < KB; ++kb) {
+				__builtin_amdgcn_sched_barrier(0);
+				convert(kb);
+			}
+		}
+		else {
+#pragma unroll
+			for (int kb = 0; kb < KB; ++kb) {
+				request(kb);
+				convert(kb);
+			}
 		}
 		xx[p] = part;
+		xm[p] = along;
 	}
 }
 
@@ -510,7 +552,7 @@ __global__ void __launch_bounds__(MFMA_WAVES * WAVE)
 assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* __restrict__ packed, const float* __restrict__ norms,
                    uint32_t* __restrict__ assignment, uint32_t* __restrict__ queue, uint32_t* __restrict__ counters,
                    uint32_t dim, uint32_t k, uint32_t kp, uint32_t n, uint32_t chunk_rows, float kd, float neg_inf, uint32_t shifted_cap,
-                   Slice... slice_argument)
+                   float kd_unmoved, Slice... slice_argument)
 {
 	static_assert(sizeof...(Slice) <= 1, "at most one slice");
 	constexpr bool SLICED = sizeof...(Slice) == 1;
@@ -524,6 +566,12 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 #pragma unroll
 		for (int j = 0; j < 4; ++j) frame.m[j] = all_norms[frame_offset(all_kp) + j];
 	}
+	__shared__ __attribute__((aligned(16))) float frame_lds[PACKED ? 4 : KB * KBLOCK]; /* unpacked rows: m, see convert_split_points */
+	if constexpr (!PACKED) {
+		for (uint32_t i = threadIdx.x; i < KB * KBLOCK; i += blockDim.x) frame_lds[i] = all_norms[frame_offset(all_kp) + i];
+	}
+	const float frame_m2 = PACKED ? 0.0f : all_norms[frame_offset(all_kp) + FRAME_DIMS];        /* |m|^2 */
+	const float frame_norm = PACKED ? 0.0f : all_norms[frame_offset(all_kp) + FRAME_DIMS + 1];  /* an upper bound of |m| */
 	__shared__ uint32_t wave_max[4][MFMA_WAVES]; /* rows 0..2: maxima per wavefront; [3][0]: items of this work-group handed out so far */
 	__shared__ uint32_t flag_list[MFMA_WAVES][2 * FLAG_CAP]; /* (point, threshold) pairs */
 	uint32_t& claimed = wave_max[3][0]; /* (kept inside an array whose size is a multiple of 16 bytes: the tiles behind the static data must stay 16-byte aligned for their 128-bit reads) */
@@ -627,7 +675,7 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 		slot = (uint32_t)__shfl((int)slot, 0);
 		/* (entries from shifted_cap on: thresholds of a moved frame mean nothing to the kernels that will read them) */
 		for (uint32_t i = lane; i < 2 * flagged; i += WAVE)
-			queue[2 * (size_t)slot + i] = (PACKED && (i & 1u) && slot + i / 2 >= shifted_cap) ? __float_as_uint(__builtin_inff()) : flag_list[wave][i];
+			queue[2 * (size_t)slot + i] = ((i & 1u) && slot + i / 2 >= shifted_cap) ? __float_as_uint(__builtin_inff()) : flag_list[wave][i];
 		__builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
 		__builtin_amdgcn_wave_barrier();
 		flagged = 0;
@@ -740,13 +788,14 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 		}
 	};
 
-	auto sweep = [&](const SplitPoints<KB> (&b)[P], const float (&xx)[P], uint32_t base) {
-		float x2[P];
+	auto sweep = [&](const SplitPoints<KB> (&b)[P], const float (&xx)[P], const float (&xalong)[P], uint32_t base) {
+		float x2[P], along_m[P];
 		Track st[P];
 #pragma unroll
 		for (int p = 0; p < P; ++p) {
 			/* PACKED: the half-waves hold |x|^2 and sum_i xrest_i^2 of the same point; the pair is taken apart again below */
 			x2[p] = PACKED ? xx[p] : xx[p] + __shfl_xor(xx[p], 32);
+			along_m[p] = PACKED ? 0.0f : xalong[p] + __shfl_xor(xalong[p], 32); /* (x - m) . m of the point */
 			st[p].m1 = __builtin_inff();
 			st[p].m2 = __builtin_inff();
 			st[p].tile = 0;
@@ -1103,6 +1152,7 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 				xsq = x2[p];
 				tau = cert_tau(kd, xsq, xmid2, cert);
 			}
+			const float along = along_m[p];
 			const uint32_t pt = base + p * TILE + col;
 			const bool mine = h == 0 && pt < n;
 			if constexpr (SLICED) {
@@ -1136,7 +1186,10 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 				if (flag) {
 					const uint32_t at = 2 * (flagged + __builtin_popcountll(mask & ((1ull << lane) - 1ull)));
 					flag_list[wave][at] = pt;
-					flag_list[wave][at + 1] = screening_threshold(first, tau);
+					/* kd_unmoved > 0: for kernels that evaluate in the frame of the data (certificate.h) */
+					flag_list[wave][at + 1] = kd_unmoved > 0.0f
+						? screening_threshold(cert_unmoved_threshold(first, tau, xsq, along, c2max, frame_m2, frame_norm, kd_unmoved), 0.0f)
+						: screening_threshold(first, tau);
 				}
 				flagged += add;
 			}
@@ -1144,9 +1197,13 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 	};
 
 	static_assert(!PACKED || KB == 1, "the packed form is one block of 16 slots");
-	auto load_points = [&](SplitPoints<KB> (&bb)[P], float (&xs)[P], uint32_t first) {
-		if constexpr (PACKED) load_packed_points<P, LD, VEC>(bb, xs, data, stride, first, col, h, dim, n, frame);
-		else load_split_points<KB, P, LD, VEC>(bb, xs, data, stride, first, col, h, dim, n);
+	auto load_points = [&](SplitPoints<KB> (&bb)[P], float (&xs)[P], float (&xa)[P], uint32_t first) {
+		if constexpr (PACKED) {
+			load_packed_points<P, LD, VEC>(bb, xs, data, stride, first, col, h, dim, n, frame);
+#pragma unroll
+			for (int p = 0; p < P; ++p) xa[p] = 0.0f; /* (the thresholds of the packed rows stay in the moved frame) */
+		}
+		else load_split_points<KB, P, LD, VEC, (KB > 4)>(bb, xs, xa, data, stride, first, col, h, dim, n, frame_lds);
 	};
 
 	/*
@@ -1179,14 +1236,18 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 		/* one set of split operands; the raw coordinates of the next item travel while the current one is swept */
 		RawPoints<KB, PACKED> raw[P];
 		SplitPoints<KB> b0[P];
-		float xx0[P];
+		float xx0[P], xm0[P];
 		auto request_points = [&](uint32_t first) {
 			if constexpr (PACKED) request_packed_points<P, LD, VEC>(raw, data, stride, first, col, dim, n);
 			else request_split_points<KB, P, LD, VEC>(raw, data, stride, first, col, h, dim, n);
 		};
 		auto convert_points = [&]() {
-			if constexpr (PACKED) convert_packed_points<P>(b0, xx0, raw, h, frame);
-			else convert_split_points<KB, P>(b0, xx0, raw);
+			if constexpr (PACKED) {
+				convert_packed_points<P>(b0, xx0, raw, h, frame);
+#pragma unroll
+				for (int p = 0; p < P; ++p) xm0[p] = 0.0f;
+			}
+			else convert_split_points<KB, P>(b0, xx0, xm0, raw, frame_lds, h);
 		};
 		uint32_t item = uniform(claim());
 		uint32_t next = uniform(claim());
@@ -1197,7 +1258,7 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 		while (item < items) {
 			const uint32_t after = claim();
 			if (next < items) request_points(first_point(next));
-			sweep(b0, xx0, first_point(item));
+			sweep(b0, xx0, xm0, first_point(item));
 			item = next;
 			next = uniform(after);
 			if (item < items) convert_points();
@@ -1205,12 +1266,12 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 	}
 	else {
 		SplitPoints<KB> b0[P];
-		float xx0[P];
+		float xx0[P], xm0[P];
 		uint32_t item = uniform(claim());
 		while (item < items) {
 			const uint32_t after = claim();
-			load_points(b0, xx0, first_point(item));
-			sweep(b0, xx0, first_point(item));
+			load_points(b0, xx0, xm0, first_point(item));
+			sweep(b0, xx0, xm0, first_point(item));
 			item = uniform(after);
 		}
 	}
@@ -1238,7 +1299,7 @@ static __device__ __attribute__((noinline)) void evaluate_pair_of_row(const floa
 }
 
 template <int KB, int P, bool PACKED = false>
-__global__ void __launch_bounds__(SCREEN_WAVES * WAVE) __attribute__((amdgpu_waves_per_eu(KB <= 3 ? 2 : 1)))
+__global__ void __launch_bounds__(SCREEN_WAVES * WAVE) __attribute__((amdgpu_waves_per_eu((KB <= 3 || KB == 8) ? 2 : 1)))
 screen_bf16_kernel(const float* __restrict__ rows, const float* __restrict__ packed, const float* __restrict__ norms,
                    const float* __restrict__ means_t, const uint32_t* __restrict__ row_queue, const uint32_t* __restrict__ row_count,
                    uint32_t* __restrict__ pairs, uint32_t* __restrict__ item_pairs,
@@ -1294,7 +1355,11 @@ screen_bf16_kernel(const float* __restrict__ rows, const float* __restrict__ pac
 		SplitPoints<KB> b[P];
 		float xx[P];
 		if constexpr (PACKED) load_packed_points<P, KMX_AOS, false>(b, xx, rows, dim, base, col, h, dim, count, frame);
-		else load_split_points<KB, P, KMX_AOS, false>(b, xx, rows, dim, base, col, h, dim, count);
+		else {
+			float along[P]; /* (not needed here: the thresholds of these rows are values of the moved frame) */
+			load_split_points<KB, P, KMX_AOS, false, false>(b, xx, along, rows, dim, base, col, h, dim, count, norms + frame_offset(kp));
+			__builtin_amdgcn_sched_barrier(0); /* (the operands of the first tiles are not requested before the rows are split) */
+		}
 		float thr[P];
 		bool valid[P];
 #pragma unroll
@@ -1489,9 +1554,9 @@ static int launch_bf16_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 	const uint32_t unit_points = MFMA_WAVES * (stream_mode ? P : PR) * TILE;
 	const uint32_t units = (a.n + unit_points - 1) / unit_points;
 	void (*kernel)(const float*, size_t, const float*, const float*, uint32_t*, uint32_t*, uint32_t*,
-	               uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, float, float, uint32_t) = nullptr;
+	               uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, float, float, uint32_t, float) = nullptr;
 	void (*sliced_kernel)(const float*, size_t, const float*, const float*, uint32_t*, uint32_t*, uint32_t*,
-	                      uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, float, float, uint32_t, CentroidSlice) = nullptr;
+	                      uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, float, float, uint32_t, float, CentroidSlice) = nullptr;
 	if constexpr (KB == 4) {
 		if (slices > 1) sliced_kernel = assign_bf16_kernel<KB, PR, LD, VEC, false, false, PF, PACKED, CentroidSlice>;
 	}
@@ -1515,12 +1580,13 @@ static int launch_bf16_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 	per_cu = std::max(1, std::min(per_cu, 4));
 	const uint32_t grid = std::min(units, dev.compute_units * (uint32_t)per_cu);
 	exec->block_count = grid;
+	const float kd_unmoved = a.unmoved_thresholds ? cert_kd_unmoved(a.dim) : 0.0f;
 	int rc = profile_begin(0);
 	if (rc) return rc;
 	if (slices == 1) {
 		KMX_LAUNCH_KERNEL(kernel, dim3(grid), dim3(MFMA_WAVES * WAVE), lds_bytes, stream(),
 		                   a.data, a.stride, ws->packed_means, ws->norms, a.assignment, ws->queue, ws->counters,
-		                   a.dim, a.k, kp, a.n, chunk_rows, kd, -__builtin_inff(), a.shifted_cap);
+		                   a.dim, a.k, kp, a.n, chunk_rows, kd, -__builtin_inff(), a.shifted_cap, kd_unmoved);
 		KMX_LAUNCH_CHECK("assign_bf16_kernel");
 	}
 	else {
@@ -1532,7 +1598,7 @@ static int launch_bf16_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 			KMX_LAUNCH_KERNEL(sliced_kernel, dim3(grid), dim3(MFMA_WAVES * WAVE), lds_bytes, stream(),
 			                   a.data, a.stride, ws->packed_means + packed_row(row0, RS), ws->norms + (size_t)(row0 / TILE) * NORM_TILE,
 			                   a.assignment, ws->queue, ws->counters,
-			                   a.dim, std::min(a.k - std::min(a.k, row0), rows), rows, a.n, rows, kd, -__builtin_inff(), a.shifted_cap, slice);
+			                   a.dim, std::min(a.k - std::min(a.k, row0), rows), rows, a.n, rows, kd, -__builtin_inff(), a.shifted_cap, kd_unmoved, slice);
 			KMX_LAUNCH_CHECK("assign_bf16_kernel (a slice of the centroids)");
 		}
 	}

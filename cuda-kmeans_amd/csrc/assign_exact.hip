@@ -585,6 +585,9 @@ static int launch_recheck_dpad(const AssignArgs& a, Workspace* ws, uint32_t kp)
 	return launch_recheck_reg<LD, L, 2, 64>(a, ws, kp);
 }
 
+/* |c|^2 of the centroids as given (a sweep in a moved frame keeps the norms of the moved centroids in ws->norms) */
+static const float* exact_norms(const Workspace* ws) { return ws->exact_norms ? ws->exact_norms : ws->norms; }
+
 template <int LD, int DPAD>
 static int launch_recheck_points(const AssignArgs& a, Workspace* ws, uint32_t kp)
 {
@@ -595,7 +598,7 @@ static int launch_recheck_points(const AssignArgs& a, Workspace* ws, uint32_t kp
 	const dim3 grid(DPAD <= 32 ? 512 : 256); /* two work-groups fit a compute unit while the rows of a lane take at most 64 registers */
 #define KMX_RECHECK_POINTS(FULL, C) \
 	KMX_LAUNCH_KERNEL((recheck_points_kernel<LD, DPAD, FULL, C>), grid, dim3(threads), 0, stream(), \
-	                   a.data, a.stride, ws->means_t, ws->norms, a.assignment, a.dim, a.k, kp, ws->queue, ws->counters)
+	                   a.data, a.stride, ws->means_t, exact_norms(ws), a.assignment, a.dim, a.k, kp, ws->queue, ws->counters)
 	if (a.dim == DPAD) { if (two) KMX_RECHECK_POINTS(true, CPL); else KMX_RECHECK_POINTS(true, 1); }
 	else { if (two) KMX_RECHECK_POINTS(false, CPL); else KMX_RECHECK_POINTS(false, 1); }
 #undef KMX_RECHECK_POINTS
@@ -610,10 +613,10 @@ static int launch_recheck_sliced(const AssignArgs& a, Workspace* ws, uint32_t kp
 	const dim3 grid(256);
 	if (a.dim % SLICE == 0)
 		KMX_LAUNCH_KERNEL((recheck_sliced_kernel<LD, true>), grid, dim3(threads), 0, stream(),
-		                   a.data, a.stride, ws->means_t, ws->norms, a.assignment, a.dim, a.k, kp, ws->queue, ws->counters);
+		                   a.data, a.stride, ws->means_t, exact_norms(ws), a.assignment, a.dim, a.k, kp, ws->queue, ws->counters);
 	else
 		KMX_LAUNCH_KERNEL((recheck_sliced_kernel<LD, false>), grid, dim3(threads), 0, stream(),
-		                   a.data, a.stride, ws->means_t, ws->norms, a.assignment, a.dim, a.k, kp, ws->queue, ws->counters);
+		                   a.data, a.stride, ws->means_t, exact_norms(ws), a.assignment, a.dim, a.k, kp, ws->queue, ws->counters);
 	KMX_LAUNCH_CHECK("recheck_sliced_kernel");
 	return KMX_OK;
 }

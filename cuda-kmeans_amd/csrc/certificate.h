@@ -105,6 +105,29 @@ KMX_HD float cert_tau(float kd, float x2, float xpart2, const CertCoeffs& c)
 	return kd * (x2 + c.c2max) + (c.a * cert_sqrt_upper(xpart2) + c.b * cert_sqrt_upper(x2));
 }
 
+/*
+ * The screening threshold of a sweep in a moved frame, taken back to the frame of the data for a kernel that evaluates
+ * a_r[j] ~ A_j = |c_j|^2 - 2 c_j . x there, as a chain of fused multiply-adds. With x' = x - m, c' = c - m:
+ *      A'_j = |c'_j|^2 - 2 c'_j . x' = A_j + sh,    sh = 2 x . m - |m|^2 = 2 x' . m + |m|^2      (the same for every j),
+ * so a centroid can be the serial result only if A_j <= first' + tau' - sh (first' and tau' of the moved frame), and
+ * the kernel may drop j only if a_r[j] exceeds that by more than its own error and the error of the computed sh:
+ *   - the chain: (2 d + 7) u (|c_j|^2 + 2 |c_j||x|) <= (2 d + 7) u' Q with Q >= |x|^2 + max_j |c_j|^2 of the data as
+ *     given; Q = (|x'| + |m|)^2 + (max_j |c'_j| + |m|)^2 from what the sweep has at hand;
+ *   - sh: d products and sums, the rounding of x' = fl(x - m) against m (u |x'||m|) and of |m|^2:
+ *     (d + 4) u' (|x'| + |m|)^2 <= (d + 4) u' Q;
+ *   - the three roundings of first' + tau' - sh + slack: 2 u' Q.
+ * Together (3 d + 13) u' Q, with d the padded length of the chains (up to 15 more than the row); the kernels add
+ * (4 d + 40) u' Q. With m = 0 this is first + tau + (4 d + 40) u' S. (The three-product form also pays 8 u' S in kd
+ * for the roundings of x' and c', as the packed form does.)
+ */
+KMX_HD float cert_kd_unmoved(unsigned dim) { return (4.0f * (float)dim + 40.0f) * CERT_UNIT; }
+KMX_HD float cert_unmoved_threshold(float first, float tau, float x2, float along, float c2max, float m2, float mnorm, float kdu)
+{
+	const float sh = 2.0f * along + m2;
+	const float xr = cert_sqrt_upper(x2) + mnorm, cr = cert_sqrt_upper(c2max) + mnorm;
+	return (first + tau) - sh + kdu * ((xr * xr + cr * cr) * 1.00001f);
+}
+
 } // namespace kmx
 
 #endif

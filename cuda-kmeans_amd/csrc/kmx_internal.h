@@ -64,6 +64,7 @@ struct Workspace {
 	float* queued_rows = nullptr;         size_t queued_rows_cap = 0;   /* floats */
 	uint32_t* queued_index = nullptr;     size_t queued_index_cap = 0;  /* words: per row 2 (queue) + 2 (assignment or 64-bit key), then the screen's pair counters and pairs */
 	uint32_t* carried = nullptr;          size_t carried_cap = 0;       /* words: per point the leader and the two smallest ranking values over the slices of centroids swept so far */
+	const float* exact_norms = nullptr; /* |c|^2 of the centroids as given, in the layout of `norms`, for the exact pass of a sweep that moved its frame (points into `norms`; null: `norms` holds them) */
 	bool fixed = false; /* the work space of the entry point that allocates nothing: its buffers never grow, a call that needs more is refused */
 };
 int workspace(Workspace** ws);
@@ -116,11 +117,13 @@ struct AssignArgs {
 	 * uncertified points (pairs of point number and threshold, length in counters[0]) to the caller. */
 	float kd_extra = 0.0f;
 	bool ranking_only = false;
-	/* Packed rows (at most 4 dimensions) whose exact pass is the screened one are swept in a frame moved to the middle of the
-	 * centroids (shift_rows): the thresholds of the queue are then values of that frame, which only the screen shares, so
-	 * entries from position shifted_cap on -- those the screen has no rows for -- get an infinite threshold. */
+	/* The split-bf16 sweep may work in a frame moved to the middle of the centroids (shift_rows). Where the screen follows,
+	 * the thresholds of the queue stay values of that frame, which only the screen shares, so entries from position
+	 * shifted_cap on -- those the screen has no rows for -- get an infinite threshold; where the other kernels of the exact
+	 * pass follow, the sweep takes the thresholds back to the frame of the data (unmoved_thresholds). */
 	bool shift_rows = false;
 	uint32_t shifted_cap = 0xFFFFFFFFu;
+	bool unmoved_thresholds = false;
 };
 
 struct UpdateArgs {

@@ -222,6 +222,27 @@ def test_centroids_swept_in_slices(km, orc, gpu, dim, k, n, lds_budget):
         assert bad.size == 0, "%s: %d mismatches, first at %s (gpu %s, oracle %s)" % (name, bad.size, bad[:5], got[bad[:5]], want[bad[:5]])
 
 
+@pytest.mark.parametrize("dim,k,n", [(32, 1024, 200000), (64, 512, 100000), (16, 256, 200000), (8, 100, 100000),
+                                     (48, 2048, 70000), (128, 300, 50000), (200, 1024, 20000)])
+@pytest.mark.parametrize("offset", [0.0, 100.0, 3000.0])
+def test_data_far_from_the_origin(km, orc, gpu, dim, k, n, offset):
+    """The split-bf16 sweep works in a frame moved to the middle of the centroids: the assignment is the oracle's wherever the
+    data lie, and the share of the points that the sweep leaves to the exact pass does not grow with their distance from
+    the origin (clusters of spread 1 inside [-10, 10]^d, moved by `offset` in every coordinate; in the frame of the data
+    the certificate would give up on every point at the last offset)."""
+    rng = np.random.default_rng(dim + k)
+    centres = rng.uniform(-10, 10, (k, dim)).astype(np.float32)
+    base = (centres[rng.integers(0, k, n)] + rng.normal(size=(n, dim)).astype(np.float32) + np.float32(offset)).astype(np.float32)
+    means = base[:k].copy()
+    want = orc.assign(base.ravel(), means.ravel(), dim, k, n, threads=0, fast=True)
+    for layout in (AOS, SOA):
+        d = base if layout == AOS else np.ascontiguousarray(base.T)
+        got, rechecked = gpu_assign(km, km.ASSIGN_MFMA_BF16X3, d.ravel(), means.ravel(), dim, k, n, layout, AOS)
+        bad = np.nonzero(got != want)[0]
+        assert bad.size == 0, "layout %d: %d mismatches, first at %s" % (layout, bad.size, bad[:5])
+        assert rechecked < n // 10, "%d of %d points left to the exact pass" % (rechecked, n)
+
+
 @pytest.mark.parametrize("dim,k,n", [(32, 256, 3000), (21, 1500, 4000), (96, 200, 1500), (4, 512, 5000)])
 def test_soa_points_in_the_exact_pass(km, orc, gpu, dim, k, n):
     """SoA points: the exact pass copies the rows of the queued points into a compact block. Inputs that queue every point
