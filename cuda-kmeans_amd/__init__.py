@@ -34,7 +34,7 @@ ABI_SYMBOLS = [
     "kmx_d2d", "kmx_sync", "kmx_set_stream", "kmx_shutdown", "kmx_fill_zero_u32", "kmx_assign_f32",
     "kmx_assign_last_rechecked", "kmx_assign_last_variant", "kmx_update_f32", "kmx_bucket_sum_f32", "kmx_fused_f32", "kmx_assign_f64", "kmx_update_f64", "kmx_fused_f64", "kmx_bucket_sum_f64", "kmx_set_queued_rows_limit",
     "kmx_graph_begin", "kmx_graph_end", "kmx_graph_launch", "kmx_graph_destroy", "kmx_event_create", "kmx_event_destroy", "kmx_event_record",
-    "kmx_event_elapsed_ms", "kmx_set_profiling", "kmx_last_kernel_ms", "kmx_last_error", "kmx_certificate_tau",
+    "kmx_event_elapsed_ms", "kmx_set_profiling", "kmx_last_kernel_ms", "kmx_last_error", "kmx_certificate_tau", "kmx_certificate_unmoved_threshold",
     "kmx_update_f32_noalloc", "kmx_reserve_f32", "kmx_prepare_points_f64", "kmx_forget_points_f64",
 ]
 
@@ -122,6 +122,7 @@ def hip_lib():
         lib.kmx_fused_f64.argtypes = lib.kmx_fused_f32.argtypes
         lib.kmx_bucket_sum_f64.argtypes = lib.kmx_bucket_sum_f32.argtypes
         lib.kmx_certificate_tau.argtypes = [ctypes.c_int, u32] + [ctypes.c_float] * 5 + [ctypes.POINTER(ctypes.c_float)]
+        lib.kmx_certificate_unmoved_threshold.argtypes = [u32] + [ctypes.c_float] * 7 + [ctypes.POINTER(ctypes.c_float)]
         lib.kmx_graph_begin.argtypes = []
         lib.kmx_graph_end.argtypes = [ctypes.POINTER(vp)]
         lib.kmx_graph_launch.argtypes = [vp]
@@ -373,6 +374,14 @@ class Graph:
         if self._g:
             check(hip_lib().kmx_graph_destroy(self._g))
             self._g = ctypes.c_void_p()
+
+
+def certificate_unmoved_threshold(dim, first, tau, x2, along, c2max, m2, mnorm):
+    """The threshold a sweep in a moved frame hands to the exact-pass kernels that evaluate in the frame of the data
+    (kmx_certificate_unmoved_threshold; host function, no device needed)."""
+    out = ctypes.c_float()
+    check(hip_lib().kmx_certificate_unmoved_threshold(dim, first, tau, x2, along, c2max, m2, mnorm, ctypes.byref(out)))
+    return float(out.value)
 
 
 def certificate_tau(form, dim, x2, xpart2, c2max, cmid2max, crest2max):

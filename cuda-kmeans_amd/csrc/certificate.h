@@ -34,10 +34,11 @@
  *        accumulation <= (4 d + 2) u' 2 S
  *        dropped = sum_i (c'hi_i + c'mid_i) xrest_i + c'rest_i x_i <= (|c'| + |c'rest|) |xrest| + |c'rest| |x|
  *     with |xrest| of the point computed when it is split.
- *     The packed sweep may work in a frame moved by a vector m (the middle of the centroids), on x' = fl(x - m) and
+ *     Both forms may work in a frame moved by a vector m (the middle of the centroids), on x' = fl(x - m) and
  *     c' = fl(c - m): distances do not depend on the frame, S becomes |x'|^2 + max_j |c'_j|^2, which is what makes tau
  *     small for data far from the origin, and the two roundings move a distance by at most 2 u (|x'| + |c'|)^2 <= 2 u' S,
- *     a difference of two distances by 4 u' S: 8 u' more in kd.
+ *     a difference of two distances by 4 u' S: 8 u' more in kd (part of the packed form's kd; the launcher adds it to
+ *     the three-product form's when that sweep moves its frame).
  * tau = kd S + TRUNC_FACTOR * (bound of the dropped products); kd = (12 d + 8 + 2 d + 12 + slack) u' and
  * (16 d + 8 + 2 d + 12 + 8 + slack) u'; TRUNC_FACTOR = 2 plus 1/16 for the fp32 roundings in the norms and square roots.
  * Values the bound does not cover (NaN, infinities, sums that overflow) make tau NaN or infinite, and the

@@ -685,6 +685,15 @@ int kmx_certificate_tau(int form, uint32_t dim, float x2, float xpart2, float c2
 	}
 }
 
+int kmx_certificate_unmoved_threshold(uint32_t dim, float first, float tau, float x2, float along, float c2max, float m2, float mnorm,
+                                      float* threshold)
+{
+	clear_error();
+	if (!threshold) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_certificate_unmoved_threshold: null pointer");
+	*threshold = cert_unmoved_threshold(first, tau, x2, along, c2max, m2, mnorm, cert_kd_unmoved(dim));
+	return KMX_OK;
+}
+
 int kmx_set_profiling(int enabled)
 {
 	clear_error();

@@ -323,10 +323,20 @@ int kmx_set_queued_rows_limit(size_t bytes);
  *   form 1: split-bf16 sweep, three products per dimension         xpart2 = sum_i xmid_i^2
  *   form 2: split-bf16 sweep, packed rows (dim <= 4, four products) xpart2 = sum_i xrest_i^2
  * x2 = |x|^2, c2max = max_j |c_j|^2, cmid2max / crest2max = max_j of the squared norms of the mid / rest parts of -2 c_j;
- * for form 2 all of them in the frame the packed sweep works in: with 128 centroids or more it subtracts the mean of the
- * (first 256) centroids from points and centroids, so the norms are those of the moved data.
+ * for forms 1 and 2 all of them in the frame the sweep works in: it subtracts a vector m from points and centroids (the
+ * mean of the first 16 centroids; for packed rows, with 128 centroids or more, of the first 256), so the norms are those
+ * of the moved data; the three-product form then adds 8 * 2^-23 * (x2 + c2max), which form 1 leaves out.
  */
 int kmx_certificate_tau(int form, uint32_t dim, float x2, float xpart2, float c2max, float cmid2max, float crest2max, float* tau);
+
+/*
+ * The screening threshold that a sweep in the moved frame hands to the kernels of the exact pass that evaluate
+ * |c_j|^2 - 2 c_j . x in the frame of the data (same purpose and conventions as kmx_certificate_tau: the kernels' own
+ * function, on the host). first, tau, x2 = |x - m|^2 and c2max = max_j |c_j - m|^2 are values of the moved frame,
+ * along = (x - m) . m, m2 = |m|^2, mnorm >= |m|. A centroid whose value exceeds the threshold cannot be the serial result.
+ */
+int kmx_certificate_unmoved_threshold(uint32_t dim, float first, float tau, float x2, float along, float c2max, float m2, float mnorm,
+                                      float* threshold);
 
 /* Message of the last failed call on this thread ("" if none). */
 const char* kmx_last_error(void);

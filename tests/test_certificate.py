@@ -306,3 +306,47 @@ def test_fp32_form_and_argument_errors(km):
         km.certificate_tau(7, 32, 1.0, 1.0, 1.0, 1.0, 1.0)
     assert not np.isfinite(km.certificate_tau(1, 8, float("inf"), 1.0, 1.0, 1.0, 1.0))
     assert np.isnan(km.certificate_tau(1, 8, float("nan"), 1.0, 1.0, 1.0, 1.0))
+
+
+@pytest.mark.parametrize("dim", [5, 16, 32, 100, 256])
+@pytest.mark.parametrize("offset", [0.0, 50.0, 3000.0, -1.0e5])
+def test_threshold_taken_back_to_the_frame_of_the_data(km, dim, offset):
+    """kmx_certificate_unmoved_threshold. A sweep in the frame moved by m knows its best moved ranking value
+    A'_j = |c_j - m|^2 - 2 (c_j - m).(x - m); the kernels of the exact pass evaluate a_r[j] = fma(-2, chain of fused
+    multiply-adds over x . c_j, |c_j|^2) on the data as given, in fp32. Here everything the kernels compute in fp32
+    is emulated in fp32, in their order (x - m and its projection on m, |m|^2, the chain), and the exact values in
+    float64. With first = the exact A'_j of a centroid and tau = 0 the threshold must not fall below that centroid's
+    own a_r[j] (it would be dropped although it attains `first`), nor exceed it by more than twice the allowance."""
+    rng = np.random.default_rng(dim + int(abs(offset)))
+    n, k = 200, 32
+    c = (rng.uniform(-10, 10, (k, dim)) + offset).astype(np.float32)
+    x = (c[rng.integers(0, k, n)] + rng.normal(size=(n, dim)) * (1 + rng.integers(0, 2, (n, 1)) * 20)).astype(np.float32)
+    m = c[:16].mean(axis=0).astype(np.float32)
+    xs = (x - m).astype(np.float32)                      # what the sweep splits
+    cs = (c - m).astype(np.float32)
+    def chain32(a, b, start=np.float32(0)):
+        acc = np.full(a.shape[:-1], start, np.float32)
+        for i in range(a.shape[-1]):                     # one rounding per fused multiply-add
+            acc = (acc.astype(np.float64) + a[..., i].astype(np.float64) * b[..., i].astype(np.float64)).astype(np.float32)
+        return acc
+    x2 = chain32(xs, xs)
+    along = chain32(xs, np.broadcast_to(m, xs.shape))
+    m2 = chain32(m[None, :], m[None, :])[0]
+    mnorm = np.float32(np.sqrt(np.float64(m2)) * 1.0001)
+    c2max = np.float32((cs.astype(np.float64) ** 2).sum(axis=1).max() * (1 + 1e-6))
+    x64, c64, m64 = x.astype(np.float64), c.astype(np.float64), m.astype(np.float64)
+    S = (x64 ** 2).sum(axis=1) + (c64 ** 2).sum(axis=1).max()
+    worst_low, worst_high = np.inf, 0.0
+    for j in range(k):
+        moved = ((c64[j] - m64) ** 2).sum() - 2.0 * ((x64 - m64) * (c64[j] - m64)).sum(axis=1)          # A'_j, exact
+        c2 = chain32(c[j][None, :], c[j][None, :])[0]
+        a_r = (np.float64(c2) - 2.0 * chain32(x, np.broadcast_to(c[j], x.shape)).astype(np.float64)).astype(np.float32)
+        thr = np.array([km.certificate_unmoved_threshold(dim, float(np.float32(moved[i])), 0.0, float(x2[i]), float(along[i]),
+                                                         float(c2max), float(m2), float(mnorm)) for i in range(n)])
+        gap = thr - a_r.astype(np.float64)
+        worst_low = min(worst_low, float((gap / S).min()))
+        worst_high = max(worst_high, float((gap / S).max()))
+    allowance = (4 * dim + 40) * U
+    assert worst_low >= 0.0, "threshold below the centroid's own value by %.3g S" % -worst_low
+    # Q, the bound of |x|^2 + max |c|^2 that the threshold uses, exceeds S by at most the triangle inequality's factor of 4
+    assert worst_high <= 4.0 * 2.0 * allowance, "threshold %.3g S above the value: more than twice the allowance" % worst_high
