@@ -83,40 +83,9 @@ pack_means_bf16_kernel(const float* __restrict__ means, size_t stride_means, flo
 		for (int q = 0; q < 4; ++q)
 			if (threadIdx.x == (uint32_t)q) norms[frame_offset(kp) + q] = frame[q];
 	}
-	/* unpacked rows: the same for rows of up to FRAME_DIMS dimensions, from the first 16 centroids (a thread per dimension,
-	 * its 16 loads in flight together: every work-group repeats this; zeros when the sweep keeps the frame of the data);
-	 * the first work-group stores it with |m|^2 and an upper bound of |m| */
+	/* unpacked rows: the same for rows of up to FRAME_DIMS dimensions (sweep_frame) */
 	__shared__ float wide_frame[FRAME_DIMS];
-	if (!(packed_slots & 1u)) {
-		constexpr uint32_t SAMPLE = 16;
-		const uint32_t sample = min(k, SAMPLE);
-		for (uint32_t q = threadIdx.x; q < dp; q += blockDim.x) {
-			float sum = 0.0f;
-			if ((packed_slots & 2u) && q < dim) {
-				float v[SAMPLE];
-#pragma unroll
-				for (uint32_t r = 0; r < SAMPLE; ++r) v[r] = r < sample ? means[elem<LM>(stride_means, r, q)] : 0.0f;
-#pragma unroll
-				for (uint32_t r = 0; r < SAMPLE; ++r) sum += __builtin_fabsf(v[r]) < __builtin_inff() ? v[r] : 0.0f;
-				sum = sum / (float)sample;
-				sum = __builtin_fabsf(sum) < __builtin_inff() ? sum : 0.0f; /* (the sum of finite values may overflow) */
-			}
-			wide_frame[q] = sum;
-		}
-		__syncthreads();
-		if (blockIdx.x == 0) {
-			for (uint32_t q = threadIdx.x; q < dp; q += blockDim.x) norms[frame_offset(kp) + q] = wide_frame[q];
-			if (threadIdx.x < WAVE) {
-				float m2 = 0.0f;
-				for (uint32_t q = lane; q < dp; q += WAVE) m2 += wide_frame[q] * wide_frame[q];
-				for (int off = WAVE / 2; off > 0; off >>= 1) m2 += __shfl_xor(m2, off);
-				if (lane == 0) {
-					norms[frame_offset(kp) + FRAME_DIMS] = m2; /* (as computed: it enters the shift of the thresholds) */
-					norms[frame_offset(kp) + FRAME_DIMS + 1] = __builtin_sqrtf(m2) * 1.0001f;
-				}
-			}
-		}
-	}
+	if (!(packed_slots & 1u)) sweep_frame<LM>(means, stride_means, dim, k, dp, (packed_slots & 2u) != 0, wide_frame, norms + frame_offset(kp));
 	if (j >= kp) return;
 	const bool packed_form = (packed_slots & 1u) != 0;
 	const uint32_t rs = packed_form ? row_floats<1, true>() : dp + ROW_PAD;

@@ -49,10 +49,7 @@ __device__ __forceinline__ float split_bf16(float v, __bf16& hi, __bf16& mid)
 /* The norms array of the split-bf16 kernels: the tiles of |c|^2 (NORM_TILE floats per tile), then per padded row
  * sum_i c'mid_i^2 and, kp floats on, sum_i c'rest_i^2 (c' = -2c; what the certificate needs, see certificate.h). */
 __host__ __device__ __forceinline__ size_t split_norms_offset(uint32_t kp) { return (size_t)(kp / TILE) * NORM_TILE; }
-/* ... and behind those the frame the rows are swept in: FRAME_DIMS coordinates of the vector m that is subtracted from
- * every point and centroid before they are split (zeros: the frame of the data), then |m|^2 and an upper bound of |m| */
-constexpr uint32_t FRAME_DIMS = 256;
-constexpr uint32_t FRAME_FLOATS = FRAME_DIMS + 4;
+/* ... and behind those the frame the rows are swept in (FRAME_FLOATS floats, see sweep_frame) */
 __host__ __device__ __forceinline__ size_t frame_offset(uint32_t kp) { return split_norms_offset(kp) + 2 * (size_t)kp; }
 /* ... and behind the frame |c|^2 of the centroids as given, in the layout of the first block (for the exact pass) */
 __host__ __device__ __forceinline__ size_t exact_norms_offset(uint32_t kp) { return frame_offset(kp) + FRAME_FLOATS; }

@@ -28,8 +28,12 @@ template <int DP, int LD, bool SCALAR>
 __global__ void __launch_bounds__(FMA_WAVES * WAVE)
 assign_lds_fma_kernel(const float* __restrict__ data, size_t stride, const float* __restrict__ packed, const float* __restrict__ norms,
                       uint32_t* __restrict__ assignment, uint32_t* __restrict__ queue, uint32_t* __restrict__ counters,
-                      uint32_t dim, uint32_t k, uint32_t kp, uint32_t n, uint32_t chunk_rows, float kd, uint32_t vec4)
+                      uint32_t dim, uint32_t k, uint32_t kp, uint32_t n, uint32_t chunk_rows, float kd, uint32_t vec4, float kd_unmoved)
 {
+	/* the frame of the sweep (sweep_frame; the packing kernel moved the centroids): the same words for every lane, so
+	 * they arrive as scalar operands */
+	const float* __restrict__ frame = norms + plain_frame_offset(kp);
+	const float frame_m2 = frame[FRAME_DIMS], frame_norm = frame[FRAME_DIMS + 1];
 	constexpr uint32_t RS = DP + ROW_PAD;
 	extern __shared__ float lds[];
 	__shared__ uint32_t wave_max[FMA_WAVES];
@@ -101,8 +105,14 @@ assign_lds_fma_kernel(const float* __restrict__ data, size_t stride, const float
 #pragma unroll
 			for (int q = 0; q < DP; ++q) x[q] = (valid && (uint32_t)q < dim) ? data[elem<LD>(stride, pt, q)] : 0.0f;
 		}
+		float along = 0.0f; /* (x - m) . m */
 #pragma unroll
-		for (int q = 0; q < DP; ++q) x2 += x[q] * x[q];
+		for (int q = 0; q < DP; ++q) {
+			const float m = frame[q];
+			x[q] -= m;
+			x2 += x[q] * x[q];
+			along += x[q] * m;
+		}
 		float m1 = __builtin_inff(), m2 = __builtin_inff();
 		uint32_t best = 0;
 		for (uint32_t chunk = 0; chunk < (SCALAR ? 1u : chunks); ++chunk) {
@@ -144,7 +154,10 @@ assign_lds_fma_kernel(const float* __restrict__ data, size_t stride, const float
 			if (flag) {
 				const uint32_t at = 2 * (flagged + __builtin_popcountll(mask & ((1ull << lane) - 1ull)));
 				flag_list[wave][at] = pt;
-				flag_list[wave][at + 1] = screening_threshold(m1, tau);
+				/* the exact pass evaluates in the frame of the data (certificate.h) */
+				flag_list[wave][at + 1] = kd_unmoved > 0.0f
+					? screening_threshold(cert_unmoved_threshold(m1, tau, x2, along, c2max, frame_m2, frame_norm, kd_unmoved), 0.0f)
+					: screening_threshold(m1, tau);
 			}
 			flagged += add;
 		}
@@ -197,25 +210,29 @@ static int launch_fma_dp(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 	const uint32_t grid = std::min(batches, dev.compute_units * per_cu);
 	exec->block_count = grid;
 	void (*kernel)(const float*, size_t, const float*, const float*, uint32_t*, uint32_t*, uint32_t*,
-	               uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, float, uint32_t) = nullptr;
+	               uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, float, uint32_t, float) = nullptr;
 	const uint32_t vec4 = (a.layout == KMX_AOS && a.dim % 4 == 0 && a.stride % 4 == 0 && ((uintptr_t)a.data % 16) == 0) ? 1u : 0u;
 	if (a.layout == KMX_AOS) kernel = scalar ? assign_lds_fma_kernel<DP, KMX_AOS, true> : assign_lds_fma_kernel<DP, KMX_AOS, false>;
 	else kernel = scalar ? assign_lds_fma_kernel<DP, KMX_SOA, true> : assign_lds_fma_kernel<DP, KMX_SOA, false>;
 	int rc = profile_begin(0);
 	if (rc) return rc;
 	KMX_LAUNCH_KERNEL(kernel, dim3(grid), dim3(FMA_WAVES * WAVE), lds_bytes, stream(),
-	                   a.data, a.stride, ws->packed_means, ws->norms, a.assignment, ws->queue, ws->counters, a.dim, a.k, kp, a.n, chunk_rows, kd, vec4);
+	                   a.data, a.stride, ws->packed_means, ws->norms, a.assignment, ws->queue, ws->counters, a.dim, a.k, kp, a.n, chunk_rows, kd, vec4, a.unmoved_thresholds ? cert_kd_unmoved(a.dim) : 0.0f);
 	KMX_LAUNCH_CHECK("assign_lds_fma_kernel");
 	return profile_end(0);
 }
 
-int launch_assign_lds_fma(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev)
+int launch_assign_lds_fma(const AssignArgs& args, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev)
 {
+	AssignArgs a = args;
+	/* the frame moves as in the fp32 MFMA sweep (launch_assign_mfma) */
+	a.shift_rows = !a.ranking_only;
+	a.unmoved_thresholds = a.shift_rows;
 	const uint32_t dp = fma_dp(a.dim);
 	const uint32_t kp = round_up(a.k, TILE);
-	int rc = launch_pack_means(a, ws, dp, kp);
+	int rc = launch_pack_means(a, ws, dp, kp, a.shift_rows);
 	if (rc) return rc;
-	const float kd = cert_kd_fma(a.dim) + a.kd_extra;
+	const float kd = cert_kd_fma(a.dim) + (a.shift_rows ? 8.0f * CERT_UNIT : 0.0f) + a.kd_extra;
 	switch (dp) {
 	case 4: rc = launch_fma_dp<4>(a, exec, ws, dev, kp, kd); break;
 	case 8: rc = launch_fma_dp<8>(a, exec, ws, dev, kp, kd); break;
@@ -228,7 +245,10 @@ int launch_assign_lds_fma(const AssignArgs& a, kmx_exec_params* exec, Workspace*
 	}
 	if (rc) return rc;
 	if (a.ranking_only) return KMX_OK; /* the caller resolves the queued points */
-	return launch_recheck(a, ws, kp);
+	ws->exact_norms = ws->norms + plain_exact_norms_offset(kp);
+	rc = launch_recheck(a, ws, kp);
+	ws->exact_norms = nullptr;
+	return rc;
 }
 
 } // namespace kmx

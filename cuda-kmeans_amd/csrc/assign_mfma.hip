@@ -58,25 +58,40 @@ static uint32_t pick_dph(uint32_t dim)
 template <int LM>
 __global__ void __launch_bounds__(256)
 pack_means_kernel(const float* __restrict__ means, size_t stride_means, float* __restrict__ packed, float* __restrict__ norms,
-                  float* __restrict__ means_t, uint32_t dim, uint32_t k, uint32_t kp, uint32_t dp, uint32_t* __restrict__ counters)
+                  float* __restrict__ means_t, uint32_t dim, uint32_t k, uint32_t kp, uint32_t dp, uint32_t moved, uint32_t* __restrict__ counters)
 {
 	const uint32_t lane = threadIdx.x & (WAVE - 1);
 	const uint32_t j = (blockIdx.x * blockDim.x + threadIdx.x) / WAVE;
 	if (blockIdx.x == 0 && threadIdx.x == 0) counters[0] = 0u; /* the recheck queue of this call starts empty */
+	/* the frame of the sweep (zeros unless `moved`): the rows are those of c - m, with their norms; the exact pass gets
+	 * the centroids and their norms as given */
+	__shared__ float frame[FRAME_DIMS];
+	sweep_frame<LM>(means, stride_means, dim, k, dp, moved != 0, frame, norms + plain_frame_offset(kp));
 	if (j >= kp) return;
 	const uint32_t rs = dp + ROW_PAD;
 	float* row = packed + packed_row(j, rs);
 	const uint32_t row_floats = rs + (j % TILE == TILE - 1 ? TILE_PAD : 0); /* the tile padding follows its last row */
-	float c2 = 0.0f;
+	float c2 = 0.0f, exact2 = 0.0f;
 	for (uint32_t q = lane; q < row_floats; q += WAVE) {
-		float v = (j < k && q < dim) ? means[elem<LM>(stride_means, j, q)] : 0.0f;
+		const float exact = (j < k && q < dim) ? means[elem<LM>(stride_means, j, q)] : 0.0f;
+		const float v = (j < k && q < dim) ? exact - frame[q] : 0.0f;
 		c2 += v * v;
+		exact2 += exact * exact;
 		row[q] = -2.0f * v;
-		if (q < dim) means_t[(size_t)q * kp + j] = v; /* exact copy for the recheck pass */
+		if (q < dim) means_t[(size_t)q * kp + j] = exact; /* exact copy for the recheck pass */
 	}
-	for (int off = WAVE / 2; off > 0; off >>= 1) c2 += __shfl_xor(c2, off);
-	if (lane == 0) norms[norm_at(j)] = j < k ? c2 : __builtin_inff();
-	if (lane < NORM_TILE - TILE && j % TILE == 0) norms[(j / TILE) * NORM_TILE + TILE + lane] = __builtin_inff();
+	for (int off = WAVE / 2; off > 0; off >>= 1) {
+		c2 += __shfl_xor(c2, off);
+		exact2 += __shfl_xor(exact2, off);
+	}
+	if (lane == 0) {
+		norms[norm_at(j)] = j < k ? c2 : __builtin_inff();
+		norms[plain_exact_norms_offset(kp) + norm_at(j)] = j < k ? exact2 : __builtin_inff();
+	}
+	if (lane < NORM_TILE - TILE && j % TILE == 0) {
+		norms[(j / TILE) * NORM_TILE + TILE + lane] = __builtin_inff();
+		norms[plain_exact_norms_offset(kp) + (j / TILE) * NORM_TILE + TILE + lane] = __builtin_inff();
+	}
 }
 
 bool mfma_supports(const AssignArgs& a, const DeviceInfo& dev)
@@ -95,33 +110,40 @@ KMX_DECLARE_MFMA_LAUNCHER(16) KMX_DECLARE_MFMA_LAUNCHER(24) KMX_DECLARE_MFMA_LAU
 KMX_DECLARE_MFMA_LAUNCHER(128)
 
 /* packs the centroids of this call into the work space (rows of dp floats, kp rows) and empties the recheck queue */
-int launch_pack_means(const AssignArgs& a, Workspace* ws, uint32_t dp, uint32_t kp)
+int launch_pack_means(const AssignArgs& a, Workspace* ws, uint32_t dp, uint32_t kp, bool moved)
 {
-	int rc = reserve_packed(ws, (size_t)(kp / TILE) * tile_floats(dp + ROW_PAD), (size_t)(kp / TILE) * NORM_TILE, (size_t)kp * a.dim);
+	int rc = reserve_packed(ws, (size_t)(kp / TILE) * tile_floats(dp + ROW_PAD), plain_norms_floats(kp), (size_t)kp * a.dim);
 	if (rc) return rc;
 	rc = reserve_queue(ws, 2 * (size_t)a.n); /* (point, threshold) pairs */
 	if (rc) return rc;
 	const uint32_t pack_blocks = (kp * WAVE + 255) / 256;
 	if (a.layout_means == KMX_AOS)
 		KMX_LAUNCH_KERNEL((pack_means_kernel<KMX_AOS>), dim3(pack_blocks), dim3(256), 0, stream(),
-		                   a.means, a.stride_means, ws->packed_means, ws->norms, ws->means_t, a.dim, a.k, kp, dp, ws->counters);
+		                   a.means, a.stride_means, ws->packed_means, ws->norms, ws->means_t, a.dim, a.k, kp, dp, moved ? 1u : 0u, ws->counters);
 	else
 		KMX_LAUNCH_KERNEL((pack_means_kernel<KMX_SOA>), dim3(pack_blocks), dim3(256), 0, stream(),
-		                   a.means, a.stride_means, ws->packed_means, ws->norms, ws->means_t, a.dim, a.k, kp, dp, ws->counters);
+		                   a.means, a.stride_means, ws->packed_means, ws->norms, ws->means_t, a.dim, a.k, kp, dp, moved ? 1u : 0u, ws->counters);
 	KMX_LAUNCH_CHECK("pack_means_kernel");
 	return KMX_OK;
 }
 
-int launch_assign_mfma(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev)
+int launch_assign_mfma(const AssignArgs& args, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev)
 {
+	AssignArgs a = args;
+	/* The sweep works in a frame moved to the middle of the centroids (sweep_frame), so that tau scales with the spread of
+	 * the data and not with its distance from the origin; the thresholds go to the exact pass in the frame of the data.
+	 * (Not for the double path: the float copies of its points are rounded relative to the origin anyway.) */
+	a.shift_rows = !a.ranking_only;
+	a.unmoved_thresholds = a.shift_rows;
 	const uint32_t dph = pick_dph(a.dim);
 	const uint32_t dp = 2 * dph;
 	const uint32_t kp = round_up(a.k, TILE);
-	int rc = launch_pack_means(a, ws, dp, kp);
+	int rc = launch_pack_means(a, ws, dp, kp, a.shift_rows);
 	if (rc) return rc;
 
-	/* tau = kd (|x|^2 + max|c|^2), kd = (8 d + 24) 2^-23 (see the bound at the top of the file) */
-	const float kd = cert_kd_fp32(a.dim) + a.kd_extra;
+	/* tau = kd (|x|^2 + max|c|^2), kd = (8 d + 24) 2^-23 (see the bound at the top of the file), 8 * 2^-23 more for the
+	 * roundings of x - m and c - m */
+	const float kd = cert_kd_fp32(a.dim) + (a.shift_rows ? 8.0f * CERT_UNIT : 0.0f) + a.kd_extra;
 	switch (dph) {
 	case 2: rc = launch_mfma_2(a, exec, ws, dev, kp, kd); break;
 	case 4: rc = launch_mfma_4(a, exec, ws, dev, kp, kd); break;
@@ -136,7 +158,10 @@ int launch_assign_mfma(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws
 	}
 	if (rc) return rc;
 	if (a.ranking_only) return KMX_OK; /* the caller resolves the queued points */
-	return launch_recheck(a, ws, kp);
+	ws->exact_norms = ws->norms + plain_exact_norms_offset(kp);
+	rc = launch_recheck(a, ws, kp);
+	ws->exact_norms = nullptr;
+	return rc;
 }
 
 } // namespace kmx

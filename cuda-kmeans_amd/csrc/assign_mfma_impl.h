@@ -7,6 +7,7 @@
 #define KMX_ASSIGN_MFMA_IMPL_H
 
 #include "kmx_internal.h"
+#include "certificate.h"
 
 #include <algorithm>
 
@@ -35,6 +36,60 @@ __device__ __forceinline__ uint32_t screening_threshold(float first, float tau)
 	return __float_as_uint(__builtin_fabsf(t) < __builtin_inff() ? t : __builtin_inff());
 }
 constexpr uint32_t COARSE_MIN_TILES = 10; /* from this many centroid tiles on, track per tile and refine */
+
+/*
+ * The frame of a sweep: FRAME_DIMS coordinates of the vector m that is subtracted from every point and centroid before
+ * the sweep uses them (zeros: the frame of the data), then |m|^2 and an upper bound of |m|. tau scales with
+ * |x - m|^2 + max |c - m|^2, so with m in the middle of the data it no longer grows with the distance of the data from
+ * the origin (certificate.h).
+ */
+constexpr uint32_t FRAME_DIMS = 256;
+constexpr uint32_t FRAME_FLOATS = FRAME_DIMS + 4;
+/* the norms array of the fp32 sweeps: the tiles of |c - m|^2, the frame, the tiles of |c|^2 (for the exact pass) */
+__host__ __device__ __forceinline__ size_t plain_frame_offset(uint32_t kp) { return (size_t)(kp / TILE) * NORM_TILE; }
+__host__ __device__ __forceinline__ size_t plain_exact_norms_offset(uint32_t kp) { return plain_frame_offset(kp) + FRAME_FLOATS; }
+__host__ __device__ __forceinline__ size_t plain_norms_floats(uint32_t kp) { return plain_exact_norms_offset(kp) + (size_t)(kp / TILE) * NORM_TILE; }
+
+/*
+ * The frame of a call, for the packing kernels (256 threads): m = the mean of the first 16 centroids, finite coordinates
+ * only (any vector would do; this one lies inside the data), a thread per dimension with its 16 loads in flight together;
+ * zeros when `moved` is false. Every work-group computes it into `m` (LDS, dp <= FRAME_DIMS floats), in the same order;
+ * the first one stores it at `stored` with |m|^2 (as computed: it enters the shift of the thresholds) and an upper
+ * bound of |m|. Ends with a barrier.
+ */
+template <int LM>
+__device__ __forceinline__ void sweep_frame(const float* __restrict__ means, size_t stride_means, uint32_t dim, uint32_t k, uint32_t dp,
+                                            bool moved, float* m, float* __restrict__ stored)
+{
+	constexpr uint32_t SAMPLE = 16;
+	const uint32_t sample = min(k, SAMPLE);
+	for (uint32_t q = threadIdx.x; q < dp; q += blockDim.x) {
+		float sum = 0.0f;
+		if (moved && q < dim) {
+			float v[SAMPLE];
+#pragma unroll
+			for (uint32_t r = 0; r < SAMPLE; ++r) v[r] = r < sample ? means[elem<LM>(stride_means, r, q)] : 0.0f;
+#pragma unroll
+			for (uint32_t r = 0; r < SAMPLE; ++r) sum += __builtin_fabsf(v[r]) < __builtin_inff() ? v[r] : 0.0f;
+			sum = sum / (float)sample;
+			sum = __builtin_fabsf(sum) < __builtin_inff() ? sum : 0.0f; /* (the sum of finite values may overflow) */
+		}
+		m[q] = sum;
+	}
+	__syncthreads();
+	if (blockIdx.x == 0) {
+		for (uint32_t q = threadIdx.x; q < dp; q += blockDim.x) stored[q] = m[q];
+		if (threadIdx.x < 64) {
+			float m2 = 0.0f;
+			for (uint32_t q = threadIdx.x; q < dp; q += 64) m2 += m[q] * m[q];
+			for (int off = 32; off > 0; off >>= 1) m2 += __shfl_xor(m2, off);
+			if (threadIdx.x == 0) {
+				stored[FRAME_DIMS] = m2;
+				stored[FRAME_DIMS + 1] = __builtin_sqrtf(m2) * 1.0001f;
+			}
+		}
+	}
+}
 
 __host__ __device__ constexpr uint32_t round_up(uint32_t v, uint32_t m) { return (v + m - 1) / m * m; }
 /* floats of one packed tile / offset of a packed row / offset of a norm */
@@ -287,11 +342,15 @@ template <int DPH, int P, int LD, bool VEC, bool STREAM, bool COARSE, bool PREFE
 __global__ void __launch_bounds__(MFMA_WAVES * WAVE)
 assign_mfma_kernel(const float* __restrict__ data, size_t stride, const float* __restrict__ packed, const float* __restrict__ norms,
                    uint32_t* __restrict__ assignment, uint32_t* __restrict__ queue, uint32_t* __restrict__ counters,
-                   uint32_t dim, uint32_t k, uint32_t kp, uint32_t n, uint32_t chunk_rows, float kd, float neg_inf)
+                   uint32_t dim, uint32_t k, uint32_t kp, uint32_t n, uint32_t chunk_rows, float kd, float neg_inf, float kd_unmoved)
 {
 	constexpr uint32_t DP = 2 * DPH;
 	constexpr uint32_t RS = DP + ROW_PAD;
 	extern __shared__ float lds[];
+	/* the frame of the sweep (sweep_frame; the packing kernel moved the centroids): m, |m|^2 and |m| */
+	__shared__ __attribute__((aligned(16))) float frame_lds[DP];
+	for (uint32_t i = threadIdx.x; i < DP; i += blockDim.x) frame_lds[i] = norms[plain_frame_offset(kp) + i];
+	const float frame_m2 = norms[plain_frame_offset(kp) + FRAME_DIMS], frame_norm = norms[plain_frame_offset(kp) + FRAME_DIMS + 1];
 	__shared__ uint32_t wave_max[MFMA_WAVES];
 	__shared__ uint32_t flag_list[MFMA_WAVES][2 * FLAG_CAP]; /* (point, threshold) pairs */
 
@@ -349,15 +408,21 @@ assign_mfma_kernel(const float* __restrict__ data, size_t stride, const float* _
 	const uint32_t unit_points = MFMA_WAVES * P * TILE;
 	const uint32_t units = (n + unit_points - 1) / unit_points;
 
-	auto sweep = [&](const float (&b)[P][DPH], uint32_t base) {
-		float x2[P];
+	auto sweep = [&](float (&b)[P][DPH], uint32_t base) {
+		float x2[P], along_m[P]; /* |x - m|^2 and (x - m) . m of the points */
 		Track st[P];
 #pragma unroll
 		for (int p = 0; p < P; ++p) {
-			float part = 0.0f;
+			float part = 0.0f, along = 0.0f;
 #pragma unroll
-			for (int s = 0; s < DPH; ++s) part += b[p][s] * b[p][s];
+			for (int s = 0; s < DPH; ++s) {
+				const float m = frame_lds[h * DPH + s];
+				b[p][s] -= m; /* the rows are swept in the moved frame (rows beyond n, read as zero, become -m: they are not written back) */
+				part += b[p][s] * b[p][s];
+				along += b[p][s] * m;
+			}
 			x2[p] = part + __shfl_xor(part, 32);
+			along_m[p] = along + __shfl_xor(along, 32);
 			st[p].m1 = __builtin_inff();
 			st[p].m2 = __builtin_inff();
 			st[p].tile = 0;
@@ -484,7 +549,10 @@ assign_mfma_kernel(const float* __restrict__ data, size_t stride, const float* _
 				if (flag) {
 					const uint32_t at = 2 * (flagged + __builtin_popcountll(mask & ((1ull << lane) - 1ull)));
 					flag_list[wave][at] = pt;
-					flag_list[wave][at + 1] = screening_threshold(first, tau);
+					/* the exact pass evaluates in the frame of the data (certificate.h) */
+					flag_list[wave][at + 1] = kd_unmoved > 0.0f
+						? screening_threshold(cert_unmoved_threshold(first, tau, x2[p], along_m[p], c2max, frame_m2, frame_norm, kd_unmoved), 0.0f)
+						: screening_threshold(first, tau);
 				}
 				flagged += add;
 			}
@@ -528,7 +596,7 @@ static int launch_mfma_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 	constexpr int P = SweepShape<DPH>::P;
 	constexpr bool PF = SweepShape<DPH>::PREFETCH;
 	uint32_t budget = exec->shared_mem_bytes ? std::min(exec->shared_mem_bytes, dev.lds_bytes) : dev.lds_bytes;
-	const uint32_t static_bytes = (2 * FLAG_CAP * MFMA_WAVES + 64) * 4; /* static LDS of the kernel */
+	const uint32_t static_bytes = (2 * FLAG_CAP * MFMA_WAVES + 64 + 2 * DPH) * 4; /* static LDS of the kernel */
 	const uint32_t tile_bytes = (tile_floats(RS) + NORM_TILE) * 4;
 	if (budget < static_bytes + tile_bytes) return fail(KMX_ERR_UNSUPPORTED, "assign (MFMA): LDS budget of %u bytes is too small", budget);
 	const uint32_t chunk_rows = std::min<uint32_t>(kp, (budget - static_bytes) / tile_bytes * TILE);
@@ -540,7 +608,7 @@ static int launch_mfma_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 	const uint32_t unit_points = MFMA_WAVES * P * TILE;
 	const uint32_t units = (a.n + unit_points - 1) / unit_points;
 	void (*kernel)(const float*, size_t, const float*, const float*, uint32_t*, uint32_t*, uint32_t*,
-	               uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, float, float) = nullptr;
+	               uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, float, float, float) = nullptr;
 	if constexpr (DPH <= 32) {
 		if (stream_mode) kernel = coarse ? assign_mfma_kernel<DPH, P, LD, VEC, true, true, PF> : assign_mfma_kernel<DPH, P, LD, VEC, true, false, PF>;
 		else kernel = coarse ? assign_mfma_kernel<DPH, P, LD, VEC, false, true, PF> : assign_mfma_kernel<DPH, P, LD, VEC, false, false, PF>;
@@ -561,7 +629,7 @@ static int launch_mfma_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 	if (rc) return rc;
 	KMX_LAUNCH_KERNEL(kernel, dim3(grid), dim3(MFMA_WAVES * WAVE), lds_bytes, stream(),
 	                   a.data, a.stride, ws->packed_means, ws->norms, a.assignment, ws->queue, ws->counters,
-	                   a.dim, a.k, kp, a.n, chunk_rows, kd, -__builtin_inff());
+	                   a.dim, a.k, kp, a.n, chunk_rows, kd, -__builtin_inff(), a.unmoved_thresholds ? cert_kd_unmoved(a.dim) : 0.0f);
 	KMX_LAUNCH_CHECK("assign_mfma_kernel");
 	return profile_end(0);
 }

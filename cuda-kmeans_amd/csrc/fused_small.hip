@@ -309,7 +309,7 @@ static int launch_fused_layouts(const AssignArgs& a, float* means_out, uint32_t*
 {
 	const uint32_t dp = fused_dp(a.dim);
 	const uint32_t kp = round_up(a.k, TILE);
-	int rc = launch_pack_means(a, ws, dp, kp);
+	int rc = launch_pack_means(a, ws, dp, kp, false);
 	if (rc) return rc;
 	const float kd = cert_kd_fma(a.dim); /* the bound of a ranking by chains of fused multiply-adds, see certificate.h */
 	switch (dp) {

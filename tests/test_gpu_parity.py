@@ -243,6 +243,26 @@ def test_data_far_from_the_origin(km, orc, gpu, dim, k, n, offset):
         assert rechecked < n // 10, "%d of %d points left to the exact pass" % (rechecked, n)
 
 
+@pytest.mark.parametrize("dim,k,n", [(2, 50, 200000), (3, 100, 200000), (2, 500, 100000), (8, 64, 200000), (4, 16, 200000),
+                                     (12, 40, 200000), (40, 300, 50000), (100, 64, 30000)])
+@pytest.mark.parametrize("offset", [0.0, 1000.0])
+def test_data_far_from_the_origin_in_the_fp32_sweeps(km, orc, gpu, dim, k, n, offset):
+    """The same for the fp32 MFMA sweep and the sweep on the vector ALU (and whatever the selector picks): they move their
+    frame too and hand the exact pass thresholds of the frame of the data."""
+    rng = np.random.default_rng(dim * 3 + k)
+    centres = rng.uniform(-10, 10, (k, dim)).astype(np.float32)
+    base = (centres[rng.integers(0, k, n)] + rng.normal(size=(n, dim)).astype(np.float32) + np.float32(offset)).astype(np.float32)
+    means = base[:k].copy()
+    want = orc.assign(base.ravel(), means.ravel(), dim, k, n, threads=0, fast=True)
+    for v in [km.ASSIGN_MFMA, km.ASSIGN_BEST] + ([km.ASSIGN_LDS_FMA] if dim <= 64 else []):
+        for layout in (AOS, SOA):
+            d = base if layout == AOS else np.ascontiguousarray(base.T)
+            got, rechecked = gpu_assign(km, v, d.ravel(), means.ravel(), dim, k, n, layout, AOS)
+            bad = np.nonzero(got != want)[0]
+            assert bad.size == 0, "variant %d, layout %d: %d mismatches, first at %s" % (v, layout, bad.size, bad[:5])
+            assert rechecked < n // 10, "variant %d: %d of %d points left to the exact pass" % (v, rechecked, n)
+
+
 @pytest.mark.parametrize("dim,k,n", [(32, 256, 3000), (21, 1500, 4000), (96, 200, 1500), (4, 512, 5000)])
 def test_soa_points_in_the_exact_pass(km, orc, gpu, dim, k, n):
     """SoA points: the exact pass copies the rows of the queued points into a compact block. Inputs that queue every point
