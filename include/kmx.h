@@ -323,9 +323,10 @@ int kmx_set_queued_rows_limit(size_t bytes);
  *   form 1: split-bf16 sweep, three products per dimension         xpart2 = sum_i xmid_i^2
  *   form 2: split-bf16 sweep, packed rows (dim <= 4, four products) xpart2 = sum_i xrest_i^2
  * x2 = |x|^2, c2max = max_j |c_j|^2, cmid2max / crest2max = max_j of the squared norms of the mid / rest parts of -2 c_j;
- * for forms 1 and 2 all of them in the frame the sweep works in: it subtracts a vector m from points and centroids (the
- * mean of the first 16 centroids; for packed rows, with 128 centroids or more, of the first 256), so the norms are those
- * of the moved data; the three-product form then adds 8 * 2^-23 * (x2 + c2max), which form 1 leaves out.
+ * all of them in the frame the sweep works in: the float sweeps subtract a vector m from points and centroids (the mean
+ * of the first 16 centroids; for packed rows, with 128 centroids or more, of the first 256; the single-pass fused kernel
+ * and the double-precision path keep m = 0), so the norms are those of the moved data; forms 0, 1 and 3 then add
+ * 8 * 2^-23 * (x2 + c2max) for the two roundings, which this function leaves out (form 2 contains it).
  */
 int kmx_certificate_tau(int form, uint32_t dim, float x2, float xpart2, float c2max, float cmid2max, float crest2max, float* tau);
 
