@@ -76,6 +76,12 @@ struct PreparedPoints {
 static PreparedPoints g_prepared;
 static double* g_means32 = nullptr;                /* float copy of the centroids */
 static size_t g_means32_cap = 0;
+/* The float copies are taken of x - m and c - m, subtracted in double: m (dim doubles, then |m|^2) is the mean of the
+ * first 16 points whose copy g_data32 holds. The float sweeps then rank data that lie around the origin whatever the
+ * doubles do, and their certificate scales with the spread of the data (certificate.h); the exact pass takes their
+ * thresholds back to the frame of the data in double. */
+static double* g_frame = nullptr;
+static size_t g_frame_cap = 0;
 
 __global__ void reset_f64_kernel(unsigned long long* __restrict__ misc)
 {
@@ -88,20 +94,46 @@ __global__ void publish_queue_length_kernel(const unsigned long long* __restrict
 	if (threadIdx.x == 0) counters[0] = queued ? (uint32_t)misc[0] : 0u;
 }
 
-/* round-to-nearest float copy; values beyond the float range become infinities, tiny ones zeros or subnormals.
- * Four elements per lane and step (two 16-byte loads, one 16-byte store); both buffers are 16-byte aligned. */
-typedef double f64x2 __attribute__((ext_vector_type(2)));
-
+/* m: a thread per dimension, the finite coordinates of the first 16 points; one work-group of 256 threads */
+template <int LD>
 __global__ void __launch_bounds__(256)
-round_to_float_kernel(const double* __restrict__ in, float* __restrict__ out, size_t count)
+point_frame_f64_kernel(const double* __restrict__ data, size_t stride, uint32_t dim, uint32_t n, double* __restrict__ frame)
 {
-	const size_t quads = count / 4;
-	for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < quads; e += (size_t)gridDim.x * blockDim.x) {
-		const f64x2 a = ((const f64x2*)in)[2 * e], b = ((const f64x2*)in)[2 * e + 1];
-		const f32x4 r = { (float)a.x, (float)a.y, (float)b.x, (float)b.y };
-		((f32x4*)out)[e] = r;
+	__shared__ double parts[256 / WAVE];
+	const uint32_t sample = min(n, 16u);
+	double m2 = 0.0;
+	for (uint32_t q = threadIdx.x; q < dim; q += blockDim.x) {
+		double sum = 0.0;
+		for (uint32_t r = 0; r < sample; ++r) {
+			const double v = data[elem<LD>(stride, r, q)];
+			sum += __builtin_fabs(v) < __builtin_inf() ? v : 0.0;
+		}
+		sum /= (double)sample;
+		sum = __builtin_fabs(sum) < __builtin_inf() ? sum : 0.0;
+		sum = (double)(float)sum; /* (a float's worth of m is enough, and x - m stays exact for more inputs) */
+		sum = __builtin_fabs(sum) < __builtin_inf() ? sum : 0.0;
+		frame[q] = sum;
+		m2 = __builtin_fma(sum, sum, m2);
 	}
-	if (blockIdx.x == 0 && threadIdx.x < count % 4) out[4 * quads + threadIdx.x] = (float)in[4 * quads + threadIdx.x];
+	for (int off = WAVE / 2; off > 0; off >>= 1) m2 += __shfl_xor(m2, off);
+	if ((threadIdx.x & (WAVE - 1)) == 0) parts[threadIdx.x / WAVE] = m2;
+	__syncthreads();
+	if (threadIdx.x == 0) frame[dim] = (parts[0] + parts[1]) + (parts[2] + parts[3]);
+}
+
+/* float copy of (in - m), subtracted in double (element e of a buffer with the layout and stride of the original) */
+template <int LD>
+__global__ void __launch_bounds__(256)
+round_moved_to_float_kernel(const double* __restrict__ in, float* __restrict__ out, size_t count, size_t stride, uint32_t dim,
+                            const double* __restrict__ frame)
+{
+	const bool narrow = count <= 0xFFFFFFFFull && stride <= 0xFFFFFFFFull; /* (32-bit division is several times cheaper) */
+	for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < count; e += (size_t)gridDim.x * blockDim.x) {
+		size_t q;
+		if (narrow) q = LD == KMX_AOS ? (uint32_t)e % (uint32_t)stride : (uint32_t)e / (uint32_t)stride;
+		else q = LD == KMX_AOS ? e % stride : e / stride;
+		out[e] = (float)(q < dim ? in[e] - frame[q] : in[e]); /* (AoS rows may be padded) */
+	}
 }
 
 /* one lane per (padded) centroid: transposed copy, |c|^2, and the largest |c|^2 as the maximum of the bit patterns
@@ -298,7 +330,8 @@ template <int LD, bool SCREEN>
 __global__ void __launch_bounds__(1024)
 requeued_batch_f64_kernel(const double* __restrict__ data, size_t stride, const double* __restrict__ means_t, const double* __restrict__ norms,
                           uint32_t* __restrict__ assignment, uint32_t dim, uint32_t k, uint32_t kp,
-                          const uint32_t* __restrict__ queue, uint32_t queue_stride, const uint32_t* __restrict__ queue_length)
+                          const uint32_t* __restrict__ queue, uint32_t queue_stride, const uint32_t* __restrict__ queue_length,
+                          const double* __restrict__ frame, const unsigned long long* __restrict__ misc)
 {
 	extern __shared__ double rows[]; /* BATCH x dim */
 	__shared__ unsigned long long chunk_min[BATCH];
@@ -323,6 +356,24 @@ requeued_batch_f64_kernel(const double* __restrict__ data, size_t stride, const 
 		}
 		__syncthreads();
 		for (uint32_t e = threadIdx.x; e < BATCH * dim; e += blockDim.x) rows[e] = data[elem<LD>(stride, point_of[e / dim], e % dim)];
+		if (SCREEN) {
+			/* The float sweep ranked x - m against c - m (frame: m, then |m|^2), where the ranking values are those of
+			 * the data as given plus sh = 2 x . m - |m|^2; the values below are of the data as given, so the threshold
+			 * comes back by sh, with an allowance for the double arithmetic on both sides (certificate.h has the
+			 * float version of this): (4 d + 40) 2^-52 (|x|^2 + max |c|^2). */
+			__syncthreads(); /* the rows are in place */
+			if (threadIdx.x < BATCH) {
+				double xm = 0.0, x2 = 0.0;
+				for (uint32_t q = 0; q < dim; ++q) {
+					const double v = rows[threadIdx.x * dim + q];
+					xm = __builtin_fma(v, frame[q], xm);
+					x2 = __builtin_fma(v, v, x2);
+				}
+				const double c2max = __longlong_as_double((long long)misc[1]);
+				const double t = threshold[threadIdx.x] - (2.0 * xm - frame[dim]) + (4.0 * dim + 40.0) * 0x1p-52 * (x2 + c2max);
+				threshold[threadIdx.x] = t == t ? t : __builtin_inf(); /* (values the bound does not cover: every centroid is evaluated) */
+			}
+		}
 		for (uint32_t base = 0; base < k; base += blockDim.x) {
 			__syncthreads(); /* rows are in place; the previous chunk is merged */
 			if (threadIdx.x < BATCH) { chunk_min[threadIdx.x] = ~0ull; chunk_arg[threadIdx.x] = NONE; }
@@ -657,10 +708,10 @@ int launch_assign_f64_ld(int variant, const double* data, size_t stride, uint32_
 	do { \
 		if (batched && float_queue) \
 			KMX_LAUNCH_KERNEL((requeued_batch_f64_kernel<LD, true>), bgrid, dim3(batch_threads), (size_t)BATCH * dim * sizeof(double), stream(), \
-			                   data, stride, g_means_t, g_norms, assignment, dim, k, kp, exact_queue, exact_stride, exact_length); \
+			                   data, stride, g_means_t, g_norms, assignment, dim, k, kp, exact_queue, exact_stride, exact_length, g_frame, misc); \
 		else if (batched) \
 			KMX_LAUNCH_KERNEL((requeued_batch_f64_kernel<LD, false>), bgrid, dim3(batch_threads), (size_t)BATCH * dim * sizeof(double), stream(), \
-			                   data, stride, g_means_t, g_norms, assignment, dim, k, kp, exact_queue, exact_stride, exact_length); \
+			                   data, stride, g_means_t, g_norms, assignment, dim, k, kp, exact_queue, exact_stride, exact_length, g_frame, misc); \
 		else if (dim > 32) KMX_F64_REQUEUED(0); \
 		else if (dim <= 8) KMX_F64_REQUEUED(8); \
 		else if (dim <= 16) KMX_F64_REQUEUED(16); \
@@ -747,13 +798,34 @@ int launch_update_f64_t(int variant, const double* data, size_t stride, const ui
 int release_f64_workspace()
 {
 	g_prepared = PreparedPoints();
-	double** buffers[] = { &g_means_t, &g_norms, &g_queue, &g_misc, &g_data32, &g_means32 };
-	size_t* caps[] = { &g_means_t_cap, &g_norms_cap, &g_queue_cap, &g_misc_cap, &g_data32_cap, &g_means32_cap };
+	double** buffers[] = { &g_means_t, &g_norms, &g_queue, &g_misc, &g_data32, &g_means32, &g_frame };
+	size_t* caps[] = { &g_means_t_cap, &g_norms_cap, &g_queue_cap, &g_misc_cap, &g_data32_cap, &g_means32_cap, &g_frame_cap };
 	for (int b = 0; b < 6; ++b) {
 		if (*buffers[b]) KMX_HIP(hipFree(*buffers[b]));
 		*buffers[b] = nullptr;
 		*caps[b] = 0;
 	}
+	return KMX_OK;
+}
+
+/* the frame of these points (g_frame) and the float copy of the moved points (g_data32) */
+static int copy_moved_points_f64(const double* data, int layout, size_t stride, uint32_t dim, uint32_t n, const DeviceInfo& dev)
+{
+	const size_t data_extent = layout == KMX_AOS ? (size_t)(n - 1) * stride + dim : (size_t)(dim - 1) * stride + n;
+	int rc = reserve_f64(&g_data32, &g_data32_cap, data_extent / 2 + 1);
+	if (rc) return rc;
+	rc = reserve_f64(&g_frame, &g_frame_cap, (size_t)dim + 1);
+	if (rc) return rc;
+	const dim3 grid((uint32_t)std::min<size_t>((data_extent + 1023) / 1024, (size_t)dev.compute_units * 32));
+	if (layout == KMX_AOS) {
+		KMX_LAUNCH_KERNEL((point_frame_f64_kernel<KMX_AOS>), dim3(1), dim3(256), 0, stream(), data, stride, dim, n, g_frame);
+		KMX_LAUNCH_KERNEL((round_moved_to_float_kernel<KMX_AOS>), grid, dim3(256), 0, stream(), data, (float*)g_data32, data_extent, stride, dim, g_frame);
+	}
+	else {
+		KMX_LAUNCH_KERNEL((point_frame_f64_kernel<KMX_SOA>), dim3(1), dim3(256), 0, stream(), data, stride, dim, n, g_frame);
+		KMX_LAUNCH_KERNEL((round_moved_to_float_kernel<KMX_SOA>), grid, dim3(256), 0, stream(), data, (float*)g_data32, data_extent, stride, dim, g_frame);
+	}
+	KMX_LAUNCH_CHECK("round_moved_to_float_kernel");
 	return KMX_OK;
 }
 
@@ -773,12 +845,8 @@ extern "C" int kmx_prepare_points_f64(const double* data, int layout, size_t str
 	const DeviceInfo* dev = nullptr;
 	rc = device_info(&dev);
 	if (rc) return rc;
-	const size_t data_extent = layout == KMX_AOS ? (size_t)(n - 1) * stride + dim : (size_t)(dim - 1) * stride + n;
-	rc = reserve_f64(&g_data32, &g_data32_cap, data_extent / 2 + 1);
+	rc = copy_moved_points_f64(data, layout, stride, dim, n, *dev);
 	if (rc) return rc;
-	KMX_LAUNCH_KERNEL(round_to_float_kernel, dim3((uint32_t)std::min<size_t>((data_extent + 1023) / 1024, (size_t)dev->compute_units * 32)), dim3(256), 0,
-	                   stream(), data, (float*)g_data32, data_extent);
-	KMX_LAUNCH_CHECK("round_to_float_kernel");
 	g_prepared.data = data; g_prepared.layout = layout; g_prepared.stride = stride; g_prepared.dim = dim; g_prepared.n = n;
 	return KMX_OK;
 }
@@ -836,20 +904,21 @@ extern "C" int kmx_assign_f64(int variant,
 	const uint32_t* float_queue_length = nullptr;
 	if (float_ranking) {
 		/* float copies with the layouts and strides of the originals */
-		const size_t data_extent = layout == KMX_AOS ? (size_t)(n - 1) * stride + dim : (size_t)(dim - 1) * stride + n;
 		const size_t means_extent = layout_means == KMX_AOS ? (size_t)(k - 1) * stride_means + dim : (size_t)(dim - 1) * stride_means + k;
 		rc = reserve_f64(&g_means32, &g_means32_cap, means_extent / 2 + 1);
 		if (rc) return rc;
 		if (!g_prepared.holds(data, layout, stride, dim, n)) {
 			g_prepared = PreparedPoints(); /* the copy is about to hold other points */
-			rc = reserve_f64(&g_data32, &g_data32_cap, data_extent / 2 + 1);
+			rc = copy_moved_points_f64(data, layout, stride, dim, n, *dev);
 			if (rc) return rc;
-			KMX_LAUNCH_KERNEL(round_to_float_kernel, dim3((uint32_t)std::min<size_t>((data_extent + 1023) / 1024, (size_t)dev->compute_units * 32)), dim3(256), 0,
-			                   stream(), data, (float*)g_data32, data_extent);
 		}
-		KMX_LAUNCH_KERNEL(round_to_float_kernel, dim3((uint32_t)std::min<size_t>((means_extent + 1023) / 1024, (size_t)dev->compute_units * 32)), dim3(256), 0,
-		                   stream(), means, (float*)g_means32, means_extent);
-		KMX_LAUNCH_CHECK("round_to_float_kernel");
+		/* the centroids in the frame of the points' copy */
+		const dim3 mgrid((uint32_t)std::min<size_t>((means_extent + 1023) / 1024, (size_t)dev->compute_units * 32));
+		if (layout_means == KMX_AOS)
+			KMX_LAUNCH_KERNEL((round_moved_to_float_kernel<KMX_AOS>), mgrid, dim3(256), 0, stream(), means, (float*)g_means32, means_extent, stride_means, dim, g_frame);
+		else
+			KMX_LAUNCH_KERNEL((round_moved_to_float_kernel<KMX_SOA>), mgrid, dim3(256), 0, stream(), means, (float*)g_means32, means_extent, stride_means, dim, g_frame);
+		KMX_LAUNCH_CHECK("round_moved_to_float_kernel");
 		Workspace* ws = nullptr;
 		rc = workspace(&ws);
 		if (rc) return rc;

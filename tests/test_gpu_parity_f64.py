@@ -96,6 +96,26 @@ def test_assignment_is_bit_exact(km, orc, gpu, dim, k, n, layout, layout_means):
         assert bad.size == 0, "variant %d: %d mismatches, first at %s" % (v, bad.size, bad[:5])
 
 
+@pytest.mark.parametrize("dim,k,n", [(32, 1024, 100000), (64, 512, 50000), (16, 256, 100000), (8, 100, 100000), (3, 300, 100000), (100, 300, 20000)])
+@pytest.mark.parametrize("offset", [0.0, 1000.0, 1.0e6])
+def test_data_far_from_the_origin(km, orc, gpu, dim, k, n, offset):
+    """The float sweeps rank float copies of x - m and c - m (m: the mean of the first points, subtracted in double), and the
+    exact pass takes their thresholds back to the frame of the data: the oracle's assignment wherever the data lie, and
+    no more points left to the exact pass far from the origin than around it."""
+    rng = np.random.default_rng(dim * 5 + k)
+    centres = rng.uniform(-10, 10, (k, dim))
+    base = centres[rng.integers(0, k, n)] + rng.normal(size=(n, dim)) + offset
+    means = base[:k].copy()
+    want = orc.assign_f64(base.ravel(), means.ravel(), dim, k, n, AOS, AOS, threads=0)
+    for v in (km.ASSIGN_BEST, km.ASSIGN_MFMA, km.ASSIGN_MFMA_BF16X3):
+        for layout in (AOS, SOA):
+            d = base if layout == AOS else np.ascontiguousarray(base.T)
+            got = gpu_assign(km, v, d.ravel(), means.ravel(), dim, k, n, layout, AOS)
+            bad = np.nonzero(got != want)[0]
+            assert bad.size == 0, "variant %d, layout %d: %d mismatches, first at %s" % (v, layout, bad.size, bad[:5])
+            assert km.last_rechecked() < n // 10, "variant %d: %d of %d points left to the exact pass" % (v, km.last_rechecked(), n)
+
+
 @pytest.mark.parametrize("dim,k,n", [(32, 2048, 66000), (48, 1100, 65536), (64, 1000, 65600)])
 @pytest.mark.parametrize("layout,layout_means", [(AOS, AOS), (SOA, SOA)])
 def test_centroids_swept_in_slices(km, orc, gpu, dim, k, n, layout, layout_means):
