@@ -85,7 +85,7 @@ pack_means_bf16_kernel(const float* __restrict__ means, size_t stride_means, flo
 	}
 	/* unpacked rows: the same for rows of up to FRAME_DIMS dimensions (sweep_frame) */
 	__shared__ float wide_frame[FRAME_DIMS];
-	if (!(packed_slots & 1u)) sweep_frame<LM>(means, stride_means, dim, k, dp, (packed_slots & 2u) != 0, wide_frame, norms + frame_offset(kp));
+	if (!(packed_slots & 1u)) sweep_frame<LM>(means, stride_means, dim, k, dp, (packed_slots & 2u) ? FRAME_MOVED : FRAME_KEPT, wide_frame, norms + frame_offset(kp));
 	if (j >= kp) return;
 	const bool packed_form = (packed_slots & 1u) != 0;
 	const uint32_t rs = packed_form ? row_floats<1, true>() : dp + ROW_PAD;

@@ -230,7 +230,7 @@ int launch_assign_lds_fma(const AssignArgs& args, kmx_exec_params* exec, Workspa
 	a.unmoved_thresholds = a.shift_rows;
 	const uint32_t dp = fma_dp(a.dim);
 	const uint32_t kp = round_up(a.k, TILE);
-	int rc = launch_pack_means(a, ws, dp, kp, a.shift_rows);
+	int rc = launch_pack_means(a, ws, dp, kp, a.shift_rows ? FRAME_MOVED : FRAME_KEPT);
 	if (rc) return rc;
 	const float kd = cert_kd_fma(a.dim) + (a.shift_rows ? 8.0f * CERT_UNIT : 0.0f) + a.kd_extra;
 	switch (dp) {

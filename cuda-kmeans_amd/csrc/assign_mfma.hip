@@ -66,7 +66,7 @@ pack_means_kernel(const float* __restrict__ means, size_t stride_means, float* _
 	/* the frame of the sweep (zeros unless `moved`): the rows are those of c - m, with their norms; the exact pass gets
 	 * the centroids and their norms as given */
 	__shared__ float frame[FRAME_DIMS];
-	sweep_frame<LM>(means, stride_means, dim, k, dp, moved != 0, frame, norms + plain_frame_offset(kp));
+	sweep_frame<LM>(means, stride_means, dim, k, dp, moved, frame, norms + plain_frame_offset(kp));
 	if (j >= kp) return;
 	const uint32_t rs = dp + ROW_PAD;
 	float* row = packed + packed_row(j, rs);
@@ -110,7 +110,7 @@ KMX_DECLARE_MFMA_LAUNCHER(16) KMX_DECLARE_MFMA_LAUNCHER(24) KMX_DECLARE_MFMA_LAU
 KMX_DECLARE_MFMA_LAUNCHER(128)
 
 /* packs the centroids of this call into the work space (rows of dp floats, kp rows) and empties the recheck queue */
-int launch_pack_means(const AssignArgs& a, Workspace* ws, uint32_t dp, uint32_t kp, bool moved)
+int launch_pack_means(const AssignArgs& a, Workspace* ws, uint32_t dp, uint32_t kp, uint32_t moved)
 {
 	int rc = reserve_packed(ws, (size_t)(kp / TILE) * tile_floats(dp + ROW_PAD), plain_norms_floats(kp), (size_t)kp * a.dim);
 	if (rc) return rc;
@@ -119,10 +119,10 @@ int launch_pack_means(const AssignArgs& a, Workspace* ws, uint32_t dp, uint32_t 
 	const uint32_t pack_blocks = (kp * WAVE + 255) / 256;
 	if (a.layout_means == KMX_AOS)
 		KMX_LAUNCH_KERNEL((pack_means_kernel<KMX_AOS>), dim3(pack_blocks), dim3(256), 0, stream(),
-		                   a.means, a.stride_means, ws->packed_means, ws->norms, ws->means_t, a.dim, a.k, kp, dp, moved ? 1u : 0u, ws->counters);
+		                   a.means, a.stride_means, ws->packed_means, ws->norms, ws->means_t, a.dim, a.k, kp, dp, moved, ws->counters);
 	else
 		KMX_LAUNCH_KERNEL((pack_means_kernel<KMX_SOA>), dim3(pack_blocks), dim3(256), 0, stream(),
-		                   a.means, a.stride_means, ws->packed_means, ws->norms, ws->means_t, a.dim, a.k, kp, dp, moved ? 1u : 0u, ws->counters);
+		                   a.means, a.stride_means, ws->packed_means, ws->norms, ws->means_t, a.dim, a.k, kp, dp, moved, ws->counters);
 	KMX_LAUNCH_CHECK("pack_means_kernel");
 	return KMX_OK;
 }
@@ -138,7 +138,7 @@ int launch_assign_mfma(const AssignArgs& args, kmx_exec_params* exec, Workspace*
 	const uint32_t dph = pick_dph(a.dim);
 	const uint32_t dp = 2 * dph;
 	const uint32_t kp = round_up(a.k, TILE);
-	int rc = launch_pack_means(a, ws, dp, kp, a.shift_rows);
+	int rc = launch_pack_means(a, ws, dp, kp, a.shift_rows ? FRAME_MOVED : FRAME_KEPT);
 	if (rc) return rc;
 
 	/* tau = kd (|x|^2 + max|c|^2), kd = (8 d + 24) 2^-23 (see the bound at the top of the file), 8 * 2^-23 more for the

@@ -53,19 +53,24 @@ __host__ __device__ __forceinline__ size_t plain_norms_floats(uint32_t kp) { ret
 /*
  * The frame of a call, for the packing kernels (256 threads): m = the mean of the first 16 centroids, finite coordinates
  * only (any vector would do; this one lies inside the data), a thread per dimension with its 16 loads in flight together;
- * zeros when `moved` is false. Every work-group computes it into `m` (LDS, dp <= FRAME_DIMS floats), in the same order;
- * the first one stores it at `stored` with |m|^2 (as computed: it enters the shift of the thresholds) and an upper
- * bound of |m|. Ends with a barrier.
+ * zeros when `moved` is FRAME_KEPT, and with FRAME_MOVED_IF_FAR also when |m|^2 is at most 16 times the mean squared
+ * distance of those centroids from m (data about the origin: a kernel that pays for the subtraction per point can then
+ * skip it). Every work-group computes it into `m` (LDS, dp <= FRAME_DIMS floats), in the same order; the first one stores
+ * it at `stored` with |m|^2 (as computed: it enters the shift of the thresholds) and an upper bound of |m|. Ends with a
+ * barrier.
  */
+constexpr uint32_t FRAME_KEPT = 0, FRAME_MOVED = 1, FRAME_MOVED_IF_FAR = 2;
 template <int LM>
 __device__ __forceinline__ void sweep_frame(const float* __restrict__ means, size_t stride_means, uint32_t dim, uint32_t k, uint32_t dp,
-                                            bool moved, float* m, float* __restrict__ stored)
+                                            uint32_t moved, float* m, float* __restrict__ stored)
 {
 	constexpr uint32_t SAMPLE = 16;
 	const uint32_t sample = min(k, SAMPLE);
+	__shared__ float frame_far[2][4]; /* per wavefront: its share of |m|^2 and of the summed squared distances */
+	float mine_m2 = 0.0f, mine_spread = 0.0f;
 	for (uint32_t q = threadIdx.x; q < dp; q += blockDim.x) {
 		float sum = 0.0f;
-		if (moved && q < dim) {
+		if (moved != FRAME_KEPT && q < dim) {
 			float v[SAMPLE];
 #pragma unroll
 			for (uint32_t r = 0; r < SAMPLE; ++r) v[r] = r < sample ? means[elem<LM>(stride_means, r, q)] : 0.0f;
@@ -73,8 +78,24 @@ __device__ __forceinline__ void sweep_frame(const float* __restrict__ means, siz
 			for (uint32_t r = 0; r < SAMPLE; ++r) sum += __builtin_fabsf(v[r]) < __builtin_inff() ? v[r] : 0.0f;
 			sum = sum / (float)sample;
 			sum = __builtin_fabsf(sum) < __builtin_inff() ? sum : 0.0f; /* (the sum of finite values may overflow) */
+			mine_m2 += sum * sum;
+#pragma unroll
+			for (uint32_t r = 0; r < SAMPLE; ++r)
+				if (r < sample && __builtin_fabsf(v[r]) < __builtin_inff()) mine_spread += (v[r] - sum) * (v[r] - sum);
 		}
 		m[q] = sum;
+	}
+	if (moved == FRAME_MOVED_IF_FAR) {
+		for (int off = 32; off > 0; off >>= 1) {
+			mine_m2 += __shfl_xor(mine_m2, off);
+			mine_spread += __shfl_xor(mine_spread, off);
+		}
+		if ((threadIdx.x & 63u) == 0) { frame_far[0][threadIdx.x / 64] = mine_m2; frame_far[1][threadIdx.x / 64] = mine_spread; }
+		__syncthreads();
+		const float m2 = (frame_far[0][0] + frame_far[0][1]) + (frame_far[0][2] + frame_far[0][3]);
+		const float spread = ((frame_far[1][0] + frame_far[1][1]) + (frame_far[1][2] + frame_far[1][3])) / (float)sample;
+		if (!(m2 > 16.0f * spread)) /* (the same decision in every work-group: the same numbers in the same order) */
+			for (uint32_t q = threadIdx.x; q < dp; q += blockDim.x) m[q] = 0.0f;
 	}
 	__syncthreads();
 	if (blockIdx.x == 0) {

@@ -37,13 +37,18 @@ constexpr uint32_t UNRESOLVED = 0xFFFFFFFFu;
 typedef float f32x4v __attribute__((ext_vector_type(4)));
 
 template <int DP, int LD, int LM, int MT>
-__global__ void __launch_bounds__(FUSED_WAVES * WAVE)
+__global__ void __launch_bounds__(FUSED_WAVES * WAVE) __attribute__((amdgpu_waves_per_eu(DP == 16 ? 7 : 1)))
 fused_small_kernel(const float* __restrict__ data, size_t stride, const float* __restrict__ packed, const float* __restrict__ norms,
                    const float* __restrict__ means_in, size_t stride_means,
                    float* __restrict__ means_out, uint32_t* __restrict__ sizes,
                    uint32_t* __restrict__ queue, uint32_t* __restrict__ counters,
-                   uint32_t dim, uint32_t k, uint32_t n, float kd, uint32_t vec4)
+                   uint32_t dim, uint32_t k, uint32_t n, float kd, uint32_t vec4, float kd_unmoved)
 {
+	/* the frame of the ranking (sweep_frame; the packing kernel moved the centroids): the same words for every lane, so they
+	 * arrive as scalar operands. Only the ranking uses the moved coordinates; the serial arithmetic and the sums take the
+	 * points as given. */
+	const float* __restrict__ frame = norms + plain_frame_offset(round_up(k, TILE));
+	const float frame_m2 = frame[FRAME_DIMS], frame_norm = frame[FRAME_DIMS + 1];
 	constexpr uint32_t RS = DP + ROW_PAD;
 	constexpr int NT = DP <= 16 ? 1 : 2;        /* tiles of 16 dimensions */
 	constexpr uint32_t PARK = NT * 16 + 1;      /* a parked row: coordinates padded with zeros to whole tiles, then the result */
@@ -116,26 +121,35 @@ fused_small_kernel(const float* __restrict__ data, size_t stride, const float* _
 #pragma unroll
 			for (int q = 0; q < DP; ++q) x[q] = (valid && (uint32_t)q < dim) ? data[elem<LD>(stride, pt, q)] : 0.0f;
 		}
-		float x2 = 0.0f;
-#pragma unroll
-		for (int q = 0; q < DP; ++q) x2 = __builtin_fmaf(x[q], x[q], x2);
-
-		/* 1. ranking: two smallest values with their centroids, third smallest value */
+		/* 1. ranking: two smallest values with their centroids, third smallest value; in the moved frame when the packing
+		 * kernel moved the centroids (the same for the whole launch), else on the coordinates as they are */
+		float x2 = 0.0f; /* |x - m|^2 */
 		float m1 = __builtin_inff(), m2 = __builtin_inff(), m3 = __builtin_inff();
 		uint32_t i1 = 0, i2 = 0;
-#pragma unroll 4
-		for (uint32_t r = 0; r < k; ++r) {
-			const float* row = packed + packed_row(r, RS); /* uniform address: scalar loads */
-			float a = norms[norm_at(r)];
+		auto rank = [&](const float (&p)[DP]) {
 #pragma unroll
-			for (int q = 0; q < DP; ++q) a = __builtin_fmaf(row[q], x[q], a);
-			const bool lt1 = a < m1, lt2 = a < m2;
-			i2 = lt1 ? i1 : (lt2 ? r : i2);
-			i1 = lt1 ? r : i1;
-			m3 = __builtin_amdgcn_fmed3f(m2, m3, a); /* third smallest of {m1, m2, m3, a} as m1 <= m2 <= m3 */
-			m2 = __builtin_amdgcn_fmed3f(m1, m2, a);
-			m1 = lt1 ? a : m1;
+			for (int q = 0; q < DP; ++q) x2 = __builtin_fmaf(p[q], p[q], x2);
+#pragma unroll 4
+			for (uint32_t r = 0; r < k; ++r) {
+				const float* row = packed + packed_row(r, RS); /* uniform address: scalar loads */
+				float a = norms[norm_at(r)];
+#pragma unroll
+				for (int q = 0; q < DP; ++q) a = __builtin_fmaf(row[q], p[q], a);
+				const bool lt1 = a < m1, lt2 = a < m2;
+				i2 = lt1 ? i1 : (lt2 ? r : i2);
+				i1 = lt1 ? r : i1;
+				m3 = __builtin_amdgcn_fmed3f(m2, m3, a); /* third smallest of {m1, m2, m3, a} as m1 <= m2 <= m3 */
+				m2 = __builtin_amdgcn_fmed3f(m1, m2, a);
+				m1 = lt1 ? a : m1;
+			}
+		};
+		if (frame_norm > 0.0f) {
+			float xs[DP];
+#pragma unroll
+			for (int q = 0; q < DP; ++q) xs[q] = x[q] - frame[q];
+			rank(xs);
 		}
+		else rank(x);
 
 		const float span = x2 + c2max;
 		const float tau = kd * span;
@@ -182,7 +196,11 @@ fused_small_kernel(const float* __restrict__ data, size_t stride, const float* _
 			if (flag) {
 				const uint32_t at = 2 * (flagged + __builtin_popcountll(mask & ((1ull << lane) - 1ull)));
 				flag_list[wave][at] = pt;
-				flag_list[wave][at + 1] = screening_threshold(m1, tau);
+				/* the exact pass evaluates in the frame of the data (certificate.h); (x - m) . m only for these few points */
+				float along = 0.0f;
+#pragma unroll
+				for (int q = 0; q < DP; ++q) along = __builtin_fmaf(x[q] - frame[q], frame[q], along);
+				flag_list[wave][at + 1] = screening_threshold(cert_unmoved_threshold(m1, tau, x2, along, c2max, frame_m2, frame_norm, kd_unmoved), 0.0f);
 			}
 			flagged += add;
 		}
@@ -289,7 +307,7 @@ static int launch_fused_t(const AssignArgs& a, float* means_out, uint32_t* sizes
 	const uint32_t static_bytes = (2 * FLAG_CAP * FUSED_WAVES + 128) * 4;
 	if (lds_bytes + static_bytes > dev.lds_bytes) return fail(KMX_ERR_UNSUPPORTED, "fused iteration: %u bytes of LDS needed", lds_bytes + static_bytes);
 	void (*kernel)(const float*, size_t, const float*, const float*, const float*, size_t, float*, uint32_t*, uint32_t*, uint32_t*,
-	               uint32_t, uint32_t, uint32_t, float, uint32_t) = mt == 1 ? fused_small_kernel<DP, LD, LM, 1> : fused_small_kernel<DP, LD, LM, 2>;
+	               uint32_t, uint32_t, uint32_t, float, uint32_t, float) = mt == 1 ? fused_small_kernel<DP, LD, LM, 1> : fused_small_kernel<DP, LD, LM, 2>;
 	const uint32_t batches = (a.n + FUSED_WAVES * WAVE - 1) / (FUSED_WAVES * WAVE);
 	const uint32_t per_cu = std::max<uint32_t>(1, std::min<uint32_t>(8, dev.lds_bytes / (lds_bytes + static_bytes)));
 	const uint32_t grid = std::min(batches, dev.compute_units * per_cu);
@@ -299,7 +317,7 @@ static int launch_fused_t(const AssignArgs& a, float* means_out, uint32_t* sizes
 	if (rc) return rc;
 	KMX_LAUNCH_KERNEL(kernel, dim3(grid), dim3(FUSED_WAVES * WAVE), lds_bytes, stream(),
 	                   a.data, a.stride, ws->packed_means, ws->norms, a.means, a.stride_means, means_out, sizes,
-	                   ws->queue, ws->counters, a.dim, a.k, a.n, kd, vec4);
+	                   ws->queue, ws->counters, a.dim, a.k, a.n, kd, vec4, cert_kd_unmoved(a.dim));
 	KMX_LAUNCH_CHECK("fused_small_kernel");
 	return profile_end(0);
 }
@@ -309,9 +327,11 @@ static int launch_fused_layouts(const AssignArgs& a, float* means_out, uint32_t*
 {
 	const uint32_t dp = fused_dp(a.dim);
 	const uint32_t kp = round_up(a.k, TILE);
-	int rc = launch_pack_means(a, ws, dp, kp, false);
+	/* the ranking works in a frame moved to the middle of the centroids when they lie far from the origin */
+	int rc = launch_pack_means(a, ws, dp, kp, FRAME_MOVED_IF_FAR);
 	if (rc) return rc;
-	const float kd = cert_kd_fma(a.dim); /* the bound of a ranking by chains of fused multiply-adds, see certificate.h */
+	/* the bound of a ranking by chains of fused multiply-adds, see certificate.h; 8 * 2^-23 for the roundings of x - m, c - m */
+	const float kd = cert_kd_fma(a.dim) + 8.0f * CERT_UNIT;
 	switch (dp) {
 	case 4: rc = launch_fused_t<4, LD, LM>(a, means_out, sizes, exec, ws, dev, kd); break;
 	case 8: rc = launch_fused_t<8, LD, LM>(a, means_out, sizes, exec, ws, dev, kd); break;
@@ -322,7 +342,9 @@ static int launch_fused_layouts(const AssignArgs& a, float* means_out, uint32_t*
 	}
 	if (rc) return rc;
 	/* the unresolved points: exact pass into the work-space assignment vector, then their share of the sums */
+	ws->exact_norms = ws->norms + plain_exact_norms_offset(kp);
 	rc = launch_recheck(a, ws, kp);
+	ws->exact_norms = nullptr;
 	if (rc) return rc;
 	KMX_LAUNCH_KERNEL((fused_fixup_kernel<LD, LM>), dim3(64), dim3(256), 0, stream(),
 	                   a.data, a.stride, a.assignment, means_out, a.stride_means, sizes, ws->queue, ws->counters, a.dim, a.k);

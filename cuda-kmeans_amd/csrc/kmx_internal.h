@@ -157,7 +157,7 @@ uint32_t screen_unit_rows(uint32_t dim);
 /* assign_mfma.hip / assign_lds_fma.hip: return KMX_ERR_UNSUPPORTED (without message side effects
  * beyond kmx_last_error) when the shape does not fit the variant. */
 /* shared by both fast variants: packed centroids (-2c rows of dp floats, kp rows), norms, transposed copy, empty queue */
-int launch_pack_means(const AssignArgs& a, Workspace* ws, uint32_t dp, uint32_t kp, bool moved);
+int launch_pack_means(const AssignArgs& a, Workspace* ws, uint32_t dp, uint32_t kp, uint32_t moved); /* FRAME_KEPT, FRAME_MOVED, FRAME_MOVED_IF_FAR (assign_mfma_impl.h) */
 bool mfma_supports(const AssignArgs& a, const DeviceInfo& dev);
 int launch_assign_mfma(const AssignArgs& a, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev);
 bool bf16_supports(const AssignArgs& a, const DeviceInfo& dev);

@@ -325,7 +325,7 @@ int kmx_set_queued_rows_limit(size_t bytes);
  * x2 = |x|^2, c2max = max_j |c_j|^2, cmid2max / crest2max = max_j of the squared norms of the mid / rest parts of -2 c_j;
  * all of them in the frame the sweep works in: the float sweeps subtract a vector m from points and centroids (the mean
  * of the first 16 centroids; for packed rows, with 128 centroids or more, of the first 256; the single-pass fused kernel
- * keeps m = 0; the double-precision path hands them float copies of data it has moved itself, in double), so the norms are those of the moved data; forms 0, 1 and 3 then add
+ * only when they lie far from the origin; the double-precision path hands them float copies of data it has moved itself, in double), so the norms are those of the moved data; forms 0, 1 and 3 then add
  * 8 * 2^-23 * (x2 + c2max) for the two roundings, which this function leaves out (form 2 contains it).
  */
 int kmx_certificate_tau(int form, uint32_t dim, float x2, float xpart2, float c2max, float cmid2max, float crest2max, float* tau);

@@ -663,6 +663,28 @@ def test_single_pass_fused_kernel(km, orc, gpu, dim, k, n, layout, layout_means)
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("dim,k,n", [(16, 16, 200000), (4, 8, 100000), (32, 32, 60000), (7, 5, 50000)])
+@pytest.mark.parametrize("offset", [30.0, 1000.0, -20000.0])
+def test_single_pass_fused_kernel_far_from_the_origin(km, orc, gpu, dim, k, n, offset):
+    """KMX_FUSED_ONE_PASS ranks in a frame moved to the middle of the centroids when they lie far from the origin, and sums
+    the points as given: the serial counts, the centroids within tolerance of float64 means of the serial assignment."""
+    rng = np.random.default_rng(dim * 17 + k)
+    centres = rng.uniform(-10, 10, (k, dim)).astype(np.float32)
+    pts = (centres[rng.integers(0, k, size=n)] + rng.normal(size=(n, dim)).astype(np.float32) + np.float32(offset)).astype(np.float32)
+    means = pts[:k].copy()
+    oa = orc.assign(pts.ravel(), means.ravel(), dim, k, n, threads=0, fast=True)
+    osz = np.bincount(oa, minlength=k).astype(np.uint32)
+    sums = np.zeros((k, dim)); np.add.at(sums, oa, pts.astype(np.float64))
+    ref = np.where(osz[:, None] > 0, sums / np.maximum(osz, 1)[:, None], 0.0).ravel()
+    for variant in (km.FUSED_ONE_PASS, km.FUSED_TWO_PASS):
+        gm, gs = fused_step(km, variant, pts.ravel(), means.ravel(), dim, k, n)
+        assert np.array_equal(gs, osz), "variant %d" % variant
+        spread = float(np.sqrt(np.mean((ref.reshape(k, dim) - ref.reshape(k, dim).mean(axis=0)) ** 2)))
+        # fp32 sums of coordinates about `offset`: their rounding is relative to the offset, not to the spread
+        assert float(np.abs(gm - ref).max()) < CENTROID_RTOL * max(spread, abs(offset)), "variant %d" % variant
+
+
+@pytest.mark.gpu
 def test_single_pass_fused_kernel_hard_inputs(km, orc, gpu):
     """Near-ties of three centroids, coincident points, NaN / inf / huge / tiny values go through the exact pass and the
     fix-up kernel; a shape the single-pass kernel does not take is refused by name."""
