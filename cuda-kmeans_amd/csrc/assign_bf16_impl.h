@@ -465,32 +465,68 @@ __device__ __forceinline__ void mfma_tile(f32x16 (&acc)[P], const StepOperands<K
 	}
 }
 
-/* A lane mask that a vector compare has just written to scalar registers, for use by select_lanes: on gfx940 and later a
+/* A lane mask that a vector compare has just written to scalar registers, for use by the masked copies below: on gfx940 and later a
  * vector instruction may read a scalar register that a vector instruction wrote only two wait states later. The compiler
  * keeps that distance for its own instructions but does not look inside inline assembly, so the wait is written out here;
- * the selections take the mask from this function's result and are thereby ordered behind it. */
+ * the copies take the mask from this function's result and are thereby ordered behind it. */
 __device__ __forceinline__ uint64_t settled_mask(uint64_t mask)
 {
 	asm volatile("s_nop 1" : "+s"(mask));
 	return mask;
 }
 
-/* `if_set` in the lanes of `mask`, `otherwise` in the others, as one v_cndmask on a mask held in scalar registers
- * (a mask from settled_mask, see there). */
-__device__ __forceinline__ float select_lanes(uint64_t mask, float if_set, float otherwise)
+/* The snapshot: the 16 results of the tile that holds a lane's smallest ranking value so far. */
+constexpr int SNAP_ROWS = 16;
+
+/* Copies in the lanes of `mask` only (a mask from settled_mask), for the lanes whose tile took the lead. The execution mask
+ * is narrowed to those lanes and restored inside one assembly statement, so nothing the compiler emits runs under the
+ * narrowed mask; in between, plain moves do what would otherwise be one v_cndmask per register, and v_mov_b64 moves two
+ * registers at the rate of one: the 16 results of a tile cost 8 instructions. The results are consecutive registers of the
+ * MFMA's accumulator, so their pairs cost no copies; the snapshot's pairs are formed here and stay pairs, as nothing else
+ * writes them. Fewer, longer statements are better than one per MFMA slot: every switch of the mask costs two scalar
+ * instructions and a wait for them. */
+#define KMX_SNAPSHOT_PAIRS(r)                                                                                                                \
+	f32x2 d0 = {snap[r], snap[r + 1]}, d1 = {snap[r + 2], snap[r + 3]}, d2 = {snap[r + 4], snap[r + 5]}, d3 = {snap[r + 6], snap[r + 7]}; \
+	const f32x2 s0 = {a[r], a[r + 1]}, s1 = {a[r + 2], a[r + 3]}, s2 = {a[r + 4], a[r + 5]}, s3 = {a[r + 6], a[r + 7]}
+#define KMX_SNAPSHOT_UNPAIR(r)                                                                                    \
+	snap[r] = d0.x, snap[r + 1] = d0.y, snap[r + 2] = d1.x, snap[r + 3] = d1.y, snap[r + 4] = d2.x, snap[r + 5] = d2.y, \
+	snap[r + 6] = d3.x, snap[r + 7] = d3.y
+
+/* in the lanes of `mask`: the smallest value so far becomes `lowest`, its tile `tile` (the same in every lane: a scalar
+ * operand), and results 0..7 of the tile replace the first half of the snapshot */
+__device__ __forceinline__ void take_lead_where(uint64_t mask, float& m1, uint32_t& leader_tile, float lowest, uint32_t tile,
+                                                float (&snap)[SNAP_ROWS], const f32x16& a)
 {
-	asm("v_cndmask_b32_e64 %0, %0, %1, %2" : "+v"(otherwise) : "v"(if_set), "s"(mask));
-	return otherwise;
-}
-__device__ __forceinline__ uint32_t select_lanes(uint64_t mask, uint32_t if_set, uint32_t otherwise)
-{
-	asm("v_cndmask_b32_e64 %0, %0, %1, %2" : "+v"(otherwise) : "v"(if_set), "s"(mask));
-	return otherwise;
+	uint64_t saved;
+	KMX_SNAPSHOT_PAIRS(0);
+	asm volatile("s_and_saveexec_b64 %[saved], %[mask]\n\tv_mov_b32 %[m1], %[lowest]\n\tv_mov_b32 %[leader], %[tile]\n\t"
+	             "v_mov_b64 %[d0], %[s0]\n\tv_mov_b64 %[d1], %[s1]\n\tv_mov_b64 %[d2], %[s2]\n\tv_mov_b64 %[d3], %[s3]\n\ts_mov_b64 exec, %[saved]"
+	             : [m1] "+v"(m1), [leader] "+v"(leader_tile), [d0] "+v"(d0), [d1] "+v"(d1), [d2] "+v"(d2), [d3] "+v"(d3), [saved] "=&s"(saved)
+	             : [lowest] "v"(lowest), [tile] "s"(tile), [s0] "v"(s0), [s1] "v"(s1), [s2] "v"(s2), [s3] "v"(s3), [mask] "s"(mask)
+	             : "scc");
+	KMX_SNAPSHOT_UNPAIR(0);
 }
 
+/* in the lanes of `mask`: results 8..15 of the tile replace the second half of the snapshot */
+__device__ __forceinline__ void copy_second_half_where(uint64_t mask, float (&snap)[SNAP_ROWS], const f32x16& a)
+{
+	uint64_t saved;
+	KMX_SNAPSHOT_PAIRS(8);
+	asm volatile("s_and_saveexec_b64 %[saved], %[mask]\n\tv_mov_b64 %[d0], %[s0]\n\tv_mov_b64 %[d1], %[s1]\n\tv_mov_b64 %[d2], %[s2]\n\t"
+	             "v_mov_b64 %[d3], %[s3]\n\ts_mov_b64 exec, %[saved]"
+	             : [d0] "+v"(d0), [d1] "+v"(d1), [d2] "+v"(d2), [d3] "+v"(d3), [saved] "=&s"(saved)
+	             : [s0] "v"(s0), [s1] "v"(s1), [s2] "v"(s2), [s3] "v"(s3), [mask] "s"(mask)
+	             : "scc");
+	KMX_SNAPSHOT_UNPAIR(8);
+}
+#undef KMX_SNAPSHOT_PAIRS
+#undef KMX_SNAPSHOT_UNPAIR
+
 /* Tracking with the snapshot: the minimum of the lane's 16 results of a tile (NaN-propagating tree, see track_tile), the two
- * smallest tile minima so far (m1 <= m2), the tile that holds m1 and its 16 results. */
-constexpr int SNAP_ROWS = 16;
+ * smallest tile minima so far (m1 <= m2), the tile that holds m1 and its 16 results. MASKED: the copies under a narrowed
+ * execution mask (above) instead of selections the compiler schedules freely; the wide-row step, whose MFMAs hide its
+ * tracking anyway, is faster with the latter (N = 1M, d = 64, k = 512: 0.182 against 0.186 ms). */
+template <bool MASKED>
 __device__ __forceinline__ void track_snapshot(const f32x16& acc, Track& s, float (&snap)[SNAP_ROWS], uint32_t tile)
 {
 	auto lowest = [](float a, float b) { return __builtin_elementwise_minimum(a, b); };
@@ -498,11 +534,18 @@ __device__ __forceinline__ void track_snapshot(const f32x16& acc, Track& s, floa
 #pragma unroll
 	for (int i = 1; i < 16; ++i) t = lowest(t, acc[i]);
 	s.m2 = __builtin_amdgcn_fmed3f(s.m1, s.m2, t); /* second smallest of {m1, m2, t} as m1 <= m2 */
-	const bool lt = t < s.m1 || tile == 0; /* tile 0 fills the snapshot, whatever its values */
-	s.tile = lt ? tile : s.tile;
-	s.m1 = lt ? t : s.m1;
+	if constexpr (MASKED) {
+		const uint64_t leads = settled_mask(tile == 0 ? ~0ull : __builtin_amdgcn_ballot_w64(t < s.m1)); /* tile 0 fills the snapshot, whatever its values */
+		take_lead_where(leads, s.m1, s.tile, t, tile, snap, acc);
+		copy_second_half_where(leads, snap, acc);
+	}
+	else {
+		const bool lt = t < s.m1 || tile == 0; /* tile 0 fills the snapshot, whatever its values */
+		s.tile = lt ? tile : s.tile;
+		s.m1 = lt ? t : s.m1;
 #pragma unroll
-	for (int i = 0; i < 16; ++i) snap[i] = lt ? acc[i] : snap[i];
+		for (int i = 0; i < 16; ++i) snap[i] = lt ? acc[i] : snap[i];
+	}
 }
 
 /* which kernel instances sweep with the fenced, prefetching step (unpacked rows of up to 48 dimensions, ten centroid tiles or
@@ -751,7 +794,7 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 				}
 #pragma unroll
 				for (int p = 0; p < P; ++p) {
-					if constexpr (WSNAP) track_snapshot(acc[p], st[p], snap[p], tile0 + t);
+					if constexpr (WSNAP) track_snapshot<false>(acc[p], st[p], snap[p], tile0 + t);
 					else track_tile<false, false>(acc[p], st[p], tile0 + t, neg_inf);
 				}
 				if constexpr (STREAM) {
@@ -831,10 +874,10 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 				const uint32_t tile0 = row0 / TILE;
 				constexpr int MFMAS = 3 * KB * P;
 				/* Tracking comes in pieces that are issued one behind each MFMA, so that a wavefront is back with its next MFMA before
-				 * the matrix pipe has finished the last one. With the snapshot a point tile costs 28 operations (SNAP_OPS), spread
+				 * the matrix pipe has finished the last one. With the snapshot a point tile costs 20 operations (SNAP_OPS), spread
 				 * evenly over its share of the step's MFMAs; without it, two pieces of 11 operations. */
 				constexpr int SLOTS = MFMAS / P;                             /* MFMAs per point tile and step */
-				constexpr int SNAP_OPS = 12 + SNAP_ROWS;
+				constexpr int SNAP_OPS = 12 + SNAP_ROWS / 2;
 				constexpr int OPS_PER_SLOT = (SNAP_OPS + SLOTS - 1) / SLOTS;
 				constexpr int CHUNKS = SNAP ? MFMAS : 2 * P;
 				constexpr int NORMS_AFTER = SNAP ? SLOTS - 1 : CHUNKS - 1;   /* acc_old[0] is free once point tile 0 has been tracked */
@@ -855,18 +898,18 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 					int issued = 0;
 					auto lowest = [](float a, float b) { return __builtin_elementwise_minimum(a, b); };
 					/* operation u of the snapshot tracking of point tile p: 0..7 the minimum of the lane's 16 results (NaN-propagating
-					 * tree, see track_tile), 8 the second smallest tile minimum so far, 9..11 the smallest and its tile, 12.. the 16
-					 * results replace the snapshot where the tile took the lead. The selections are written as v_cndmask on the mask:
-					 * from a condition the compiler makes one branch around all of them, which undoes the spreading. */
+					 * tree, see track_tile), 8 the second smallest tile minimum so far, 9 the lanes whose tile took the lead, as a mask in
+					 * scalar registers; 12 and 16 stand for the two masked statements of six and four moves that make the tile the
+					 * leader in those lanes and its results the snapshot (take_lead_where, copy_second_half_where: from a condition
+					 * the compiler makes one branch around all copies, which undoes the spreading). */
 					auto snapshot_op = [&](int p, int u) {
 						const f32x16& a = acc_old[p];
 						if (u == 0) lowest_of_tile[p] = lowest(a[0], a[1]);
 						else if (u < 8) lowest_of_tile[p] = lowest(lowest(lowest_of_tile[p], a[2 * u]), a[2 * u + 1]);
 						else if (u == 8) st[p].m2 = __builtin_amdgcn_fmed3f(st[p].m1, st[p].m2, lowest_of_tile[p]);
 						else if (u == 9) leads[p] = settled_mask(tile_old == 0 ? ~0ull : __builtin_amdgcn_ballot_w64(lowest_of_tile[p] < st[p].m1)); /* (tile 0 fills the snapshot, whatever its values) */
-						else if (u == 10) st[p].tile = select_lanes(leads[p], tile_old, st[p].tile);
-						else if (u == 11) st[p].m1 = select_lanes(leads[p], lowest_of_tile[p], st[p].m1);
-						else snap[p][u - 12] = select_lanes(leads[p], a[u - 12], snap[p][u - 12]);
+						else if (u == 12) take_lead_where(leads[p], st[p].m1, st[p].tile, lowest_of_tile[p], tile_old, snap[p], a);
+						else if (u == 16) copy_second_half_where(leads[p], snap[p], a);
 					};
 					auto after_mfma = [&](int i) {
 						__builtin_amdgcn_sched_barrier(0);
@@ -934,7 +977,7 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 					t += 2;
 				}
 				auto track = [&](const f32x16& acc, int p, uint32_t tile) {
-					if constexpr (SNAP) track_snapshot(acc, st[p], snap[p], tile);
+					if constexpr (SNAP) track_snapshot<true>(acc, st[p], snap[p], tile);
 					else track_tile<true, true>(acc, st[p], tile, neg_inf);
 				};
 				if (t + 1 < tiles) {
