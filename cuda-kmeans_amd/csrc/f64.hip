@@ -40,6 +40,7 @@
  * The order of the additions is not the serial one (it is not in the reference's kernels either).
  */
 #include "kmx_internal.h"
+#include <type_traits>
 
 #include <algorithm>
 
@@ -316,28 +317,38 @@ requeued_f64_kernel(const double* __restrict__ data, size_t stride, const double
 }
 
 /*
- * The same for many centroids: one lane per centroid (a work-group of up to 1024 lanes takes the centroids in chunks),
- * a batch of 16 queued points in LDS. For every dimension a lane loads its centroid's coordinate once (coalesced) and
- * applies it to the 16 points (broadcast LDS reads), so the centroids are read once per batch, not once per point.
- * The serial choice among the lanes of a chunk: the smallest distance by a 64-bit LDS minimum over the bit patterns
- * (distances are non-negative, so the patterns order like the values), then the lowest centroid number among the
- * lanes that hold exactly that distance; chunks are merged in ascending order with a strict comparison. NaN distances
- * take no part, except that a NaN distance to centroid 0 pins the point there (serial.hpp:21-35).
+ * The same for many centroids: four centroids per lane (a work-group of up to 256 lanes takes the centroids in chunks
+ * of four times its size), a batch of 16 queued points in LDS, coordinate by coordinate side by side. For every dimension
+ * a lane loads its centroids' coordinates once (coalesced) and applies them to the 16 points: one broadcast LDS read per
+ * point serves four multiply-adds (with one centroid per lane the LDS reads, one per multiply-add, bounded the kernel),
+ * and the centroids are read once per batch, not once per point. With thresholds from a float sweep the pairs that pass
+ * the screen are noted and evaluated afterwards, one lane per pair (N = 1M doubles, d = 256, k = 1024, 9.4 k queued points:
+ * 0.78 -> 0.36 ms with both changes; N = 2M, d = 32: 0.105 -> 0.055 ms).
+ * The serial choice: the smallest distance by a 64-bit LDS minimum over the bit patterns (distances are non-negative, so
+ * the patterns order like the values), then the lowest centroid number among those that hold exactly that distance;
+ * without the list, chunks are merged in ascending order with a strict comparison. NaN distances take no part, except
+ * that a NaN distance to centroid 0 pins the point there (serial.hpp:21-35).
  */
 constexpr int BATCH = 16;
+constexpr int BATCH_CPL = 4; /* centroids per lane: one broadcast read of a coordinate serves four multiply-adds */
+constexpr uint32_t PAIR_CAP = 1024;   /* noted pairs per batch; more than that are evaluated on the spot */
+constexpr uint32_t PAIR_SHIFT = 28;   /* 16 points of a batch above, the centroid below */
+constexpr uint32_t PAIR_MASK = (1u << PAIR_SHIFT) - 1;
 
-template <int LD, bool SCREEN>
-__global__ void __launch_bounds__(1024)
+template <int LD, bool SCREEN, int CPL>
+__global__ void __launch_bounds__(1024 / CPL)
 requeued_batch_f64_kernel(const double* __restrict__ data, size_t stride, const double* __restrict__ means_t, const double* __restrict__ norms,
                           uint32_t* __restrict__ assignment, uint32_t dim, uint32_t k, uint32_t kp,
                           const uint32_t* __restrict__ queue, uint32_t queue_stride, const uint32_t* __restrict__ queue_length,
                           const double* __restrict__ frame, const unsigned long long* __restrict__ misc)
 {
-	extern __shared__ double rows[]; /* BATCH x dim */
+	extern __shared__ double rows[]; /* dim x BATCH: coordinate q of the batch's points side by side */
 	__shared__ unsigned long long chunk_min[BATCH];
 	__shared__ uint32_t chunk_arg[BATCH];
 	__shared__ double best_dist[BATCH], threshold[BATCH];
 	__shared__ uint32_t best_arg[BATCH], pinned[BATCH], point_of[BATCH];
+	__shared__ uint32_t pair_count, pair_list[SCREEN ? PAIR_CAP : 1]; /* (point of the batch << PAIR_SHIFT) | centroid */
+	__shared__ double pair_dist[SCREEN ? PAIR_CAP : 1];
 	constexpr uint32_t NONE = 0xffffffffu;
 	const uint32_t total = *queue_length;
 	for (uint32_t first = blockIdx.x * BATCH; first < total; first += gridDim.x * BATCH) {
@@ -355,7 +366,7 @@ requeued_batch_f64_kernel(const double* __restrict__ data, size_t stride, const 
 			pinned[threadIdx.x] = 0;
 		}
 		__syncthreads();
-		for (uint32_t e = threadIdx.x; e < BATCH * dim; e += blockDim.x) rows[e] = data[elem<LD>(stride, point_of[e / dim], e % dim)];
+		for (uint32_t e = threadIdx.x; e < BATCH * dim; e += blockDim.x) rows[(e % dim) * BATCH + e / dim] = data[elem<LD>(stride, point_of[e / dim], e % dim)];
 		if (SCREEN) {
 			/* The float sweep ranked x - m against c - m (frame: m, then |m|^2), where the ranking values are those of
 			 * the data as given plus sh = 2 x . m - |m|^2; the values below are of the data as given, so the threshold
@@ -365,7 +376,7 @@ requeued_batch_f64_kernel(const double* __restrict__ data, size_t stride, const 
 			if (threadIdx.x < BATCH) {
 				double xm = 0.0, x2 = 0.0;
 				for (uint32_t q = 0; q < dim; ++q) {
-					const double v = rows[threadIdx.x * dim + q];
+					const double v = rows[q * BATCH + threadIdx.x];
 					xm = __builtin_fma(v, frame[q], xm);
 					x2 = __builtin_fma(v, v, x2);
 				}
@@ -374,75 +385,169 @@ requeued_batch_f64_kernel(const double* __restrict__ data, size_t stride, const 
 				threshold[threadIdx.x] = t == t ? t : __builtin_inf(); /* (values the bound does not cover: every centroid is evaluated) */
 			}
 		}
-		for (uint32_t base = 0; base < k; base += blockDim.x) {
-			__syncthreads(); /* rows are in place; the previous chunk is merged */
-			if (threadIdx.x < BATCH) { chunk_min[threadIdx.x] = ~0ull; chunk_arg[threadIdx.x] = NONE; }
-			const uint32_t j = base + threadIdx.x, jj = min(j, kp - 1);
-			double dist[BATCH];
-			uint32_t takes_part = 0; /* bit b: this lane's centroid is evaluated for point b */
-			if (SCREEN) {
-				double dot[BATCH];
-#pragma unroll
-				for (int b = 0; b < BATCH; ++b) dot[b] = 0.0;
-#pragma unroll 2
-				for (uint32_t q = 0; q < dim; ++q) {
-					const double c = means_t[(size_t)q * kp + jj];
-#pragma unroll
-					for (int b = 0; b < BATCH; ++b) dot[b] = __builtin_fma(rows[b * dim + q], c, dot[b]);
+		/* One pass over the centroids in chunks of blockDim.x * CPL. LISTING (a float sweep gave thresholds): the (point,
+		 * centroid) pairs within the threshold -- two or three per point -- are noted in LDS and evaluated afterwards, one
+		 * lane each (evaluating on the spot leaves the other lanes of the wavefront waiting through the serial sum, once
+		 * per point and centroid of the lane). Otherwise, and when the list overflows (thresholds that cover nothing,
+		 * many equal centroids), every lane evaluates its pairs on the spot and the chunks are merged one by one. */
+		auto scan = [&](auto listing_tag) {
+			constexpr bool LISTING = decltype(listing_tag)::value;
+			for (uint32_t base = 0; base < k; base += blockDim.x * CPL) {
+				if (!LISTING) {
+					__syncthreads(); /* rows are in place; the previous chunk is merged */
+					if (threadIdx.x < BATCH) { chunk_min[threadIdx.x] = ~0ull; chunk_arg[threadIdx.x] = NONE; }
 				}
-				const double c2 = norms[jj];
+				uint32_t j[CPL], jj[CPL]; /* this lane's centroids of the chunk, blockDim.x apart (coalesced loads) */
 #pragma unroll
-				for (int b = 0; b < BATCH; ++b) {
-					dist[b] = 0.0;
-					if (j < k && !(__builtin_fma(-2.0, dot[b], c2) > threshold[b])) { /* rare */
+				for (int c = 0; c < CPL; ++c) { j[c] = base + c * blockDim.x + threadIdx.x; jj[c] = min(j[c], kp - 1); }
+				double dist[LISTING ? 1 : CPL][LISTING ? 1 : BATCH];
+				uint32_t takes_part[CPL]; /* bit b: centroid c of this lane is evaluated for point b */
+#pragma unroll
+				for (int c = 0; c < CPL; ++c) takes_part[c] = 0;
+				if (SCREEN) {
+					double dot[CPL][BATCH];
+#pragma unroll
+					for (int c = 0; c < CPL; ++c)
+#pragma unroll
+						for (int b = 0; b < BATCH; ++b) dot[c][b] = 0.0;
+#pragma unroll 1 /* (two and four dimensions per trip measured no faster) */
+					for (uint32_t q = 0; q < dim; ++q) {
+						double cv[CPL];
+#pragma unroll
+						for (int c = 0; c < CPL; ++c) cv[c] = means_t[(size_t)q * kp + jj[c]];
+#pragma unroll
+						for (int b = 0; b < BATCH; ++b) {
+							const double x = rows[q * BATCH + b]; /* one broadcast read serves CPL multiply-adds */
+#pragma unroll
+							for (int c = 0; c < CPL; ++c) dot[c][b] = __builtin_fma(x, cv[c], dot[c][b]);
+						}
+					}
+#pragma unroll
+					for (int c = 0; c < CPL; ++c) {
+						const double c2 = norms[jj[c]];
+#pragma unroll
+						for (int b = 0; b < BATCH; ++b) {
+							const bool within = j[c] < k && !(__builtin_fma(-2.0, dot[c][b], c2) > threshold[b]);
+							if constexpr (LISTING) {
+								if (within) { /* rare */
+									const uint32_t slot = atomicAdd(&pair_count, 1u);
+									if (slot < PAIR_CAP) pair_list[slot] = ((uint32_t)b << PAIR_SHIFT) | j[c];
+								}
+							}
+							else {
+								dist[c][b] = 0.0;
+								if (within) { /* rare */
+									double sum = 0.0;
+#pragma unroll 8
+									for (uint32_t q = 0; q < dim; ++q) {
+										double diff = rows[q * BATCH + b] - means_t[(size_t)q * kp + jj[c]];
+										double sq = diff * diff;
+										sum = sum + sq;
+									}
+									dist[c][b] = __builtin_sqrt(sum);
+									takes_part[c] |= 1u << b;
+								}
+							}
+						}
+					}
+				}
+				else if constexpr (!LISTING) {
+#pragma unroll
+					for (int c = 0; c < CPL; ++c)
+#pragma unroll
+						for (int b = 0; b < BATCH; ++b) dist[c][b] = 0.0; /* the sums, then their roots */
+#pragma unroll 1
+					for (uint32_t q = 0; q < dim; ++q) {
+						double cv[CPL];
+#pragma unroll
+						for (int c = 0; c < CPL; ++c) cv[c] = means_t[(size_t)q * kp + jj[c]];
+#pragma unroll
+						for (int b = 0; b < BATCH; ++b) {
+							const double x = rows[q * BATCH + b];
+#pragma unroll
+							for (int c = 0; c < CPL; ++c) {
+								double diff = x - cv[c];
+								double sq = diff * diff;
+								dist[c][b] = dist[c][b] + sq;
+							}
+						}
+					}
+#pragma unroll
+					for (int c = 0; c < CPL; ++c) {
+#pragma unroll
+						for (int b = 0; b < BATCH; ++b) dist[c][b] = __builtin_sqrt(dist[c][b]);
+						takes_part[c] = j[c] < k ? 0xffffu : 0u;
+					}
+				}
+				if constexpr (!LISTING) {
+					__syncthreads(); /* chunk_min is reset */
+#pragma unroll
+					for (int c = 0; c < CPL; ++c) {
+#pragma unroll
+						for (int b = 0; b < BATCH; ++b) {
+							if (takes_part[c] & (1u << b)) {
+								if (dist[c][b] == dist[c][b]) atomicMin(&chunk_min[b], (unsigned long long)__double_as_longlong(dist[c][b]));
+								else if (j[c] == 0) pinned[b] = 1;
+							}
+						}
+					}
+					__syncthreads();
+#pragma unroll
+					for (int c = 0; c < CPL; ++c) {
+#pragma unroll
+						for (int b = 0; b < BATCH; ++b)
+							if ((takes_part[c] & (1u << b)) && dist[c][b] == dist[c][b] && (unsigned long long)__double_as_longlong(dist[c][b]) == chunk_min[b])
+								atomicMin(&chunk_arg[b], j[c]);
+					}
+					__syncthreads();
+					if (threadIdx.x < BATCH && chunk_arg[threadIdx.x] != NONE) {
+						const double d = __longlong_as_double((long long)chunk_min[threadIdx.x]);
+						if (best_arg[threadIdx.x] == NONE || best_dist[threadIdx.x] > d) { best_dist[threadIdx.x] = d; best_arg[threadIdx.x] = chunk_arg[threadIdx.x]; }
+					}
+				}
+			}
+		};
+		bool listed = false;
+		if constexpr (SCREEN) {
+			if (k <= PAIR_MASK) {
+				if (threadIdx.x == 0) pair_count = 0;
+				if (threadIdx.x < BATCH) { chunk_min[threadIdx.x] = ~0ull; chunk_arg[threadIdx.x] = NONE; }
+				__syncthreads(); /* rows and thresholds are in place, the list is empty */
+				scan(std::true_type{});
+				__syncthreads();
+				const uint32_t found = pair_count;
+				listed = found <= PAIR_CAP;
+				if (listed) {
+					/* one lane per pair: the serial sum, then the smallest distance per point and the lowest centroid that has it */
+					for (uint32_t slot = threadIdx.x; slot < found; slot += blockDim.x) {
+						const uint32_t entry = pair_list[slot], b = entry >> PAIR_SHIFT, j = entry & PAIR_MASK;
 						double sum = 0.0;
 #pragma unroll 8
 						for (uint32_t q = 0; q < dim; ++q) {
-							double diff = rows[b * dim + q] - means_t[(size_t)q * kp + jj];
+							double diff = rows[q * BATCH + b] - means_t[(size_t)q * kp + j];
 							double sq = diff * diff;
 							sum = sum + sq;
 						}
-						dist[b] = __builtin_sqrt(sum);
-						takes_part |= 1u << b;
+						const double d = __builtin_sqrt(sum);
+						pair_dist[slot] = d;
+						if (d == d) atomicMin(&chunk_min[b], (unsigned long long)__double_as_longlong(d));
+						else if (j == 0) pinned[b] = 1;
+					}
+					__syncthreads();
+					for (uint32_t slot = threadIdx.x; slot < found; slot += blockDim.x) {
+						const uint32_t entry = pair_list[slot], b = entry >> PAIR_SHIFT, j = entry & PAIR_MASK;
+						const double d = pair_dist[slot];
+						if (d == d && (unsigned long long)__double_as_longlong(d) == chunk_min[b]) atomicMin(&chunk_arg[b], j);
+					}
+					__syncthreads();
+					if (threadIdx.x < BATCH && chunk_arg[threadIdx.x] != NONE) {
+						best_dist[threadIdx.x] = __longlong_as_double((long long)chunk_min[threadIdx.x]);
+						best_arg[threadIdx.x] = chunk_arg[threadIdx.x];
 					}
 				}
-			}
-			else {
-				double sum[BATCH];
-#pragma unroll
-				for (int b = 0; b < BATCH; ++b) sum[b] = 0.0;
-#pragma unroll 2
-				for (uint32_t q = 0; q < dim; ++q) {
-					const double c = means_t[(size_t)q * kp + jj];
-#pragma unroll
-					for (int b = 0; b < BATCH; ++b) {
-						double diff = rows[b * dim + q] - c;
-						double sq = diff * diff;
-						sum[b] = sum[b] + sq;
-					}
-				}
-#pragma unroll
-				for (int b = 0; b < BATCH; ++b) dist[b] = __builtin_sqrt(sum[b]);
-				takes_part = j < k ? 0xffffu : 0u;
-			}
-			__syncthreads(); /* chunk_min is reset */
-#pragma unroll
-			for (int b = 0; b < BATCH; ++b) {
-				if (takes_part & (1u << b)) {
-					if (dist[b] == dist[b]) atomicMin(&chunk_min[b], (unsigned long long)__double_as_longlong(dist[b]));
-					else if (j == 0) pinned[b] = 1;
-				}
-			}
-			__syncthreads();
-#pragma unroll
-			for (int b = 0; b < BATCH; ++b)
-				if ((takes_part & (1u << b)) && dist[b] == dist[b] && (unsigned long long)__double_as_longlong(dist[b]) == chunk_min[b]) atomicMin(&chunk_arg[b], j);
-			__syncthreads();
-			if (threadIdx.x < BATCH && chunk_arg[threadIdx.x] != NONE) {
-				const double d = __longlong_as_double((long long)chunk_min[threadIdx.x]);
-				if (best_arg[threadIdx.x] == NONE || best_dist[threadIdx.x] > d) { best_dist[threadIdx.x] = d; best_arg[threadIdx.x] = chunk_arg[threadIdx.x]; }
 			}
 		}
+		if (!listed) scan(std::false_type{});
 		__syncthreads();
 		if (threadIdx.x < here)
 			assignment[point_of[threadIdx.x]] = (pinned[threadIdx.x] || best_arg[threadIdx.x] == NONE) ? 0u : best_arg[threadIdx.x];
@@ -651,6 +756,78 @@ update_ranges_f64_kernel(const double* __restrict__ data, size_t stride, const u
 		if (counts[e]) atomicAdd(&sizes[c0 + e], counts[e]);
 }
 
+/*
+ * The same for AoS rows of 128 dimensions and more: the work-group has one lane per dimension (at most 1024 lanes; longer
+ * rows take several dimensions per lane) and all of them add ONE listed row at a time, ROWS_IN_FLIGHT row loads in flight
+ * (the last batch of a piece included: loads one after the other wait for HBM each). No two lanes ever meet at an element
+ * of the sums, so the additions are plain reads and writes of LDS instead of atomics (an LDS floating-point atomic
+ * serialises its lanes): N = 1M doubles, k = 1024: d = 256 0.98 -> 0.54 ms, d = 128 0.41 ms with 8 loads in flight, 0.36 ms
+ * with 16 (rows of 512 dimensions: 0.25 ms with 8, 0.27 ms with 16). Pieces of 2048 points keep the list at 8 KB, so that
+ * four work-groups share a compute unit; pieces of 4096 and 8192 points measured 25-50 % slower. The ranges differ in their
+ * numbers of points (the clusters of a Lloyd iteration are far from equal), so the launch holds twice as many work-groups
+ * as are resident and the slices are half as long: at benchmark configuration 4 (N = 1M, d = 256, k = 1024, the assignment of
+ * the iteration) 0.55 ms against 0.72 ms with as many as are resident and 1.28 ms with half of that; 16 and 32 per compute unit
+ * are no better, and on equal clusters the number makes no difference.
+ */
+constexpr uint32_t ROWS_PIECE_POINTS = 2048;
+constexpr uint32_t ROWS_MIN_DIM = 128;
+constexpr uint32_t ROWS_GROUPS_PER_CU = 8; /* work-groups of the launch per compute unit (four are resident) */
+
+template <int LM, int ROWS_IN_FLIGHT>
+__global__ void __launch_bounds__(1024)
+update_ranges_rows_f64_kernel(const double* __restrict__ data, size_t stride, const uint32_t* __restrict__ assignment,
+                              double* __restrict__ means, size_t stride_means, uint32_t* __restrict__ sizes,
+                              uint32_t dim, uint32_t k, uint32_t n, uint32_t range_size, uint32_t slices)
+{
+	extern __shared__ double sums[]; /* range_size * dim doubles, range_size counts, ROWS_PIECE_POINTS list entries */
+	__shared__ uint32_t listed;
+	uint32_t* counts = (uint32_t*)(sums + (size_t)range_size * dim);
+	uint32_t* list = counts + range_size;
+	const uint32_t slice = blockIdx.x % slices, range = blockIdx.x / slices;
+	const uint32_t c0 = range * range_size, cn = min(range_size, k - c0);
+	for (uint32_t e = threadIdx.x; e < cn * dim; e += blockDim.x) sums[e] = 0.0;
+	for (uint32_t e = threadIdx.x; e < cn; e += blockDim.x) counts[e] = 0;
+	const uint32_t per_slice = (n + slices - 1) / slices;
+	const uint32_t s0 = min(slice * per_slice, n), s1 = min(s0 + per_slice, n);
+	for (uint32_t p0 = s0; p0 < s1; p0 += ROWS_PIECE_POINTS) {
+		__syncthreads(); /* sums are zero / the previous piece is added */
+		if (threadIdx.x == 0) listed = 0;
+		__syncthreads();
+		const uint32_t p1 = min(p0 + ROWS_PIECE_POINTS, s1);
+		for (uint32_t i = p0 + threadIdx.x; i < p1; i += blockDim.x) {
+			const uint32_t c = assignment[i] - c0;
+			if (c < cn) {
+				list[atomicAdd(&listed, 1u)] = (i - p0) | (c << 13);
+				atomicAdd(&counts[c], 1u);
+			}
+		}
+		__syncthreads();
+		const uint32_t members = listed;
+		for (uint32_t q = threadIdx.x; q < dim; q += blockDim.x) {
+			for (uint32_t m = 0; m < members; m += ROWS_IN_FLIGHT) {
+				double v[ROWS_IN_FLIGHT];
+				uint32_t at[ROWS_IN_FLIGHT];
+#pragma unroll
+				for (int i = 0; i < ROWS_IN_FLIGHT; ++i) { /* the last batch repeats its first row where it has no more */
+					const uint32_t entry = list[m + i < members ? m + i : m];
+					at[i] = (entry >> 13) * dim + q;
+					v[i] = data[(size_t)(p0 + (entry & (PIECE_POINTS - 1))) * stride + q];
+				}
+#pragma unroll
+				for (int i = 0; i < ROWS_IN_FLIGHT; ++i) /* in order: two of the rows may belong to one cluster */
+					if (m + i < members) sums[at[i]] += v[i];
+			}
+		}
+	}
+	__syncthreads();
+	for (uint32_t e = threadIdx.x; e < cn * dim; e += blockDim.x) {
+		const double v = sums[e];
+		if (v != 0.0) unsafeAtomicAdd(&means[elem<LM>(stride_means, c0 + e / dim, e % dim)], v);
+	}
+	for (uint32_t e = threadIdx.x; e < cn; e += blockDim.x)
+		if (counts[e]) atomicAdd(&sizes[c0 + e], counts[e]);
+}
+
 /* serial.hpp:66-72: divide by the member count, empty clusters stay at zero */
 template <int LM>
 __global__ void __launch_bounds__(256)
@@ -693,7 +870,7 @@ int launch_assign_f64_ld(int variant, const double* data, size_t stride, uint32_
 	/* queued points: many centroids and rows long enough to pay for the work-group-wide minimum -> batches of points
 	 * against one lane per centroid; else 16 lanes (2 for few centroids) share a point */
 	const bool batched = k >= 256 && dim >= 16 && (size_t)BATCH * dim * sizeof(double) <= 48 * 1024; /* dynamic + static LDS stay below 64 KB */
-	const uint32_t batch_threads = std::min<uint32_t>(1024, (k + WAVE - 1) / WAVE * WAVE);
+	const uint32_t batch_threads = std::min<uint32_t>(1024 / BATCH_CPL, ((k + BATCH_CPL - 1) / BATCH_CPL + WAVE - 1) / WAVE * WAVE);
 	const dim3 bgrid(std::min<uint32_t>((n + BATCH - 1) / BATCH, dev.compute_units * 2));
 	const bool many = k >= 256;
 	const dim3 qgrid((uint32_t)std::min<size_t>(((size_t)n * (many ? 16 : 2) + 255) / 256, (size_t)dev.compute_units * 8));
@@ -707,10 +884,10 @@ int launch_assign_f64_ld(int variant, const double* data, size_t stride, uint32_
 #define KMX_F64_REQUEUED_BY_DIM() \
 	do { \
 		if (batched && float_queue) \
-			KMX_LAUNCH_KERNEL((requeued_batch_f64_kernel<LD, true>), bgrid, dim3(batch_threads), (size_t)BATCH * dim * sizeof(double), stream(), \
+			KMX_LAUNCH_KERNEL((requeued_batch_f64_kernel<LD, true, BATCH_CPL>), bgrid, dim3(batch_threads), (size_t)BATCH * dim * sizeof(double), stream(), \
 			                   data, stride, g_means_t, g_norms, assignment, dim, k, kp, exact_queue, exact_stride, exact_length, g_frame, misc); \
 		else if (batched) \
-			KMX_LAUNCH_KERNEL((requeued_batch_f64_kernel<LD, false>), bgrid, dim3(batch_threads), (size_t)BATCH * dim * sizeof(double), stream(), \
+			KMX_LAUNCH_KERNEL((requeued_batch_f64_kernel<LD, false, BATCH_CPL>), bgrid, dim3(batch_threads), (size_t)BATCH * dim * sizeof(double), stream(), \
 			                   data, stride, g_means_t, g_norms, assignment, dim, k, kp, exact_queue, exact_stride, exact_length, g_frame, misc); \
 		else if (dim > 32) KMX_F64_REQUEUED(0); \
 		else if (dim <= 8) KMX_F64_REQUEUED(8); \
@@ -768,7 +945,22 @@ int launch_update_f64_t(int variant, const double* data, size_t stride, const ui
 	const dim3 grid(std::max<uint32_t>(wanted, 1));
 	exec->block_size = block.x;
 	exec->block_count = grid.x;
-	if (n > 0 && use_ranges) {
+	if (n > 0 && use_ranges && LD == KMX_AOS && dim >= ROWS_MIN_DIM) {
+		const size_t range_bytes = (size_t)range_size * dim * sizeof(double) + (size_t)range_size * sizeof(uint32_t) + ROWS_PIECE_POINTS * sizeof(uint32_t);
+		const dim3 lanes(std::min<uint32_t>(1024, (dim + WAVE - 1) / WAVE * WAVE)); /* one per dimension */
+		const size_t per_slice = std::max<size_t>(1024, 16 * (size_t)range_size * dim);
+		const uint32_t slices = (uint32_t)std::max<size_t>(1, std::min<size_t>((total + per_slice - 1) / per_slice, std::max<size_t>(1, (size_t)dev.compute_units * ROWS_GROUPS_PER_CU / ranges)));
+		exec->block_size = lanes.x;
+		exec->block_count = slices * ranges;
+		if (dim <= 256)
+			KMX_LAUNCH_KERNEL((update_ranges_rows_f64_kernel<LM, 16>), dim3(slices * ranges), lanes, range_bytes, stream(),
+			                   data, stride, assignment, means, stride_means, sizes, dim, k, n, range_size, slices);
+		else
+			KMX_LAUNCH_KERNEL((update_ranges_rows_f64_kernel<LM, 8>), dim3(slices * ranges), lanes, range_bytes, stream(),
+			                   data, stride, assignment, means, stride_means, sizes, dim, k, n, range_size, slices);
+		KMX_LAUNCH_CHECK("update_ranges_rows_f64_kernel");
+	}
+	else if (n > 0 && use_ranges) {
 		const size_t range_bytes = (size_t)range_size * dim * sizeof(double) + (size_t)range_size * sizeof(uint32_t) + PIECE_POINTS * sizeof(uint32_t);
 		const dim3 wide(1024);
 		const size_t per_slice = std::max<size_t>(1024, 16 * (size_t)range_size * dim);

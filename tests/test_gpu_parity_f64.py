@@ -171,7 +171,7 @@ def test_hard_inputs(km, orc, gpu, dim, k, n):
 
 
 UPDATE_SHAPES = [(8, 64, 65536), (20, 128, 10240), (3, 5, 257), (32, 1024, 50000), (4, 4096, 100000), (16, 16, 300000),
-                 (256, 1024, 4096), (33, 7, 1000), (300, 260, 3000), (5000, 3, 64)]
+                 (256, 1024, 4096), (33, 7, 1000), (300, 260, 3000), (5000, 3, 64), (128, 700, 30000), (130, 33, 5000), (1100, 40, 2500)]
 
 
 @pytest.mark.parametrize("dim,k,n", UPDATE_SHAPES)
