@@ -189,11 +189,13 @@ int dispatch_assign(int variant, const AssignArgs& a, kmx_exec_params* exec, Wor
 		 * The plain-VALU variant, which reads a small centroid block through the scalar cache, wins with at most 16
 		 * centroids of at most 16 dimensions (d = 16, k = 16: 0.086 against 0.105 ms; d = 8, k = 8: 0.049 against 0.080 ms)
 		 * and loses from there on (d = 16, k = 32: 0.128 against 0.110 ms; d = 32, k = 16: 0.183 against 0.161 ms).
-		 * The double path, which pays more per queued point: no packed form (2.35 against 1.91 ms); the plain-VALU variant
+		 * The double path, which pays more per queued point: the packed form from 256 centroids on, where its exact pass
+		 * works in batches (N = 4M doubles, d = 4, k = 4096: 1.09 against 1.64 ms per call; d = 3, k = 1024: 0.40 against
+		 * 0.52 ms; d = 4, k = 256: 0.25 against 0.29 ms; d = 2, k = 1024: level); the plain-VALU variant
 		 * up to 32 centroids (N = 2M doubles, d = 16, k = 32: 0.134 against 0.153 ms; d = 32, k = 16: level); the split
 		 * sweep from there as for floats (d = 64, k = 48: 0.547 against 0.625 ms; d = 32, k = 33: 0.302 against 0.326 ms;
 		 * d = 5, k = 1024: 0.427 against 0.438 ms). */
-		const bool packed_wins = !a.ranking_only && ((a.dim >= 3 && a.dim <= 4 && a.k >= 128) || (a.dim == 2 && a.k >= 512));
+		const bool packed_wins = (a.dim >= 3 && a.dim <= 4 && a.k >= (a.ranking_only ? 256u : 128u)) || (a.dim == 2 && a.k >= 512);
 		const bool split_wins = a.dim >= 16 || (a.dim >= 5 && a.k > 64);
 		const bool few = a.ranking_only ? a.k <= 32 : (a.k <= 16 && a.dim <= 16);
 		if (few && lds_fma_supports(a, dev) && lds_fma_reads_through_scalar_cache(a)) variant = KMX_ASSIGN_LDS_FMA;

@@ -76,7 +76,8 @@ def test_first_pass_equals_reference_golden(km, gpu, golden, name):
 
 
 SHAPES = [(20, 128, 10240), (3, 5, 257), (7, 33, 1000), (2, 2, 128), (16, 16, 5000), (32, 1000, 4099), (64, 96, 2048),
-          (100, 40, 1500), (256, 300, 700), (1, 7, 300), (5, 4100, 777), (9, 8, 64), (33, 9, 513), (4, 1, 100), (3, 5, 1), (40, 1, 1), (300, 260, 300), (400, 256, 200)]
+          (100, 40, 1500), (256, 300, 700), (1, 7, 300), (5, 4100, 777), (9, 8, 64), (33, 9, 513), (4, 1, 100), (3, 5, 1), (40, 1, 1), (300, 260, 300), (400, 256, 200),
+          (4, 4096, 3000), (3, 300, 70001), (2, 700, 5000), (12, 1024, 9000), (8, 256, 20000)]
 
 
 @pytest.mark.parametrize("dim,k,n", SHAPES)
@@ -134,7 +135,7 @@ def test_centroids_swept_in_slices(km, orc, gpu, dim, k, n, layout, layout_means
         assert bad.size == 0, "variant %d: %d mismatches, first at %s" % (v, bad.size, bad[:5])
 
 
-@pytest.mark.parametrize("dim,k,n", [(8, 64, 4096), (32, 256, 3000), (40, 70, 1000)])
+@pytest.mark.parametrize("dim,k,n", [(8, 64, 4096), (32, 256, 3000), (40, 70, 1000), (4, 300, 5000), (2, 600, 4000), (8, 512, 3000)])
 def test_hard_inputs(km, orc, gpu, dim, k, n):
     """Exact ties, duplicated centroids, coincident points, NaN / inf / huge / tiny values, float-invisible gaps."""
     rng = np.random.default_rng(99 + dim)
