@@ -369,6 +369,8 @@ requeued_f64_kernel(const double* __restrict__ data, size_t stride, const double
  */
 constexpr int BATCH = 16;
 constexpr int BATCH_CPL = 4; /* centroids per lane: one broadcast read of a coordinate serves four multiply-adds */
+constexpr int AHEAD = 2; /* dimensions between the request for the centroids' coordinates and their use (1: 13 % slower at d = 256, 4: level) */
+constexpr uint32_t THRESHOLD_PARTS = 16; /* lanes that share a row when the thresholds are taken back (fewer in a work-group of fewer than 256) */
 constexpr uint32_t PAIR_CAP = 1024;   /* noted pairs per batch; more than that are evaluated on the spot */
 constexpr uint32_t PAIR_SHIFT = 28;   /* 16 points of a batch above, the centroid below */
 constexpr uint32_t PAIR_MASK = (1u << PAIR_SHIFT) - 1;
@@ -385,6 +387,7 @@ requeued_batch_f64_kernel(const double* __restrict__ data, size_t stride, const 
 	__shared__ uint32_t chunk_arg[BATCH];
 	__shared__ double best_dist[BATCH], threshold[BATCH];
 	__shared__ uint32_t best_arg[BATCH], pinned[BATCH], point_of[BATCH];
+	__shared__ double part_xm[SCREEN ? THRESHOLD_PARTS : 1][BATCH], part_x2[SCREEN ? THRESHOLD_PARTS : 1][BATCH];
 	__shared__ uint32_t pair_count, pair_list[SCREEN ? PAIR_CAP : 1]; /* (point of the batch << PAIR_SHIFT) | centroid */
 	__shared__ double pair_dist[SCREEN ? PAIR_CAP : 1];
 	constexpr uint32_t NONE = 0xffffffffu;
@@ -411,12 +414,26 @@ requeued_batch_f64_kernel(const double* __restrict__ data, size_t stride, const 
 			 * comes back by sh, with an allowance for the double arithmetic on both sides (certificate.h has the
 			 * float version of this): (4 d + 40) 2^-52 (|x|^2 + max |c|^2). */
 			__syncthreads(); /* the rows are in place */
-			if (threadIdx.x < BATCH) {
+			/* x . m and |x|^2 of every point: up to 16 lanes share a row, each with an interleaved part of it (a single lane
+			 * per point walked 256 dimensions one LDS round trip at a time) */
+			const uint32_t parts = min(THRESHOLD_PARTS, blockDim.x / BATCH);
+			if (threadIdx.x < BATCH * parts) {
+				const uint32_t b = threadIdx.x % BATCH, part = threadIdx.x / BATCH;
 				double xm = 0.0, x2 = 0.0;
-				for (uint32_t q = 0; q < dim; ++q) {
-					const double v = rows[q * BATCH + threadIdx.x];
+				for (uint32_t q = part; q < dim; q += parts) {
+					const double v = rows[q * BATCH + b];
 					xm = __builtin_fma(v, frame[q], xm);
 					x2 = __builtin_fma(v, v, x2);
+				}
+				part_xm[part][b] = xm;
+				part_x2[part][b] = x2;
+			}
+			__syncthreads();
+			if (threadIdx.x < BATCH) {
+				double xm = 0.0, x2 = 0.0;
+				for (uint32_t part = 0; part < parts; ++part) {
+					xm += part_xm[part][threadIdx.x];
+					x2 += part_x2[part][threadIdx.x];
 				}
 				const double c2max = __longlong_as_double((long long)misc[1]);
 				const double t = threshold[threadIdx.x] - (2.0 * xm - frame[dim]) + (4.0 * dim + 40.0) * 0x1p-52 * (x2 + c2max);
@@ -448,16 +465,31 @@ requeued_batch_f64_kernel(const double* __restrict__ data, size_t stride, const 
 					for (int c = 0; c < CPL; ++c)
 #pragma unroll
 						for (int b = 0; b < BATCH; ++b) dot[c][b] = 0.0;
-#pragma unroll 1 /* (two and four dimensions per trip measured no faster) */
-					for (uint32_t q = 0; q < dim; ++q) {
-						double cv[CPL];
+					/* the centroids' coordinates are requested AHEAD dimensions before they are used (unrolling alone left
+					 * every trip waiting for its own loads) */
+					double ahead[AHEAD][CPL];
 #pragma unroll
-						for (int c = 0; c < CPL; ++c) cv[c] = means_t[(size_t)q * kp + jj[c]];
+					for (int d = 0; d < AHEAD; ++d)
 #pragma unroll
-						for (int b = 0; b < BATCH; ++b) {
-							const double x = rows[q * BATCH + b]; /* one broadcast read serves CPL multiply-adds */
+						for (int c = 0; c < CPL; ++c) ahead[d][c] = means_t[(size_t)min((uint32_t)d, dim - 1) * kp + jj[c]];
+					for (uint32_t q0 = 0; q0 < dim; q0 += AHEAD) {
 #pragma unroll
-							for (int c = 0; c < CPL; ++c) dot[c][b] = __builtin_fma(x, cv[c], dot[c][b]);
+						for (int d = 0; d < AHEAD; ++d) {
+							const uint32_t q = q0 + d;
+							if (q < dim) {
+								double cv[CPL];
+#pragma unroll
+								for (int c = 0; c < CPL; ++c) {
+									cv[c] = ahead[d][c];
+									ahead[d][c] = means_t[(size_t)min(q + AHEAD, dim - 1) * kp + jj[c]];
+								}
+#pragma unroll
+								for (int b = 0; b < BATCH; ++b) {
+									const double x = rows[q * BATCH + b]; /* one broadcast read serves CPL multiply-adds */
+#pragma unroll
+									for (int c = 0; c < CPL; ++c) dot[c][b] = __builtin_fma(x, cv[c], dot[c][b]);
+								}
+							}
 						}
 					}
 #pragma unroll
