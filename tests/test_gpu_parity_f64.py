@@ -172,7 +172,8 @@ def test_hard_inputs(km, orc, gpu, dim, k, n):
 
 
 UPDATE_SHAPES = [(8, 64, 65536), (20, 128, 10240), (3, 5, 257), (32, 1024, 50000), (4, 4096, 100000), (16, 16, 300000),
-                 (256, 1024, 4096), (33, 7, 1000), (300, 260, 3000), (5000, 3, 64), (128, 700, 30000), (130, 33, 5000), (1100, 40, 2500)]
+                 (256, 1024, 4096), (33, 7, 1000), (300, 260, 3000), (5000, 3, 64), (128, 700, 30000), (130, 33, 5000), (1100, 40, 2500),
+                 (17, 300, 40000), (64, 1000, 70001), (100, 90, 33000), (127, 513, 9000), (40, 2000, 20000)]
 
 
 @pytest.mark.parametrize("dim,k,n", UPDATE_SHAPES)
