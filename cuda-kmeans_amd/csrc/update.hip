@@ -952,7 +952,10 @@ static int launch_update_tuned(const UpdateArgs& u, kmx_exec_params* exec, Works
 		const uint32_t gw = whole_rows ? std::max<uint32_t>(16, pow2_at_least(u.dim / 4)) : (u.dim > 16 ? 32 : pow2_at_least(std::max<uint32_t>(u.dim, 4))) / vec;
 		const uint32_t pieces_bytes = 1024u * (vec + 1) * 4; /* sums of clusters cut by a range boundary, and a flag per lane group */
 		const uint32_t max_points = std::min<uint32_t>(1u << SORT_SHIFT, (budget - (u.k + 36) * 4 - pieces_bytes) / 4 / 1024 * 1024);
-		uint32_t chunks = std::max<uint32_t>(1, dev.compute_units / slices);
+		/* one chunk per compute unit; two for rows of at most 16 bytes, whose chunks are bound by the sorting, not by their
+		 * traffic (N = 4M, d = 4: k = 256 0.056 -> 0.045 ms, k = 1024 0.057 -> 0.048 ms, k = 4096 0.070 -> 0.066 ms; rows of
+		 * 8 and 16 dimensions: no gain, and four per compute unit lose) */
+		uint32_t chunks = std::max<uint32_t>(1, dev.compute_units * (u.dim <= 4 ? 2u : 1u) / slices);
 		uint32_t chunk_points = (u.n + chunks - 1) / chunks;
 		chunk_points = std::min(max_points, (chunk_points + 1023) / 1024 * 1024);
 		chunks = (u.n + chunk_points - 1) / chunk_points;
