@@ -24,6 +24,7 @@ ASSIGN_BASE, ASSIGN_LDS_FMA, ASSIGN_MFMA, ASSIGN_BEST, ASSIGN_MFMA_BF16X3 = 0, 1
 FUSED_TWO_PASS, FUSED_ONE_PASS, FUSED_BEST = 0, 1, 2
 UPDATE_ATOMIC_POINT, UPDATE_ATOMIC_FINE, UPDATE_ATOMIC_SHM, UPDATE_BASE, UPDATE_ATOMIC_WARP = 0, 1, 2, 3, 4
 UPDATE_ATOMIC_SHM2, UPDATE_FAKE, UPDATE_FAKE_SHM = 5, 6, 7  # the remaining kernels of the update micro-benchmark
+UPDATE_SERIAL_ORDER = 8  # the sums of the serial loop (ascending point number inside a cluster), bit for bit, in O(n dim)
 UPDATE_EMULATED_ATOMICS = 0x100  # flag for the point, fine and wavefront variants: compare-and-swap loops
 
 KMX_OK, KMX_ERR_INVALID_ARGUMENT, KMX_ERR_UNSUPPORTED, KMX_ERR_DEVICE, KMX_ERR_NO_DEVICE = 0, 1, 2, 3, 4
@@ -477,7 +478,9 @@ class HipKMeansAlgorithm:
 
     def update_step(self, nxt):
         # the tuned float update clears or overwrites its outputs itself (kmx_update_f32, KMX_UPDATE_ATOMIC_SHM)
-        if not (self.update_variant == UPDATE_ATOMIC_SHM and np.dtype(self.dtype) == np.float32):
+        self_clearing = (self.update_variant == UPDATE_ATOMIC_SHM and np.dtype(self.dtype) == np.float32) or \
+            self.update_variant == UPDATE_SERIAL_ORDER
+        if not self_clearing:
             self.cu_means[nxt].zero()
             self.cu_sizes.zero()
         update(self.update_variant, self.cu_data, self.layout, self.stride, self.cu_assignment[nxt], self.cu_means[nxt],

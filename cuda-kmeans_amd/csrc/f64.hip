@@ -1198,12 +1198,26 @@ int release_f64_workspace()
 	g_prepared = PreparedPoints();
 	double** buffers[] = { &g_means_t, &g_norms, &g_queue, &g_misc, &g_data32, &g_means32, &g_frame };
 	size_t* caps[] = { &g_means_t_cap, &g_norms_cap, &g_queue_cap, &g_misc_cap, &g_data32_cap, &g_means32_cap, &g_frame_cap };
-	for (int b = 0; b < 6; ++b) {
+	for (size_t b = 0; b < sizeof(buffers) / sizeof(buffers[0]); ++b) {
 		if (*buffers[b]) KMX_HIP(hipFree(*buffers[b]));
 		*buffers[b] = nullptr;
 		*caps[b] = 0;
 	}
 	return KMX_OK;
+}
+
+/* The announced points are about to change or go away: [dst, dst + bytes) is being written or released. If it touches
+ * them, the float copy must not outlive them -- hipMalloc readily hands the same address out again, and the sweeps
+ * would rank the new contents against the old copy. bytes = 0: extent unknown, anything at or below the points counts. */
+void forget_prepared_points_f64(const void* dst, size_t bytes)
+{
+	if (!g_prepared.data || !dst) return;
+	const size_t extent = g_prepared.layout == KMX_AOS ? (size_t)(g_prepared.n - 1) * g_prepared.stride + g_prepared.dim
+	                                                   : (size_t)(g_prepared.dim - 1) * g_prepared.stride + g_prepared.n;
+	const uintptr_t lo = (uintptr_t)g_prepared.data, hi = lo + extent * sizeof(double);
+	const uintptr_t a = (uintptr_t)dst;
+	const bool touches = bytes == 0 ? a < hi : (a < hi && a + bytes > lo);
+	if (touches) g_prepared = PreparedPoints();
 }
 
 /* the frame of these points (g_frame) and the float copy of the moved points (g_data32) */
@@ -1234,8 +1248,8 @@ using namespace kmx;
 extern "C" int kmx_prepare_points_f64(const double* data, int layout, size_t stride, uint32_t dim, uint32_t n)
 {
 	clear_error();
+	g_prepared = PreparedPoints(); /* whatever happens below, the old announcement is over */
 	if (dim == 0) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_prepare_points_f64: dim must be positive");
-	g_prepared = PreparedPoints();
 	if (n == 0) return KMX_OK;
 	if (!data) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_prepare_points_f64: null device pointer");
 	int rc = check_layout_f64("kmx_prepare_points_f64", "data", layout, stride, n, dim);
@@ -1367,14 +1381,20 @@ static int update_f64_call(const char* who, bool divide, int variant,
 	if (rc) return rc;
 	rc = check_layout_f64(who, "means", layout_means, stride_means, k, dim);
 	if (rc) return rc;
-	if (variant < KMX_UPDATE_ATOMIC_POINT || variant > KMX_UPDATE_ATOMIC_SHM)
-		return fail(KMX_ERR_INVALID_ARGUMENT, "%s: unknown variant %d (doubles: ATOMIC_POINT, ATOMIC_FINE, ATOMIC_SHM)", who, variant);
+	if ((variant < KMX_UPDATE_ATOMIC_POINT || variant > KMX_UPDATE_ATOMIC_SHM) && variant != KMX_UPDATE_SERIAL_ORDER)
+		return fail(KMX_ERR_INVALID_ARGUMENT, "%s: unknown variant %d (doubles: ATOMIC_POINT, ATOMIC_FINE, ATOMIC_SHM, SERIAL_ORDER)", who, variant);
 	if (exec->privatized_copies > 1)
 		return fail(KMX_ERR_UNSUPPORTED, "%s: privatized copies in global memory are not built for doubles", who);
 	if ((uint64_t)k * dim > 0xffffffffull) return fail(KMX_ERR_UNSUPPORTED, "%s: k * dim does not fit 32 bits", who);
 	const DeviceInfo* dev = nullptr;
 	rc = device_info(&dev);
 	if (rc) return rc;
+	if (variant == KMX_UPDATE_SERIAL_ORDER) {
+		Workspace* ws = nullptr;
+		rc = workspace(&ws);
+		if (rc) return rc;
+		return launch_update_serial_order<double>(data, layout, stride, assignment, means, layout_means, stride_means, cluster_sizes, dim, k, n, divide, exec, ws);
+	}
 
 	rc = profile_begin(1);
 	if (rc) return rc;

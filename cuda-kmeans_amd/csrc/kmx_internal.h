@@ -172,10 +172,22 @@ int noalloc_workspace(Workspace** ws);
 int launch_update(int variant, const UpdateArgs& u, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev);
 int launch_divide_means(const UpdateArgs& u);
 
+/* update_ordered.hip: KMX_UPDATE_SERIAL_ORDER for floats and doubles -- stable counting sort of the point numbers by
+ * cluster, then one lane per (cluster, coordinate) adds the members in ascending point order and divides: the bits of
+ * the serial loop. Scratch (chunk histograms, cluster starts, the sorted point numbers: about n + 2^21 words) is taken
+ * from ws->partials. */
+template <typename F>
+int launch_update_serial_order(const F* data, int layout, size_t stride, const uint32_t* assignment,
+                               F* means, int layout_means, size_t stride_means, uint32_t* cluster_sizes,
+                               uint32_t dim, uint32_t k, uint32_t n, bool divide, kmx_exec_params* exec, Workspace* ws);
+
 /* f64.hip: the double-precision calls keep their own transposed centroids; the runtime grows the buffer under the
  * rules of the work space (not while a graph is recorded, after the stream has drained) and releases it on shutdown */
 int reserve_f64(double** ptr, size_t* cap, size_t doubles);
 int release_f64_workspace();
+/* [dst, dst + bytes) is about to be written or released (bytes = 0: extent unknown): if the points announced by
+ * kmx_prepare_points_f64 lie there, their float copy is forgotten */
+void forget_prepared_points_f64(const void* dst, size_t bytes);
 
 /* fused_small.hip: one pass over the points for a handful of centroids. a.assignment is a scratch vector of n entries
  * (only the entries of the points left to the exact pass are written); means_out and sizes are zero on entry and hold

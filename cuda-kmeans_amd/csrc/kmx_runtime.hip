@@ -296,6 +296,16 @@ int kmx_free(void* dptr)
 	clear_error();
 	KMX_NOT_WHILE_CAPTURING("kmx_free");
 	if (!dptr) return KMX_OK;
+	{
+		/* points announced with kmx_prepare_points_f64 that live in this allocation are gone with it */
+		void* base = nullptr;
+		size_t size = 0;
+		if (hipMemGetAddressRange(&base, &size, dptr) == hipSuccess && base && size) forget_prepared_points_f64(base, size);
+		else {
+			(void)hipGetLastError();
+			forget_prepared_points_f64(dptr, 0);
+		}
+	}
 	KMX_HIP(hipFree(dptr));
 	return KMX_OK;
 }
@@ -306,6 +316,7 @@ int kmx_h2d(void* dst_device, const void* src_host, size_t bytes)
 	KMX_NOT_WHILE_CAPTURING("kmx_h2d");
 	if (bytes == 0) return KMX_OK;
 	if (!dst_device || !src_host) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_h2d: null pointer");
+	forget_prepared_points_f64(dst_device, bytes);
 	KMX_HIP(hipMemcpyAsync(dst_device, src_host, bytes, hipMemcpyHostToDevice, stream()));
 	return KMX_OK;
 }
@@ -327,6 +338,7 @@ int kmx_d2d(void* dst_device, const void* src_device, size_t bytes)
 	KMX_NOT_WHILE_CAPTURING("kmx_d2d");
 	if (bytes == 0) return KMX_OK;
 	if (!dst_device || !src_device) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_d2d: null pointer");
+	forget_prepared_points_f64(dst_device, bytes);
 	KMX_HIP(hipMemcpyAsync(dst_device, src_device, bytes, hipMemcpyDeviceToDevice, stream()));
 	return KMX_OK;
 }
@@ -360,6 +372,7 @@ int kmx_fill_zero_u32(void* dptr, size_t count)
 	clear_error();
 	if (count == 0) return KMX_OK;
 	if (!dptr) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_fill_zero_u32: null pointer");
+	forget_prepared_points_f64(dptr, count * sizeof(uint32_t));
 	const unsigned block = 256;
 	size_t blocks = (count + block - 1) / block;
 	if (blocks > 4096) blocks = 4096;
@@ -372,11 +385,12 @@ int kmx_fill_zero_u32(void* dptr, size_t count)
 static int check_update_variant(const char* who, int variant, bool bucket_sum)
 {
 	const int base = variant & ~KMX_UPDATE_EMULATED_ATOMICS;
-	if (base < KMX_UPDATE_ATOMIC_POINT || base > KMX_UPDATE_FAKE_SHM) return fail(KMX_ERR_INVALID_ARGUMENT, "%s: unknown variant %d", who, variant);
+	if (base < KMX_UPDATE_ATOMIC_POINT || base > KMX_UPDATE_SERIAL_ORDER) return fail(KMX_ERR_INVALID_ARGUMENT, "%s: unknown variant %d", who, variant);
 	if ((base == KMX_UPDATE_FAKE || base == KMX_UPDATE_FAKE_SHM) && !bucket_sum)
 		return fail(KMX_ERR_INVALID_ARGUMENT, "%s: variant %d ignores its inputs; it exists for kmx_bucket_sum_f32 only", who, variant);
 	if ((variant & KMX_UPDATE_EMULATED_ATOMICS) &&
-	    (base == KMX_UPDATE_ATOMIC_SHM || base == KMX_UPDATE_BASE || base == KMX_UPDATE_ATOMIC_SHM2 || base == KMX_UPDATE_FAKE_SHM))
+	    (base == KMX_UPDATE_ATOMIC_SHM || base == KMX_UPDATE_BASE || base == KMX_UPDATE_ATOMIC_SHM2 || base == KMX_UPDATE_FAKE_SHM ||
+	     base == KMX_UPDATE_SERIAL_ORDER))
 		return fail(KMX_ERR_UNSUPPORTED, "%s: emulated atomics exist for the point, fine, wavefront and fake variants only", who);
 	return KMX_OK;
 }

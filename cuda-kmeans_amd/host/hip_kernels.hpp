@@ -209,7 +209,7 @@ template<typename F, typename IDX_T, class LAYOUT, class LAYOUT_MEANS, int EMUL 
 class NAME {\
 public:\
 	/* false: the runner clears or overwrites its outputs itself, the driver may leave out the two runFillZeros calls */\
-	static constexpr bool needsZeroedOutput = !(SELF_CLEARING && std::is_same<F, float>::value);\
+	static constexpr bool needsZeroedOutput = !(SELF_CLEARING == 2 || (SELF_CLEARING == 1 && std::is_same<F, float>::value));\
 	static void run(const UpdateProblemInstance<F, IDX_T>& in, HipExecParameters& exec)\
 	{\
 		static_assert(!(EMUL && CAN_EMULATE) || std::is_same<F, float>::value, "emulated atomics are built for floats");\
@@ -217,8 +217,11 @@ public:\
 	}\
 };
 
-KMX_DEFINE_UPDATE_KERNEL(UpdateAtomicPointKernel, KMX_UPDATE_ATOMIC_POINT, true, false) /* kernels.cu:726-761 */
-KMX_DEFINE_UPDATE_KERNEL(UpdateAtomicFineKernel, KMX_UPDATE_ATOMIC_FINE, true, false)   /* kernels.cu:770-809 */
-KMX_DEFINE_UPDATE_KERNEL(UpdateAtomicShmKernel, KMX_UPDATE_ATOMIC_SHM, false, true)    /* kernels.cu:817-878 */
+/* SELF_CLEARING: 0 = the outputs must be zero on entry, 1 = not for floats, 2 = for neither element type */
+KMX_DEFINE_UPDATE_KERNEL(UpdateAtomicPointKernel, KMX_UPDATE_ATOMIC_POINT, true, 0) /* kernels.cu:726-761 */
+KMX_DEFINE_UPDATE_KERNEL(UpdateAtomicFineKernel, KMX_UPDATE_ATOMIC_FINE, true, 0)   /* kernels.cu:770-809 */
+KMX_DEFINE_UPDATE_KERNEL(UpdateAtomicShmKernel, KMX_UPDATE_ATOMIC_SHM, false, 1)    /* kernels.cu:817-878 */
+/* no kernel of the reference: the sums of SerialKMeansAlgorithm::updateMeans (serial.hpp:44-73) in its order, on the device */
+KMX_DEFINE_UPDATE_KERNEL(UpdateSerialOrderKernel, KMX_UPDATE_SERIAL_ORDER, false, 2)
 
 #endif

@@ -21,6 +21,7 @@
 
 #include <chrono>
 #include <cstdio>
+#include <cstring>
 #include <cstdint>
 #include <iostream>
 #include <map>
@@ -164,6 +165,7 @@ void run_kmeans(const ProgramArguments& args, std::vector<F>& data, std::vector<
 	using MfmaBf16 = MfmaBf16AssignmentKernel<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC>;
 	using Point = UpdateAtomicPointKernel<F, IDX_T, LAYOUT, LAYOUT_MEANS>;
 	using Shm = UpdateAtomicShmKernel<F, IDX_T, LAYOUT, LAYOUT_MEANS>;
+	using Ordered = UpdateSerialOrderKernel<F, IDX_T, LAYOUT, LAYOUT_MEANS>;
 	using map_t = std::map<std::string, std::unique_ptr<IKMeansAlgorithm<F, IDX_T>>>;
 	map_t algorithms;
 	algorithms["serial"].reset(new SerialKMeansAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC>(threads));
@@ -172,6 +174,8 @@ void run_kmeans(const ProgramArguments& args, std::vector<F>& data, std::vector<
 	algorithms["hip_mfma"].reset(new HipKMeansAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC, Mfma, Shm>(exec, json, graph));
 	algorithms["hip_mfma_bf16"].reset(new HipKMeansAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC, MfmaBf16, Shm>(exec, json, graph));
 	algorithms["hip_best"].reset(new HipKMeansAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC, Best, Shm>(exec, json, graph));
+	/* the fastest assignment with the update that adds in the serial order: the whole run has the bits of `serial` */
+	algorithms["hip_best_serial_order"].reset(new HipKMeansAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC, Best, Ordered>(exec, json, graph));
 	algorithms["hip_fused"].reset(new HipFusedKMeansAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC>(exec));
 
 	auto it = algorithms.find(algoName);
@@ -206,7 +210,7 @@ void run_kmeans(const ProgramArguments& args, std::vector<F>& data, std::vector<
 
 	std::size_t errors = 0, mismatches = 0;
 	double centroidErr = 0.0;
-	bool verified = false;
+	bool verified = false, identical = false;
 	if (args.getBool("verify") && algoName != "serial") {
 		std::cerr << "Verifying results ... "; std::cerr.flush();
 		SerialKMeansAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC> base(threads);
@@ -224,7 +228,11 @@ void run_kmeans(const ProgramArguments& args, std::vector<F>& data, std::vector<
 		errors = mismatches + verify_means<F, LAYOUT_MEANS>(algorithm->getMeans(), base.getMeans(), dim, k);
 		centroidErr = centroid_error<F, LAYOUT_MEANS>(algorithm->getMeans(), base.getMeans(), dim, k);
 		verified = true;
-		std::cerr << (errors == 0 ? "OK" : "FAILED") << " (centroid error relative to rms coordinate: " << centroidErr << ")" << std::endl;
+		/* the same bits as the serial run: every assignment equal and the centroid buffers equal byte for byte */
+		identical = mismatches == 0 && algorithm->getMeans().size() == base.getMeans().size()
+			&& std::memcmp(algorithm->getMeans().data(), base.getMeans().data(), base.getMeans().size() * sizeof(F)) == 0;
+		std::cerr << (errors == 0 ? "OK" : "FAILED") << " (centroid error relative to rms coordinate: " << centroidErr
+			<< (identical ? "; bit-identical to the serial run" : "") << ")" << std::endl;
 	}
 
 	if (args.isPresent("dump")) {
@@ -234,14 +242,17 @@ void run_kmeans(const ProgramArguments& args, std::vector<F>& data, std::vector<
 
 	if (json) {
 		auto* hip = dynamic_cast<HipKMeansAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC, Best, Shm>*>(algorithm.get());
+		auto* ordered = dynamic_cast<HipKMeansAlgorithm<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC, Best, Ordered>*>(algorithm.get());
 		std::cout << "{\"algorithm\": \"" << algoName << "\", \"n\": " << n << ", \"dim\": " << dim << ", \"k\": " << k
 			<< ", \"iterations\": " << iters << ", \"init_ms\": " << initMs << ", \"ms_per_iteration\": " << msPerIter
 			<< ", \"ns_per_input_float\": " << nsPerFloat
 			<< ", \"points_centroids_dims_per_s\": " << (double)n * (double)k * (double)dim / (msPerIter * 1e-3);
 		if (hip) std::cout << ", \"assign_ms\": " << hip->assignMs() / (double)iters << ", \"update_ms\": " << hip->updateMs() / (double)iters
 			<< ", \"rechecked_points\": " << hip->recheckedPoints();
+		if (ordered) std::cout << ", \"assign_ms\": " << ordered->assignMs() / (double)iters << ", \"update_ms\": " << ordered->updateMs() / (double)iters
+			<< ", \"rechecked_points\": " << ordered->recheckedPoints();
 		if (verified) std::cout << ", \"verify_errors\": " << errors << ", \"assignment_mismatches\": " << mismatches
-			<< ", \"centroid_error\": " << centroidErr;
+			<< ", \"centroid_error\": " << centroidErr << ", \"bit_identical\": " << (identical ? "true" : "false");
 		std::cout << "}" << std::endl;
 	}
 	algorithm->cleanup();
@@ -307,7 +318,7 @@ int main(int argc, char* argv[])
 		args.registerInt("seed", "Random generator seed.", 42, 0);
 		args.registerBool("assignmentOnly", "Run only assignment part of the algorithm (microbenchmark).");
 		args.conflicts("assignmentOnly", "iterations");
-		args.registerString("algorithm", "Which algorithm is to be tested (serial, hip_base, hip_base_shm, hip_mfma, hip_mfma_bf16, hip_best, hip_fused; assignment only: hip_lds_fma).", "serial");
+		args.registerString("algorithm", "Which algorithm is to be tested (serial, hip_base, hip_base_shm, hip_mfma, hip_mfma_bf16, hip_best, hip_best_serial_order, hip_fused; assignment only: hip_lds_fma).", "serial");
 		args.registerEnum("layout", "Type of data layout.", "aos", { "aos", "soa" });
 		args.registerEnum("layoutMeans", "Type of data layout (override for means only).", "aos", { "aos", "soa" });
 		args.registerBool("double", "Use doubles instead of floats.");

@@ -89,6 +89,13 @@ typedef enum kmx_update_variant {
 	 * 0.1 to dimension i mod dim of bucket (i / dim) mod k, so result[b][d] = 0.1 * #{points congruent to b modulo k} */
 	KMX_UPDATE_FAKE = 6,         /* AtomicFakeKernel: global atomics (may be or-ed with KMX_UPDATE_EMULATED_ATOMICS) */
 	KMX_UPDATE_FAKE_SHM = 7,     /* AtomicShmFakeKernel: the first shared_mem_bytes / (dim 4) buckets cached in LDS */
+	/* no kernel of the reference: the sums of its SERIAL loop (serial.hpp:44-73) -- the members of a cluster added one after
+	 * the other in ascending point number, then the guarded divide -- in O(n dim) work: stable counting sort of the point
+	 * numbers by cluster, then one lane per (cluster, coordinate) walks its members in order. Same bits as
+	 * SerialKMeansAlgorithm (and as KMX_UPDATE_BASE, which costs O(n k dim)), so a whole run with this update and any
+	 * assignment variant equals the reference's serial run bit for bit. No precondition on the outputs. Floats and doubles.
+	 * Time grows with the largest cluster (a chain of that many dependent additions). */
+	KMX_UPDATE_SERIAL_ORDER = 8,
 	/* flag, or-ed to ATOMIC_POINT / ATOMIC_FINE / ATOMIC_WARP / FAKE: additions as compare-and-swap loops instead of the hardware
 	 * atomic (the micro-benchmark's --emul, AtomicEmulTrait, bucketing-cuda/kernels/kernels.cu:83-91) */
 	KMX_UPDATE_EMULATED_ATOMICS = 0x100

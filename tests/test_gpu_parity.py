@@ -539,6 +539,138 @@ def test_free_running_loop_reports_only_near_ties(km, orc, gpu):
         assert np.array_equal(gs, osz) and rel_err(gm, o_means) < CENTROID_RTOL
 
 
+# ---------------------------------------------------------------- whole runs with the bits of the serial run
+
+GOLDEN_CASES = ["cfg1_full", "cfg1_soa_soa", "cfg1_aos_soa", "cfg1_soa_aos", "cfg2_small", "cfg3_small", "cfg4_small", "cfg5_small"]
+
+
+@pytest.mark.parametrize("name", GOLDEN_CASES)
+@pytest.mark.parametrize("update_variant", ["base", "serial_order"])
+def test_whole_runs_equal_the_reference_golden(km, gpu, golden, name, update_variant):
+    """A free-running Lloyd run (no teacher forcing) with the selector's assignment and an update that adds in the
+    serial order, against what the REFERENCE's SerialKMeansAlgorithm left after the same number of iterations
+    (tests/golden/make_golden.py): final assignment, counts and centroids bit for bit."""
+    index, arrays = golden
+    c = index[name]
+    spec = km.baseline_config(c["config"])
+    data = km.generate_points(spec, c["n"], layout=c["layout"])
+    means0 = km.first_k_means(spec, c["layout_means"])
+    uv = km.UPDATE_BASE if update_variant == "base" else km.UPDATE_SERIAL_ORDER
+    alg = km.HipKMeansAlgorithm(km.ASSIGN_BEST, uv, layout=c["layout"], layout_means=c["layout_means"])
+    alg.initialize(c["dim"], c["k"], c["n"], c["iterations"], data, means0)
+    alg.run()
+    means, asg, sizes = alg.getMeans(), alg.getAssignment(), alg.getClusterSizes()
+    alg.cleanup()
+    want = arrays[name + "_assignment"].astype(np.uint32)
+    assert np.array_equal(asg, want), "%d points differ from the reference's final assignment" % int((asg != want).sum())
+    assert np.array_equal(sizes, arrays[name + "_counts"])
+    head = arrays[name + "_means_head"]
+    assert np.array_equal(means[:head.size].view(np.uint32), head.view(np.uint32))
+    assert "%016x" % km.fnv1a64(means) == c["means_fnv1a64"]
+
+
+@pytest.mark.parametrize("dim,k,n", UPDATE_SHAPES + [(8, 64, 0), (5, 20000, 30000), (1, 1, 1000), (16, 16, 1 << 20)])
+@pytest.mark.parametrize("layout,layout_means", [(AOS, AOS), (SOA, SOA), (AOS, SOA), (SOA, AOS)])
+def test_serial_order_update_has_the_bits_of_the_serial_loop(km, orc, gpu, dim, k, n, layout, layout_means):
+    """KMX_UPDATE_SERIAL_ORDER against the oracle's update, bit for bit, on random assignments with empty clusters, one
+    very large cluster and outputs full of leftovers (the variant has no precondition on them)."""
+    rng = np.random.default_rng(dim * 1000003 + k * 101 + n)
+    data = (rng.standard_normal(max(n, 1) * dim) * 3 + 1).astype(np.float32)[:n * dim]
+    asg = rng.integers(0, k, size=n, dtype=np.uint32)
+    if k > 2 and n:
+        asg[asg == 1] = 0                                    # cluster 1 stays empty
+        asg[rng.random(n) < 0.3] = k - 1                     # one cluster with a third of the points
+    if layout == SOA:
+        data = np.ascontiguousarray(data.reshape(n, dim).T).ravel()
+    means, sizes = gpu_update(km, km.UPDATE_SERIAL_ORDER, data, asg, dim, k, n, layout, layout_means, dirty=True)
+    want_means, want_sizes = orc.update(data, asg, dim, k, n, layout, layout_means, threads=0)
+    assert np.array_equal(sizes, want_sizes)
+    assert np.array_equal(means.view(np.uint32), want_means.view(np.uint32)), \
+        "%d of %d centroid coordinates differ in their bits" % (int((means.view(np.uint32) != want_means.view(np.uint32)).sum()), means.size)
+
+
+FULL_RUNS = [(1, None), (2, None), (3, None), (4, None), (5, 1 << 20)]
+
+
+@pytest.mark.parametrize("cid,n", FULL_RUNS)
+def test_full_runs_are_identical_to_the_serial_run(km, orc, gpu, cid, n):
+    """The benchmark configurations at their full size (configuration 5: the first 2^20 points) and full iteration
+    count, free-running: selector's assignment + serial-order update on the device against the oracle's whole serial
+    run (all cores; the same per-element operations as one core). Zero mismatches, counts equal, centroids bit-equal."""
+    spec = km.baseline_config(cid)
+    n = int(spec.n) if n is None else n
+    dim, k, iters = spec.dim, spec.k, spec.iterations
+    data, means0 = km.generate_points(spec, n), km.first_k_means(spec)
+    alg = km.HipKMeansAlgorithm(km.ASSIGN_BEST, km.UPDATE_SERIAL_ORDER)
+    alg.initialize(dim, k, n, iters, data, means0)
+    alg.run()
+    gm, ga, gs = alg.getMeans(), alg.getAssignment(), alg.getClusterSizes()
+    alg.cleanup()
+    om, oa, osz = orc.kmeans(data, means0, dim, k, n, iters, threads=0, fast=True)
+    differ = int((ga != oa).sum())
+    print("configuration %d, N = %d, %d iterations free-running with the serial-order update: %d assignment mismatches, "
+          "centroids %s" % (cid, n, iters, differ, "bit-equal" if np.array_equal(gm.view(np.uint32), om.view(np.uint32)) else "differ"))
+    assert differ == 0
+    assert np.array_equal(gs, osz)
+    assert np.array_equal(gm.view(np.uint32), om.view(np.uint32))
+
+
+@pytest.mark.parametrize("cid,n", FULL_RUNS)
+def test_free_running_default_parts_from_the_serial_run_only_at_near_ties(km, orc, gpu, cid, n):
+    """The fast default (tuned update, sums in another order) free-running beside the run with the serial-order update,
+    which the test above holds bit-identical to the serial run and which therefore stands for it here, iteration by
+    iteration. Where the two part for the first time both still hold centroids that agree to rounding, and every point
+    that differs there must be a near-tie of the serial centroids (best and second-best serial distance closer than
+    1e-5 relative) or lie within the distance between the two runs' centroids. The line printed at the end is the figure of record: mismatches and centroid error after the full
+    iteration count."""
+    spec = km.baseline_config(cid)
+    n = int(spec.n) if n is None else n
+    dim, k, iters = spec.dim, spec.k, spec.iterations
+    data, means0 = km.generate_points(spec, n), km.first_k_means(spec)
+    fast = km.HipKMeansAlgorithm(km.ASSIGN_BEST, km.UPDATE_ATOMIC_SHM)
+    ref = km.HipKMeansAlgorithm(km.ASSIGN_BEST, km.UPDATE_SERIAL_ORDER)
+    fast.initialize(dim, k, n, iters, data, means0)
+    ref.initialize(dim, k, n, iters, data, means0)
+    first_split, split_points, near_ties, largest_gap = None, 0, 0, 0.0
+    for it in range(iters):
+        r_prev, f_prev = ref.getMeans(), fast.getMeans()
+        fa_buf, ra_buf = fast.iteration(), ref.iteration()
+        fa = fast.cu_assignment[fa_buf].read(np.uint32, n)
+        ra = ref.cu_assignment[ra_buf].read(np.uint32, n)
+        fast.update_step(fa_buf)
+        ref.update_step(ra_buf)
+        differ = np.nonzero(fa != ra)[0]
+        if it == 0:
+            assert differ.size == 0, "the first assignment reads identical centroids and must be identical"
+        if differ.size and first_split is None:
+            first_split, split_points = it, int(differ.size)
+            sub = np.ascontiguousarray(data.reshape(n, dim)[differ]).ravel()
+            _, best, second = orc.assign(sub, r_prev, dim, k, differ.size, threads=0, fast=False, detail=True)
+            gaps = (second.astype(np.float64) - best) / np.maximum(second.astype(np.float64), 1e-30)
+            largest_gap, near_ties = float(gaps.max()), int((gaps < NEAR_TIE).sum())
+            # Whatever is no near-tie must be explained by how far the two runs' centroids already lie apart (the serial
+            # fp32 sum of a very large cluster is itself 1e-3 off its exact value, configuration 5): moving centroid j
+            # by |delta_j| changes a distance by at most |delta_j|, so the point can only go from a to b if
+            # d_b - d_a <= |delta_a| + |delta_b| (distances to the serial centroids, in float64).
+            x = sub.reshape(differ.size, dim).astype(np.float64)
+            rc, fc = r_prev.reshape(k, dim).astype(np.float64), f_prev.reshape(k, dim).astype(np.float64)
+            a, b = ra[differ], fa[differ]
+            d_a, d_b = np.sqrt(((x - rc[a]) ** 2).sum(1)), np.sqrt(((x - rc[b]) ** 2).sum(1))
+            moved = np.sqrt(((fc - rc) ** 2).sum(1))
+            unexplained = (d_b - d_a) > moved[a] + moved[b] + NEAR_TIE * d_b
+            assert not unexplained.any(), "%d differing points are neither near-ties nor within the distance between the two runs' centroids" % int(unexplained.sum())
+    fm, fa, fs = fast.getMeans(), fast.getAssignment(), fast.getClusterSizes()
+    rm, ra = ref.getMeans(), ref.getAssignment()
+    fast.cleanup(); ref.cleanup()
+    assert int(fs.sum()) == n and np.array_equal(fs, np.bincount(fa, minlength=k).astype(np.uint32))
+    print("free-running default, configuration %d, N = %d: parts from the serial run at iteration %s (%d points, %d of them near-ties "
+          "below 1e-5, largest relative gap %.2e, the rest within the distance between the two runs' centroids); after %d iterations "
+          "%d of %d points differ, centroid error %.3e of the rms coordinate"
+          % (cid, n, first_split, split_points, near_ties, largest_gap, iters, int((fa != ra).sum()), n, rel_err(fm, rm)))
+    if first_split is None:
+        assert rel_err(fm, rm) < CENTROID_RTOL
+
+
 # ---------------------------------------------------------------- full benchmark sizes: every point against the oracle
 
 @pytest.mark.parametrize("cid", [1, 2, 3, 4, 5])

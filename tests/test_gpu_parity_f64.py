@@ -220,6 +220,84 @@ def test_every_iteration_matches_oracle(km, orc, gpu, cid, n, iters):
     alg.cleanup()
 
 
+@pytest.mark.parametrize("dim,k,n", [(8, 64, 65536), (3, 5, 257), (32, 1024, 50000), (4, 4096, 100000), (16, 16, 300000), (256, 1024, 4096),
+                                     (2, 70000, 4096), (8, 64, 0)])
+@pytest.mark.parametrize("layout,layout_means", [(AOS, AOS), (SOA, SOA), (AOS, SOA), (SOA, AOS)])
+def test_serial_order_update_has_the_bits_of_the_serial_loop(km, orc, gpu, dim, k, n, layout, layout_means):
+    """KMX_UPDATE_SERIAL_ORDER on doubles against the oracle's update, bit for bit."""
+    rng = np.random.default_rng(dim * 7 + k + n)
+    data = rng.normal(size=n * dim) * 2.0 + 1.0
+    asg = rng.integers(0, k, size=n, dtype=np.uint32)
+    if k > 2 and n:
+        asg[asg == 1] = 0
+        asg[rng.random(n) < 0.3] = k - 1
+    want_m, want_s = orc.update_f64(data, asg, dim, k, n, layout, layout_means, threads=0)
+    got_m, got_s = gpu_update(km, km.UPDATE_SERIAL_ORDER, data, asg, dim, k, n, layout, layout_means)
+    assert np.array_equal(got_s, want_s)
+    assert np.array_equal(got_m.view(np.uint64), want_m.view(np.uint64))
+
+
+def test_whole_runs_equal_the_reference_golden(km, gpu, golden):
+    """Free-running double-precision runs with the serial-order update against what the REFERENCE's
+    SerialKMeansAlgorithm<double> left (tests/golden/make_golden_f64.py): assignment, counts, centroids bit for bit."""
+    index, arrays = golden
+    for name, c in sorted(index.items()):
+        spec = km.baseline_config(c["config"])
+        data = km.widen_points(km.generate_points(spec, c["n"], layout=c["layout"]))
+        means0 = km.widen_points(km.first_k_means(spec, c["layout_means"]))
+        alg = km.HipKMeansAlgorithm(km.ASSIGN_BEST, km.UPDATE_SERIAL_ORDER, layout=c["layout"], layout_means=c["layout_means"], dtype=np.float64)
+        alg.initialize(c["dim"], c["k"], c["n"], c["iterations"], data, means0)
+        alg.run()
+        means, asg, sizes = alg.getMeans(), alg.getAssignment(), alg.getClusterSizes()
+        alg.cleanup()
+        assert np.array_equal(asg, arrays[name + "_assignment"].astype(np.uint32)), name
+        assert np.array_equal(sizes, arrays[name + "_counts"]), name
+        head = arrays[name + "_means_head"]
+        assert np.array_equal(means[:head.size].view(np.uint64), head.view(np.uint64)), name
+        assert "%016x" % km.fnv1a64(means) == c["means_fnv1a64"], name
+
+
+def test_prepared_points_do_not_outlive_their_buffer(km, orc, gpu):
+    """The float copy made by kmx_prepare_points_f64 is dropped when the announced buffer is rewritten through the library
+    (kmx_h2d, kmx_d2d, kmx_fill_zero_u32) or released (kmx_free): a later call on the same address, which hipMalloc readily
+    hands out again, must see the new contents."""
+    dim, k, n = 16, 128, 20000
+    rng = np.random.default_rng(5)
+    first = rng.normal(size=n * dim) * 3
+    other = rng.normal(size=n * dim) * 3 + 1
+    means = first.reshape(n, dim)[:k].copy().ravel()
+    lib = km.hip_lib()
+    m = km.DeviceBuffer(8 * k * dim); m.write(means)
+    a = km.DeviceBuffer(4 * n)
+    spare = km.DeviceBuffer(8 * n * dim); spare.write(other)
+
+    def run(buf):
+        km.assign(km.ASSIGN_BEST, buf, km.AOS, dim, m, km.AOS, dim, a, dim, k, n, dtype=np.float64)
+        km.sync()
+        return a.read(np.uint32, n)
+
+    want_first = orc.assign_f64(first, means, dim, k, n, threads=0)
+    want_other = orc.assign_f64(other, means, dim, k, n, threads=0)
+    want_zero = orc.assign_f64(np.zeros(n * dim), means, dim, k, n, threads=0)
+    d = km.DeviceBuffer(8 * n * dim); d.write(first)
+    km.check(lib.kmx_prepare_points_f64(d.ptr, km.AOS, dim, dim, n))
+    assert np.array_equal(run(d), want_first)
+    d.write(other)                                       # rewritten in place through kmx_h2d, no kmx_forget_points_f64
+    assert np.array_equal(run(d), want_other)
+    km.check(lib.kmx_prepare_points_f64(d.ptr, km.AOS, dim, dim, n))
+    km.check(lib.kmx_d2d(d.ptr, spare.ptr, 8 * n * dim)) # the same contents again: harmless, but the copy is dropped
+    d.zero()                                             # kmx_fill_zero_u32
+    assert np.array_equal(run(d), want_zero)
+    d.write(first)
+    km.check(lib.kmx_prepare_points_f64(d.ptr, km.AOS, dim, dim, n))
+    d.free()                                             # kmx_free: the announcement goes with the buffer
+    d = km.DeviceBuffer(8 * n * dim)                     # very likely the same address
+    d.write(other)
+    assert np.array_equal(run(d), want_other)
+    for b in (d, m, a, spare):
+        b.free()
+
+
 def test_fused_call_and_argument_errors(km, orc, gpu):
     spec = km.baseline_config(1)
     n = 20000
