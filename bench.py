@@ -216,7 +216,9 @@ def main():
     ap.add_argument("--config", type=int, default=2, help="benchmark configuration 1..5 (2 = headline)")
     ap.add_argument("--cpu-sample", type=int, default=0, help="points in the CPU baseline sample (0 = about 12 s of work)")
     ap.add_argument("--assign-variant", default="best", choices=["base", "lds_fma", "mfma", "mfma_bf16x3", "best"])
-    ap.add_argument("--update-variant", default="atomic_shm", choices=["atomic_point", "atomic_fine", "atomic_shm"])
+    ap.add_argument("--update-variant", default="atomic_shm", choices=["atomic_point", "atomic_fine", "atomic_shm", "serial_order"],
+                    help="serial_order: sums in the order of the reference's serial loop (whole runs bit-identical to it); "
+                         "its roofline_update covers all kernels of the variant (sort + sums)")
     ap.add_argument("--fused", action="store_true",
                     help="time the fused iteration (kmx_fused_f32: one call per iteration, no assignment vector; a single "
                          "pass over the points where k <= 32) instead of assignment + update")
@@ -246,7 +248,7 @@ def main():
     assign_variant = {"base": km.ASSIGN_BASE, "lds_fma": km.ASSIGN_LDS_FMA, "mfma": km.ASSIGN_MFMA, "mfma_bf16x3": km.ASSIGN_MFMA_BF16X3,
                       "best": km.ASSIGN_BEST}[args.assign_variant]
     update_variant = {"atomic_point": km.UPDATE_ATOMIC_POINT, "atomic_fine": km.UPDATE_ATOMIC_FINE,
-                      "atomic_shm": km.UPDATE_ATOMIC_SHM}[args.update_variant]
+                      "atomic_shm": km.UPDATE_ATOMIC_SHM, "serial_order": km.UPDATE_SERIAL_ORDER}[args.update_variant]
     if args.fused:
         return fused_main(km, args, spec, data, means0)
     if args.double:

@@ -1393,7 +1393,7 @@ static int update_f64_call(const char* who, bool divide, int variant,
 		Workspace* ws = nullptr;
 		rc = workspace(&ws);
 		if (rc) return rc;
-		return launch_update_serial_order<double>(data, layout, stride, assignment, means, layout_means, stride_means, cluster_sizes, dim, k, n, divide, exec, ws);
+		return launch_update_serial_order<double>(data, layout, stride, assignment, means, layout_means, stride_means, cluster_sizes, dim, k, n, divide, exec, ws, *dev);
 	}
 
 	rc = profile_begin(1);

@@ -179,7 +179,7 @@ int launch_divide_means(const UpdateArgs& u);
 template <typename F>
 int launch_update_serial_order(const F* data, int layout, size_t stride, const uint32_t* assignment,
                                F* means, int layout_means, size_t stride_means, uint32_t* cluster_sizes,
-                               uint32_t dim, uint32_t k, uint32_t n, bool divide, kmx_exec_params* exec, Workspace* ws);
+                               uint32_t dim, uint32_t k, uint32_t n, bool divide, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev);
 
 /* f64.hip: the double-precision calls keep their own transposed centroids; the runtime grows the buffer under the
  * rules of the work space (not while a graph is recorded, after the stream has drained) and releases it on shutdown */

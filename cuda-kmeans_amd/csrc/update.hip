@@ -1195,7 +1195,7 @@ int launch_update(int variant, const UpdateArgs& u, kmx_exec_params* exec, Works
 {
 	if (variant == KMX_UPDATE_SERIAL_ORDER)
 		return launch_update_serial_order<float>(u.data, u.layout, u.stride, u.assignment, u.means, u.layout_means, u.stride_means, u.cluster_sizes,
-		                                         u.dim, u.k, u.n, u.divide, exec, ws);
+		                                         u.dim, u.k, u.n, u.divide, exec, ws, dev);
 	/* (the fixed work space has no room for a copy of the points: SoA points then stay with the element-wise kernels) */
 	if (!ws->fixed && u.layout == KMX_SOA && (variant & ~KMX_UPDATE_EMULATED_ATOMICS) == KMX_UPDATE_ATOMIC_SHM && u.n > 0 && u.dim >= 8 &&
 	    (size_t)u.n * u.dim * sizeof(float) <= ROWS_COPY_MAX_BYTES) {

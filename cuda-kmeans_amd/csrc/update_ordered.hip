@@ -27,7 +27,6 @@ namespace kmx {
 constexpr uint32_t ORDERED_LDS_CLUSTERS = 16384; /* up to here a chunk's counters live in LDS (64 KB per wavefront-sized work-group) */
 constexpr uint32_t ORDERED_HIST_WORDS = 1u << 21; /* bound of chunks x k */
 constexpr uint32_t ORDERED_MAX_CHUNKS = 4096;
-constexpr int ORDERED_UNROLL = 8;
 
 /*
  * Histogram of one chunk of points: hist[chunk][cluster]. One wavefront per chunk, the same chunks as the scatter.
@@ -177,42 +176,74 @@ ordered_scatter_kernel(const uint32_t* __restrict__ assignment, uint32_t* __rest
 }
 
 /*
- * One lane per (cluster, coordinate): the members' coordinates added one after the other in the order of the sorted
- * list, i.e. in ascending point number, starting from zero like the serial loop (serial.hpp:57-63), then the guarded
- * divide (serial.hpp:65-71). The loads of ORDERED_UNROLL rows are in flight together; the additions stay a chain.
+ * One lane per cluster and piece of VEC consecutive coordinates (VEC = 1, or a 16-byte piece of an AoS row): the members'
+ * coordinates added one after the other in the order of the sorted list, i.e. in ascending point number, starting from
+ * zero like the serial loop (serial.hpp:57-63), then the guarded divide (serial.hpp:65-71). The additions of a
+ * coordinate are a chain; what can overlap are the loads: the pieces of UNROLL rows are in flight together, and the
+ * point numbers of the next UNROLL rows are requested before the current ones are added (a chain is as many sums as
+ * the machine runs at once here, so the time is the latency of a load divided by the loads in flight).
  */
-template <typename F, int LD, int LM>
-__global__ void __launch_bounds__(256)
+template <typename F, int VEC> struct alignas(sizeof(F) * VEC) OrderedPiece { F v[VEC]; };
+
+template <typename F, int LD, int LM, int VEC, int UNROLL>
+__global__ void __launch_bounds__(64)
 ordered_sum_kernel(const F* __restrict__ data, size_t stride, const uint32_t* __restrict__ sorted, const uint32_t* __restrict__ starts,
                    const uint32_t* __restrict__ sizes, F* __restrict__ means, size_t stride_means, uint32_t dim, uint32_t k, uint32_t divide)
 {
-	const size_t e = (size_t)blockIdx.x * 256 + threadIdx.x;
-	if (e >= (size_t)k * dim) return;
-	const uint32_t c = (uint32_t)(e / dim), d = (uint32_t)(e % dim);
+	static_assert(VEC == 1 || LD == KMX_AOS, "pieces of several coordinates are pieces of AoS rows");
+	typedef OrderedPiece<F, VEC> piece_t;
+	const uint32_t pieces = dim / VEC; /* the launcher picks VEC among the divisors of dim */
+	const size_t e = (size_t)blockIdx.x * WAVE + threadIdx.x;
+	if (e >= (size_t)k * pieces) return;
+	const uint32_t c = (uint32_t)(e / pieces), d = (uint32_t)(e % pieces) * VEC;
 	const uint32_t members = sizes[c];
 	const uint32_t begin = starts[c], end = begin + members;
-	F sum = (F)0;
-	for (uint32_t j = begin; j < end; j += ORDERED_UNROLL) {
-		uint32_t point[ORDERED_UNROLL];
-		F v[ORDERED_UNROLL];
+	piece_t sum;
 #pragma unroll
-		for (int u = 0; u < ORDERED_UNROLL; ++u) point[u] = sorted[min(j + u, end - 1)];
+	for (int i = 0; i < VEC; ++i) sum.v[i] = (F)0;
+	if (members) {
+		uint32_t point[UNROLL];
 #pragma unroll
-		for (int u = 0; u < ORDERED_UNROLL; ++u) v[u] = data[elem<LD>(stride, point[u], d)];
+		for (int u = 0; u < UNROLL; ++u) point[u] = sorted[min(begin + u, end - 1)];
+		for (uint32_t j = begin; j < end; j += UNROLL) {
+			piece_t v[UNROLL];
 #pragma unroll
-		for (int u = 0; u < ORDERED_UNROLL; ++u)
-			if (j + u < end) sum = sum + v[u];
+			for (int u = 0; u < UNROLL; ++u) v[u] = *(const piece_t*)(data + elem<LD>(stride, point[u], d));
+#pragma unroll
+			for (int u = 0; u < UNROLL; ++u) point[u] = sorted[min(j + UNROLL + u, end - 1)];
+#pragma unroll
+			for (int u = 0; u < UNROLL; ++u) {
+				if (j + u < end) {
+#pragma unroll
+					for (int i = 0; i < VEC; ++i) sum.v[i] = sum.v[i] + v[u].v[i];
+				}
+			}
+		}
 	}
-	means[elem<LM>(stride_means, c, d)] = !divide ? sum : (members ? sum / (F)members : (F)0);
+#pragma unroll
+	for (int i = 0; i < VEC; ++i)
+		means[elem<LM>(stride_means, c, d + i)] = !divide ? sum.v[i] : (members ? sum.v[i] / (F)members : (F)0);
 }
 
+/* Work-groups of one wavefront: what bounds this kernel is the number of cache lines a compute unit keeps in flight, so
+ * the chains are spread over as many compute units as there are wavefronts (measured at N = 2M, d = 32, k = 1024: 32
+ * work-groups of four wavefronts with 16-byte pieces 0.85 ms). The 16-byte pieces, which need a quarter of the lanes, are
+ * taken only where they still leave two wavefronts per compute unit. */
 template <typename F, int LD, int LM>
 static int launch_ordered_sum(const F* data, size_t stride, const uint32_t* sorted, const uint32_t* starts, const uint32_t* sizes,
-                              F* means, size_t stride_means, uint32_t dim, uint32_t k, bool divide)
+                              F* means, size_t stride_means, uint32_t dim, uint32_t k, bool divide, const DeviceInfo& dev)
 {
-	const size_t total = (size_t)k * dim;
-	KMX_LAUNCH_KERNEL((ordered_sum_kernel<F, LD, LM>), dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, stream(),
-	                   data, stride, sorted, starts, sizes, means, stride_means, dim, k, divide ? 1u : 0u);
+	constexpr int WIDE = 16 / sizeof(F);
+	const bool fits = LD == KMX_AOS && dim % WIDE == 0 && stride % WIDE == 0 && ((uintptr_t)data & 15) == 0;
+	const bool wide = fits && (size_t)k * (dim / WIDE) >= (size_t)2 * WAVE * dev.compute_units;
+	const size_t total = (size_t)k * (wide ? dim / WIDE : dim);
+	const dim3 grid((uint32_t)((total + WAVE - 1) / WAVE));
+	if (wide)
+		KMX_LAUNCH_KERNEL((ordered_sum_kernel<F, KMX_AOS, LM, WIDE, 32>), grid, dim3(WAVE), 0, stream(),
+		                   data, stride, sorted, starts, sizes, means, stride_means, dim, k, divide ? 1u : 0u);
+	else
+		KMX_LAUNCH_KERNEL((ordered_sum_kernel<F, LD, LM, 1, 32>), grid, dim3(WAVE), 0, stream(),
+		                   data, stride, sorted, starts, sizes, means, stride_means, dim, k, divide ? 1u : 0u);
 	KMX_LAUNCH_CHECK("ordered_sum_kernel");
 	return KMX_OK;
 }
@@ -220,10 +251,10 @@ static int launch_ordered_sum(const F* data, size_t stride, const uint32_t* sort
 template <typename F>
 int launch_update_serial_order(const F* data, int layout, size_t stride, const uint32_t* assignment,
                                F* means, int layout_means, size_t stride_means, uint32_t* cluster_sizes,
-                               uint32_t dim, uint32_t k, uint32_t n, bool divide, kmx_exec_params* exec, Workspace* ws)
+                               uint32_t dim, uint32_t k, uint32_t n, bool divide, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev)
 {
 	if (n > 0xFFFFFFFFu - (1u << 20)) return fail(KMX_ERR_UNSUPPORTED, "the serial-order update takes fewer than 2^32 - 2^20 points");
-	if ((uint64_t)k * dim > 0xFFFFFFFFull * 256) return fail(KMX_ERR_UNSUPPORTED, "the serial-order update: k * dim is too large for one launch");
+	if ((uint64_t)k * dim > 0xFFFFFFFFull * WAVE) return fail(KMX_ERR_UNSUPPORTED, "the serial-order update: k * dim is too large for one launch");
 	/* chunks: one wavefront each, a multiple of 64 points, few enough that chunks x k counters stay small */
 	uint32_t chunks = 0, chunk_points = WAVE;
 	if (n > 0) {
@@ -274,15 +305,15 @@ int launch_update_serial_order(const F* data, int layout, size_t stride, const u
 			KMX_LAUNCH_KERNEL((ordered_scatter_kernel<false>), dim3(chunks), dim3(WAVE), 0, stream(), assignment, hist, starts, sorted, k, n, chunk_points);
 		KMX_LAUNCH_CHECK("ordered_scatter_kernel");
 	}
-	if (layout == KMX_AOS && layout_means == KMX_AOS) rc = launch_ordered_sum<F, KMX_AOS, KMX_AOS>(data, stride, sorted, starts, cluster_sizes, means, stride_means, dim, k, divide);
-	else if (layout == KMX_AOS) rc = launch_ordered_sum<F, KMX_AOS, KMX_SOA>(data, stride, sorted, starts, cluster_sizes, means, stride_means, dim, k, divide);
-	else if (layout_means == KMX_AOS) rc = launch_ordered_sum<F, KMX_SOA, KMX_AOS>(data, stride, sorted, starts, cluster_sizes, means, stride_means, dim, k, divide);
-	else rc = launch_ordered_sum<F, KMX_SOA, KMX_SOA>(data, stride, sorted, starts, cluster_sizes, means, stride_means, dim, k, divide);
+	if (layout == KMX_AOS && layout_means == KMX_AOS) rc = launch_ordered_sum<F, KMX_AOS, KMX_AOS>(data, stride, sorted, starts, cluster_sizes, means, stride_means, dim, k, divide, dev);
+	else if (layout == KMX_AOS) rc = launch_ordered_sum<F, KMX_AOS, KMX_SOA>(data, stride, sorted, starts, cluster_sizes, means, stride_means, dim, k, divide, dev);
+	else if (layout_means == KMX_AOS) rc = launch_ordered_sum<F, KMX_SOA, KMX_AOS>(data, stride, sorted, starts, cluster_sizes, means, stride_means, dim, k, divide, dev);
+	else rc = launch_ordered_sum<F, KMX_SOA, KMX_SOA>(data, stride, sorted, starts, cluster_sizes, means, stride_means, dim, k, divide, dev);
 	if (rc) return rc;
 	return profile_end(1);
 }
 
-template int launch_update_serial_order<float>(const float*, int, size_t, const uint32_t*, float*, int, size_t, uint32_t*, uint32_t, uint32_t, uint32_t, bool, kmx_exec_params*, Workspace*);
-template int launch_update_serial_order<double>(const double*, int, size_t, const uint32_t*, double*, int, size_t, uint32_t*, uint32_t, uint32_t, uint32_t, bool, kmx_exec_params*, Workspace*);
+template int launch_update_serial_order<float>(const float*, int, size_t, const uint32_t*, float*, int, size_t, uint32_t*, uint32_t, uint32_t, uint32_t, bool, kmx_exec_params*, Workspace*, const DeviceInfo&);
+template int launch_update_serial_order<double>(const double*, int, size_t, const uint32_t*, double*, int, size_t, uint32_t*, uint32_t, uint32_t, uint32_t, bool, kmx_exec_params*, Workspace*, const DeviceInfo&);
 
 } // namespace kmx
