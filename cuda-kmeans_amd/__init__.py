@@ -36,7 +36,7 @@ ABI_SYMBOLS = [
     "kmx_assign_last_rechecked", "kmx_assign_last_variant", "kmx_update_f32", "kmx_bucket_sum_f32", "kmx_fused_f32", "kmx_assign_f64", "kmx_update_f64", "kmx_fused_f64", "kmx_bucket_sum_f64", "kmx_set_queued_rows_limit",
     "kmx_graph_begin", "kmx_graph_end", "kmx_graph_launch", "kmx_graph_destroy", "kmx_event_create", "kmx_event_destroy", "kmx_event_record",
     "kmx_event_elapsed_ms", "kmx_set_profiling", "kmx_last_kernel_ms", "kmx_last_error", "kmx_certificate_tau", "kmx_certificate_unmoved_threshold",
-    "kmx_update_f32_noalloc", "kmx_reserve_f32", "kmx_prepare_points_f64", "kmx_forget_points_f64",
+    "kmx_update_f32_noalloc", "kmx_reserve_f32", "kmx_prepare_points_f64", "kmx_forget_points_f64", "kmx_probe_matrix_chain",
 ]
 
 
@@ -135,6 +135,7 @@ def hip_lib():
         lib.kmx_set_profiling.argtypes = [ctypes.c_int]
         lib.kmx_set_queued_rows_limit.argtypes = [ctypes.c_size_t]
         lib.kmx_last_kernel_ms.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_float)]
+        lib.kmx_probe_matrix_chain.argtypes = [ctypes.c_int, vp, vp, vp, vp, u32]
         _hip = lib
     return _hip
 
@@ -390,6 +391,25 @@ def certificate_tau(form, dim, x2, xpart2, c2max, cmid2max, crest2max):
     out = ctypes.c_float()
     check(hip_lib().kmx_certificate_tau(form, dim, x2, xpart2, c2max, cmid2max, crest2max, ctypes.byref(out)))
     return out.value
+
+
+def probe_matrix_chain(kind, a, b, c):
+    """kmx_probe_matrix_chain on host arrays: a (32, depth), b (32, depth: row j = column j of B), c (32, 32), all
+    float32; returns d = c + a b^T as the matrix cores accumulate it, block by block (kind 0: fp32, 1: bf16 operands)."""
+    a, b, c = (np.ascontiguousarray(v, dtype=np.float32) for v in (a, b, c))
+    depth = a.shape[1]
+    block = 2 if kind == 0 else 16
+    assert a.shape == (32, depth) and b.shape == (32, depth) and c.shape == (32, 32) and depth % block == 0
+    bufs = [DeviceBuffer(v.nbytes) for v in (a, b, c, c)]
+    try:
+        for buf, v in zip(bufs, (a, b, c)):
+            buf.write(v)
+        check(hip_lib().kmx_probe_matrix_chain(kind, bufs[0].ptr, bufs[1].ptr, bufs[2].ptr, bufs[3].ptr, depth // block))
+        sync()
+        return bufs[3].read(np.float32, 32 * 32).reshape(32, 32)
+    finally:
+        for buf in bufs:
+            buf.free()
 
 
 def reserve(assign_variant, update_variant, layout, layout_means, dim, k, n):

@@ -1534,6 +1534,65 @@ static int launch_screen_bf16_kb(const float* rows, const Workspace* ws, const u
 	return KMX_OK;
 }
 
+/* static LDS of assign_bf16_kernel: the flag lists, wave_max (4 x MFMA_WAVES words) and the frame of the rows */
+template <int KB, bool PACKED> constexpr uint32_t sweep_static_lds_bytes()
+{
+	return (2 * FLAG_CAP * MFMA_WAVES + 4 * MFMA_WAVES + (PACKED ? 4 : KB * KBLOCK)) * 4;
+}
+
+/*
+ * What a sweep is about to be launched with, checked on the host against what the kernel assumes: every offset the
+ * kernel forms from these numbers -- the packed rows and norms of each chunk or slice, the frame behind the norms, the
+ * two LDS buffers, the staged pieces, the values carried between slices, the queue -- must lie inside its allocation.
+ * A kernel that runs off one of them faults the GPU for everybody; a launch refused here costs an error message.
+ */
+struct SweepPlan {
+	uint32_t kb, rs, kp, k, n, chunk_rows, slices, lds_bytes, static_bytes, grid;
+	bool stream_mode, packed_form, wide;
+};
+
+inline int check_sweep_plan(const SweepPlan& p, const Workspace* ws, const DeviceInfo& dev, const void* data, bool vec)
+{
+#define KMX_PLAN(cond) do { if (!(cond)) return fail(KMX_ERR_DEVICE, "assign (split-bf16 MFMA): launch refused, the plan breaks \"%s\" (dim blocks %u, k %u, kp %u, n %u, chunk rows %u, slices %u, LDS %u + %u)", \
+	#cond, p.kb, p.k, p.kp, p.n, p.chunk_rows, p.slices, p.lds_bytes, p.static_bytes); } while (0)
+	const uint32_t tile_words = tile_floats(p.rs);
+	KMX_PLAN(p.kp % TILE == 0 && p.kp >= p.k && p.kp - p.k < TILE);
+	KMX_PLAN(p.chunk_rows > 0 && p.chunk_rows % TILE == 0 && p.chunk_rows <= p.kp);
+	KMX_PLAN(tile_words % 4 == 0 && NORM_TILE % 4 == 0);                                  /* 16-byte copies of tiles and norms */
+	KMX_PLAN(p.grid >= 1 && p.n >= 1);
+	KMX_PLAN((uint64_t)p.lds_bytes + p.static_bytes <= dev.lds_bytes);
+	KMX_PLAN(ws->packed_means && (size_t)(p.kp / TILE) * tile_words <= ws->packed_cap);  /* the last chunk or slice ends with the block */
+	KMX_PLAN(ws->norms && split_norms_floats(p.kp) <= ws->norms_cap);
+	KMX_PLAN(p.packed_form || (p.kb * KBLOCK <= FRAME_DIMS && FRAME_DIMS + 2 <= FRAME_FLOATS)); /* the frame read behind the norms */
+	KMX_PLAN(ws->queue && 2 * (size_t)p.n <= ws->queue_cap && ws->counters);
+	KMX_PLAN(!vec || ((uintptr_t)data & 15) == 0);
+	const uint32_t chunk_tiles = p.chunk_rows / TILE;
+	if (p.slices > 1) {
+		KMX_PLAN(!p.stream_mode && p.slices <= SLICED_MAX_SLICES);
+		KMX_PLAN(ws->carried && 3 * (size_t)p.n <= ws->carried_cap);
+		KMX_PLAN((uint64_t)(p.slices - 1) * p.chunk_rows < p.kp);                         /* the last slice is not empty */
+		KMX_PLAN((uint64_t)chunk_tiles * (tile_words + NORM_TILE) * 4 <= p.lds_bytes);
+	}
+	else if (!p.stream_mode) {
+		KMX_PLAN(p.chunk_rows == p.kp);
+		KMX_PLAN((uint64_t)chunk_tiles * (tile_words + NORM_TILE) * 4 <= p.lds_bytes);
+	}
+	else {
+		KMX_PLAN((uint64_t)2 * chunk_tiles * (tile_words + NORM_TILE) * 4 <= p.lds_bytes); /* two buffers */
+		KMX_PLAN(chunk_tiles * NORM_TILE / 4 <= MFMA_WAVES * WAVE);                        /* one 16-byte piece of norms per lane */
+		if (!p.wide)
+			KMX_PLAN((uint64_t)chunk_tiles * tile_words / 4 <= (uint64_t)STAGE_VECS * MFMA_WAVES * WAVE); /* a chunk staged in registers */
+		/* every chunk, the short last one too: whole tiles inside the block */
+		for (uint32_t row0 = 0; row0 < p.kp; row0 += p.chunk_rows) {
+			const uint32_t rows = std::min(p.chunk_rows, p.kp - row0);
+			KMX_PLAN(rows % TILE == 0 && packed_row(row0, p.rs) + (size_t)(rows / TILE) * tile_words <= ws->packed_cap);
+			KMX_PLAN((size_t)(row0 / TILE + rows / TILE) * NORM_TILE <= split_norms_offset(p.kp));
+		}
+	}
+#undef KMX_PLAN
+	return KMX_OK;
+}
+
 /* point tiles per wavefront and sweep, and whether the next sweep's points are prefetched: bounded by the register file */
 template <int KB> struct SplitSweepShape {
 	static constexpr int P = KB <= 8 ? 2 : 1; /* (rows of 65 to 128 dimensions: 128 registers of split operands; measured 6 % faster than one tile, whose centroid operands serve half the MFMAs) */
@@ -1551,7 +1610,7 @@ static int launch_bf16_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 	constexpr int PR = (!PACKED && KB == 2 && KMX_SNAPSHOT_FROM_KB > 2) ? 3 : P; /* a third point tile fits where the tracking keeps no snapshot */
 	constexpr bool PF = SplitSweepShape<KB>::PREFETCH;
 	uint32_t budget = exec->shared_mem_bytes ? std::min(exec->shared_mem_bytes, dev.lds_bytes) : dev.lds_bytes;
-	const uint32_t static_bytes = (2 * FLAG_CAP * MFMA_WAVES + 64) * 4;
+	const uint32_t static_bytes = sweep_static_lds_bytes<KB, PACKED>();
 	const uint32_t tile_bytes = (tile_floats(RS) + NORM_TILE) * 4;
 	if (budget < static_bytes + tile_bytes) return fail(KMX_ERR_UNSUPPORTED, "assign (split-bf16 MFMA): LDS budget of %u bytes is too small", budget);
 	/* everything resident if it fits (rows up to 64 dimensions only: the wider kernels always stream); otherwise two
@@ -1621,8 +1680,13 @@ static int launch_bf16_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 	const uint32_t grid = std::min(units, dev.compute_units * (uint32_t)per_cu);
 	exec->block_count = grid;
 	const float kd_unmoved = a.unmoved_thresholds ? cert_kd_unmoved(a.dim) : 0.0f;
-	int rc = profile_begin(0);
-	if (rc) return rc;
+	int rc = KMX_OK;
+	if (!sizing_only()) {
+		const SweepPlan plan = { (uint32_t)KB, RS, kp, a.k, a.n, chunk_rows, slices, lds_bytes, static_bytes, grid, stream_mode, PACKED, wide_rows_sweep<KB>() };
+		if ((rc = check_sweep_plan(plan, ws, dev, a.data, VEC))) return rc;
+		if (slices > 1 ? !sliced_kernel : !kernel) return fail(KMX_ERR_DEVICE, "assign (split-bf16 MFMA): no kernel instance for this plan");
+	}
+	if ((rc = profile_begin(0))) return rc;
 	if (slices == 1) {
 		KMX_LAUNCH_KERNEL(kernel, dim3(grid), dim3(MFMA_WAVES * WAVE), lds_bytes, stream(),
 		                   a.data, a.stride, ws->packed_means, ws->norms, a.assignment, ws->queue, ws->counters,
@@ -1634,6 +1698,7 @@ static int launch_bf16_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 			const uint32_t row0 = s * chunk_rows;
 			const uint32_t rows = std::min(chunk_rows, kp - row0);
 			const CentroidSlice slice = { ws->norms, ws->carried, a.k, kp, row0, (s > 0 ? CARRY_IN : 0u) | (s + 1 < slices ? CARRY_OUT : 0u) };
+			if (row0 >= kp || rows == 0 || rows % TILE != 0) return fail(KMX_ERR_DEVICE, "assign (split-bf16 MFMA): slice %u of %u is empty or ragged", s, slices);
 			/* (the kernel's view: `rows` resident centroids, all of them one chunk) */
 			KMX_LAUNCH_KERNEL(sliced_kernel, dim3(grid), dim3(MFMA_WAVES * WAVE), lds_bytes, stream(),
 			                   a.data, a.stride, ws->packed_means + packed_row(row0, RS), ws->norms + (size_t)(row0 / TILE) * NORM_TILE,

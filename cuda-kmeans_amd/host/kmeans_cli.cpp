@@ -25,6 +25,7 @@
 #include <cstdint>
 #include <iostream>
 #include <map>
+#include <vector>
 #include <memory>
 #include <string>
 
@@ -74,6 +75,32 @@ void getHipExecParameters(const ProgramArguments& args, HipExecParameters& exec)
 	exec.regsCache = (std::uint32_t)args.getInt("regsCache");
 }
 
+/*
+ * The reference's launch parameters (k-means.cpp:318-326) shape the launches of the kernels that have that freedom:
+ * hip_base (one lane per point) and the global-atomic update behind it. The tuned kernels fix their own work-group
+ * shape (8 wavefronts around the LDS-resident centroids, 16 around a sorted chunk, the MFMA tile as register tile), so
+ * a value given for one of these options changes nothing there: say so instead of leaving a parameter sweep to wonder
+ * why its times do not move.
+ */
+void warnIgnoredLaunchParameters(const ProgramArguments& args, const std::string& algoName)
+{
+	static const std::map<std::string, std::vector<const char*>> ignored = {
+		{ "hip_base", { "regsCache" } },
+		{ "hip_base_shm", { "regsCache", "privatizedCopies" } },
+		{ "hip_lds_fma", { "cudaBlockSize", "itemsPerThread", "regsCache", "privatizedCopies" } },
+		{ "hip_mfma", { "cudaBlockSize", "itemsPerThread", "regsCache", "privatizedCopies" } },
+		{ "hip_mfma_bf16", { "cudaBlockSize", "itemsPerThread", "regsCache", "privatizedCopies" } },
+		{ "hip_best", { "cudaBlockSize", "itemsPerThread", "regsCache", "privatizedCopies" } },
+		{ "hip_best_serial_order", { "cudaBlockSize", "itemsPerThread", "regsCache", "privatizedCopies" } },
+		{ "hip_fused", { "cudaBlockSize", "itemsPerThread", "regsCache", "privatizedCopies" } },
+	};
+	auto it = ignored.find(algoName);
+	if (it == ignored.end()) return;
+	for (const char* name : it->second)
+		if (args.isPresent(name))
+			std::cerr << "Warning: --" << name << " is ignored by " << algoName << " (its kernels fix their own launch shape)." << std::endl;
+}
+
 /* capability checks of the reference's getCudaExecParameters (k-means.cpp:27-41), once a device algorithm is chosen */
 void checkDevice(const HipExecParameters& exec)
 {
@@ -111,6 +138,7 @@ void run_assignment(const ProgramArguments& args, std::vector<F>& data, std::vec
 
 	auto it = algorithms.find(algoName);
 	if (it == algorithms.end()) throw std::runtime_error("Unkown algorithm '" + algoName + "'.");
+	warnIgnoredLaunchParameters(args, algoName);
 	if (algoName != "serial") checkDevice(exec);
 	std::cerr << "Selected assignment-only algorithm: " << algoName << std::endl;
 	auto algorithm = std::move(it->second);
@@ -180,6 +208,7 @@ void run_kmeans(const ProgramArguments& args, std::vector<F>& data, std::vector<
 
 	auto it = algorithms.find(algoName);
 	if (it == algorithms.end()) throw std::runtime_error("Unkown algorithm '" + algoName + "'.");
+	warnIgnoredLaunchParameters(args, algoName);
 	if (algoName != "serial") checkDevice(exec);
 	std::cerr << "Selected k-means algorithm: " << algoName << std::endl;
 	auto algorithm = std::move(it->second);
@@ -325,7 +354,7 @@ int main(int argc, char* argv[])
 		args.registerBool("verify", "Verify results against base (serial) algorithm.");
 		args.registerInt("privatizedCopies", "Number of privatized copies in global memory (relevant only to some algorithms).", 1, 1, 4096);
 		args.registerInt("itemsPerThread", "Number of computations performed per thread.", 1, 1, 4096);
-		args.registerInt("regsCache", "Size of the registry cache (kept for compatibility; unused).", 1, 1);
+		args.registerInt("regsCache", "Size of the registry cache (accepted for compatibility; no kernel of this build reads it, a warning says so).", 1, 1);
 		args.registerInt("cudaBlockSize", "Number of threads in each block.", 256, 1, 4096);
 		args.alias("hipBlockSize", "cudaBlockSize");
 		args.registerInt("cudaBlockCount", "Number of blocks executed in a grid (algorithms choose their own).", 0, 0);

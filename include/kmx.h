@@ -346,6 +346,18 @@ int kmx_certificate_tau(int form, uint32_t dim, float x2, float xpart2, float c2
 int kmx_certificate_unmoved_threshold(uint32_t dim, float first, float tau, float x2, float along, float c2max, float m2, float mnorm,
                                       float* threshold);
 
+/*
+ * What the matrix cores do with a chain of accumulations (no counterpart in the reference; a diagnostic the tests use to
+ * hold the hardware to the assumption the certificates make about it: at most one 2^-23 of the running magnitude per
+ * accumulated product, however the instruction rounds or truncates inside). One wavefront computes
+ *      d[i][j] = c[i][j] + sum_q a[i][q] b[j][q],   i, j < 32,  q < depth,
+ * block by block in ascending q, one instruction per block, with the instructions, operand layout and order of the
+ * sweeps: kind 0 = v_mfma_f32_32x32x2_f32 (depth = 2 blocks), kind 1 = v_mfma_f32_32x32x16_bf16 (depth = 16 blocks; the
+ * values of a and b must be exactly representable in bf16, the low 16 bits of their words are dropped).
+ * a: 32 x depth row-major; b: 32 x depth, the depth values of column j contiguous; c, d: 32 x 32 row-major. Device pointers.
+ */
+int kmx_probe_matrix_chain(int kind, const float* a, const float* b, const float* c, float* d, uint32_t blocks);
+
 /* Message of the last failed call on this thread ("" if none). */
 const char* kmx_last_error(void);
 

@@ -350,3 +350,80 @@ def test_threshold_taken_back_to_the_frame_of_the_data(km, dim, offset):
     assert worst_low >= 0.0, "threshold below the centroid's own value by %.3g S" % -worst_low
     # Q, the bound of |x|^2 + max |c|^2 that the threshold uses, exceeds S by at most the triangle inequality's factor of 4
     assert worst_high <= 4.0 * 2.0 * allowance, "threshold %.3g S above the value: more than twice the allowance" % worst_high
+
+
+# ---------------------------------------------------------------- the accumulation inside the matrix cores
+#
+# The certificates allow one u' = 2^-23 of the running magnitude per accumulated product "for any rounding or truncation
+# inside the matrix core" (csrc/certificate.h). The running magnitude is bounded by M = |c| + sum_q |a_q b_q| (which
+# |c_j|^2 + 2 |c_j||x| of the derivation bounds in turn, by Cauchy-Schwarz), so the assumption reads
+#       |d - (c + sum_q a_q b_q)|  <=  steps * u' * M        for a chain of `steps` products.
+# The operand sets below are chosen so that an accumulator that merely truncates after every product -- the worst the
+# assumption admits -- uses most of that allowance: they fail a bound of half a u' per step under that model (shown here, on
+# the CPU), and tests/test_gpu_certificate.py holds the hardware's own results on the same operands to the full bound.
+
+def accumulation_cases(kind):
+    """Operand sets for kmx_probe_matrix_chain: name -> (a[32, depth], b[32, depth], c[32, 32]) in float32.
+    kind 1: a and b hold bf16 values (products exact in fp32); kind 0: full fp32 mantissas."""
+    rng = np.random.default_rng(1234 + kind)
+    block = 2 if kind == 0 else 16
+    quant = (lambda v: np.asarray(v, np.float32)) if kind == 0 else bf16_round
+    cases = {}
+
+    def mant(shape):   # mantissas in [1, 2) with all their bits in use
+        return 1.0 + rng.integers(0, 1 << 23, size=shape) * 2.0 ** -23
+
+    for blocks in (1, 3, 12, 48):
+        depth = blocks * block
+        # products of very different exponents inside one block: 2^0 ... 2^-20
+        ea, eb = rng.integers(0, 11, size=(32, depth)), rng.integers(0, 11, size=(32, depth))
+        a = quant(mant((32, depth)) * 2.0 ** -ea * rng.choice([-1.0, 1.0], size=(32, depth)))
+        b = quant(mant((32, depth)) * 2.0 ** -eb * rng.choice([-1.0, 1.0], size=(32, depth)))
+        cases["wide_exponents_%d" % blocks] = (a, b, (rng.normal(size=(32, 32)) * 0.5).astype(np.float32))
+        # cancelling pairs next to a small term: +A, -A, +eps, ... ; the accumulator starts small as well
+        a = quant(mant((32, depth)))
+        b = quant(mant((32, depth)))
+        a[:, 1::2] = -a[:, 0::2][:, : a[:, 1::2].shape[1]]
+        b[:, 1::2] = b[:, 0::2][:, : b[:, 1::2].shape[1]]
+        last = depth - 1 if depth % 2 else depth - 2
+        a[:, last:] = quant(mant((32, depth - last)) * 2.0 ** -20)        # the terms that must survive the cancellation
+        b[:, last:] = quant(mant((32, depth - last)))
+        cases["cancelling_pairs_%d" % blocks] = (a, b, (rng.normal(size=(32, 32)) * 2.0 ** -18).astype(np.float32))
+        # a large accumulator and products just below its unit in the last place, all of one sign: what truncation loses most of
+        c = ((1.0 + rng.integers(0, 1 << 22, size=(32, 32)) * 2.0 ** -23) * 1024.0).astype(np.float32)   # ulp(c) = 2^-13
+        a = quant((1.0 + rng.integers(0, 4, size=(32, depth)) * 2.0 ** -7) * 2.0 ** -7)
+        b = quant(np.full((32, depth), 0.96875 * 2.0 ** -6))             # a_q b_q in (0.96, 0.995) ulp(c)
+        cases["small_addends_%d" % blocks] = (a, b, c)
+    return cases
+
+
+def exact_chain(a, b, c):
+    """c + a b^T in float64 (every product of two fp32 values is exact there) and M = |c| + sum_q |a_q b_q|."""
+    a64, b64, c64 = a.astype(np.float64), b.astype(np.float64), c.astype(np.float64)
+    return c64 + a64 @ b64.T, np.abs(c64) + np.abs(a64) @ np.abs(b64).T
+
+
+def chopped_chain(a, b, c):
+    """The worst accumulator the assumption admits: fp32, one product at a time, every sum truncated towards zero."""
+    s = c.astype(np.float32).copy()
+    for q in range(a.shape[1]):
+        v = s.astype(np.float64) + np.outer(a[:, q].astype(np.float64), b[:, q].astype(np.float64))
+        r = v.astype(np.float32)
+        over = np.abs(r.astype(np.float64)) > np.abs(v)
+        r[over] = np.nextafter(r[over], np.float32(0))
+        s = r
+    return s
+
+
+@pytest.mark.parametrize("kind", [0, 1])
+def test_accumulation_cases_use_the_allowance_of_one_unit_per_step(kind):
+    """A truncating accumulator stays within steps * u' * M on every operand set and exceeds half of that on some:
+    the operands have teeth against a bound of half a u' per step."""
+    beyond_half = 0
+    for name, (a, b, c) in accumulation_cases(kind).items():
+        exact, m = exact_chain(a, b, c)
+        err = np.abs(chopped_chain(a, b, c).astype(np.float64) - exact)
+        steps = a.shape[1]
+        assert np.all(err <= steps * U * m), name
+        beyond_half += int((err > 0.5 * steps * U * m).sum())
+    assert beyond_half > 1000, "only %d results of the truncating model exceed half a unit per step" % beyond_half

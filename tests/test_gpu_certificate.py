@@ -10,7 +10,7 @@ scan's index bit for bit where random data never probes the bound.
 import numpy as np
 import pytest
 
-from test_certificate import near_ties, worst_case_inputs
+from test_certificate import U, accumulation_cases, exact_chain, near_ties, worst_case_inputs
 
 pytestmark = pytest.mark.gpu
 
@@ -96,6 +96,47 @@ def test_gap_sweep(km, orc, gpu, dim, offset):
     data = np.empty((n, dim), np.float32)
     for first in range(0, n, chunk):                 # the generator works in float64: in pieces
         data[first:first + chunk], _ = near_ties(dim, chunk, k, rng, offset, centroids=c)
+    means = np.ascontiguousarray(c).ravel()
+    want = orc.assign(data.ravel(), means, dim, k, n, threads=0, fast=True)
+    d = km.DeviceBuffer(data.nbytes); d.write(data.ravel())
+    for v in variants(km, dim):
+        got, rechecked = assign_all(km, d, means, dim, k, n, v)
+        bad = np.nonzero(got != want)[0]
+        assert bad.size == 0, "variant %d: %d of %d points differ (first %s), %d went to the exact pass" % (v, bad.size, n, bad[:5], rechecked)
+    d.free()
+
+
+@pytest.mark.parametrize("kind", [0, 1])
+def test_matrix_core_accumulation_stays_within_one_unit_per_step(km, gpu, kind):
+    """The hardware assumption of the certificates (csrc/certificate.h: one u' of the running magnitude per accumulated
+    product covers whatever the matrix core rounds or truncates), measured: chains of v_mfma_f32_32x32x2_f32 (kind 0) and
+    v_mfma_f32_32x32x16_bf16 (kind 1) on products of exponents 2^0..2^-20 inside a block, cancelling pairs next to a term
+    of 2^-20, a large accumulator with addends below its last place, up to 48 blocks. tests/test_certificate.py shows that
+    an accumulator which truncates after every product fails half of this bound on the same operands."""
+    worst = 0.0
+    for name, (a, b, c) in accumulation_cases(kind).items():
+        d = km.probe_matrix_chain(kind, a, b, c).astype(np.float64)
+        exact, m = exact_chain(a, b, c)
+        steps = a.shape[1]
+        per_step = np.abs(d - exact) / (steps * U * m)
+        assert per_step.max() <= 1.0, "%s: %.3f u' of the running magnitude per step" % (name, float(per_step.max()))
+        worst = max(worst, float(per_step.max()))
+    print("matrix cores, kind %d: at most %.4f u' of the running magnitude per accumulated product" % (kind, worst))
+
+
+@pytest.mark.parametrize("dim", [16, 32, 64, 256])
+def test_gap_sweep_with_coordinates_of_very_different_exponents(km, orc, gpu, dim):
+    """Near-ties (true gaps log-uniform over 1e-9..1e-3 of |ca|^2 + |cb|^2, on both sides of every tau) between centroids
+    whose coordinates span 2^0..2^-10 inside every block of 16 dimensions with alternating signs, so that the products of
+    one matrix-core block span 2^0..2^-20 and partly cancel: every variant must return the serial scan's index."""
+    n, k, chunk = 1 << 18, 128, 1 << 16
+    rng = np.random.default_rng(dim)
+    scale = (2.0 ** -(np.arange(dim) % 11)).astype(np.float32)
+    sign = np.where(np.arange(dim) % 2 == 0, 1.0, -1.0).astype(np.float32)
+    c = ((1.0 + rng.random(size=(k, dim))) * scale * sign * rng.choice([1.0, 1.0, 1.0, -1.0], size=(k, dim))).astype(np.float32)
+    data = np.empty((n, dim), np.float32)
+    for first in range(0, n, chunk):
+        data[first:first + chunk], _ = near_ties(dim, chunk, k, rng, 0.0, centroids=c)
     means = np.ascontiguousarray(c).ravel()
     want = orc.assign(data.ravel(), means, dim, k, n, threads=0, fast=True)
     d = km.DeviceBuffer(data.nbytes); d.write(data.ravel())

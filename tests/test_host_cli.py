@@ -105,6 +105,35 @@ def test_no_device_is_an_error_not_a_fallback(harness, km):
     assert rc == 2 and "No HIP devices found!" in out
 
 
+def test_launch_parameters_that_an_algorithm_ignores_are_named(harness):
+    """--regsCache / --itemsPerThread / --cudaBlockSize (k-means.cpp:318-326) shape the launches of hip_base only; given to
+    a tuned algorithm they change nothing, and the harness says so on stderr (before it looks for a device)."""
+    rc, out, err = run(harness, "--algorithm", "hip_best", "--regsCache", "4", "--itemsPerThread", "2", "--cudaBlockSize", "128")
+    for name in ("regsCache", "itemsPerThread", "cudaBlockSize"):
+        assert "Warning: --%s is ignored by hip_best" % name in err, err
+    rc, out, err = run(harness, "--algorithm", "cuda_cached_regs", "--assignmentOnly", "--regsCache", "4")
+    assert "Warning: --regsCache is ignored by hip_mfma" in err, err
+    rc, out, err = run(harness, "--algorithm", "hip_base", "--itemsPerThread", "2", "--cudaBlockSize", "128", "--regsCache", "2")
+    assert "--itemsPerThread is ignored" not in err and "--cudaBlockSize is ignored" not in err and "--regsCache is ignored by hip_base" in err, err
+    rc, out, err = run(harness, "--algorithm", "hip_best")
+    assert "Warning" not in err, err
+    rc, out, err = run(harness, "--algorithm", "serial", "--regsCache", "4", "--N", "1k", "--k", "8", "--dim", "4")
+    assert rc == 0 and "Warning" not in err, err
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("config,iters,extra", [("1", "10", []), ("2", "5", ["--N", "64k"]), ("5", "6", ["--N", "256k"]), ("3", "4", ["--N", "128k", "--layout", "soa"])])
+def test_serial_order_algorithm_is_bit_identical_to_the_serial_run(harness, gpu, config, iters, extra):
+    """hip_best_serial_order: the selector's assignment with the update that adds in the serial order; --verify then finds
+    the whole run (several iterations, free-running) equal to the serial algorithm's bit for bit."""
+    rc, out, err = run(harness, "--config", config, "--algorithm", "hip_best_serial_order", "--iterations", iters, "--verify",
+                       "--serialThreads", "8", "--json", *extra)
+    assert rc == 0, out + err
+    rep = json.loads(out)
+    assert rep["bit_identical"] is True and rep["assignment_mismatches"] == 0 and rep["centroid_error"] == 0.0, rep
+    assert "bit-identical to the serial run" in err
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("algo", ["hip_best", "hip_mfma", "hip_mfma_bf16", "hip_base", "hip_base_shm", "cuda_best", "hip_fused",
                                   "cuda_fused_regs"])
