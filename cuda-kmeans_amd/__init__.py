@@ -36,7 +36,7 @@ ABI_SYMBOLS = [
     "kmx_assign_last_rechecked", "kmx_assign_last_variant", "kmx_update_f32", "kmx_bucket_sum_f32", "kmx_fused_f32", "kmx_assign_f64", "kmx_update_f64", "kmx_fused_f64", "kmx_bucket_sum_f64", "kmx_set_queued_rows_limit",
     "kmx_graph_begin", "kmx_graph_end", "kmx_graph_launch", "kmx_graph_destroy", "kmx_event_create", "kmx_event_destroy", "kmx_event_record",
     "kmx_event_elapsed_ms", "kmx_set_profiling", "kmx_last_kernel_ms", "kmx_last_error", "kmx_certificate_tau", "kmx_certificate_unmoved_threshold",
-    "kmx_update_f32_noalloc", "kmx_reserve_f32", "kmx_prepare_points_f64", "kmx_forget_points_f64", "kmx_probe_matrix_chain",
+    "kmx_update_f32_noalloc", "kmx_reserve_f32", "kmx_prepare_points_f64", "kmx_forget_points_f64", "kmx_probe_matrix_chain", "kmx_set_two_level_sweep",
 ]
 
 
@@ -136,6 +136,7 @@ def hip_lib():
         lib.kmx_set_queued_rows_limit.argtypes = [ctypes.c_size_t]
         lib.kmx_last_kernel_ms.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_float)]
         lib.kmx_probe_matrix_chain.argtypes = [ctypes.c_int, vp, vp, vp, vp, u32]
+        lib.kmx_set_two_level_sweep.argtypes = [ctypes.c_int]
         _hip = lib
     return _hip
 
@@ -420,6 +421,11 @@ def reserve(assign_variant, update_variant, layout, layout_means, dim, k, n):
 def set_queued_rows_limit(nbytes):
     """Bound of the block of copied rows the exact pass keeps for SoA points (kmx_set_queued_rows_limit)."""
     check(hip_lib().kmx_set_queued_rows_limit(ctypes.c_size_t(nbytes)))
+
+
+def set_two_level_sweep(mode):
+    """kmx_set_two_level_sweep: 0 = one level always, 1 = two levels where they pay (default), 2 = wherever the kernels allow."""
+    check(hip_lib().kmx_set_two_level_sweep(mode))
 
 
 def set_profiling(enabled):

@@ -56,7 +56,10 @@ pack_means_bf16_kernel(const float* __restrict__ means, size_t stride_means, flo
 {
 	const uint32_t lane = threadIdx.x & (WAVE - 1);
 	const uint32_t j = (blockIdx.x * blockDim.x + threadIdx.x) / WAVE;
-	if (blockIdx.x == 0 && threadIdx.x == 0) counters[0] = 0u; /* the recheck queue of this call starts empty */
+	if (blockIdx.x == 0 && threadIdx.x == 0) {
+		counters[0] = 0u; /* the recheck queue of this call starts empty */
+		counters[LISTED_COUNTER] = 0u; /* and so does the list of points the first level of a two-level sweep passes on */
+	}
 	/* packed rows: the frame of the sweep, the mean of the first centroids (up to 256 of them, one per lane; the finite
 	 * coordinates; any vector would do, this one is near the middle of the data). Every work-group computes it, in the same order. */
 	__shared__ float frame_parts[4][4];

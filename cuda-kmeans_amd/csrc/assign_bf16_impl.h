@@ -24,6 +24,12 @@ constexpr uint32_t SLICED_MAX_SLICES = 8;
  * two slices, 0.422 ms streamed; k = 2048: the same; k = 4096: 1.50 against 1.45 ms), and SoA points cost more to read
  * twice than the slices save (d = 56, k = 1024: 0.434 against 0.380 ms) */
 constexpr uint32_t SLICED_MAX_SLICES_WIDE = 2;
+/* The two-level sweep (LevelOne / ListedPoints below) pays when the first level settles most points and the sweep, not
+ * the launches, is what the call costs. */
+#ifndef KMX_TWO_LEVEL_MIN_POINTS
+#define KMX_TWO_LEVEL_MIN_POINTS (1u << 18)
+#endif
+constexpr uint32_t TWO_LEVEL_MIN_TILES = 4; /* centroid tiles (from 97 centroids on) */
 constexpr int STAGE_VECS = 9;   /* 16-byte pieces of a streamed chunk per lane: a chunk holds at most 9 * 512 * 16 bytes of tiles */
 
 /* Floats per packed centroid row. The PACKED form (rows of at most 4 dimensions) has 16 slots = 8 floats per row and no
@@ -128,14 +134,18 @@ __device__ __forceinline__ void load_packed_points(SplitPoints<1> (&b)[P], float
 	convert_packed_points<P>(b, xx, raw, h, frame);
 }
 
-template <int KB, int P, int LD, bool VEC>
+/* LISTED: the sweep covers the points of a list (entries of two words, the first one the point number); position
+ * base + p TILE + col of the list stands where the point number itself stands otherwise, n is the length of the list */
+template <int KB, int P, int LD, bool VEC, bool LISTED = false>
 __device__ __forceinline__ void request_split_points(RawPoints<KB, false> (&raw)[P], const float* __restrict__ data, size_t stride,
-                                                     uint32_t base, uint32_t col, uint32_t h, uint32_t dim, uint32_t n)
+                                                     uint32_t base, uint32_t col, uint32_t h, uint32_t dim, uint32_t n,
+                                                     const uint32_t* __restrict__ list = nullptr)
 {
 #pragma unroll
 	for (int p = 0; p < P; ++p) {
-		const uint32_t pt = base + p * TILE + col;
-		const bool valid = pt < n;
+		const uint32_t slot = base + p * TILE + col;
+		const bool valid = slot < n;
+		const uint32_t pt = LISTED ? (valid ? list[2 * (size_t)slot] : 0u) : slot;
 #pragma unroll
 		for (int kb = 0; kb < KB; ++kb) {
 			const uint32_t d0 = kb * KBLOCK + h * 8;
@@ -170,13 +180,15 @@ __device__ __forceinline__ void request_split_points(RawPoints<KB, false> (&raw)
 /* The rows are swept as x - m (`frame`: the FRAME_DIMS coordinates of m, zero beyond the row; the packing kernel moved the
  * centroids alike). xx = the lane's share of |x - m|^2, xm = its share of (x - m) . m (which takes a threshold back to the
  * frame of the data, see unmoved_threshold). */
-template <int KB, int P>
+/* LEVEL1 (the first level of the two-level sweep, which multiplies the hi parts only): xl = the lane's share of
+ * sum_i (v_i - hi_i)^2, what its certificate needs of the point (the subtraction is exact); the mid parts go unused. */
+template <int KB, int P, bool LEVEL1 = false>
 __device__ __forceinline__ void convert_split_points(SplitPoints<KB> (&b)[P], float (&xx)[P], float (&xm)[P], const RawPoints<KB, false> (&raw)[P],
-                                                     const float* frame, uint32_t h)
+                                                     const float* frame, uint32_t h, float* xl = nullptr)
 {
 #pragma unroll
 	for (int p = 0; p < P; ++p) {
-		float part = 0.0f, along = 0.0f;
+		float part = 0.0f, along = 0.0f, low = 0.0f;
 #pragma unroll
 		for (int kb = 0; kb < KB; ++kb) {
 			const f32x4 m0 = *(const f32x4*)(frame + kb * KBLOCK + h * 8), m1 = *(const f32x4*)(frame + kb * KBLOCK + h * 8 + 4);
@@ -190,10 +202,15 @@ __device__ __forceinline__ void convert_split_points(SplitPoints<KB> (&b)[P], fl
 				split_bf16(v, hi, mid);
 				b[p].hi[kb][j] = hi;
 				b[p].mid[kb][j] = mid;
+				if constexpr (LEVEL1) {
+					const float r = v - (float)hi;
+					low += r * r;
+				}
 			}
 		}
 		xx[p] = part;
 		xm[p] = along;
+		if constexpr (LEVEL1) xl[p] = low;
 	}
 }
 
@@ -423,7 +440,8 @@ template <int KB> struct StepOperands {
 	bf16x8 chi[KB], cmid[KB];
 };
 
-template <int KB>
+/* HI_ONLY: the first level of the two-level sweep multiplies the hi parts only and leaves the mid parts in LDS */
+template <int KB, bool HI_ONLY = false>
 __device__ __forceinline__ void fetch_operands(StepOperands<KB>& o, const float* __restrict__ lds_tiles, uint32_t tile, uint32_t col, uint32_t h)
 {
 	constexpr uint32_t RS = row_floats<KB, false>();
@@ -431,7 +449,7 @@ __device__ __forceinline__ void fetch_operands(StepOperands<KB>& o, const float*
 #pragma unroll
 	for (int kb = 0; kb < KB; ++kb) {
 		o.chi[kb] = row_unit(arow, 4 * kb + 2 * h);
-		o.cmid[kb] = row_unit(arow, 4 * kb + 2 * h + 1);
+		if constexpr (!HI_ONLY) o.cmid[kb] = row_unit(arow, 4 * kb + 2 * h + 1);
 	}
 }
 
@@ -447,9 +465,17 @@ __device__ __forceinline__ void fetch_norms(f32x16& c, const float* __restrict__
 
 /* The MFMAs of one centroid tile for P point tiles: per block of 16 dimensions hi*mid, mid*hi, hi*hi (small terms
  * first). On entry acc[0] holds the tile's norms: they start every accumulator (acc[0] itself last). */
-template <int KB, int P>
+template <int KB, int P, bool HI_ONLY = false>
 __device__ __forceinline__ void mfma_tile(f32x16 (&acc)[P], const StepOperands<KB>& o, const SplitPoints<KB> (&b)[P])
 {
+	if constexpr (HI_ONLY) { /* one product per dimension */
+#pragma unroll
+		for (int kb = 0; kb < KB; ++kb) {
+#pragma unroll
+			for (int p = P - 1; p >= 0; --p) acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(o.chi[kb], b[p].hi[kb], kb == 0 ? acc[0] : acc[p], 0, 0, 0);
+		}
+		return;
+	}
 #pragma unroll
 	for (int p = P - 1; p >= 0; --p) acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(o.chi[0], b[p].mid[0], acc[0], 0, 0, 0);
 #pragma unroll
@@ -583,20 +609,50 @@ struct CentroidSlice {
 	uint32_t mode;          /* CARRY_IN: earlier slices have been swept; CARRY_OUT: later ones follow, nothing is decided yet */
 };
 constexpr uint32_t CARRY_IN = 1u, CARRY_OUT = 2u;
+
+/*
+ * The two-level sweep (rows of 17 to 32 dimensions, resident centroids, many points). Level 1 multiplies the hi parts only:
+ * a third of the matrix work, half the operand registers and LDS reads, and a certificate about two hundred times wider
+ * (cert_coeffs_level1), which still settles the points whose two nearest centroids are far apart -- 86 % at the headline
+ * configuration. The points it cannot settle go to a list (`queue` and `counters` of that launch are the list and its
+ * length), and level 2, the three-product sweep, covers the points of that list instead of all points; what level 2
+ * cannot settle goes to the exact pass as before. A point's result does not depend on the level that settles it: every
+ * level writes the serial scan's index or passes the point on.
+ */
+struct LevelOne {
+	uint32_t unused;
+};
+struct ListedPoints {
+	const uint32_t* list;    /* entries of two words, the first one the point number */
+	const uint32_t* length;  /* entries in the list (written by the launch of level 1) */
+};
+template <class T, class... Extra> constexpr bool extra_is() { return sizeof...(Extra) == 1 && (std::is_same<T, Extra>::value || ...); }
 __device__ __forceinline__ CentroidSlice slice_of() { return CentroidSlice{ nullptr, nullptr, 0u, 0u, 0u, 0u }; }
 __device__ __forceinline__ CentroidSlice slice_of(const CentroidSlice& s) { return s; }
+__device__ __forceinline__ CentroidSlice slice_of(const LevelOne&) { return slice_of(); }
+__device__ __forceinline__ CentroidSlice slice_of(const ListedPoints&) { return slice_of(); }
+__device__ __forceinline__ ListedPoints listed_of() { return ListedPoints{ nullptr, nullptr }; }
+__device__ __forceinline__ ListedPoints listed_of(const ListedPoints& l) { return l; }
+template <class T> __device__ __forceinline__ ListedPoints listed_of(const T&) { return listed_of(); }
 
-/* (Slice: nothing, or CentroidSlice for the instances that sweep slices; the others are compiled without any of it) */
+/* (Slice: nothing; CentroidSlice for the instances that sweep slices; LevelOne / ListedPoints for the two levels of the
+ * two-level sweep; the others are compiled without any of it) */
 template <int KB, int P, int LD, bool VEC, bool STREAM, bool COARSE, bool PREFETCH, bool PACKED = false, class... Slice>
 __global__ void __launch_bounds__(MFMA_WAVES * WAVE)
 assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* __restrict__ packed, const float* __restrict__ norms,
                    uint32_t* __restrict__ assignment, uint32_t* __restrict__ queue, uint32_t* __restrict__ counters,
-                   uint32_t dim, uint32_t k, uint32_t kp, uint32_t n, uint32_t chunk_rows, float kd, float neg_inf, uint32_t shifted_cap,
+                   uint32_t dim, uint32_t k, uint32_t kp, uint32_t n_given, uint32_t chunk_rows, float kd, float neg_inf, uint32_t shifted_cap,
                    float kd_unmoved, Slice... slice_argument)
 {
 	static_assert(sizeof...(Slice) <= 1, "at most one slice");
-	constexpr bool SLICED = sizeof...(Slice) == 1;
+	constexpr bool SLICED = extra_is<CentroidSlice, Slice...>();
+	constexpr bool LEVEL1 = extra_is<LevelOne, Slice...>();
+	constexpr bool LISTED = extra_is<ListedPoints, Slice...>();
+	static_assert(!(LEVEL1 || LISTED) || (COARSE && !PACKED && !STREAM && KB <= 3 && PREFETCH), "the two-level sweep is built on the pipelined step with prefetched points");
 	[[maybe_unused]] const CentroidSlice slice = slice_of(slice_argument...);
+	[[maybe_unused]] const ListedPoints listed = listed_of(slice_argument...);
+	/* LISTED: the points of the list (never more than the caller's n) */
+	const uint32_t n = LISTED ? min(listed.length[0], n_given) : n_given;
 	const float* __restrict__ all_norms = SLICED ? slice.all_norms : norms;
 	const uint32_t all_k = SLICED ? slice.all_k : k, all_kp = SLICED ? slice.all_kp : kp;
 	constexpr uint32_t RS = row_floats<KB, PACKED>();
@@ -644,7 +700,7 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 			for (uint32_t w = 0; w < MFMA_WAVES; ++w) cmax[q] = max(cmax[q], wave_max[q][w]);
 		}
 		const CentroidBounds cb{ __uint_as_float(cmax[0]), __uint_as_float(cmax[1]), __uint_as_float(cmax[2]) };
-		cert = PACKED ? cert_coeffs_packed(cb) : cert_coeffs_split(cb);
+		cert = PACKED ? cert_coeffs_packed(cb) : LEVEL1 ? cert_coeffs_level1(cb) : cert_coeffs_split(cb);
 		/* the same in every lane of the work-group: kept in scalar registers */
 		cert.c2max = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(cert.c2max)));
 		cert.a = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(cert.a)));
@@ -828,7 +884,7 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 		}
 	};
 
-	auto sweep = [&](const SplitPoints<KB> (&b)[P], const float (&xx)[P], const float (&xalong)[P], uint32_t base) {
+	auto sweep = [&](const SplitPoints<KB> (&b)[P], const float (&xx)[P], const float (&xalong)[P], uint32_t base, [[maybe_unused]] const float* xlow = nullptr) {
 		float x2[P], along_m[P];
 		Track st[P];
 #pragma unroll
@@ -872,7 +928,7 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 				const float* lds_norms = lds_tiles + (size_t)chunk_tiles * tile_floats(RS);
 				const uint32_t tiles = rows / TILE;
 				const uint32_t tile0 = row0 / TILE;
-				constexpr int MFMAS = 3 * KB * P;
+				constexpr int MFMAS = (LEVEL1 ? 1 : 3) * KB * P;
 				/* Tracking comes in pieces that are issued one behind each MFMA, so that a wavefront is back with its next MFMA before
 				 * the matrix pipe has finished the last one. With the snapshot a point tile costs 20 operations (SNAP_OPS), spread
 				 * evenly over its share of the step's MFMAs; without it, two pieces of 11 operations. */
@@ -890,7 +946,7 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 				 * acc_old[0] has been tracked: the remaining MFMAs give its answer time to arrive. */
 				auto step = [&](StepOperands<KB>& fetch_into, uint32_t t_new, f32x16 (&acc_new)[P], const StepOperands<KB>& use,
 				                f32x16 (&acc_old)[P], uint32_t tile_old) {
-					fetch_operands<KB>(fetch_into, lds_tiles, min(t_new + 1, tiles - 1), col, h);
+					fetch_operands<KB, LEVEL1>(fetch_into, lds_tiles, min(t_new + 1, tiles - 1), col, h);
 					__builtin_amdgcn_sched_barrier(0);
 					bool better[P][2];
 					float lowest_of_tile[P];
@@ -938,6 +994,17 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 							__builtin_amdgcn_sched_barrier(0);
 						}
 					};
+					if constexpr (LEVEL1) {
+#pragma unroll
+						for (int kb = 0; kb < KB; ++kb) {
+#pragma unroll
+							for (int p = P - 1; p >= 0; --p) {
+								acc_new[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(use.chi[kb], b[p].hi[kb], kb == 0 ? acc_new[0] : acc_new[p], 0, 0, 0);
+								after_mfma(issued++);
+							}
+						}
+					}
+					else {
 #pragma unroll
 					for (int p = P - 1; p >= 0; --p) {
 						acc_new[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(use.chi[0], b[p].mid[0], acc_new[0], 0, 0, 0);
@@ -963,13 +1030,14 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 							after_mfma(issued++);
 						}
 					}
+					}
 				};
 				StepOperands<KB> o0, o1;
-				fetch_operands<KB>(o0, lds_tiles, 0, col, h);
+				fetch_operands<KB, LEVEL1>(o0, lds_tiles, 0, col, h);
 				fetch_norms(acc0[0], lds_norms, 0, h);
-				fetch_operands<KB>(o1, lds_tiles, min(1u, tiles - 1), col, h);
+				fetch_operands<KB, LEVEL1>(o1, lds_tiles, min(1u, tiles - 1), col, h);
 				fetch_norms(acc1[0], lds_norms, min(1u, tiles - 1), h);
-				mfma_tile<KB, P>(acc0, o0, b);
+				mfma_tile<KB, P, LEVEL1>(acc0, o0, b);
 				uint32_t t = 0; /* acc0 holds tile t, not yet tracked; o1 and acc1[0] hold the centroid parts and norms of tile t + 1 */
 				while (t + 2 < tiles) {
 					step(o0, t + 1, acc1, o1, acc0, tile0 + t);
@@ -981,7 +1049,7 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 					else track_tile<true, true>(acc, st[p], tile, neg_inf);
 				};
 				if (t + 1 < tiles) {
-					mfma_tile<KB, P>(acc1, o1, b);
+					mfma_tile<KB, P, LEVEL1>(acc1, o1, b);
 #pragma unroll
 					for (int p = 0; p < P; ++p) track(acc0[p], p, tile0 + t);
 #pragma unroll
@@ -1180,6 +1248,10 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 				xsq = h == 0 ? x2[p] : other;
 				tau = cert_tau(kd, xsq, h == 0 ? other : x2[p], cert);
 			}
+			else if constexpr (LEVEL1) {
+				xsq = x2[p];
+				tau = cert_tau(kd, xsq, xlow[p] + __shfl_xor(xlow[p], 32), cert);
+			}
 			else {
 				float xmid2 = 0.0f;
 #pragma unroll
@@ -1193,8 +1265,9 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 				tau = cert_tau(kd, xsq, xmid2, cert);
 			}
 			const float along = along_m[p];
-			const uint32_t pt = base + p * TILE + col;
-			const bool mine = h == 0 && pt < n;
+			const uint32_t slot = base + p * TILE + col;
+			const bool mine = h == 0 && slot < n;
+			const uint32_t pt = LISTED ? (mine ? listed.list[2 * (size_t)slot] : 0u) : slot;
 			if constexpr (SLICED) {
 			idx += slice.row_base;
 			if (slice.mode & CARRY_IN) {
@@ -1279,15 +1352,16 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 		float xx0[P], xm0[P];
 		auto request_points = [&](uint32_t first) {
 			if constexpr (PACKED) request_packed_points<P, LD, VEC>(raw, data, stride, first, col, dim, n);
-			else request_split_points<KB, P, LD, VEC>(raw, data, stride, first, col, h, dim, n);
+			else request_split_points<KB, P, LD, VEC, LISTED>(raw, data, stride, first, col, h, dim, n, listed.list);
 		};
+		[[maybe_unused]] float xl0[P];
 		auto convert_points = [&]() {
 			if constexpr (PACKED) {
 				convert_packed_points<P>(b0, xx0, raw, h, frame);
 #pragma unroll
 				for (int p = 0; p < P; ++p) xm0[p] = 0.0f;
 			}
-			else convert_split_points<KB, P>(b0, xx0, xm0, raw, frame_lds, h);
+			else convert_split_points<KB, P, LEVEL1>(b0, xx0, xm0, raw, frame_lds, h, xl0);
 		};
 		uint32_t item = uniform(claim());
 		uint32_t next = uniform(claim());
@@ -1298,7 +1372,8 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 		while (item < items) {
 			const uint32_t after = claim();
 			if (next < items) request_points(first_point(next));
-			sweep(b0, xx0, xm0, first_point(item));
+			if constexpr (LEVEL1) sweep(b0, xx0, xm0, first_point(item), xl0);
+			else sweep(b0, xx0, xm0, first_point(item));
 			item = next;
 			next = uniform(after);
 			if (item < items) convert_points();
@@ -1672,6 +1747,24 @@ static int launch_bf16_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 	else {
 		kernel = assign_bf16_kernel<KB, P, LD, VEC, true, false, PF>;
 	}
+	/* two levels: hi * hi for everybody, then the three products for the points that level could not settle */
+	constexpr bool TWO_LEVEL_BUILT = KB == 2 && !PACKED && PF;
+	[[maybe_unused]] void (*level1_kernel)(const float*, size_t, const float*, const float*, uint32_t*, uint32_t*, uint32_t*,
+	                                      uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, float, float, uint32_t, float, LevelOne) = nullptr;
+	[[maybe_unused]] void (*level2_kernel)(const float*, size_t, const float*, const float*, uint32_t*, uint32_t*, uint32_t*,
+	                                      uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, float, float, uint32_t, float, ListedPoints) = nullptr;
+	bool two_level = false;
+	if constexpr (TWO_LEVEL_BUILT) {
+		const int mode = two_level_mode(); /* kmx_set_two_level_sweep: 0 never, 1 where it pays, 2 wherever the kernels allow it */
+		two_level = !stream_mode && slices == 1 && coarse && a.two_level && mode != 0 &&
+		            (mode == 2 || (swept_tiles >= TWO_LEVEL_MIN_TILES && a.n >= KMX_TWO_LEVEL_MIN_POINTS));
+		level1_kernel = assign_bf16_kernel<KB, PR, LD, VEC, false, true, PF, PACKED, LevelOne>;
+		level2_kernel = assign_bf16_kernel<KB, PR, LD, VEC, false, true, PF, PACKED, ListedPoints>;
+	}
+	if (two_level) {
+		int rc = reserve_listed(ws, 2 * (size_t)a.n);
+		if (rc) return rc;
+	}
 	const void* launched = slices > 1 ? (const void*)sliced_kernel : (const void*)kernel;
 	KMX_HIP(hipFuncSetAttribute(launched, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
 	int per_cu = 1;
@@ -1687,7 +1780,26 @@ static int launch_bf16_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 		if (slices > 1 ? !sliced_kernel : !kernel) return fail(KMX_ERR_DEVICE, "assign (split-bf16 MFMA): no kernel instance for this plan");
 	}
 	if ((rc = profile_begin(0))) return rc;
-	if (slices == 1) {
+	if (two_level) {
+		if constexpr (TWO_LEVEL_BUILT) {
+			if (!sizing_only() && (!ws->listed || ws->listed_cap < 2 * (size_t)a.n)) return fail(KMX_ERR_DEVICE, "assign (split-bf16 MFMA): no list for the two levels");
+			KMX_HIP(hipFuncSetAttribute((const void*)level1_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+			KMX_HIP(hipFuncSetAttribute((const void*)level2_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+			/* level 1: its "queue" is the list, its counter the list's length; thresholds mean nothing there */
+			const float kd1 = kd - cert_kd_split(a.dim) + cert_kd_level1(a.dim);
+			KMX_LAUNCH_KERNEL(level1_kernel, dim3(grid), dim3(MFMA_WAVES * WAVE), lds_bytes, stream(),
+			                   a.data, a.stride, ws->packed_means, ws->norms, a.assignment, ws->listed, ws->counters + LISTED_COUNTER,
+			                   a.dim, a.k, kp, a.n, chunk_rows, kd1, -__builtin_inff(), 0xFFFFFFFFu, 0.0f, LevelOne{ 0u });
+			KMX_LAUNCH_CHECK("assign_bf16_kernel (first level)");
+			/* level 2: the listed points only; as many work-groups as the device runs at once, those without work leave */
+			const ListedPoints listed = { ws->listed, ws->counters + LISTED_COUNTER };
+			KMX_LAUNCH_KERNEL(level2_kernel, dim3(std::min(grid, dev.compute_units * (uint32_t)per_cu)), dim3(MFMA_WAVES * WAVE), lds_bytes, stream(),
+			                   a.data, a.stride, ws->packed_means, ws->norms, a.assignment, ws->queue, ws->counters,
+			                   a.dim, a.k, kp, a.n, chunk_rows, kd, -__builtin_inff(), a.shifted_cap, kd_unmoved, listed);
+			KMX_LAUNCH_CHECK("assign_bf16_kernel (second level)");
+		}
+	}
+	else if (slices == 1) {
 		KMX_LAUNCH_KERNEL(kernel, dim3(grid), dim3(MFMA_WAVES * WAVE), lds_bytes, stream(),
 		                   a.data, a.stride, ws->packed_means, ws->norms, a.assignment, ws->queue, ws->counters,
 		                   a.dim, a.k, kp, a.n, chunk_rows, kd, -__builtin_inff(), a.shifted_cap, kd_unmoved);

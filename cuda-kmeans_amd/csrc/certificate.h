@@ -39,6 +39,13 @@
  *     small for data far from the origin, and the two roundings move a distance by at most 2 u (|x'| + |c'|)^2 <= 2 u' S,
  *     a difference of two distances by 4 u' S: 8 u' more in kd (part of the packed form's kd; the launcher adds it to
  *     the three-product form's when that sweep moves its frame).
+ *   - one-product form (the first level of the two-level sweep: hi*hi only, d products and the norm):
+ *        accumulation <= (d + 2) u' 2 S
+ *        dropped = sum_i c'hi_i (x_i - xhi_i) + (c'_i - c'hi_i) x_i <= |c'hi| |xlo| + |c'lo| |x|
+ *     with xlo = x - xhi, whose norm the lane computes when it splits the point (the subtraction is exact in fp32),
+ *     |c'hi| <= (1 + 2^-8) |c'| and |c'lo| <= |c'mid| + |c'rest| from the packing kernel. The bound is about 2^-8 |c'||x|,
+ *     two hundred times the three-product one: this level settles the points whose two nearest centroids are far apart
+ *     (86 % at the headline configuration) with a third of the matrix work, the others are swept again with three products.
  * tau = kd S + TRUNC_FACTOR * (bound of the dropped products); kd = (12 d + 8 + 2 d + 12 + slack) u' and
  * (16 d + 8 + 2 d + 12 + 8 + slack) u'; TRUNC_FACTOR = 2 plus 1/16 for the fp32 roundings in the norms and square roots.
  * Values the bound does not cover (NaN, infinities, sums that overflow) make tau NaN or infinite, and the
@@ -68,6 +75,7 @@ KMX_HD float cert_kd_fp32(unsigned dim) { return (8.0f * (float)dim + 24.0f) * C
 KMX_HD float cert_kd_fma(unsigned dim) { return (4.0f * (float)dim + 24.0f) * CERT_UNIT; }
 KMX_HD float cert_kd_split(unsigned dim) { return (14.0f * (float)dim + 28.0f) * CERT_UNIT; }
 KMX_HD float cert_kd_packed(unsigned dim) { return (18.0f * (float)dim + 36.0f) * CERT_UNIT; }
+KMX_HD float cert_kd_level1(unsigned dim) { return (6.0f * (float)dim + 28.0f) * CERT_UNIT; } /* 4 d + 8 accumulation, 2 d + 12 serial margin, slack */
 
 /* The bound in the form the kernels evaluate per point: tau = kd (x2 + c2max) + a sqrt(xpart2) + b sqrt(x2), with
  * xpart2 = sum_i xmid_i^2 (three-product form) or sum_i xrest_i^2 (packed form); a and b depend on the centroids only. */
@@ -80,6 +88,14 @@ KMX_HD CertCoeffs cert_coeffs_split(const CentroidBounds& c)
 	const float cnorm = 2.0f * __builtin_sqrtf(c.c2max); /* |c'| */
 	const float cmid = __builtin_sqrtf(c.mid2max), crest = __builtin_sqrtf(c.rest2max);
 	return CertCoeffs{ c.c2max, CERT_TRUNC_FACTOR * (cmid + (cnorm + crest) * CERT_BF16_UNIT), CERT_TRUNC_FACTOR * crest };
+}
+
+/* one-product form: tau = kd (x2 + c2max) + a sqrt(sum_i (x_i - xhi_i)^2) + b sqrt(x2) */
+KMX_HD CertCoeffs cert_coeffs_level1(const CentroidBounds& c)
+{
+	const float cnorm = 2.0f * __builtin_sqrtf(c.c2max); /* |c'| */
+	const float clo = __builtin_sqrtf(c.mid2max) + __builtin_sqrtf(c.rest2max); /* >= |c' - c'hi| */
+	return CertCoeffs{ c.c2max, CERT_TRUNC_FACTOR * (cnorm * (1.0f + CERT_BF16_UNIT)), CERT_TRUNC_FACTOR * clo };
 }
 
 KMX_HD CertCoeffs cert_coeffs_packed(const CentroidBounds& c)

@@ -43,7 +43,7 @@ int device_info(const DeviceInfo** out);
 /*
  * Work space owned by the library (grown on demand, released by kmx_shutdown):
  *   recheck queue : indices of the points the fast assignment kernels hand to the exact pass
- *   counters      : [0] = queue length of the current call
+ *   counters      : [0] = queue length of the current call, [4] = length of the list between the two levels of a two-level sweep
  *   packed means  : centroids re-laid-out (scaled by -2, padded) for the fast assignment kernels
  *   norms         : |c|^2 per (padded) centroid followed by max_j |c_j|^2
  *   partials      : per-work-group partial sums/counts of the update kernels that need them
@@ -64,6 +64,7 @@ struct Workspace {
 	float* queued_rows = nullptr;         size_t queued_rows_cap = 0;   /* floats */
 	uint32_t* queued_index = nullptr;     size_t queued_index_cap = 0;  /* words: per row 2 (queue) + 2 (assignment or 64-bit key), then the screen's pair counters and pairs */
 	uint32_t* carried = nullptr;          size_t carried_cap = 0;       /* words: per point the leader and the two smallest ranking values over the slices of centroids swept so far */
+	uint32_t* listed = nullptr;           size_t listed_cap = 0;        /* words: two per point the first level of a two-level sweep could not settle (its length: counters[LISTED_COUNTER]) */
 	const float* exact_norms = nullptr; /* |c|^2 of the centroids as given, in the layout of `norms`, for the exact pass of a sweep that moved its frame (points into `norms`; null: `norms` holds them) */
 	bool fixed = false; /* the work space of the entry point that allocates nothing: its buffers never grow, a call that needs more is refused */
 };
@@ -76,6 +77,9 @@ int reserve_bucket_sizes(Workspace* ws, size_t entries);
 int reserve_rows_copy(Workspace* ws, size_t floats);
 int reserve_queued_rows(Workspace* ws, size_t rows, size_t dim, size_t extra_words);
 int reserve_carried(Workspace* ws, size_t words);
+int reserve_listed(Workspace* ws, size_t words);
+int two_level_mode(); /* kmx_set_two_level_sweep */
+constexpr uint32_t LISTED_COUNTER = 4; /* word of Workspace::counters that holds the length of Workspace::listed */
 
 #define KMX_HIP(call)                                                                                         \
 	do {                                                                                                      \
@@ -124,6 +128,9 @@ struct AssignArgs {
 	bool shift_rows = false;
 	uint32_t shifted_cap = 0xFFFFFFFFu;
 	bool unmoved_thresholds = false;
+	/* rows of 17 to 32 dimensions: the sweep may run in two levels (one product per dimension for all points, three for
+	 * those the first level cannot settle); off for measurements of the one-level sweep */
+	bool two_level = true;
 };
 
 struct UpdateArgs {

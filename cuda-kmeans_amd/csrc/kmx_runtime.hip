@@ -140,6 +140,9 @@ int reserve_queued_rows(Workspace* ws, size_t rows, size_t dim, size_t extra_wor
 }
 
 int reserve_carried(Workspace* ws, size_t words) { return grow(&ws->carried, &ws->carried_cap, words); }
+int reserve_listed(Workspace* ws, size_t words) { return grow(&ws->listed, &ws->listed_cap, words); }
+static int g_two_level_mode = 1;
+int two_level_mode() { return g_two_level_mode; }
 
 static int release_workspace()
 {
@@ -155,6 +158,7 @@ static int release_workspace()
 	if (g_ws.queued_rows) KMX_HIP(hipFree(g_ws.queued_rows));
 	if (g_ws.queued_index) KMX_HIP(hipFree(g_ws.queued_index));
 	if (g_ws.carried) KMX_HIP(hipFree(g_ws.carried));
+	if (g_ws.listed) KMX_HIP(hipFree(g_ws.listed));
 	g_ws = Workspace();
 	return release_f64_workspace();
 }
@@ -697,6 +701,7 @@ int kmx_certificate_tau(int form, uint32_t dim, float x2, float xpart2, float c2
 	case 3: *tau = cert_kd_fma(dim) * (x2 + c2max); return KMX_OK;
 	case 1: *tau = cert_tau(cert_kd_split(dim), x2, xpart2, cert_coeffs_split(cb)); return KMX_OK;
 	case 2: *tau = cert_tau(cert_kd_packed(dim), x2, xpart2, cert_coeffs_packed(cb)); return KMX_OK;
+	case 4: *tau = cert_tau(cert_kd_level1(dim), x2, xpart2, cert_coeffs_level1(cb)); return KMX_OK;
 	default: return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_certificate_tau: unknown form %d", form);
 	}
 }
@@ -707,6 +712,14 @@ int kmx_certificate_unmoved_threshold(uint32_t dim, float first, float tau, floa
 	clear_error();
 	if (!threshold) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_certificate_unmoved_threshold: null pointer");
 	*threshold = cert_unmoved_threshold(first, tau, x2, along, c2max, m2, mnorm, cert_kd_unmoved(dim));
+	return KMX_OK;
+}
+
+int kmx_set_two_level_sweep(int mode)
+{
+	clear_error();
+	if (mode < 0 || mode > 2) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_set_two_level_sweep: mode %d (0 = never, 1 = where it pays, 2 = wherever the kernels allow it)", mode);
+	g_two_level_mode = mode;
 	return KMX_OK;
 }
 

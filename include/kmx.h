@@ -321,6 +321,15 @@ int kmx_last_kernel_ms(int which, float* ms);
 int kmx_set_queued_rows_limit(size_t bytes);
 
 /*
+ * The split-bf16 sweep of rows of 17 to 32 dimensions may run in two levels (no counterpart in the reference): one product
+ * per dimension (hi * hi) for all points, a third of the matrix work, with a certificate wide enough for it; then the three
+ * products for the points that level could not settle; then the exact pass as always. The results are the same at every
+ * setting. mode 0: one level always; 1 (default): two levels where they pay (resident centroids, 97 centroids or more,
+ * 2^18 points or more); 2: two levels wherever the kernels allow it (for tests and measurements on small inputs).
+ */
+int kmx_set_two_level_sweep(int mode);
+
+/*
  * The certification bound of the ranking sweeps, evaluated on the host by the very function the kernels use (no
  * counterpart in the reference, whose kernels evaluate every pair directly; no device needed). A sweep decides a point
  * without the serial arithmetic only if its two smallest ranking values differ by more than tau; the tests check tau
@@ -329,6 +338,7 @@ int kmx_set_queued_rows_limit(size_t bytes);
  *   form 3: sweeps on the vector ALU (KMX_ASSIGN_LDS_FMA, the single-pass fused kernel): the same with a smaller kd
  *   form 1: split-bf16 sweep, three products per dimension         xpart2 = sum_i xmid_i^2
  *   form 2: split-bf16 sweep, packed rows (dim <= 4, four products) xpart2 = sum_i xrest_i^2
+ *   form 4: first level of the two-level split-bf16 sweep (one product per dimension, hi * hi) xpart2 = sum_i (x_i - xhi_i)^2
  * x2 = |x|^2, c2max = max_j |c_j|^2, cmid2max / crest2max = max_j of the squared norms of the mid / rest parts of -2 c_j;
  * all of them in the frame the sweep works in: the float sweeps subtract a vector m from points and centroids (the mean
  * of the first 16 centroids; for packed rows, with 128 centroids or more, of the first 256; the single-pass fused kernel

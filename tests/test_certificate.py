@@ -179,6 +179,51 @@ def test_tau_covers_the_split_and_the_serial_margin(km, dim, packed, kind):
     assert not wrong.any(), "%d certified pairs contradict the serial comparison" % int(wrong.sum())
 
 
+@pytest.mark.parametrize("dim", [17, 20, 32])
+@pytest.mark.parametrize("kind", ["adversarial", "pairs", "ties0", "ties100", "ties10000"])
+def test_tau_of_the_first_level_covers_one_product_per_dimension(km, dim, kind):
+    """The first level of the two-level sweep keeps hi * hi only: a1[j] = |c_j|^2 + sum_i c'hi_i xhi_i. Its tau (form 4, with
+    sum_i (x_i - xhi_i)^2 of the point) must cover twice what that drops plus the accumulation allowance of d products
+    plus the serial margin, and every pair it would certify must be a strict win of the serial comparison."""
+    rng = np.random.default_rng(dim * 17)
+    n, k = 4096, 16
+    if kind == "adversarial":
+        x, c = adversarial(dim, n, k, rng)
+    elif kind == "pairs":
+        if dim != 32:
+            pytest.skip("the construction exists for 32 dimensions")
+        x, c = worst_case_inputs(dim, 8192)
+        n = x.shape[0]
+    else:
+        x, c = near_ties(dim, n, k, rng, float(kind[4:]))
+    xh = split(x)[0]
+    cp = (np.float32(-2) * c).astype(np.float32)
+    ch, cm, cr = (p.astype(np.float64) for p in split(cp))
+    c2 = (c.astype(np.float32) ** 2).sum(1, dtype=np.float32).astype(np.float64)
+    a1 = c2[:, None] + ch @ xh.astype(np.float64).T
+    exact = (c.astype(np.float64) ** 2).sum(1)[:, None] + cp.astype(np.float64) @ x.astype(np.float64).T
+    xlo = (x - xh).astype(np.float32)                                   # exact in fp32, as in the kernel
+    x2 = (x.astype(np.float32) ** 2).sum(1, dtype=np.float32)
+    xlo2 = (xlo ** 2).sum(1, dtype=np.float32)
+    c2max, cmid2max, crest2max = float(c2.max()), float((cm ** 2).sum(1).max()), float((cr ** 2).sum(1).max())
+    tau = np.array([km.certificate_tau(4, dim, float(x2[i]), float(xlo2[i]), c2max, cmid2max, crest2max) for i in range(n)], np.float64)
+    s_all = x2.astype(np.float64) + c2max
+    accumulation = (dim + 2) * U * 2 * s_all
+    margin = (2 * dim + 12) * U * s_all
+    dropped = np.abs(a1 - exact).max(0)
+    need = 2 * dropped + 2 * accumulation + margin
+    assert np.all(need <= tau), "tau misses %d of %d points (worst ratio %.3f)" % (int((need > tau).sum()), n, float((need / tau).max()))
+    # the bound is not slack by orders of magnitude either: on the adversarial mantissas it is within 8x of what is dropped
+    if kind == "adversarial":
+        assert float((tau / np.maximum(need, 1e-30)).min()) < 8.0
+    dist = serial_distances(x, c)
+    j1 = a1.argmin(0)
+    certified = (a1 - a1[j1, np.arange(n)][None, :]) + 2 * accumulation[None, :] > tau[None, :]
+    certified[j1, np.arange(n)] = False
+    wrong = certified & ~(dist[j1, np.arange(n)][None, :] < dist)
+    assert not wrong.any(), "%d certified pairs contradict the serial comparison" % int(wrong.sum())
+
+
 @pytest.mark.parametrize("dim", [2, 4, 8, 16, 32, 64])
 @pytest.mark.parametrize("kind", ["adversarial", "ties0", "ties100", "ties10000"])
 def test_tau_of_the_vector_alu_sweeps_covers_a_chain_of_fused_multiply_adds(km, dim, kind):
