@@ -176,6 +176,7 @@ int launch_assign_lds_fma(const AssignArgs& a, kmx_exec_params* exec, Workspace*
 /* update.hip */
 /* the work space of kmx_update_f32_noalloc on the current device: `partials` is the library's static scratch array */
 int noalloc_workspace(Workspace** ws);
+bool recording_graph(); /* between kmx_graph_begin and kmx_graph_end */
 int launch_update(int variant, const UpdateArgs& u, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev);
 int launch_divide_means(const UpdateArgs& u);
 

@@ -31,6 +31,7 @@ static hipStream_t g_capture_stream = nullptr;
 static bool g_capturing = false;
 
 hipStream_t stream() { return g_capturing ? g_capture_stream : g_stream; }
+bool recording_graph() { return g_capturing; }
 
 #define KMX_NOT_WHILE_CAPTURING(name)                                                                          \
 	do {                                                                                                       \
@@ -261,7 +262,10 @@ int kmx_set_device(int device)
 		return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_set_device: the library holds a work space on device %d; call kmx_shutdown() before moving to device %d",
 		            g_dev.device, device);
 	KMX_HIP(hipSetDevice(device));
-	return KMX_OK;
+	/* the address of this device's scratch array of kmx_update_f32_noalloc, now rather than inside its first call (looking
+	 * it up loads the library's code onto the device, which is no work for a call that promises to allocate nothing) */
+	Workspace* scratch = nullptr;
+	return noalloc_workspace(&scratch);
 }
 
 int kmx_device_props(kmx_props* props)
@@ -455,6 +459,10 @@ int kmx_reserve_f32(int assign_variant, int update_variant, int layout, int layo
 		Workspace* ws = nullptr;
 		rc = workspace(&ws);
 		if (rc == KMX_OK) rc = reserve_fused_assignment(ws, n); /* kmx_fused_f32 keeps its assignment vector in the work space */
+	}
+	if (rc == KMX_OK) {
+		Workspace* scratch = nullptr;
+		rc = noalloc_workspace(&scratch); /* kmx_update_f32_noalloc: the address of its scratch array on this device */
 	}
 	g_sizing = false;
 	g_last_assign_variant = last_variant;

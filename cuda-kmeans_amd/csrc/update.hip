@@ -1180,6 +1180,10 @@ int noalloc_workspace(Workspace** ws)
 	if (device < 0 || device >= NOALLOC_MAX_DEVICES) return fail(KMX_ERR_UNSUPPORTED, "kmx_update_f32_noalloc: device %d is beyond the %d devices the library keeps scratch pointers for", device, NOALLOC_MAX_DEVICES);
 	Workspace& w = g_noalloc_ws[device];
 	if (!w.partials) {
+		/* the first look-up on a device loads the library's code and its 64 MiB array there: not under a recording */
+		if (recording_graph())
+			return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_update_f32_noalloc: the first call on a device sets up its scratch array, which cannot happen while a graph "
+			                                      "is recorded: call kmx_set_device, kmx_reserve_f32 or kmx_update_f32_noalloc once before kmx_graph_begin");
 		float* ptr = nullptr;
 		KMX_HIP(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)));
 		if (!ptr) return fail(KMX_ERR_DEVICE, "kmx_update_f32_noalloc: the scratch array has no address on device %d", device);

@@ -189,6 +189,9 @@ int kmx_update_f32(int variant,
  * kmx_update_f32 makes of them and run the element-wise kernels (slower, same results). Per-kernel profiling
  * (kmx_set_profiling) does not cover this call. All calls on one GPU share that GPU's array: calls that overlap in
  * time on one GPU (different streams, different threads) race; calls on the library's one stream do not.
+ * The address of a device's array is looked up once per device: by kmx_set_device, by kmx_reserve_f32, or else by the
+ * first call of this function on the device, which is therefore refused (KMX_ERR_INVALID_ARGUMENT) between kmx_graph_begin
+ * and kmx_graph_end -- make one of those calls before recording.
  */
 #define KMX_UPDATE_NOALLOC_SCRATCH_BYTES (64u << 20)
 int kmx_update_f32_noalloc(int variant,

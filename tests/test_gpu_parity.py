@@ -181,6 +181,9 @@ def test_hard_inputs(km, orc, gpu, dim, k, n):
     (33, 300, 65600, 40000),    # a small LDS budget: many short slices
     (17, 250, 70000, 24000),
     (20, 3000, 70001, 0),
+    (32, 800, 66000, 27700),    # LDS for four tiles: 25 tiles in six slices of four and a last slice of ONE tile under the pipelined step
+    (48, 800, 66000, 35900),    # the same for rows of 33..48 dimensions
+    (24, 130, 66000, 13400),    # LDS for one tile: five slices of one tile each
 ])
 def test_centroids_swept_in_slices(km, orc, gpu, dim, k, n, lds_budget):
     """From 65536 points on, rows of 17 to 64 dimensions whose centroids do not fit the LDS are swept once per slice of

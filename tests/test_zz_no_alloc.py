@@ -55,6 +55,46 @@ def test_noalloc_update_equals_update(km, orc, gpu, dim, k, n1, n2, layout, layo
         d.free(); a.free()
 
 
+def device_memory_in_use():
+    """Bytes of device memory in use, asked of the HIP runtime this process has loaded (hipMemGetInfo)."""
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so")
+    free, total = ctypes.c_size_t(0), ctypes.c_size_t(0)
+    assert hip.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+    return total.value - free.value
+
+
+def test_noalloc_update_allocates_nothing_and_records(km, orc, gpu):
+    """After the device has been set up (kmx_set_device looks up the scratch array), calls of the entry point leave the
+    device's memory in use unchanged -- under a graph recording too, whose replays give the eager call's result."""
+    dim, k, n = 32, 1024, 200000
+    rng = np.random.default_rng(3)
+    pts = rng.normal(size=(n, dim)).astype(np.float32)
+    asg = rng.integers(0, k, size=n).astype(np.uint32)
+    d = km.DeviceBuffer(pts.nbytes); d.write(pts.ravel())
+    a = km.DeviceBuffer(4 * n); a.write(asg)
+    m = km.DeviceBuffer(4 * k * dim); s = km.DeviceBuffer(4 * k)
+    km.sync()
+    before = device_memory_in_use()
+    km.update_noalloc(km.UPDATE_ATOMIC_SHM, d, AOS, dim, a, m, AOS, dim, s, dim, k, n)
+    km.sync()
+    assert device_memory_in_use() == before
+    want_m, want_s = m.read(np.float32, k * dim), s.read(np.uint32, k)
+    om, osz = orc.update(pts.ravel(), asg, dim, k, n, threads=0)
+    assert np.array_equal(want_s, osz) and rel_err(want_m, om) < CENTROID_RTOL
+    with km.Graph() as g:
+        km.update_noalloc(km.UPDATE_ATOMIC_SHM, d, AOS, dim, a, m, AOS, dim, s, dim, k, n)
+    for _ in range(3):
+        m.write(np.full(k * dim, 0x7FC00001, np.uint32)); s.write(np.full(k, 7, np.uint32))   # eager work between the replays
+        g.launch()
+        km.sync()
+        assert np.array_equal(s.read(np.uint32, k), want_s)
+        assert rel_err(m.read(np.float32, k * dim), want_m) < 1e-5   # (the order of the additions inside a cluster varies from run to run)
+    g.destroy()   # (the runtime keeps memory of its own for a graph: nothing to compare after this point)
+    for b in (d, a, m, s):
+        b.free()
+
+
 def test_noalloc_update_refuses_what_does_not_fit(km, gpu):
     dim, k, n = 64, 16384, 1 << 20                       # 32 chunks x 2 slices... x 16384 x 65 words: beyond 64 MiB
     d = km.DeviceBuffer(4 * n * dim); d.zero()
