@@ -207,6 +207,47 @@ def double_main(km, args, spec, data, means0):
     print(json.dumps(out))
 
 
+def single_pass_report(km, args, spec, alg, means0, ms_per_step, data):
+    """The default pair of kernels went through kmx_iteration_f32's single pass (k <= 32, dim <= 32): one kernel reads every
+    point once, assigns it, accumulates it and writes its assignment. There is no assignment / update split to report; the
+    dominant kernel is that one, bound by HBM."""
+    n, dim, k = int(spec.n), spec.dim, spec.k
+    alg.reset(means0)
+    km.set_profiling(True)
+    k_ms, rechecked = 0.0, 0
+    for _ in range(args.steps):
+        alg.step()
+        k_ms += km.last_kernel_ms(0)
+        rechecked += km.last_rechecked()
+    km.set_profiling(False)
+    k_ms /= args.steps
+    alg.cleanup()
+    traffic = measured_traffic(args.config)
+    algorithmic = 4.0 * (n * dim + n + 2 * k * dim + k)     # points in, assignment out, centroids in and out, counts
+    gbs = algorithmic / (k_ms * 1e-3) / 1e9
+    out = {
+        "metric": "ms per k-means iteration (assign+update), benchmark configuration %d" % args.config,
+        "value": round(ms_per_step, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "benchmark configuration %d: N=%d d=%d k=%d, %s, initial centroids = first k points, seed %d"
+                               % (args.config, n, dim, k, "Gaussian mixture" if spec.kind != 1 else "uniform", spec.seed),
+                   "layout": "aos", "assignment": "hip_best", "update": "atomic_shm",
+                   "launch": "one kmx_iteration_f32 call per iteration: a single pass over the points"},
+        "assign_ms": None, "update_ms": None,
+        "points_centroids_dims_per_s": round(float(n) * k * dim / (ms_per_step * 1e-3), 0),
+        "rechecked_points_per_iteration": round(rechecked / args.steps, 1),
+        "roofline": {"kernel": "single-pass iteration kernel (ranking, serial arithmetic on the two leaders, sums on the matrix cores)",
+                     "bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4),
+                     "traffic": traffic.get("iteration"), "algorithmic_bytes": algorithmic, "avg_kernel_ms": round(k_ms, 4)},
+    }
+    if not args.no_cpu_baseline:
+        per_point_s = 0.45e-9 * k * dim
+        n_sample = args.cpu_sample or int(min(n, max(1024, 12.0 / per_point_s)))
+        out["cpu_baseline"] = cpu_baseline(km, spec, n_sample, data, means0)
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -273,6 +314,9 @@ def main():
     ms_per_step = wall_ms / args.steps
     counts = alg.getClusterSizes()
     assert int(counts.sum()) == n, "cluster counts do not sum to N"
+
+    if alg.one_call() and km.last_iteration_passes() == 1:
+        return single_pass_report(km, args, spec, alg, means0, ms_per_step, data)
 
     # 3. instrumented repeat of the same iterations
     alg.reset(means0)

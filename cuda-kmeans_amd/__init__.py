@@ -36,7 +36,7 @@ ABI_SYMBOLS = [
     "kmx_assign_last_rechecked", "kmx_assign_last_variant", "kmx_update_f32", "kmx_bucket_sum_f32", "kmx_fused_f32", "kmx_assign_f64", "kmx_update_f64", "kmx_fused_f64", "kmx_bucket_sum_f64", "kmx_set_queued_rows_limit",
     "kmx_graph_begin", "kmx_graph_end", "kmx_graph_launch", "kmx_graph_destroy", "kmx_event_create", "kmx_event_destroy", "kmx_event_record",
     "kmx_event_elapsed_ms", "kmx_set_profiling", "kmx_last_kernel_ms", "kmx_last_error", "kmx_certificate_tau", "kmx_certificate_unmoved_threshold",
-    "kmx_update_f32_noalloc", "kmx_reserve_f32", "kmx_prepare_points_f64", "kmx_forget_points_f64", "kmx_probe_matrix_chain", "kmx_set_two_level_sweep",
+    "kmx_update_f32_noalloc", "kmx_reserve_f32", "kmx_prepare_points_f64", "kmx_forget_points_f64", "kmx_probe_matrix_chain", "kmx_set_two_level_sweep", "kmx_iteration_f32", "kmx_iteration_last_passes",
 ]
 
 
@@ -137,6 +137,8 @@ def hip_lib():
         lib.kmx_last_kernel_ms.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_float)]
         lib.kmx_probe_matrix_chain.argtypes = [ctypes.c_int, vp, vp, vp, vp, u32]
         lib.kmx_set_two_level_sweep.argtypes = [ctypes.c_int]
+        lib.kmx_iteration_f32.argtypes = [vp, ctypes.c_int, sz, vp, vp, ctypes.c_int, sz, vp, vp, u32, u32, u32, ctypes.POINTER(ExecParams)]
+        lib.kmx_iteration_last_passes.argtypes = [ctypes.POINTER(ctypes.c_int)]
         _hip = lib
     return _hip
 
@@ -352,6 +354,22 @@ def fused(variant, data_buf, layout, stride, means_in_buf, means_out_buf, layout
     return ex
 
 
+def iteration(data_buf, layout, stride, means_in_buf, means_out_buf, layout_means, stride_means, assignment_buf, sizes_buf,
+              dim, k, n, exec_params=None):
+    """kmx_iteration_f32: assignment (selector) and update (tuned) of one Lloyd iteration in one call; enqueues and returns."""
+    ex = exec_params if exec_params is not None else ExecParams()
+    check(hip_lib().kmx_iteration_f32(data_buf.ptr, layout, stride, means_in_buf.ptr, means_out_buf.ptr, layout_means, stride_means,
+                                      assignment_buf.ptr, sizes_buf.ptr, dim, k, n, ctypes.byref(ex)))
+    return ex
+
+
+def last_iteration_passes():
+    """Passes over the points the last kmx_iteration_f32 call made (1: the single-pass kernel, 2: assignment, then update)."""
+    p = ctypes.c_int(0)
+    check(hip_lib().kmx_iteration_last_passes(ctypes.byref(p)))
+    return p.value
+
+
 class Graph:
     """A recording of library calls (kmx_graph_begin .. kmx_graph_end) that can be launched as one unit."""
 
@@ -513,29 +531,45 @@ class HipKMeansAlgorithm:
                self.layout_means, self.stride_means, self.cu_sizes, self.dim, self.k, self.n, self.exec, self.dtype)
         self.last = nxt
 
+    def one_call(self):
+        """The default pair of kernels on floats goes through kmx_iteration_f32, which reads the points once where it can."""
+        return self.assign_variant == ASSIGN_BEST and self.update_variant == UPDATE_ATOMIC_SHM and self.dtype == np.dtype(np.float32)
+
+    def step(self):
+        """One whole iteration: one kmx_iteration_f32 call for the default pair of kernels, else assignment, then update."""
+        if not self.one_call():
+            self.update_step(self.iteration())
+            return
+        nxt = (self.last + 1) % 2
+        iteration(self.cu_data, self.layout, self.stride, self.cu_means[self.last], self.cu_means[nxt], self.layout_means,
+                  self.stride_means, self.cu_assignment[nxt], self.cu_sizes, self.dim, self.k, self.n, self.exec)
+        self.last = nxt
+
     def run(self, iters=None, collect_rechecked=False, use_graph=False):
         """All iterations, one sync at the end. use_graph: the first iteration runs call by call (it sizes the work
         space), then two ping-pong iterations are recorded once and replayed; an odd one out runs call by call."""
         todo = self.iters if iters is None else iters
         if use_graph and not collect_rechecked and todo >= 3:
-            self.update_step(self.iteration())
+            self.step()
             pairs = (todo - 1) // 2
             with Graph() as g:
                 for _ in range(2):
-                    self.update_step(self.iteration())
+                    self.step()
             for _ in range(pairs):
                 g.launch()
             todo -= 1 + 2 * pairs
             for _ in range(todo):
-                self.update_step(self.iteration())
+                self.step()
             sync()
             g.destroy()
             return
         for _ in range(todo):
-            nxt = self.iteration()
             if collect_rechecked:
+                nxt = self.iteration()
                 self.rechecked.append(last_rechecked())
-            self.update_step(nxt)
+                self.update_step(nxt)
+            else:
+                self.step()
         sync()
 
     def getMeans(self):

@@ -36,13 +36,16 @@ constexpr uint32_t UNRESOLVED = 0xFFFFFFFFu;
 
 typedef float f32x4v __attribute__((ext_vector_type(4)));
 
-template <int DP, int LD, int LM, int MT>
+/* EMIT: the result of every point the kernel settles is also written to `assignment` (the points it leaves to the exact
+ * pass are written there by that pass): the iteration then hands out the assignment vector the reference's unfused driver
+ * keeps (cuda.hpp:26,72-85), for one more coalesced store of 4 n bytes. */
+template <int DP, int LD, int LM, int MT, bool EMIT>
 __global__ void __launch_bounds__(FUSED_WAVES * WAVE) __attribute__((amdgpu_waves_per_eu(DP == 16 ? 7 : 1)))
 fused_small_kernel(const float* __restrict__ data, size_t stride, const float* __restrict__ packed, const float* __restrict__ norms,
                    const float* __restrict__ means_in, size_t stride_means,
                    float* __restrict__ means_out, uint32_t* __restrict__ sizes,
                    uint32_t* __restrict__ queue, uint32_t* __restrict__ counters,
-                   uint32_t dim, uint32_t k, uint32_t n, float kd, uint32_t vec4, float kd_unmoved)
+                   uint32_t dim, uint32_t k, uint32_t n, float kd, uint32_t vec4, float kd_unmoved, uint32_t* __restrict__ assignment)
 {
 	/* the frame of the ranking (sweep_frame; the packing kernel moved the centroids): the same words for every lane, so they
 	 * arrive as scalar operands. Only the ranking uses the moved coordinates; the serial arithmetic and the sums take the
@@ -187,6 +190,9 @@ fused_small_kernel(const float* __restrict__ data, size_t stride, const float* _
 			if (!decided) result = two ? of_two : UNRESOLVED;
 		}
 		if (!valid) result = UNRESOLVED;
+		if constexpr (EMIT) {
+			if (result != UNRESOLVED) assignment[pt] = result;
+		}
 
 		const bool flag = valid && result == UNRESOLVED;
 		const unsigned long long mask = __ballot(flag);
@@ -307,7 +313,9 @@ static int launch_fused_t(const AssignArgs& a, float* means_out, uint32_t* sizes
 	const uint32_t static_bytes = (2 * FLAG_CAP * FUSED_WAVES + 128) * 4;
 	if (lds_bytes + static_bytes > dev.lds_bytes) return fail(KMX_ERR_UNSUPPORTED, "fused iteration: %u bytes of LDS needed", lds_bytes + static_bytes);
 	void (*kernel)(const float*, size_t, const float*, const float*, const float*, size_t, float*, uint32_t*, uint32_t*, uint32_t*,
-	               uint32_t, uint32_t, uint32_t, float, uint32_t, float) = mt == 1 ? fused_small_kernel<DP, LD, LM, 1> : fused_small_kernel<DP, LD, LM, 2>;
+	               uint32_t, uint32_t, uint32_t, float, uint32_t, float, uint32_t*) =
+		a.emit_assignment ? (mt == 1 ? fused_small_kernel<DP, LD, LM, 1, true> : fused_small_kernel<DP, LD, LM, 2, true>)
+		                  : (mt == 1 ? fused_small_kernel<DP, LD, LM, 1, false> : fused_small_kernel<DP, LD, LM, 2, false>);
 	const uint32_t batches = (a.n + FUSED_WAVES * WAVE - 1) / (FUSED_WAVES * WAVE);
 	const uint32_t per_cu = std::max<uint32_t>(1, std::min<uint32_t>(8, dev.lds_bytes / (lds_bytes + static_bytes)));
 	const uint32_t grid = std::min(batches, dev.compute_units * per_cu);
@@ -317,7 +325,7 @@ static int launch_fused_t(const AssignArgs& a, float* means_out, uint32_t* sizes
 	if (rc) return rc;
 	KMX_LAUNCH_KERNEL(kernel, dim3(grid), dim3(FUSED_WAVES * WAVE), lds_bytes, stream(),
 	                   a.data, a.stride, ws->packed_means, ws->norms, a.means, a.stride_means, means_out, sizes,
-	                   ws->queue, ws->counters, a.dim, a.k, a.n, kd, vec4, cert_kd_unmoved(a.dim));
+	                   ws->queue, ws->counters, a.dim, a.k, a.n, kd, vec4, cert_kd_unmoved(a.dim), a.assignment);
 	KMX_LAUNCH_CHECK("fused_small_kernel");
 	return profile_end(0);
 }
@@ -352,7 +360,9 @@ static int launch_fused_layouts(const AssignArgs& a, float* means_out, uint32_t*
 	return KMX_OK;
 }
 
-/* a.assignment must be the work-space vector of n entries; means_out and sizes are zero on entry; the caller divides */
+/* a.assignment: a vector of n entries -- the work-space vector (only the entries of the points left to the exact pass are
+ * written), or with a.emit_assignment the caller's, which then receives every point's result; means_out and sizes are zero
+ * on entry; the caller divides */
 int launch_fused_small(const AssignArgs& a, float* means_out, uint32_t* sizes, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev)
 {
 	if (a.layout == KMX_AOS && a.layout_means == KMX_AOS) return launch_fused_layouts<KMX_AOS, KMX_AOS>(a, means_out, sizes, exec, ws, dev);

@@ -131,6 +131,8 @@ struct AssignArgs {
 	/* rows of 17 to 32 dimensions: the sweep may run in two levels (one product per dimension for all points, three for
 	 * those the first level cannot settle); off for measurements of the one-level sweep */
 	bool two_level = true;
+	/* the single-pass fused kernel: write the result of every point to `assignment`, not only those of the exact pass */
+	bool emit_assignment = false;
 };
 
 struct UpdateArgs {
@@ -179,6 +181,7 @@ int noalloc_workspace(Workspace** ws);
 bool recording_graph(); /* between kmx_graph_begin and kmx_graph_end */
 int launch_update(int variant, const UpdateArgs& u, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev);
 int launch_divide_means(const UpdateArgs& u);
+int clear_update_outputs(const UpdateArgs& u); /* means (replica 0) and cluster sizes := 0 in one launch */
 
 /* update_ordered.hip: KMX_UPDATE_SERIAL_ORDER for floats and doubles -- stable counting sort of the point numbers by
  * cluster, then one lane per (cluster, coordinate) adds the members in ascending point order and divides: the bits of

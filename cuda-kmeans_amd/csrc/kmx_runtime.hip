@@ -637,6 +637,55 @@ int kmx_fused_f32(int variant,
 	                      cluster_sizes, dim, k, n, exec);
 }
 
+static int g_last_iteration_passes = 0;
+
+int kmx_iteration_f32(const float* data, int layout, size_t stride,
+                      const float* means_in, float* means_out, int layout_means, size_t stride_means,
+                      uint32_t* assignment, uint32_t* cluster_sizes,
+                      uint32_t dim, uint32_t k, uint32_t n, kmx_exec_params* exec)
+{
+	clear_error();
+	if (!exec) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_iteration_f32: exec is null");
+	if (dim == 0 || k == 0) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_iteration_f32: dim and k must be positive");
+	if (!means_in || !means_out || !cluster_sizes) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_iteration_f32: null device pointer");
+	if (n > 0 && (!data || !assignment)) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_iteration_f32: null device pointer");
+	if (means_in == means_out) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_iteration_f32: means_in and means_out must differ");
+	g_last_iteration_passes = 2;
+	if (fused_small_supports(dim, k) && n > 0) {
+		int rc = check_layout("kmx_iteration_f32", "data", layout, stride, n, dim);
+		if (rc) return rc;
+		rc = check_layout("kmx_iteration_f32", "means", layout_means, stride_means, k, dim);
+		if (rc) return rc;
+		const DeviceInfo* dev = nullptr;
+		rc = device_info(&dev);
+		if (rc) return rc;
+		Workspace* ws = nullptr;
+		rc = workspace(&ws);
+		if (rc) return rc;
+		UpdateArgs u{ data, layout, stride, assignment, means_out, layout_means, stride_means, cluster_sizes, dim, k, n };
+		rc = clear_update_outputs(u); /* the single-pass kernel accumulates into them */
+		if (rc) return rc;
+		AssignArgs a{ data, layout, stride, means_in, layout_means, stride_means, assignment, dim, k, n };
+		a.emit_assignment = true;
+		g_last_assign_variant = KMX_ASSIGN_LDS_FMA; /* the ranking of the single-pass kernel: fused multiply-adds on scalar operands */
+		rc = launch_fused_small(a, means_out, cluster_sizes, exec, ws, *dev);
+		if (rc) return rc;
+		g_last_iteration_passes = 1;
+		return launch_divide_means(u);
+	}
+	int rc = kmx_assign_f32(KMX_ASSIGN_BEST, data, layout, stride, means_in, layout_means, stride_means, nullptr, assignment, dim, k, n, exec);
+	if (rc) return rc;
+	return kmx_update_f32(KMX_UPDATE_ATOMIC_SHM, data, layout, stride, assignment, means_out, layout_means, stride_means, cluster_sizes, dim, k, n, exec);
+}
+
+int kmx_iteration_last_passes(int* passes)
+{
+	clear_error();
+	if (!passes) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_iteration_last_passes: null pointer");
+	*passes = g_last_iteration_passes;
+	return KMX_OK;
+}
+
 int kmx_graph_begin(void)
 {
 	clear_error();

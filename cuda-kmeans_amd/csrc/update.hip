@@ -1195,6 +1195,8 @@ int noalloc_workspace(Workspace** ws)
 	return KMX_OK;
 }
 
+int clear_update_outputs(const UpdateArgs& u) { return clear_outputs(u); }
+
 int launch_update(int variant, const UpdateArgs& u, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev)
 {
 	if (variant == KMX_UPDATE_SERIAL_ORDER)

@@ -121,6 +121,14 @@ inline int fused_call(int variant, const double* data, int ld, std::size_t strid
 	std::size_t strideMeans, std::uint32_t* sizes, std::uint32_t dim, std::uint32_t k, std::uint32_t n, kmx_exec_params* exec)
 { return kmx_fused_f64(variant, data, ld, stride, meansIn, meansOut, lm, strideMeans, sizes, dim, k, n, exec); }
 
+/* kmx_iteration_f32: the default pair of kernels in one call (floats); see HipKMeansAlgorithm */
+inline int iteration_call(const float* data, int ld, std::size_t stride, const float* meansIn, float* meansOut, int lm, std::size_t strideMeans,
+	std::uint32_t* assignment, std::uint32_t* sizes, std::uint32_t dim, std::uint32_t k, std::uint32_t n, kmx_exec_params* exec)
+{ return kmx_iteration_f32(data, ld, stride, meansIn, meansOut, lm, strideMeans, assignment, sizes, dim, k, n, exec); }
+inline int iteration_call(const double*, int, std::size_t, const double*, double*, int, std::size_t, std::uint32_t*, std::uint32_t*,
+	std::uint32_t, std::uint32_t, std::uint32_t, kmx_exec_params*)
+{ return KMX_ERR_UNSUPPORTED; } /* never reached: the driver takes the one call for floats only */
+
 /* The points of a run are uploaded once and never change (cuda.hpp:54-64): the double-precision entry points are told so and
  * keep the float copy their ranking sweeps work on, instead of converting the points in every call. Floats need nothing. */
 inline int prepare_points_call(const float*, int, std::size_t, std::uint32_t, std::uint32_t) { return KMX_OK; }
@@ -171,6 +179,17 @@ void fused(int variant, const FusedProblemInstance<F, IDX_T>& in, HipExecParamet
 		in.data, LAYOUT::ID, LAYOUT::precomputeConstants(in.n, in.dim),
 		in.meansIn, in.meansOut, LAYOUT_MEANS::ID, LAYOUT_MEANS::precomputeConstants(in.k, in.dim),
 		(std::uint32_t*)in.clusterSizes, in.dim, in.k, in.n, reinterpret_cast<kmx_exec_params*>(&exec)));
+}
+
+/* assignment + update of one iteration in one call (kmx_iteration_f32) */
+template<typename F, typename IDX_T, class LAYOUT, class LAYOUT_MEANS>
+void iteration(const F* data, const F* meansIn, F* meansOut, IDX_T* assignment, IDX_T* sizes, std::size_t dim, std::size_t k, std::size_t n,
+	HipExecParameters& exec)
+{
+	static_assert(sizeof(IDX_T) == 4, "built for 32-bit indices");
+	KMX_CHECK(iteration_call(data, LAYOUT::ID, LAYOUT::precomputeConstants(n, dim), meansIn, meansOut, LAYOUT_MEANS::ID,
+		LAYOUT_MEANS::precomputeConstants(k, dim), (std::uint32_t*)assignment, (std::uint32_t*)sizes,
+		(std::uint32_t)dim, (std::uint32_t)k, (std::uint32_t)n, reinterpret_cast<kmx_exec_params*>(&exec)));
 }
 
 } // namespace hip_detail

@@ -94,6 +94,13 @@ class HipKMeansAlgorithm : public IKMeansAlgorithm<F, IDX_T>
 
 	std::size_t meansSize() const { return LAYOUT_MEANS::size(this->mK, this->mDim); }
 
+	/* The default pair of kernels on floats -- the selector's assignment and the tuned update -- is one library call
+	 * (kmx_iteration_f32), which reads the points once where a single kernel can hold all centroids; the loop body of
+	 * cuda.hpp:72-85 otherwise. With the timing split the two halves stay two calls: there is nothing to split in one kernel. */
+	static constexpr bool kOneCall = std::is_same<F, float>::value
+		&& std::is_same<ASGN_KERNEL, BestCachedAssignmentKernel<F, IDX_T, LAYOUT, LAYOUT_MEANS, METRIC>>::value
+		&& std::is_same<UPDATE_KERNEL, UpdateAtomicShmKernel<F, IDX_T, LAYOUT, LAYOUT_MEANS, false>>::value;
+
 	void fetchResult()
 	{
 		if (mResultReady) return;
@@ -133,6 +140,12 @@ private:
 	{
 		const std::size_t copies = mExecParams.privatizedCopies ? mExecParams.privatizedCopies : 1;
 		const unsigned next = (mLast + 1) % 2;
+		if (kOneCall) {
+			hip_detail::iteration<F, IDX_T, LAYOUT, LAYOUT_MEANS>(*mDevData, *mDevMeans[mLast], *mDevMeans[next], *mDevAssignment[next],
+				*mDevClusterSizes, this->mDim, this->mK, this->mN, mExecParams);
+			mLast = next;
+			return;
+		}
 		AssignmentProblemInstance<F, IDX_T> assignment(*mDevData, *mDevMeans[mLast], *mDevAssignment[mLast],
 			*mDevAssignment[next], this->mDim, this->mK, this->mN);
 		ASGN_KERNEL::run(assignment, mExecParams);
@@ -173,6 +186,11 @@ public:
 	void run() override
 	{
 		if (mUseGraph && !mTimeSplit && this->mIters >= 3) { runRecorded(); return; }
+		if (kOneCall && !mTimeSplit) {
+			for (std::size_t iter = 0; iter < this->mIters; ++iter) iterate();
+			KMX_CHECK(kmx_sync());
+			return;
+		}
 		void* ev[3] = { nullptr, nullptr, nullptr };
 		if (mTimeSplit) for (auto& e : ev) KMX_CHECK(kmx_event_create(&e));
 		const std::size_t copies = mExecParams.privatizedCopies ? mExecParams.privatizedCopies : 1;

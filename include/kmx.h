@@ -239,6 +239,22 @@ int kmx_fused_f32(int variant,
                   uint32_t dim, uint32_t k, uint32_t n, kmx_exec_params* exec);
 
 /*
+ * ---- one iteration of CudaKMeansAlgorithm::run's loop (cuda.hpp:72-85: assignment kernel, two zero-fills, update kernel) in
+ *      one call, with the selector's assignment and the tuned update ----
+ * assignment[i] = the nearest centroid of means_in (exactly as kmx_assign_f32), means_out / cluster_sizes = the centroids and
+ * member counts of that assignment (as kmx_update_f32 with KMX_UPDATE_ATOMIC_SHM). No precondition on the outputs. What the
+ * one call buys: where a single kernel can hold all centroids (k <= 32, dim <= 32 -- the shapes bound by HBM, where reading
+ * the points twice is what an iteration costs) it reads every point ONCE, assigns it, accumulates it and writes its
+ * assignment; everywhere else the call is the two calls it stands for. kmx_iteration_last_passes tells which of the two
+ * ran (1 or 2 passes over the points; 0 before the first call).
+ */
+int kmx_iteration_f32(const float* data, int layout, size_t stride,
+                      const float* means_in, float* means_out, int layout_means, size_t stride_means,
+                      uint32_t* assignment, uint32_t* cluster_sizes,
+                      uint32_t dim, uint32_t k, uint32_t n, kmx_exec_params* exec);
+int kmx_iteration_last_passes(int* passes);
+
+/*
  * ---- the same runners instantiated with F = double: the reference's --double switch (k-means.cpp:341-342) selects
  *      the <double> instantiations of every kernel (kernels.cu:1200-1261) ----
  * Arguments as for the _f32 entry points, with doubles for data and centroids (strides in elements).

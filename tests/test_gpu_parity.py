@@ -758,6 +758,63 @@ def test_full_size_properties(km, orc, gpu, cid):
     assert rechecked < n // 10
 
 
+# ---------------------------------------------------------------- one call per iteration
+
+@pytest.mark.parametrize("dim,k,n", [(16, 16, 100000), (3, 5, 257), (8, 32, 5000), (20, 7, 3333), (32, 32, 4099), (4, 2, 70000),
+                                     (16, 33, 20000), (40, 16, 9000), (32, 1024, 30000)])   # the last three: two passes
+@pytest.mark.parametrize("layout,layout_means", [(AOS, AOS), (SOA, SOA), (AOS, SOA), (SOA, AOS)])
+def test_one_call_iteration(km, orc, gpu, dim, k, n, layout, layout_means):
+    """kmx_iteration_f32 (cuda.hpp:72-85 in one call): the assignment is the serial scan's, counts exact, centroids within
+    tolerance, outputs full of leftovers on entry; a single pass over the points where k <= 32 and dim <= 32."""
+    rng = np.random.default_rng(dim * 977 + k)
+    centres = rng.uniform(-10, 10, size=(max(k // 2, 1), dim))
+    pts = (centres[rng.integers(0, centres.shape[0], size=n)] + rng.normal(size=(n, dim))).astype(np.float32)
+    means = pts[:k].copy()
+    if k > 3:
+        means[2] = means[1]                                  # a duplicate: exact ties
+    data = np.ascontiguousarray(pts if layout == AOS else pts.T).ravel()
+    cents = np.ascontiguousarray(means if layout_means == AOS else means.T).ravel()
+    d = km.DeviceBuffer(data.nbytes); d.write(data)
+    m_in = km.DeviceBuffer(cents.nbytes); m_in.write(cents)
+    m_out = km.DeviceBuffer(cents.nbytes); m_out.write(np.full(cents.size, 0x7FC12345, np.uint32))
+    a = km.DeviceBuffer(4 * n); a.write(np.full(n, 0xFFFFFFF0, np.uint32))
+    s = km.DeviceBuffer(4 * k); s.write(np.full(k, 0xDEADBEEF, np.uint32))
+    km.iteration(d, layout, km.layout_stride(layout, n, dim), m_in, m_out, layout_means, km.layout_stride(layout_means, k, dim), a, s, dim, k, n)
+    km.sync()
+    assert km.last_iteration_passes() == (1 if k <= 32 and dim <= 32 else 2)
+    got_a, got_m, got_s = a.read(np.uint32, n), m_out.read(np.float32, cents.size), s.read(np.uint32, k)
+    for b in (d, m_in, m_out, a, s):
+        b.free()
+    want_a = orc.assign(data, cents, dim, k, n, layout, layout_means, threads=0, fast=True)
+    bad = np.nonzero(got_a != want_a)[0]
+    assert bad.size == 0, "%d of %d points differ (first %s: %s, oracle %s)" % (bad.size, n, bad[:5], got_a[bad[:5]], want_a[bad[:5]])
+    want_m, want_s = orc.update(data, want_a, dim, k, n, layout, layout_means, threads=0)
+    assert np.array_equal(got_s, want_s)
+    assert rel_err(got_m, want_m) < CENTROID_RTOL
+
+
+@pytest.mark.parametrize("cid,n,iters", [(5, 1 << 18, 4), (1, 65536, 3), (2, 65536, 2)])
+def test_whole_runs_through_the_one_call(km, orc, gpu, cid, n, iters):
+    """HipKMeansAlgorithm.run() with the default pair of kernels goes through kmx_iteration_f32: every iteration against
+    the oracle fed with the centroids the device used."""
+    spec = km.baseline_config(cid)
+    dim, k = spec.dim, spec.k
+    data, means0 = km.generate_points(spec, n), km.first_k_means(spec)
+    alg = km.HipKMeansAlgorithm(km.ASSIGN_BEST, km.UPDATE_ATOMIC_SHM)
+    alg.initialize(dim, k, n, iters, data, means0)
+    assert alg.one_call()
+    for it in range(iters):
+        prev = alg.getMeans()
+        alg.step()
+        km.sync()
+        ga, gm, gs = alg.getAssignment(), alg.getMeans(), alg.getClusterSizes()
+        oa = orc.assign(data, prev, dim, k, n, threads=0, fast=True)
+        assert np.array_equal(ga, oa), "iteration %d: %d mismatches" % (it, int((ga != oa).sum()))
+        om, osz = orc.update(data, oa, dim, k, n, threads=0)
+        assert np.array_equal(gs, osz) and rel_err(gm, om) < CENTROID_RTOL
+    alg.cleanup()
+
+
 # ---------------------------------------------------------------- recorded iterations (HIP graph)
 
 def fused_step(km, variant, data, means, dim, k, n, layout=AOS, layout_means=AOS):
