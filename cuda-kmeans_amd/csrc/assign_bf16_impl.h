@@ -218,14 +218,16 @@ __device__ __forceinline__ void convert_split_points(SplitPoints<KB> (&b)[P], fl
  * registers): all coordinates of a point are requested first, then the blocks of 16 dimensions are converted one at a time
  * behind a fence each, so that the coordinates of the frame are not requested ahead and held as well. Otherwise the
  * scheduler is left to interleave the blocks. */
-template <int KB, int P, int LD, bool VEC, bool FENCED = false>
+template <int KB, int P, int LD, bool VEC, bool FENCED = false, bool LISTED = false, bool LEVEL1 = false>
 __device__ __forceinline__ void load_split_points(SplitPoints<KB> (&b)[P], float (&xx)[P], float (&xm)[P], const float* __restrict__ data, size_t stride,
-                                                  uint32_t base, uint32_t col, uint32_t h, uint32_t dim, uint32_t n, const float* frame)
+                                                  uint32_t base, uint32_t col, uint32_t h, uint32_t dim, uint32_t n, const float* frame,
+                                                  const uint32_t* __restrict__ list = nullptr, float* xl = nullptr)
 {
 #pragma unroll
 	for (int p = 0; p < P; ++p) {
-		const uint32_t pt = base + p * TILE + col;
-		const bool valid = pt < n;
+		const uint32_t slot = base + p * TILE + col;
+		const bool valid = slot < n;
+		const uint32_t pt = LISTED ? (valid ? list[2 * (size_t)slot] : 0u) : slot; /* (see request_split_points) */
 		float v[KB][8];
 		auto request = [&](int kb) {
 			const uint32_t d0 = kb * KBLOCK + h * 8;
@@ -253,7 +255,7 @@ __device__ __forceinline__ void load_split_points(SplitPoints<KB> (&b)[P], float
 				for (int j = 0; j < 8; ++j) v[kb][j] = (valid && d0 + j < dim) ? data[elem<LD>(stride, pt, d0 + j)] : 0.0f;
 			}
 		};
-		float part = 0.0f, along = 0.0f;
+		float part = 0.0f, along = 0.0f, low = 0.0f;
 		auto convert = [&](int kb) {
 			const uint32_t d0 = kb * KBLOCK + h * 8;
 			const f32x4 m0 = *(const f32x4*)(frame + d0), m1 = *(const f32x4*)(frame + d0 + 4);
@@ -263,10 +265,19 @@ __device__ __forceinline__ void load_split_points(SplitPoints<KB> (&b)[P], float
 				const float w = v[kb][j] - m[j];
 				part += w * w;
 				along += w * m[j];
-				__bf16 hi, mid;
-				split_bf16(w, hi, mid);
-				b[p].hi[kb][j] = hi;
-				b[p].mid[kb][j] = mid;
+				if constexpr (LEVEL1) { /* the first level multiplies the hi parts only (convert_split_points): no mid part, |w - hi|^2 instead */
+					const __bf16 hi = (__bf16)w;
+					/* hi as a float: its 16 bits in the upper half of the word */
+					const float r = w - __uint_as_float((uint32_t)__builtin_bit_cast(unsigned short, hi) << 16);
+					low = __builtin_fmaf(r, r, low);
+					b[p].hi[kb][j] = hi;
+				}
+				else {
+					__bf16 hi, mid;
+					split_bf16(w, hi, mid);
+					b[p].hi[kb][j] = hi;
+					b[p].mid[kb][j] = mid;
+				}
 			}
 		};
 		if (FENCED) {
@@ -287,6 +298,12 @@ __device__ __forceinline__ void load_split_points(SplitPoints<KB> (&b)[P], float
 		}
 		xx[p] = part;
 		xm[p] = along;
+		if constexpr (LEVEL1) {
+			/* the sum exists here, in a register: left alone the compiler moves the additions behind the sweep, where the
+			 * sum is used, and keeps all coordinates alive until then (150 to 900 spilled registers at 256 dimensions) */
+			asm volatile("" : "+v"(low));
+			xl[p] = low;
+		}
 	}
 }
 
@@ -648,7 +665,8 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 	constexpr bool SLICED = extra_is<CentroidSlice, Slice...>();
 	constexpr bool LEVEL1 = extra_is<LevelOne, Slice...>();
 	constexpr bool LISTED = extra_is<ListedPoints, Slice...>();
-	static_assert(!(LEVEL1 || LISTED) || (COARSE && !PACKED && !STREAM && KB <= 3 && PREFETCH), "the two-level sweep is built on the pipelined step with prefetched points");
+	static_assert(!(LEVEL1 || LISTED) || (COARSE && !PACKED && !STREAM && KB <= 3 && PREFETCH) || (wide_rows_sweep<KB>() && STREAM && !PREFETCH),
+	              "the two-level sweep is built on the pipelined step with prefetched points and on the wide-row step");
 	[[maybe_unused]] const CentroidSlice slice = slice_of(slice_argument...);
 	[[maybe_unused]] const ListedPoints listed = listed_of(slice_argument...);
 	/* LISTED: the points of the list (never more than the caller's n) */
@@ -829,22 +847,24 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 				}
 #pragma unroll
 				for (int p = 1; p < P; ++p) acc[p] = acc[0];
-				bf16x8 chi[KB], cmid[KB];
+				bf16x8 chi[KB], cmid[LEVEL1 ? 1 : KB]; /* (the first level of a two-level sweep multiplies the hi parts only) */
 #pragma unroll
 				for (int kb = 0; kb < AHEAD; ++kb) {
 					chi[kb] = row_unit(arow, 4 * kb + 2 * h);
-					cmid[kb] = row_unit(arow, 4 * kb + 2 * h + 1);
+					if constexpr (!LEVEL1) cmid[kb] = row_unit(arow, 4 * kb + 2 * h + 1);
 				}
 #pragma unroll
 				for (int kb = 0; kb < KB; ++kb) {
 					if (kb + AHEAD < KB) {
 						chi[kb + AHEAD] = row_unit(arow, 4 * (kb + AHEAD) + 2 * h);
-						cmid[kb + AHEAD] = row_unit(arow, 4 * (kb + AHEAD) + 2 * h + 1);
+						if constexpr (!LEVEL1) cmid[kb + AHEAD] = row_unit(arow, 4 * (kb + AHEAD) + 2 * h + 1);
 					}
+					if constexpr (!LEVEL1) {
 #pragma unroll
-					for (int p = 0; p < P; ++p) acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(chi[kb], x[p].mid[kb], acc[p], 0, 0, 0);
+						for (int p = 0; p < P; ++p) acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(chi[kb], x[p].mid[kb], acc[p], 0, 0, 0);
 #pragma unroll
-					for (int p = 0; p < P; ++p) acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cmid[kb], x[p].hi[kb], acc[p], 0, 0, 0);
+						for (int p = 0; p < P; ++p) acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cmid[kb], x[p].hi[kb], acc[p], 0, 0, 0);
+					}
 #pragma unroll
 					for (int p = 0; p < P; ++p) acc[p] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(chi[kb], x[p].hi[kb], acc[p], 0, 0, 0);
 				}
@@ -861,12 +881,13 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 				}
 				/* the order of the step: global requests; norms and AHEAD blocks of operands; then per block its MFMAs
 				 * and the request for the block AHEAD blocks on; tracking and the LDS writes come last by their dependences */
+				constexpr int PARTS = LEVEL1 ? 1 : 2, PRODUCTS = LEVEL1 ? 1 : 3; /* LDS reads and MFMAs per block of 16 dimensions */
 				if constexpr (STREAM) __builtin_amdgcn_sched_group_barrier(0x020, PIECE_VECS + 1, 0);
-				__builtin_amdgcn_sched_group_barrier(0x100, 4 + 2 * AHEAD, 0);
+				__builtin_amdgcn_sched_group_barrier(0x100, 4 + PARTS * AHEAD, 0);
 #pragma unroll
 				for (int kb = 0; kb < KB; ++kb) {
-					__builtin_amdgcn_sched_group_barrier(0x008, 3 * P, 0);
-					if (kb + AHEAD < KB) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+					__builtin_amdgcn_sched_group_barrier(0x008, PRODUCTS * P, 0);
+					if (kb + AHEAD < KB) __builtin_amdgcn_sched_group_barrier(0x100, PARTS, 0);
 				}
 			}
 			if constexpr (STREAM) {
@@ -1310,13 +1331,13 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 	};
 
 	static_assert(!PACKED || KB == 1, "the packed form is one block of 16 slots");
-	auto load_points = [&](SplitPoints<KB> (&bb)[P], float (&xs)[P], float (&xa)[P], uint32_t first) {
+	auto load_points = [&](SplitPoints<KB> (&bb)[P], float (&xs)[P], float (&xa)[P], uint32_t first, [[maybe_unused]] float* xlp = nullptr) {
 		if constexpr (PACKED) {
 			load_packed_points<P, LD, VEC>(bb, xs, data, stride, first, col, h, dim, n, frame);
 #pragma unroll
 			for (int p = 0; p < P; ++p) xa[p] = 0.0f; /* (the thresholds of the packed rows stay in the moved frame) */
 		}
-		else load_split_points<KB, P, LD, VEC, (KB > 4)>(bb, xs, xa, data, stride, first, col, h, dim, n, frame_lds);
+		else load_split_points<KB, P, LD, VEC, (KB > 4), LISTED, LEVEL1>(bb, xs, xa, data, stride, first, col, h, dim, n, frame_lds, listed.list, xlp);
 	};
 
 	/*
@@ -1382,11 +1403,18 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 	else {
 		SplitPoints<KB> b0[P];
 		float xx0[P], xm0[P];
+		[[maybe_unused]] float xl0[P];
 		uint32_t item = uniform(claim());
 		while (item < items) {
 			const uint32_t after = claim();
-			load_points(b0, xx0, xm0, first_point(item));
-			sweep(b0, xx0, xm0, first_point(item));
+			if constexpr (LEVEL1) {
+				load_points(b0, xx0, xm0, first_point(item), xl0);
+				sweep(b0, xx0, xm0, first_point(item), xl0);
+			}
+			else {
+				load_points(b0, xx0, xm0, first_point(item));
+				sweep(b0, xx0, xm0, first_point(item));
+			}
 			item = uniform(after);
 		}
 	}
@@ -1748,7 +1776,9 @@ static int launch_bf16_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 		kernel = assign_bf16_kernel<KB, P, LD, VEC, true, false, PF>;
 	}
 	/* two levels: hi * hi for everybody, then the three products for the points that level could not settle */
-	constexpr bool TWO_LEVEL_BUILT = KB == 2 && !PACKED && PF;
+	constexpr bool TWO_LEVEL_WIDE = KB == 16; /* rows of 129 to 256 dimensions: the wide-row step */
+	constexpr bool TWO_LEVEL_BUILT = (KB == 2 && !PACKED && PF) || TWO_LEVEL_WIDE;
+	constexpr int P1 = TWO_LEVEL_WIDE ? 1 : PR; /* point tiles per wavefront in the first level (two tiles of hi parts would fit the registers of 256-dimension rows by count, but the compiler spills 300 to 700 of them) */
 	[[maybe_unused]] void (*level1_kernel)(const float*, size_t, const float*, const float*, uint32_t*, uint32_t*, uint32_t*,
 	                                      uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, float, float, uint32_t, float, LevelOne) = nullptr;
 	[[maybe_unused]] void (*level2_kernel)(const float*, size_t, const float*, const float*, uint32_t*, uint32_t*, uint32_t*,
@@ -1756,10 +1786,16 @@ static int launch_bf16_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 	bool two_level = false;
 	if constexpr (TWO_LEVEL_BUILT) {
 		const int mode = two_level_mode(); /* kmx_set_two_level_sweep: 0 never, 1 where it pays, 2 wherever the kernels allow it */
-		two_level = !stream_mode && slices == 1 && coarse && a.two_level && mode != 0 &&
+		two_level = (TWO_LEVEL_WIDE ? stream_mode : (!stream_mode && coarse)) && slices == 1 && a.two_level && mode != 0 &&
 		            (mode == 2 || (swept_tiles >= TWO_LEVEL_MIN_TILES && a.n >= KMX_TWO_LEVEL_MIN_POINTS));
-		level1_kernel = assign_bf16_kernel<KB, PR, LD, VEC, false, true, PF, PACKED, LevelOne>;
-		level2_kernel = assign_bf16_kernel<KB, PR, LD, VEC, false, true, PF, PACKED, ListedPoints>;
+		if constexpr (TWO_LEVEL_WIDE) {
+			level1_kernel = assign_bf16_kernel<KB, P1, LD, VEC, true, false, PF, PACKED, LevelOne>;
+			level2_kernel = assign_bf16_kernel<KB, P, LD, VEC, true, false, PF, PACKED, ListedPoints>;
+		}
+		else {
+			level1_kernel = assign_bf16_kernel<KB, PR, LD, VEC, false, true, PF, PACKED, LevelOne>;
+			level2_kernel = assign_bf16_kernel<KB, PR, LD, VEC, false, true, PF, PACKED, ListedPoints>;
+		}
 	}
 	if (two_level) {
 		int rc = reserve_listed(ws, 2 * (size_t)a.n);
@@ -1787,7 +1823,9 @@ static int launch_bf16_t(const AssignArgs& a, kmx_exec_params* exec, Workspace* 
 			KMX_HIP(hipFuncSetAttribute((const void*)level2_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
 			/* level 1: its "queue" is the list, its counter the list's length; thresholds mean nothing there */
 			const float kd1 = kd - cert_kd_split(a.dim) + cert_kd_level1(a.dim);
-			KMX_LAUNCH_KERNEL(level1_kernel, dim3(grid), dim3(MFMA_WAVES * WAVE), lds_bytes, stream(),
+			const uint32_t unit_points1 = MFMA_WAVES * (stream_mode ? P1 : PR) * TILE;
+			const uint32_t grid1 = std::min((a.n + unit_points1 - 1) / unit_points1, dev.compute_units * (uint32_t)per_cu);
+			KMX_LAUNCH_KERNEL(level1_kernel, dim3(grid1), dim3(MFMA_WAVES * WAVE), lds_bytes, stream(),
 			                   a.data, a.stride, ws->packed_means, ws->norms, a.assignment, ws->listed, ws->counters + LISTED_COUNTER,
 			                   a.dim, a.k, kp, a.n, chunk_rows, kd1, -__builtin_inff(), 0xFFFFFFFFu, 0.0f, LevelOne{ 0u });
 			KMX_LAUNCH_CHECK("assign_bf16_kernel (first level)");

@@ -1,4 +1,4 @@
-"""The two-level split-bf16 sweep (rows of 17 to 32 dimensions): one product per dimension for all points, three for those the
+"""The two-level split-bf16 sweep (rows of 17 to 32 and of 129 to 256 dimensions): one product per dimension for all points, three for those the
 first level cannot settle, the exact pass for the rest. By default it runs from 2^18 points on; here it is forced
 (kmx_set_two_level_sweep(2)) so that the inputs aimed at the certificates and the hard inputs of the other modules, which are
 smaller, pass through both levels. Every result must be the serial scan's index, as with one level."""
@@ -22,7 +22,7 @@ def two_levels(km):
 
 
 @pytest.mark.parametrize("dim,k,n", [(32, 1024, 50000), (17, 130, 9000), (20, 100, 3000), (24, 700, 20000), (32, 33, 5000), (31, 4000, 30000),
-                                     (32, 1056, 70000), (28, 64, 4097)])
+                                     (32, 1056, 70000), (28, 64, 4097), (256, 1024, 20000), (200, 300, 9000), (129, 40, 3000), (256, 2100, 5000)])
 @pytest.mark.parametrize("layout,layout_means", [(AOS, AOS), (SOA, SOA), (AOS, SOA)])
 def test_assignment_is_bit_exact(km, orc, gpu, two_levels, dim, k, n, layout, layout_means):
     rng = np.random.default_rng(dim * 131 + k)
@@ -57,7 +57,7 @@ def test_both_settings_return_the_same_and_the_first_level_settles_most_points(k
     assert counts[2] == counts[1] and abs(counts[2] - counts[0]) <= max(64, counts[0] // 2), counts
 
 
-@pytest.mark.parametrize("dim,k,n", [(32, 256, 3000), (21, 1500, 4000), (32, 1024, 4096)])
+@pytest.mark.parametrize("dim,k,n", [(32, 256, 3000), (21, 1500, 4000), (32, 1024, 4096), (200, 160, 2000), (256, 300, 1500)])
 def test_hard_inputs(km, orc, gpu, two_levels, dim, k, n):
     parity_tests.test_hard_inputs(km, orc, gpu, dim, k, n)
 
@@ -66,13 +66,15 @@ def test_worst_case_pairs_match_the_serial_scan(km, orc, gpu, two_levels):
     certificate_tests.test_worst_case_pairs_match_the_serial_scan(km, orc, gpu, 32)
 
 
+@pytest.mark.parametrize("dim", [32, 256])
 @pytest.mark.parametrize("offset", [0.0, 1e2, 1e4])
-def test_gap_sweep(km, orc, gpu, two_levels, offset):
-    certificate_tests.test_gap_sweep(km, orc, gpu, 32, offset)
+def test_gap_sweep(km, orc, gpu, two_levels, dim, offset):
+    certificate_tests.test_gap_sweep(km, orc, gpu, dim, offset)
 
 
-def test_gap_sweep_with_coordinates_of_very_different_exponents(km, orc, gpu, two_levels):
-    certificate_tests.test_gap_sweep_with_coordinates_of_very_different_exponents(km, orc, gpu, 32)
+@pytest.mark.parametrize("dim", [32, 256])
+def test_gap_sweep_with_coordinates_of_very_different_exponents(km, orc, gpu, two_levels, dim):
+    certificate_tests.test_gap_sweep_with_coordinates_of_very_different_exponents(km, orc, gpu, dim)
 
 
 @pytest.mark.parametrize("offset", [0.0, 100.0, 3000.0])
