@@ -269,6 +269,8 @@ def main():
     ap.add_argument("--graph", action="store_true",
                     help="replay a recorded pair of iterations (HIP graph) instead of launching every kernel of the timed "
                          "iterations one by one (measured: no gain on this runtime, 0.042 vs 0.035 ms at configuration 1)")
+    ap.add_argument("--two-level", type=int, default=1, choices=[0, 1, 2],
+                    help="the split-bf16 sweep in two levels: 0 never, 1 where it pays (default), 2 wherever the kernels allow it")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="one device-to-device copy of the point array before the timed region (a copy kernel of known "
                          "size, to scale FETCH_SIZE / WRITE_SIZE counter readings)")
@@ -281,6 +283,7 @@ def main():
         km.build(force=False)
     if km.device_count() == 0:
         sys.exit("bench.py: no HIP device visible")
+    km.set_two_level_sweep(args.two_level)
     spec = km.baseline_config(args.config)
     n, dim, k = int(spec.n), spec.dim, spec.k
     data = km.generate_points(spec)
@@ -389,6 +392,7 @@ def main():
                                % (args.config, n, dim, k, "Gaussian mixture" if spec.kind != 1 else "uniform", spec.seed),
                    "layout": "aos", "assignment": "hip_" + args.assign_variant,
                    "assignment_kernel": VARIANT_NAMES.get(ran_variant, str(ran_variant)), "update": args.update_variant,
+                   "two_level_sweep": {0: "never", 1: "where it pays", 2: "wherever the kernels allow it"}[args.two_level],
                    "launch": "call by call" if not args.graph or args.steps < 3 else "first iteration call by call, then a recorded pair of iterations replayed (HIP graph)"},
         "assign_ms": round(t_assign, 4), "update_ms": round(t_update, 4),
         "points_centroids_dims_per_s": round(float(n) * k * dim / (ms_per_step * 1e-3), 0),
