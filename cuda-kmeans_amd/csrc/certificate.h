@@ -75,6 +75,10 @@ KMX_HD float cert_kd_fp32(unsigned dim) { return (8.0f * (float)dim + 24.0f) * C
 KMX_HD float cert_kd_fma(unsigned dim) { return (4.0f * (float)dim + 24.0f) * CERT_UNIT; }
 KMX_HD float cert_kd_split(unsigned dim) { return (14.0f * (float)dim + 28.0f) * CERT_UNIT; }
 KMX_HD float cert_kd_packed(unsigned dim) { return (18.0f * (float)dim + 36.0f) * CERT_UNIT; }
+/* ranking values whose lowest `bits` mantissa bits are replaced (by the centroid's number): a value a moves by less than 2^bits
+ * units in its last place, at most 2^bits u' |a|, and |a| = ||c'|^2 - 2 c'.x'| <= 2 |c'|^2 + |x'|^2 <= 2 S; a difference of two
+ * values by twice that; the factor's slack covers the roundings inside a. */
+KMX_HD float cert_kd_keyed(unsigned bits) { return 2.0f * CERT_TRUNC_FACTOR * (float)(1u << bits) * CERT_UNIT; }
 KMX_HD float cert_kd_level1(unsigned dim) { return (6.0f * (float)dim + 28.0f) * CERT_UNIT; } /* 4 d + 8 accumulation, 2 d + 12 serial margin, slack */
 
 /* The bound in the form the kernels evaluate per point: tau = kd (x2 + c2max) + a sqrt(xpart2) + b sqrt(x2), with
