@@ -237,7 +237,7 @@ def single_pass_report(km, args, spec, alg, means0, ms_per_step, data):
         "assign_ms": None, "update_ms": None,
         "points_centroids_dims_per_s": round(float(n) * k * dim / (ms_per_step * 1e-3), 0),
         "rechecked_points_per_iteration": round(rechecked / args.steps, 1),
-        "roofline": {"kernel": "single-pass iteration kernel (ranking, serial arithmetic on the two leaders, sums on the matrix cores)",
+        "roofline": {"kernel": "single-pass iteration kernel (ranking and sums on the matrix cores, the next batch of rows in flight)",
                      "bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4),
                      "traffic": traffic.get("iteration"), "algorithmic_bytes": algorithmic, "avg_kernel_ms": round(k_ms, 4)},
     }

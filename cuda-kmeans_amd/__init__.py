@@ -414,10 +414,11 @@ def certificate_tau(form, dim, x2, xpart2, c2max, cmid2max, crest2max):
 
 def probe_matrix_chain(kind, a, b, c):
     """kmx_probe_matrix_chain on host arrays: a (32, depth), b (32, depth: row j = column j of B), c (32, 32), all
-    float32; returns d = c + a b^T as the matrix cores accumulate it, block by block (kind 0: fp32, 1: bf16 operands)."""
+    float32; returns d = c + a b^T as the matrix cores accumulate it, block by block (kind 0: fp32 32x32x2, 1: bf16
+    operands 32x32x16, 2: fp32 16x16x4)."""
     a, b, c = (np.ascontiguousarray(v, dtype=np.float32) for v in (a, b, c))
     depth = a.shape[1]
-    block = 2 if kind == 0 else 16
+    block = {0: 2, 1: 16, 2: 4}[kind]
     assert a.shape == (32, depth) and b.shape == (32, depth) and c.shape == (32, 32) and depth % block == 0
     bufs = [DeviceBuffer(v.nbytes) for v in (a, b, c, c)]
     try:

@@ -203,7 +203,7 @@ void forget_prepared_points_f64(const void* dst, size_t bytes);
 /* fused_small.hip: one pass over the points for a handful of centroids. a.assignment is a scratch vector of n entries
  * (only the entries of the points left to the exact pass are written); means_out and sizes are zero on entry and hold
  * sums and counts on return (the caller divides). */
-bool fused_small_supports(uint32_t dim, uint32_t k);
+bool fused_small_supports(uint32_t dim, uint32_t k, int layout, size_t stride, uint32_t n);
 int launch_fused_small(const AssignArgs& a, float* means_out, uint32_t* sizes, kmx_exec_params* exec, Workspace* ws, const DeviceInfo& dev);
 
 } // namespace kmx

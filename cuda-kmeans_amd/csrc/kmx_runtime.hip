@@ -611,7 +611,7 @@ int kmx_fused_f32(int variant,
 	rc = reserve_fused_assignment(ws, n);
 	if (rc) return rc;
 
-	const bool one_pass_fits = fused_small_supports(dim, k);
+	const bool one_pass_fits = fused_small_supports(dim, k, layout, stride, n);
 	if (variant == KMX_FUSED_ONE_PASS && !one_pass_fits)
 		return fail(KMX_ERR_UNSUPPORTED, "kmx_fused_f32: shape dim=%u k=%u is not supported by the single-pass kernel", dim, k);
 	if (variant != KMX_FUSED_TWO_PASS && one_pass_fits && n > 0) {
@@ -651,7 +651,7 @@ int kmx_iteration_f32(const float* data, int layout, size_t stride,
 	if (n > 0 && (!data || !assignment)) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_iteration_f32: null device pointer");
 	if (means_in == means_out) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_iteration_f32: means_in and means_out must differ");
 	g_last_iteration_passes = 2;
-	if (fused_small_supports(dim, k) && n > 0) {
+	if (fused_small_supports(dim, k, layout, stride, n) && n > 0) {
 		int rc = check_layout("kmx_iteration_f32", "data", layout, stride, n, dim);
 		if (rc) return rc;
 		rc = check_layout("kmx_iteration_f32", "means", layout_means, stride_means, k, dim);
@@ -759,6 +759,11 @@ int kmx_certificate_tau(int form, uint32_t dim, float x2, float xpart2, float c2
 	case 1: *tau = cert_tau(cert_kd_split(dim), x2, xpart2, cert_coeffs_split(cb)); return KMX_OK;
 	case 2: *tau = cert_tau(cert_kd_packed(dim), x2, xpart2, cert_coeffs_packed(cb)); return KMX_OK;
 	case 4: *tau = cert_tau(cert_kd_level1(dim), x2, xpart2, cert_coeffs_level1(cb)); return KMX_OK;
+	case 5: /* the single-pass iteration kernels: forms 3 and 0 with the lowest xpart2 (4 or 5) bits of a value replaced by its centroid's number */
+	case 6:
+		if (!(xpart2 == 4.0f || xpart2 == 5.0f)) return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_certificate_tau: forms 5 and 6 take 4 or 5 replaced bits in xpart2");
+		*tau = ((form == 5 ? cert_kd_fma(dim) : cert_kd_fp32(dim)) + cert_kd_keyed((unsigned)xpart2)) * (x2 + c2max);
+		return KMX_OK;
 	default: return fail(KMX_ERR_INVALID_ARGUMENT, "kmx_certificate_tau: unknown form %d", form);
 	}
 }

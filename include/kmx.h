@@ -354,7 +354,10 @@ int kmx_set_two_level_sweep(int mode);
  * without the serial arithmetic only if its two smallest ranking values differ by more than tau; the tests check tau
  * against an emulation of the split operands on adversarial inputs.
  *   form 0: fp32 MFMA sweep (KMX_ASSIGN_MFMA)                      tau = kd (x2 + c2max); xpart2, cmid2max, crest2max ignored
- *   form 3: sweeps on the vector ALU (KMX_ASSIGN_LDS_FMA, the single-pass fused kernel): the same with a smaller kd
+ *   form 3: sweeps on the vector ALU (KMX_ASSIGN_LDS_FMA): the same with a smaller kd
+ *   forms 5, 6: the single-pass iteration kernels (narrow rows: the chain of form 3; rows of 8, 16, 32 floats: the matrix
+ *           instruction of form 0), whose ranking values carry the centroid's number in their lowest bits: xpart2 = the
+ *           number of replaced bits, 4 (up to 16 centroids) or 5
  *   form 1: split-bf16 sweep, three products per dimension         xpart2 = sum_i xmid_i^2
  *   form 2: split-bf16 sweep, packed rows (dim <= 4, four products) xpart2 = sum_i xrest_i^2
  *   form 4: first level of the two-level split-bf16 sweep (one product per dimension, hi * hi) xpart2 = sum_i (x_i - xhi_i)^2
@@ -382,7 +385,8 @@ int kmx_certificate_unmoved_threshold(uint32_t dim, float first, float tau, floa
  *      d[i][j] = c[i][j] + sum_q a[i][q] b[j][q],   i, j < 32,  q < depth,
  * block by block in ascending q, one instruction per block, with the instructions, operand layout and order of the
  * sweeps: kind 0 = v_mfma_f32_32x32x2_f32 (depth = 2 blocks), kind 1 = v_mfma_f32_32x32x16_bf16 (depth = 16 blocks; the
- * values of a and b must be exactly representable in bf16, the low 16 bits of their words are dropped).
+ * values of a and b must be exactly representable in bf16, the low 16 bits of their words are dropped), kind 2 =
+ * v_mfma_f32_16x16x4_f32 (depth = 4 blocks; the 32 x 32 result as four tiles of 16 x 16).
  * a: 32 x depth row-major; b: 32 x depth, the depth values of column j contiguous; c, d: 32 x 32 row-major. Device pointers.
  */
 int kmx_probe_matrix_chain(int kind, const float* a, const float* b, const float* c, float* d, uint32_t blocks);

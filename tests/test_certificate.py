@@ -259,6 +259,57 @@ def test_tau_of_the_vector_alu_sweeps_covers_a_chain_of_fused_multiply_adds(km, 
     assert not wrong.any(), "%d certified pairs contradict the serial comparison" % int(wrong.sum())
 
 
+@pytest.mark.parametrize("dim", [4, 16, 32])
+@pytest.mark.parametrize("k", [16, 32])
+@pytest.mark.parametrize("kind", ["adversarial", "ties0", "ties100"])
+def test_tau_of_the_single_pass_kernels_pays_for_the_centroid_number_in_the_low_bits(km, dim, k, kind):
+    """The single-pass iteration kernels replace the lowest 4 (k <= 16) or 5 bits of every ranking value by the centroid's
+    number and track minima of the result (forms 5 and 6 of kmx_certificate_tau). The chain is emulated as for form 3, the
+    bits are replaced as the kernels do, and twice the distance of the keyed values from the exact ones plus the serial
+    margin must stay below tau; what tau certifies on the keyed values is a strict serial win, and the centroid read back
+    from the low bits of the minimum is the centroid of that value."""
+    bits = 4 if k <= 16 else 5
+    rng = np.random.default_rng(dim * 19 + k + len(kind))
+    n = 4096
+    x, c = adversarial(dim, n, k, rng) if kind == "adversarial" else near_ties(dim, n, k, rng, float(kind[4:]))
+    cp = (np.float32(-2) * c).astype(np.float32)
+    c2 = np.zeros(k, np.float32)
+    for q in range(dim):
+        c2 = (c2 + (c[:, q] * c[:, q]).astype(np.float32)).astype(np.float32)
+    a = np.repeat(c2[:, None], n, 1)
+    for q in range(dim):
+        a = (cp[:, q].astype(np.float64)[:, None] * x[:, q].astype(np.float64)[None, :] + a.astype(np.float64)).astype(np.float32)
+    mask = np.uint32((1 << bits) - 1)
+    keyed = ((a.view(np.uint32) & ~mask) | np.arange(k, dtype=np.uint32)[:, None]).view(np.float32)
+    exact = (c.astype(np.float64) ** 2).sum(1)[:, None] + cp.astype(np.float64) @ x.astype(np.float64).T
+    x2 = (x.astype(np.float32) ** 2).sum(1, dtype=np.float32)
+    c2max = float(c2.max())
+    s_all = x2.astype(np.float64) + c2max
+    tau5 = np.array([km.certificate_tau(5, dim, float(x2[i]), float(bits), c2max, 0.0, 0.0) for i in range(n)], np.float64)
+    tau6 = np.array([km.certificate_tau(6, dim, float(x2[i]), float(bits), c2max, 0.0, 0.0) for i in range(n)], np.float64)
+    tau3 = np.array([km.certificate_tau(3, dim, float(x2[i]), 0.0, c2max, 0.0, 0.0) for i in range(n)], np.float64)
+    assert np.all(tau6 >= tau5) and np.all(tau5 > tau3)
+    assert tau5[0] == pytest.approx(tau3[0] + 4.125 * (1 << bits) * U * s_all[0], rel=1e-5)
+    moved = np.abs(keyed.astype(np.float64) - a.astype(np.float64))
+    assert np.all(moved.max(0) <= 2.0625 * (1 << bits) * U * s_all)            # one value's share of the allowance
+    assert moved.max() > 0.25 * (1 << bits) * U * np.abs(a).max() * 0.5            # and the bits do move the values
+    margin = (2 * dim + 12) * U * s_all
+    off = np.abs(keyed.astype(np.float64) - exact).max(0)
+    assert np.all(2 * off + margin <= tau5)
+    dist = serial_distances(x, c)
+    j1 = keyed.argmin(0)
+    assert np.array_equal(keyed[j1, np.arange(n)].view(np.uint32) & mask, j1.astype(np.uint32))
+    certified = (keyed.astype(np.float64) - keyed[j1, np.arange(n)].astype(np.float64)[None, :]) > tau5[None, :]
+    certified[j1, np.arange(n)] = False
+    wrong = certified & ~(dist[j1, np.arange(n)][None, :] < dist)
+    assert not wrong.any(), "%d certified pairs contradict the serial comparison" % int(wrong.sum())
+    if dim == 4 and kind == "adversarial":
+        # teeth: with few dimensions the replaced bits take the values out of the bound of the chain itself
+        assert np.any(off > (2 * dim + 7) * (U / 2) * s_all)
+    with pytest.raises(Exception):
+        km.certificate_tau(5, dim, 1.0, 3.0, 1.0, 0.0, 0.0)
+
+
 @pytest.mark.parametrize("dim", [2, 3, 4])
 @pytest.mark.parametrize("kind", ["ties0", "ties100", "ties10000", "uniform", "mirrored pairs"])
 def test_tau_in_a_moved_frame_covers_the_distances_of_the_data(km, dim, kind):
@@ -409,10 +460,10 @@ def test_threshold_taken_back_to_the_frame_of_the_data(km, dim, offset):
 
 def accumulation_cases(kind):
     """Operand sets for kmx_probe_matrix_chain: name -> (a[32, depth], b[32, depth], c[32, 32]) in float32.
-    kind 1: a and b hold bf16 values (products exact in fp32); kind 0: full fp32 mantissas."""
+    kind 1: a and b hold bf16 values (products exact in fp32); kinds 0 and 2: full fp32 mantissas."""
     rng = np.random.default_rng(1234 + kind)
-    block = 2 if kind == 0 else 16
-    quant = (lambda v: np.asarray(v, np.float32)) if kind == 0 else bf16_round
+    block = {0: 2, 1: 16, 2: 4}[kind]
+    quant = bf16_round if kind == 1 else (lambda v: np.asarray(v, np.float32))
     cases = {}
 
     def mant(shape):   # mantissas in [1, 2) with all their bits in use
@@ -460,7 +511,7 @@ def chopped_chain(a, b, c):
     return s
 
 
-@pytest.mark.parametrize("kind", [0, 1])
+@pytest.mark.parametrize("kind", [0, 1, 2])
 def test_accumulation_cases_use_the_allowance_of_one_unit_per_step(kind):
     """A truncating accumulator stays within steps * u' * M on every operand set and exceeds half of that on some:
     the operands have teeth against a bound of half a u' per step."""

@@ -106,11 +106,11 @@ def test_gap_sweep(km, orc, gpu, dim, offset):
     d.free()
 
 
-@pytest.mark.parametrize("kind", [0, 1])
+@pytest.mark.parametrize("kind", [0, 1, 2])
 def test_matrix_core_accumulation_stays_within_one_unit_per_step(km, gpu, kind):
     """The hardware assumption of the certificates (csrc/certificate.h: one u' of the running magnitude per accumulated
-    product covers whatever the matrix core rounds or truncates), measured: chains of v_mfma_f32_32x32x2_f32 (kind 0) and
-    v_mfma_f32_32x32x16_bf16 (kind 1) on products of exponents 2^0..2^-20 inside a block, cancelling pairs next to a term
+    product covers whatever the matrix core rounds or truncates), measured: chains of v_mfma_f32_32x32x2_f32 (kind 0),
+    v_mfma_f32_32x32x16_bf16 (kind 1) and v_mfma_f32_16x16x4_f32 (kind 2) on products of exponents 2^0..2^-20 inside a block, cancelling pairs next to a term
     of 2^-20, a large accumulator with addends below its last place, up to 48 blocks. tests/test_certificate.py shows that
     an accumulator which truncates after every product fails half of this bound on the same operands."""
     worst = 0.0

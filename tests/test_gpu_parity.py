@@ -877,11 +877,13 @@ def test_single_pass_fused_kernel_far_from_the_origin(km, orc, gpu, dim, k, n, o
 
 
 @pytest.mark.gpu
-def test_single_pass_fused_kernel_hard_inputs(km, orc, gpu):
+@pytest.mark.parametrize("dim,k", [(8, 16), (4, 16), (16, 20), (24, 10), (32, 32)])
+def test_single_pass_fused_kernel_hard_inputs(km, orc, gpu, dim, k):
     """Near-ties of three centroids, coincident points, NaN / inf / huge / tiny values go through the exact pass and the
-    fix-up kernel; a shape the single-pass kernel does not take is refused by name."""
-    dim, k, n = 8, 16, 4096
-    rng = np.random.default_rng(77)
+    fix-up kernel; a shape the single-pass kernel does not take is refused by name. Rows of 4 and 24 floats take the
+    lane-per-point kernel, rows of 8, 16 and 32 the kernel that ranks on the matrix cores."""
+    n = 4096
+    rng = np.random.default_rng(77 + dim)
     base = rng.normal(size=(n, dim)).astype(np.float32)
     means = rng.normal(size=(k, dim)).astype(np.float32)
     cases = {}
