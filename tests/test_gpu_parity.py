@@ -793,6 +793,32 @@ def test_one_call_iteration(km, orc, gpu, dim, k, n, layout, layout_means):
     assert rel_err(got_m, want_m) < CENTROID_RTOL
 
 
+def test_single_pass_kernel_is_bounded_by_what_a_buffer_descriptor_spans(km, gpu):
+    """The single-pass kernel reads its points through one buffer descriptor (up to 0xF0000000 bytes): a larger array is
+    refused by name when the kernel is asked for, and kmx_iteration_f32 takes two passes. The points are zeros: every
+    point ties between all centroids, the serial scan returns centroid 0, and only the first centroid gets members."""
+    dim, k = 16, 4
+    n = (0xF0000000 // (4 * dim)) + 4096                   # just past the bound: 4.03 GB of points
+    d = km.DeviceBuffer(4 * n * dim); d.zero()
+    cents = np.zeros(k * dim, np.float32); cents[dim:] = 1.0   # centroid 0 at the origin, the others away from it
+    m_in = km.DeviceBuffer(cents.nbytes); m_in.write(cents)
+    m_out = km.DeviceBuffer(cents.nbytes); m_out.zero()
+    s = km.DeviceBuffer(4 * k); s.zero()
+    a = km.DeviceBuffer(4 * n)
+    try:
+        with pytest.raises(km.KmxError, match="single-pass"):
+            km.fused(km.FUSED_ONE_PASS, d, AOS, dim, m_in, m_out, AOS, dim, s, dim, k, n)
+        km.iteration(d, AOS, dim, m_in, m_out, AOS, dim, a, s, dim, k, n)
+        km.sync()
+        assert km.last_iteration_passes() == 2
+        sizes = s.read(np.uint32, k)
+        assert sizes.tolist() == [n, 0, 0, 0]
+        assert not a.read(np.uint32, n).any()
+    finally:
+        for b in (d, m_in, m_out, s, a):
+            b.free()
+
+
 @pytest.mark.parametrize("cid,n,iters", [(5, 1 << 18, 4), (1, 65536, 3), (2, 65536, 2)])
 def test_whole_runs_through_the_one_call(km, orc, gpu, cid, n, iters):
     """HipKMeansAlgorithm.run() with the default pair of kernels goes through kmx_iteration_f32: every iteration against
