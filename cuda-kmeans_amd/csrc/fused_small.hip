@@ -44,12 +44,13 @@ constexpr uint32_t FUSED_LATER_DRAIN = WAVE / 2;
 
 typedef float f32x4v __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 constexpr size_t FUSED_MAX_DATA_BYTES = 0xF0000000u; /* what one buffer descriptor spans, less room for a batch past the end */
 
 /* LDS words per wavefront of the matrix-ranking kernel: parked rows (or the sums at the end) and the membership rows */
 __host__ __device__ constexpr uint32_t fused_matrix_wave_floats(uint32_t nt, uint32_t mt)
 {
-	return (WAVE * (nt * 16 + 1) > mt * 16 * nt * 16 ? WAVE * (nt * 16 + 1) : mt * 16 * nt * 16) + WAVE * mt * 16;
+	return (WAVE * (nt * 16 + 2) > mt * 16 * nt * 16 ? WAVE * (nt * 16 + 2) : mt * 16 * nt * 16) + WAVE * mt * 16 / 2;
 }
 
 __host__ __device__ constexpr uint32_t fused_key_bits(uint32_t mt) { return mt == 1 ? 4u : 5u; } /* 16 centroids per MT */
@@ -370,8 +371,10 @@ fused_matrix_kernel(const float* __restrict__ data, size_t stride, const float* 
 	const float frame_m2 = frame[FRAME_DIMS], frame_norm = frame[FRAME_DIMS + 1];
 	constexpr uint32_t RS = DP + ROW_PAD;
 	constexpr int CH = (DP + 15) / 16;          /* chunks of 16 dimensions: one 16-byte piece per quad */
+	constexpr bool DEEP = CH == 1;              /* two batches of rows requested ahead (their pieces wait in registers) */
+	constexpr uint32_t AHEAD = DEEP ? 2 : 1;
 	constexpr int NT = CH;                      /* tiles of 16 dimensions of the sums */
-	constexpr uint32_t PARK = NT * 16 + 1;      /* a parked row: coordinates padded with zeros to whole tiles, then the result */
+	constexpr uint32_t PARK = NT * 16 + 2;      /* a parked row: coordinates padded with zeros to whole tiles; rows 8 apart start 16 banks apart */
 	constexpr uint32_t EX = DP + 1;             /* row stride of the exact centroid copy: odd, so that different rows start in different banks */
 	constexpr uint32_t SUM_ROWS = MT * 16, SUM_COLS = NT * 16;
 	constexpr uint32_t KEY = (1u << fused_key_bits(MT)) - 1u;
@@ -380,23 +383,31 @@ fused_matrix_kernel(const float* __restrict__ data, size_t stride, const float* 
 	__shared__ uint32_t flag_list[FUSED_WAVES][2 * FUSED_FLAG_CAP];
 	__shared__ uint32_t later_list[FUSED_WAVES][2 * FUSED_LATER_CAP];
 	__shared__ uint32_t members[32];
+	__shared__ __attribute__((aligned(16))) float start_norms[32]; /* what the ranking chains start from */
 	const uint32_t lane = threadIdx.x & (WAVE - 1);
 	const uint32_t wave = threadIdx.x / WAVE;
 	const uint32_t col = lane & 15, quad = lane >> 4;
-	const unsigned long long lanes_below = (1ull << lane) - 1ull;
+	/* how many of the lanes below this one are set in a mask */
+	auto below = [](unsigned long long mask) -> uint32_t {
+		return __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
+	};
 
-	/* LDS: [exact centroids k x EX][per wavefront: 64 parked rows, later its SUM_ROWS x SUM_COLS sums; 64 rows of SUM_ROWS
-	 * membership words: 1.0 at a point's cluster while its batch is summed, zeros otherwise] */
+	/* LDS: [exact centroids k x EX][per wavefront: 64 parked rows, later its SUM_ROWS x SUM_COLS sums; SUM_ROWS rows of 64
+	 * membership halfwords: bf16 1.0 at a point's place in its cluster's row while its batch is summed, zeros otherwise] */
 	constexpr uint32_t WAVE_FLOATS = fused_matrix_wave_floats(NT, MT);
 	float* exact = lds;
 	float* parked = exact + (size_t)k * EX + (size_t)wave * WAVE_FLOATS;
-	float* member_of = parked + WAVE * PARK;
+	unsigned short* member_of = (unsigned short*)(parked + (WAVE * PARK > SUM_ROWS * SUM_COLS ? WAVE * PARK : SUM_ROWS * SUM_COLS));
 	for (uint32_t i = threadIdx.x; i < k * EX; i += blockDim.x) {
 		const uint32_t j = i / EX, q = i - j * EX;
 		exact[i] = q < dim ? means_in[elem<LM>(stride_means, j, q)] : 0.0f;
 	}
 	for (uint32_t i = lane; i < WAVE_FLOATS; i += WAVE) parked[i] = 0.0f; /* the padding columns and the membership words stay zero */
-	if (threadIdx.x < 32) members[threadIdx.x] = 0u;
+	if (threadIdx.x < 32) {
+		members[threadIdx.x] = 0u;
+		/* rows past k never win: a large finite norm (an infinity would turn into a NaN under the key) */
+		start_norms[threadIdx.x] = threadIdx.x < k ? norms[threadIdx.x] : 3.0e38f;
+	}
 
 	uint32_t cmax = 0;
 	for (uint32_t j = threadIdx.x; j < k; j += blockDim.x) cmax = max(cmax, __float_as_uint(norms[norm_at(j)]));
@@ -407,10 +418,10 @@ fused_matrix_kernel(const float* __restrict__ data, size_t stride, const float* 
 	for (uint32_t w = 0; w < FUSED_WAVES; ++w) cmax = max(cmax, wave_max[w]);
 	const float c2max = __uint_as_float(cmax);
 
-	/* the operands that stay: this lane's pieces of centroid rows mt * 16 + col (A), of the frame, and the norms and the
-	 * numbers of centroids mt * 16 + 4 quad + 0..3 (the rows of D this lane holds). Rows past k never win: a large finite
-	 * norm (an infinity would turn into a NaN under the key). k <= 32: one tile of packed rows, RS floats apart. */
-	float ca[MT][CH][4], fr[CH][4], cn[MT][4];
+	/* the operands that stay: this lane's pieces of centroid rows mt * 16 + col (A) and of the frame, and the numbers of
+	 * centroids mt * 16 + 4 quad + 0..3 (the rows of D this lane holds; their norms are read from LDS where a chain
+	 * starts). k <= 32: one tile of packed rows, RS floats apart. */
+	float ca[MT][CH][4], fr[CH][4];
 	uint32_t key[MT][4];
 #pragma unroll
 	for (int j = 0; j < CH; ++j)
@@ -428,9 +439,7 @@ fused_matrix_kernel(const float* __restrict__ data, size_t stride, const float* 
 	for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
 		for (int i = 0; i < 4; ++i) {
-			const uint32_t r = mt * 16 + 4 * quad + i;
-			cn[mt][i] = r < k ? norms[r] : 3.0e38f;
-			key[mt][i] = r;
+			key[mt][i] = mt * 16 + 4 * quad + i;
 		}
 
 	uint32_t flagged = 0; /* wave-uniform */
@@ -447,13 +456,11 @@ fused_matrix_kernel(const float* __restrict__ data, size_t stride, const float* 
 	};
 
 	/* sums: MT x NT tiles of 16 clusters x 16 dimensions; this lane holds dimension col of clusters 4 quad + 0..3 of every tile */
-	f32x4v acc[2][MT][NT]; /* two sets, taken in turn: consecutive instructions do not wait for each other's result */
+	f32x4v acc[MT][NT];
 #pragma unroll
-	for (int half = 0; half < 2; ++half)
+	for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-		for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-			for (int nt = 0; nt < NT; ++nt) acc[half][mt][nt] = f32x4v{ 0.0f, 0.0f, 0.0f, 0.0f };
+		for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = f32x4v{ 0.0f, 0.0f, 0.0f, 0.0f };
 
 	/* one lane per point: the whole row (the points that are settled later, the points for the recheck queue) */
 	auto load_row = [&](float (&x)[DP], uint32_t pt, bool valid) {
@@ -471,35 +478,62 @@ fused_matrix_kernel(const float* __restrict__ data, size_t stride, const float* 
 		}
 	};
 
-	/* 3. the parked rows (row l: point l of the batch, zeros unless it is accumulated here): membership x coordinates on
-	 * the MFMA; both operands come straight from LDS */
+	/* 3. the parked rows (row l: point l of the batch, zeros unless it is accumulated here): membership x coordinates on the
+	 * bf16 matrix instruction (v_mfma_f32_16x16x32_bf16: 32 points per instruction, sixteen times the rate of the fp32 one,
+	 * and it runs beside the vector ALU, which the fp32 one does not). A coordinate is the exact sum of three bf16 values --
+	 * its upper 16 bits, the upper 16 bits of what that leaves, and the rest, at most 8 significant bits each -- and
+	 * 1.0 * part is exact, so the three products add up to the coordinate in the fp32 accumulator as 1.0 * x did; only the
+	 * order of the additions differs from the serial one (parts below 2^-126 are flushed by the instruction: far below
+	 * the tolerance of any sum). This lane feeds dimension col of points 32 blk + 8 quad + 0..7 (B) and their membership
+	 * of cluster col (A). */
 	auto add_parked = [&](uint32_t result) {
 		const bool counted = result != UNRESOLVED;
-		float* mine = member_of + (size_t)lane * SUM_ROWS + (counted ? result : 0u);
+		unsigned short* mine = member_of + (size_t)(counted ? result : 0u) * WAVE + lane;
 		if (counted) {
-			*mine = 1.0f;
+			*mine = 0x3F80u; /* bf16 1.0 */
 			atomicAdd(&members[result], 1u);
 		}
 		__builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
 		__builtin_amdgcn_wave_barrier();
-#pragma unroll 4
-		for (uint32_t s = 0; s < WAVE / 4; ++s) {
-			/* this lane feeds point 4 s + quad: its membership of cluster col (A) and its coordinate col (B) */
-			const float* row = parked + (size_t)(4 * s + quad) * PARK;
-			const float* in = member_of + (size_t)(4 * s + quad) * SUM_ROWS;
-			float b[NT];
 #pragma unroll
-			for (int nt = 0; nt < NT; ++nt) b[nt] = row[nt * 16 + col];
+		for (uint32_t blk = 0; blk < 2; ++blk) {
+			bf16x8 hi[NT], mid[NT], lo[NT];
+#pragma unroll
+			for (int nt = 0; nt < NT; ++nt) {
+				uint32_t ph[8], pm[8], pl[8];
+#pragma unroll
+				for (int i = 0; i < 8; ++i) {
+					const float v = parked[(size_t)(32 * blk + 8 * quad + i) * PARK + nt * 16 + col];
+					ph[i] = __float_as_uint(v) & 0xFFFF0000u;
+					const float r = v - __uint_as_float(ph[i]);
+					pm[i] = __float_as_uint(r) & 0xFFFF0000u;
+					pl[i] = __float_as_uint(r - __uint_as_float(pm[i]));
+				}
+				u32x4 wh, wm, wl; /* the upper halves of two words side by side: __builtin_amdgcn_perm(hi word, lo word, selector) */
+#pragma unroll
+				for (int i = 0; i < 4; ++i) {
+					wh[i] = __builtin_amdgcn_perm(ph[2 * i + 1], ph[2 * i], 0x07060302u);
+					wm[i] = __builtin_amdgcn_perm(pm[2 * i + 1], pm[2 * i], 0x07060302u);
+					wl[i] = __builtin_amdgcn_perm(pl[2 * i + 1], pl[2 * i], 0x07060302u);
+				}
+				hi[nt] = __builtin_bit_cast(bf16x8, wh);
+				mid[nt] = __builtin_bit_cast(bf16x8, wm);
+				lo[nt] = __builtin_bit_cast(bf16x8, wl);
+			}
 #pragma unroll
 			for (int mt = 0; mt < MT; ++mt) {
-				const float a = in[mt * 16 + col];
+				const bf16x8 in = *(const bf16x8*)(member_of + (size_t)(mt * 16 + col) * WAVE + 32 * blk + 8 * quad);
 #pragma unroll
-				for (int nt = 0; nt < NT; ++nt) acc[s & 1][mt][nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b[nt], acc[s & 1][mt][nt], 0, 0, 0);
+				for (int nt = 0; nt < NT; ++nt) {
+					acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(in, hi[nt], acc[mt][nt], 0, 0, 0);
+					acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(in, mid[nt], acc[mt][nt], 0, 0, 0);
+					acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(in, lo[nt], acc[mt][nt], 0, 0, 0);
+				}
 			}
 		}
 		__builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
 		__builtin_amdgcn_wave_barrier();
-		if (counted) *mine = 0.0f;
+		if (counted) *mine = 0u;
 	};
 
 	/* 2. the serial arithmetic on the two leaders of the points that wait for it (rows of the exact copy in LDS, one row per
@@ -584,12 +618,9 @@ fused_matrix_kernel(const float* __restrict__ data, size_t stride, const float* 
 			}
 		}
 	};
-	/* the rows of the batch after this one are on their way while this one is worked on: what a compute unit keeps in
-	 * flight, not its arithmetic, decides how much of the memory's bandwidth it sees */
-	uint32_t ahead[4][CH][4];
-	load_pieces(ahead, blockIdx.x, blockIdx.x >= batches);
 	const bool padded = dim < (uint32_t)DP; /* then the pieces hold words of other rows past `dim` */
-	for (uint32_t batch = blockIdx.x; batch < batches; batch += gridDim.x) {
+	/* one batch whose pieces have been requested into `ahead`; the same registers then take the batch two further on */
+	auto batch_step = [&](uint32_t (&ahead)[4][CH][4], uint32_t batch) {
 		if (waiting >= FUSED_LATER_DRAIN) settle_waiting(); /* before this batch's registers are live */
 		const uint32_t first = batch * batch_points + wave * WAVE;
 		float x[4][CH][4];
@@ -625,7 +656,7 @@ fused_matrix_kernel(const float* __restrict__ data, size_t stride, const float* 
 			for (int g = g0; g < g0 + 2; ++g) {
 				f32x4v d[MT];
 #pragma unroll
-				for (int mt = 0; mt < MT; ++mt) d[mt] = f32x4v{ cn[mt][0], cn[mt][1], cn[mt][2], cn[mt][3] };
+				for (int mt = 0; mt < MT; ++mt) d[mt] = *(const f32x4v*)(start_norms + mt * 16 + 4 * quad);
 				float sq = 0.0f;
 #pragma unroll
 				for (int j = 0; j < CH; ++j)
@@ -661,7 +692,6 @@ fused_matrix_kernel(const float* __restrict__ data, size_t stride, const float* 
 		else { rank_pair(std::false_type{}, 0); rank_pair(std::false_type{}, 2); }
 		swap_rows32(m1[0], m1[2]); swap_rows32(m2[0], m2[2]); swap_rows32(m3[0], m3[2]); swap_rows32(x2[0], x2[2]);
 		merge_triples(m1[0], m2[0], m3[0], m1[2], m2[2], m3[2]);
-		load_pieces(ahead, batch + gridDim.x, batch + gridDim.x >= batches); /* x is not read past this line */
 		const float best = m1[0], second = m2[0], third = m3[0];
 		const float xx = x2[0] + x2[2];
 
@@ -675,15 +705,23 @@ fused_matrix_kernel(const float* __restrict__ data, size_t stride, const float* 
 		const bool two = (third - best > tau) && covered;
 		const uint32_t result = decided ? i1 : UNRESOLVED;
 		if constexpr (EMIT) {
-			if (decided) assignment[pt] = result;
+			/* whole lines: the lanes without a result store UNRESOLVED, which the wavefront (settle_waiting) or the exact pass
+			 * overwrites later. Through a descriptor of the n results: the lanes past n aim past its end, where stores are
+			 * dropped. (The stores cost more than their 4 bytes per point: 0.284 against 0.249 ms at N = 16.7M, d = 16 -- the
+			 * compiler makes every wait for rows a wait for the store in flight as well; issuing it a step later, or as
+			 * assembly the compiler does not count, measured the same.) */
+			const __amdgpu_buffer_rsrc_t results = __builtin_amdgcn_make_buffer_rsrc(assignment, 0, n * 4u, 0x00020000);
+			__builtin_amdgcn_raw_buffer_store_b32(result, results, pt * 4u, 0, 0);
 		}
+		/* the next requests into the registers of this batch (x is not read past this line) */
+		load_pieces(ahead, batch + AHEAD * gridDim.x, batch + AHEAD * gridDim.x >= batches);
 
 		/* the points with two candidates wait for the arithmetic on those (what the list cannot take goes the way of the
 		 * points with three: the list has room for 32 more whenever a batch starts) */
 		bool later = valid && !decided && two;
 		const unsigned long long later_mask = __ballot(later);
 		if (later_mask) {
-			const uint32_t at = waiting + __builtin_popcountll(later_mask & lanes_below);
+			const uint32_t at = waiting + below(later_mask);
 			later = later && at < FUSED_LATER_CAP;
 			if (later) {
 				later_list[wave][2 * at] = pt;
@@ -697,7 +735,7 @@ fused_matrix_kernel(const float* __restrict__ data, size_t stride, const float* 
 			const uint32_t add = (uint32_t)__builtin_popcountll(flag_mask);
 			if (flagged + add > FUSED_FLAG_CAP) flush_flags();
 			if (flag) {
-				const uint32_t at = 2 * (flagged + __builtin_popcountll(flag_mask & lanes_below));
+				const uint32_t at = 2 * (flagged + below(flag_mask));
 				flag_list[wave][at] = pt;
 				/* the exact pass evaluates in the frame of the data (certificate.h); (x - m) . m only for these few points,
 				 * from their rows in memory */
@@ -715,6 +753,22 @@ fused_matrix_kernel(const float* __restrict__ data, size_t stride, const float* 
 			}
 		}
 		add_parked(result);
+	};
+	/* one batch, or with rows of up to 16 floats two, on their way while another is worked on: what a compute unit keeps in
+	 * flight, not its arithmetic, decides how much of the memory's bandwidth it sees */
+	if constexpr (DEEP) {
+		uint32_t even[4][CH][4], odd[4][CH][4];
+		load_pieces(even, blockIdx.x, blockIdx.x >= batches);
+		load_pieces(odd, blockIdx.x + gridDim.x, blockIdx.x + gridDim.x >= batches);
+		for (uint32_t batch = blockIdx.x; batch < batches; batch += 2 * gridDim.x) {
+			batch_step(even, batch);
+			if (batch + gridDim.x < batches) batch_step(odd, batch + gridDim.x);
+		}
+	}
+	else {
+		uint32_t ahead[4][CH][4];
+		load_pieces(ahead, blockIdx.x, blockIdx.x >= batches);
+		for (uint32_t batch = blockIdx.x; batch < batches; batch += gridDim.x) batch_step(ahead, batch);
 	}
 	while (waiting) settle_waiting();
 	if (flagged) flush_flags();
@@ -727,7 +781,7 @@ fused_matrix_kernel(const float* __restrict__ data, size_t stride, const float* 
 #pragma unroll
 		for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-			for (int r = 0; r < 4; ++r) parked[(size_t)(mt * 16 + 4 * quad + r) * SUM_COLS + nt * 16 + col] = acc[0][mt][nt][r] + acc[1][mt][nt][r];
+			for (int r = 0; r < 4; ++r) parked[(size_t)(mt * 16 + 4 * quad + r) * SUM_COLS + nt * 16 + col] = acc[mt][nt][r];
 	__syncthreads();
 	const float* sums = exact + (size_t)k * EX;
 	for (uint32_t e = threadIdx.x; e < k * dim; e += blockDim.x) {
@@ -795,7 +849,7 @@ static int launch_fused_t(const AssignArgs& a, float* means_out, uint32_t* sizes
 	const uint32_t mt = a.k <= 16 ? 1 : 2;
 	const uint32_t wave_floats = std::max<uint32_t>(WAVE * (NT * 16 + 1), mt * 16 * NT * 16);
 	const uint32_t lds_bytes = (a.k * (DP + 1) + FUSED_WAVES * (fused_matrix_rows(DP) ? fused_matrix_wave_floats(NT, mt) : wave_floats)) * 4;
-	const uint32_t static_bytes = (2 * (FUSED_FLAG_CAP + FUSED_LATER_CAP) * FUSED_WAVES + 128) * 4;
+	const uint32_t static_bytes = (2 * (FUSED_FLAG_CAP + FUSED_LATER_CAP) * FUSED_WAVES + 128 + 32) * 4;
 	if (lds_bytes + static_bytes > dev.lds_bytes) return fail(KMX_ERR_UNSUPPORTED, "fused iteration: %u bytes of LDS needed", lds_bytes + static_bytes);
 	void (*kernel)(const float*, size_t, const float*, const float*, const float*, size_t, float*, uint32_t*, uint32_t*, uint32_t*,
 	               uint32_t, uint32_t, uint32_t, float, uint32_t, float, uint32_t*, uint32_t) = nullptr;
