@@ -145,3 +145,32 @@ def test_gap_sweep_with_coordinates_of_very_different_exponents(km, orc, gpu, di
         bad = np.nonzero(got != want)[0]
         assert bad.size == 0, "variant %d: %d of %d points differ (first %s), %d went to the exact pass" % (v, bad.size, n, bad[:5], rechecked)
     d.free()
+
+
+@pytest.mark.parametrize("dim,k", [(16, 16), (32, 32), (8, 20), (4, 16), (24, 9), (16, 3)])
+@pytest.mark.parametrize("offset", [0.0, 1e2, 1e4])
+def test_gap_sweep_through_the_single_pass_iteration(km, orc, gpu, dim, k, offset):
+    """The gap sweep (points next to bisectors, true gaps log-uniform over 1e-9..1e-3 on both sides of every tau) through
+    kmx_iteration_f32 where it reads the points once: the ranking values of those kernels carry the centroid's number in
+    their low bits (csrc/certificate.h: cert_kd_keyed), the rows of 8, 16 and 32 floats rank on v_mfma_f32_16x16x4_f32.
+    The assignment is the serial scan's, the counts are exact."""
+    n, chunk = 1 << 19, 1 << 16
+    rng = np.random.default_rng(int(dim * 11 + k + offset))
+    _, c = near_ties(dim, 1, k, rng, offset)
+    data = np.empty((n, dim), np.float32)
+    for first in range(0, n, chunk):
+        data[first:first + chunk], _ = near_ties(dim, chunk, k, rng, offset, centroids=c)
+    means = np.ascontiguousarray(c).ravel()
+    want = orc.assign(data.ravel(), means, dim, k, n, threads=0, fast=True)
+    d = km.DeviceBuffer(data.nbytes); d.write(data.ravel())
+    m = km.DeviceBuffer(means.nbytes); m.write(means)
+    out = km.DeviceBuffer(means.nbytes); a = km.DeviceBuffer(4 * n); sizes = km.DeviceBuffer(4 * k)
+    km.iteration(d, 0, dim, m, out, 0, dim, a, sizes, dim, k, n)
+    km.sync()
+    assert km.last_iteration_passes() == 1
+    got = a.read(np.uint32, n)
+    bad = np.nonzero(got != want)[0]
+    assert bad.size == 0, "%d of %d points differ (first %s)" % (bad.size, n, bad[:5])
+    assert np.array_equal(sizes.read(np.uint32, k), np.bincount(want, minlength=k))
+    for b in (d, m, out, a, sizes):
+        b.free()
