@@ -3,7 +3,9 @@
  * floats): the shapes where the iteration is bound by HBM and reading the points twice (assignment, then
  * update) costs the most. Role of the reference's fused kernels (kernels.cu:883-1190).
  *
- * One lane owns one point, its coordinates in registers.
+ * Two kernels, by the width of the rows (launch_fused_t): fused_small_kernel, one lane per point, for rows of 4 and 24
+ * floats, and fused_matrix_kernel (described where it stands), which ranks on the matrix cores, for rows of 8, 16 and 32.
+ * fused_small_kernel: one lane owns one point, its coordinates in registers.
  *   1. Ranking a[j] = |c_j|^2 - 2 c_j.x with plain fused multiply-adds; the packed centroid rows are read with
  *      wave-uniform addresses (scalar loads, scalar operands). The low bits of a value's
  *      mantissa are replaced by the centroid's number, so the lane tracks its three smallest values with one
@@ -25,8 +27,8 @@
  *      LDS atomics. At the end the four wavefronts' accumulators meet in LDS: one global atomic per element and
  *      work-group.
  *
- * Floating-point contraction is off for the whole file (the serial arithmetic must not fuse); the ranking uses
- * explicit fused multiply-adds.
+ * Floating-point contraction is off for the whole file (the serial arithmetic must not fuse); the rankings use
+ * explicit fused multiply-adds and matrix instructions.
  */
 #include <type_traits>
 #include "certificate.h"
