@@ -709,9 +709,10 @@ fused_matrix_kernel(const float* __restrict__ data, size_t stride, const float* 
 		if constexpr (EMIT) {
 			/* whole lines: the lanes without a result store UNRESOLVED, which the wavefront (settle_waiting) or the exact pass
 			 * overwrites later. Through a descriptor of the n results: the lanes past n aim past its end, where stores are
-			 * dropped. (The stores cost more than their 4 bytes per point: 0.284 against 0.249 ms at N = 16.7M, d = 16 -- the
-			 * compiler makes every wait for rows a wait for the store in flight as well; issuing it a step later, or as
-			 * assembly the compiler does not count, measured the same.) */
+			 * dropped. (The kernel with the output costs more than the output's 4 bytes per point: 0.284 against 0.249 ms at
+			 * N = 16.7M, d = 16, of which 0.011 ms go when the stores are switched off at run time. The waits are not the
+			 * reason: as compiled, every wait for rows is a wait for all that is in flight, the store included, and a loop
+			 * laid out so that the waits count the requests exactly measured the same with and without the output.) */
 			const __amdgpu_buffer_rsrc_t results = __builtin_amdgcn_make_buffer_rsrc(assignment, 0, n * 4u, 0x00020000);
 			__builtin_amdgcn_raw_buffer_store_b32(result, results, pt * 4u, 0, 0);
 		}
