@@ -1351,7 +1351,14 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 	 * work-group has to arrive at the barrier of every chunk, so all of them sweep the same number of times.
 	 */
 	const uint32_t my_units = blockIdx.x < units ? (units - blockIdx.x + gridDim.x - 1) / gridDim.x : 0u;
-	const uint32_t items = STREAM ? my_units : my_units * MFMA_WAVES;
+	/* The listed points of a second level are few units per work-group (14 % of N = 2M points: 567 units for 256
+	 * work-groups, three for some and two for the others): there the work-groups share the ITEMS evenly, a contiguous
+	 * range each (N = 2M, d = 32, k = 1024: 0.077 -> 0.072 ms). */
+	constexpr bool EVEN_ITEMS = LISTED && !STREAM;
+	const uint32_t all_items = (n + P * TILE - 1) / (P * TILE);
+	const uint32_t item0 = (uint32_t)((uint64_t)blockIdx.x * all_items / gridDim.x);
+	const uint32_t item1 = (uint32_t)((uint64_t)(blockIdx.x + 1) * all_items / gridDim.x);
+	const uint32_t items = EVEN_ITEMS ? item1 - item0 : STREAM ? my_units : my_units * MFMA_WAVES;
 	uint32_t static_item = 0;
 	auto claim = [&]() -> uint32_t {
 		if (STREAM) return static_item++;
@@ -1362,6 +1369,7 @@ assign_bf16_kernel(const float* __restrict__ data, size_t stride, const float* _
 	auto uniform = [&](uint32_t v) -> uint32_t { return STREAM ? v : (uint32_t)__builtin_amdgcn_readfirstlane((int)v); };
 	/* first point of an item: unit blockIdx.x + (item / 8) gridDim.x, slice item % 8 (streamed: the wavefront's own slice of unit `item`) */
 	auto first_point = [&](uint32_t item) -> uint32_t {
+		if (EVEN_ITEMS) return (item0 + item) * P * TILE;
 		const uint32_t unit = blockIdx.x + (STREAM ? item : item / MFMA_WAVES) * gridDim.x;
 		const uint32_t slice = STREAM ? wave : item % MFMA_WAVES;
 		return (unit * MFMA_WAVES + slice) * P * TILE;
