@@ -709,10 +709,14 @@ fused_matrix_kernel(const float* __restrict__ data, size_t stride, const float* 
 		if constexpr (EMIT) {
 			/* whole lines: the lanes without a result store UNRESOLVED, which the wavefront (settle_waiting) or the exact pass
 			 * overwrites later. Through a descriptor of the n results: the lanes past n aim past its end, where stores are
-			 * dropped. (The kernel with the output costs more than the output's 4 bytes per point: 0.284 against 0.249 ms at
-			 * N = 16.7M, d = 16, of which 0.011 ms go when the stores are switched off at run time. The waits are not the
-			 * reason: as compiled, every wait for rows is a wait for all that is in flight, the store included, and a loop
-			 * laid out so that the waits count the requests exactly measured the same with and without the output.) */
+			 * dropped. (What the output costs is the stores themselves, not the code around them: N = 16.7M, d = 16, one
+			 * GPU, the kernel compiled with the output and the stores replaced by statements that only keep their operands
+			 * alive: 0.249 ms as without the output; these stores alone 0.276 ms; those of settle_waiting alone 0.272 ms;
+			 * both 0.285 ms. 64 MB written next to 1.07 GB read cost as much as 110 MB of reads -- a copy runs at three
+			 * quarters of the bandwidth of a read on this memory as well -- and the results of the points settled later,
+			 * 5 % of all, as much again when they stand alone: a word stored into a line that has left the caches makes the
+			 * memory read and write the line. Holding the lines back in LDS until their last point is settled takes those
+			 * away (0.278 ms) but costs 3 to 10 % on data with few or very many such points, and was dropped.) */
 			const __amdgpu_buffer_rsrc_t results = __builtin_amdgcn_make_buffer_rsrc(assignment, 0, n * 4u, 0x00020000);
 			__builtin_amdgcn_raw_buffer_store_b32(result, results, pt * 4u, 0, 0);
 		}
